@@ -1,0 +1,193 @@
+/*
+ * kten_hip.h — C ABI of libkten_hip.so, the MI355X (gfx950) device side of a kten
+ * backend. The Kotlin `HipRawTensor` / `HipTensorOperations` classes (or any FFI host:
+ * Panama FFM, JNI, ctypes) bind exactly these entry points; each one names the member of
+ * the reference's backend contract it serves. Reference paths are relative to the
+ * reference root:
+ *
+ *   RAW = kten-api/src/main/kotlin/eu/redbean/kten/api/tensor/store/AbstractRawTensor.kt
+ *   OPS = kten-api/src/main/kotlin/eu/redbean/kten/api/tensor/operations/TensorOperations.kt
+ *   JVM = backend/kten-jvm/src/main/kotlin/eu/redbean/kten/jvm/tensor/store/JVMRawTensor.kt
+ *   OCL = backend/kten-opencl/src/main/kotlin/eu/redbean/kten/opencl/tensor
+ *
+ * Conventions
+ *   - Every call returns 0 (KTH_OK) or a negative KTH_E_* code; kth_last_error() gives
+ *     the calling thread's message for the last failure. No exception crosses the ABI.
+ *   - A buffer handle is an opaque uint64_t naming a device-resident fp32 store. All
+ *     data is fp32, row-major contiguous; shapes are int32 with at most KTH_MAX_DIMS
+ *     dims (OCL/platform/kernels/OCLKernelConstant.kt:4) and fewer than 2^31 elements
+ *     (kten-api/.../autograd/utils/ShapeFunctions.kt:344).
+ *   - Shapes travel by value inside the kernel arguments; nothing is uploaded per launch.
+ *   - All launches are asynchronous on one internal in-order stream. The only blocking
+ *     calls are kth_upload, kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
+ *     kth_timer_end and kth_shutdown.
+ *   - Shape / argument errors are reported before anything is launched, as the
+ *     reference throws IllegalArgumentException host-side before computing
+ *     (JVM:89-93, ShapeFunctions.kt:187-201).
+ *   - Calls are serialised by one internal mutex; the reference is single-threaded by
+ *     convention (kten-api/.../tensor/platform/PlatformProvider.kt:42-46).
+ */
+#ifndef KTEN_HIP_H
+#define KTEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KTH_MAX_DIMS 10
+
+/* status codes */
+#define KTH_OK            0
+#define KTH_E_NOT_INIT   -1   /* kth_init has not succeeded */
+#define KTH_E_HANDLE     -2   /* unknown, stale or released handle */
+#define KTH_E_ARGUMENT   -3   /* bad op code, size, range, dims > KTH_MAX_DIMS, null pointer */
+#define KTH_E_SHAPE      -4   /* shapes do not broadcast / do not match */
+#define KTH_E_MEMORY     -5   /* device allocation failed or pool cap exceeded */
+#define KTH_E_DEVICE     -6   /* a HIP runtime call failed */
+
+/* Operation codes. Numbering follows OCL/platform/kernels/OCLKernelConstant.kt:5-43 so a
+ * Kotlin host can reuse that enum; KTH_NEG (unaryMinus, RAW:51) has no OpenCL code. */
+enum kth_op {
+    KTH_PLUS = 0, KTH_MINUS = 1, KTH_TIMES = 2, KTH_DIV = 3, KTH_POW = 4,
+    KTH_RECIPROCAL = 5, KTH_LOG = 6,
+    KTH_SUM = 7, KTH_MEAN = 8, KTH_MAX = 9, KTH_MIN = 10, KTH_ARG_MAX = 11, KTH_ARG_MIN = 12,
+    KTH_LT = 13, KTH_LTE = 14, KTH_GT = 15, KTH_GTE = 16, KTH_EQ = 17, KTH_NEQ = 18,
+    KTH_EXP = 19, KTH_TANH = 20, KTH_SIGMOID = 21, KTH_SINH = 22, KTH_COSH = 23, KTH_ABS = 24,
+    KTH_SIGN = 25, KTH_SQRT = 26, KTH_SIN = 27, KTH_COS = 28, KTH_TAN = 29, KTH_ASIN = 30,
+    KTH_ACOS = 31, KTH_ATAN = 32, KTH_FLOOR = 33, KTH_CEIL = 34, KTH_ROUND = 35, KTH_TRUNC = 36,
+    KTH_RSQRT = 37,
+    KTH_NEG = 40
+};
+
+/* ------------------------------------------------------------------ platform bring-up */
+
+/* Select the device, create the stream and the buffer pool. Idempotent for the same
+ * device. Serves the PlatformInitializer of a backend
+ * (OCL/platform/OCLPlatformInitializer.kt:20-41, OCL/platform/OCLEnvironment.kt:203-300). */
+int kth_init(int device);
+
+/* Drain the stream and free every device buffer, live or pooled. */
+int kth_shutdown(void);
+
+/* Message for the calling thread's last failed call ("" if none). */
+const char* kth_last_error(void);
+
+/* Device name, total memory, compute-unit count and wavefront width: the fields a
+ * backend puts into PlatformInfo (kten-api/.../tensor/platform/PlatformInfo.kt:3-9). */
+int kth_device_info(char* name, size_t cap, uint64_t* total_mem, int* compute_units, int* wave_size);
+
+/* PlatformProvider.epsilon (PlatformProvider.kt:12), used by EQ/NEQ as |a-b| < eps
+ * (JVM:371-377,387-393). Default 1e-7f. */
+int kth_set_epsilon(float eps);
+
+/* PlatformProvider.memoryUsageScaleHint (PlatformProvider.kt:23-29): fraction of device
+ * memory that live + pooled buffers may occupy; pooled buffers are freed first, then
+ * kth_alloc fails with KTH_E_MEMORY. Default 0.85. */
+int kth_set_memory_scale_hint(double fraction);
+
+/* ------------------------------------------------------------------ stores */
+
+/* A store of n_floats fp32 values (contents undefined), reference count 1. Buffers
+ * come from a size-keyed reuse pool, the role of OCLEnvironment's reuse pool
+ * (OCL/platform/OCLEnvironment.kt:36-200). Serves createRaw(shape) (OPS:16). */
+int kth_alloc(uint64_t n_floats, uint64_t* handle);
+
+/* incrementRef (OPS:28) and the store-sharing of copy(shallow=true) / view
+ * (OCL/store/OCLRawTensor.kt:252-263). */
+int kth_retain(uint64_t handle);
+
+/* release (OPS:22): at zero the buffer returns to the pool (OCL/store/OCLRawTensor.kt:37-48). */
+int kth_release(uint64_t handle);
+
+/* Host -> device. Serves createRaw(shape, init) (OPS:11), fromCommonSerializable
+ * (OPS:135) and the JVM -> device platform transformer. Blocking. */
+int kth_upload(uint64_t handle, uint64_t offset, const float* src, uint64_t n);
+
+/* Device -> host after draining the stream. Serves toSerializableData (OPS:133) and
+ * the device -> JVM platform transformer. */
+int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n);
+
+/* getSingleValue (RAW:166) / Tensor.item(). Blocking. */
+int kth_read_scalar(uint64_t handle, uint64_t index, float* out);
+
+/* copy(shallow=false) (RAW:168, JVM:257-262) and contiguous slice moves. */
+int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n);
+
+/* inplaceFill (RAW:244), zerosLike / zeroOut (OPS:24-26), createRawFill (OPS:18-20),
+ * set(range, Float) on a contiguous range (RAW:35-37). */
+int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value);
+
+/* containsNan (RAW:240, JVM:520-522). Blocking. */
+int kth_contains_nan(uint64_t handle, uint64_t n, int* out);
+
+/* ------------------------------------------------------------------ elementwise */
+
+/* plus/minus/times/div/pow(tensor) (RAW:39,47,53,61,67; JVM:81-87,110-138) with the
+ * broadcast fused into the kernel, and lt..neq(tensor) (RAW:194-199; JVM:355-377).
+ * oshape must be the common shape of RAW:170-192; each operand must broadcast to it by
+ * the rule of ShapeFunctions.kt:187-201 (else KTH_E_SHAPE). `out` must not alias an
+ * operand unless all three shapes are equal. op: KTH_PLUS..KTH_POW, KTH_LT..KTH_NEQ. */
+int kth_binary(int op,
+               uint64_t a, const int32_t* ashape, int adims,
+               uint64_t b, const int32_t* bshape, int bdims,
+               uint64_t out, const int32_t* oshape, int odims);
+
+/* plusAssign / timesAssign(tensor) (RAW:43,55; JVM:89-97,114,126): a[i] = a[i] op b[i]
+ * on equal shapes (the host checks shape equality and throws, JVM:90-93). */
+int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n);
+
+/* plus/minus/times/div/pow(Float) (RAW:41,49,57,63,69; JVM:99-103,112-140) and
+ * lt..neq(Float) (RAW:201-206; JVM:379-393): out[i] = a[i] op c. reverse != 0 computes
+ * c op a[i]; the contract needs it for TensorOperations.pow(constant, raw) (OPS:39).
+ * out == a is allowed and gives plusAssign/timesAssign/divAssign(Float)
+ * (RAW:45,59,65; JVM:105-108,116,130,136). */
+int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t n);
+
+/* unaryMinus, reciprocal, log (RAW:51,71,73; JVM:122,142,144) and exp..rsqrt
+ * (RAW:208-227; JVM:395-435). op: KTH_NEG, KTH_RECIPROCAL, KTH_LOG, KTH_EXP..KTH_RSQRT.
+ * out == a is allowed. */
+int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n);
+
+/* clamp (RAW:215; JVM:409-411): min(max(x, lo), hi) with java.lang.Math NaN rules. */
+int kth_clamp(uint64_t a, uint64_t out, uint64_t n, float lo, float hi);
+
+/* broadcastTo (RAW:25; JVM:51-73): materialise src at dshape. The host returns `this`
+ * without calling when the shapes are equal (JVM:52-53). */
+int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
+                     uint64_t dst, const int32_t* dshape, int ddims);
+
+/* ------------------------------------------------------------------ reductions */
+
+/* aggregateOverAxis (RAW:75,92-119; JVM:154-225) on a tensor seen as
+ * [outer, axis, inner] -> [outer, 1, inner]. op: KTH_SUM, KTH_MEAN, KTH_MAX, KTH_MIN,
+ * KTH_ARG_MAX, KTH_ARG_MIN (indices stored as float, JVM:180; axis must be <= 2^24).
+ * Deterministic: the same input gives the same bits on every call. */
+int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner);
+
+/* sum() / mean() (RAW:121-122; JVM:146-152) of n values into out[0]. op: KTH_SUM, KTH_MEAN. */
+int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
+
+/* ------------------------------------------------------------------ control and metrics */
+
+/* Wait for everything launched so far. */
+int kth_sync(void);
+
+/* PlatformMetricsProvider.getMetrics (kten-api/.../operations/PlatformMetricsProvider.kt:3-6,
+ * OCL/platform/OCLEnvironment.kt:89-96): bytes in live stores, bytes parked in the pool,
+ * kernel launches so far, and the algorithmic bytes those launches moved (operands at
+ * their un-broadcast size plus the output, 4 bytes each). Any pointer may be NULL. */
+int kth_metrics(uint64_t* live_bytes, uint64_t* pool_bytes, uint64_t* launches, uint64_t* bytes_moved);
+
+/* Device-side stopwatch on the internal stream (a HIP event pair), for benchmarks that
+ * must time the stream the kernels run on. No counterpart in the reference, which has
+ * no timing facility. kth_timer_end blocks until the second event completes. */
+int kth_timer_begin(void);
+int kth_timer_end(float* milliseconds);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KTEN_HIP_H */

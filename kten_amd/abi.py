@@ -1,0 +1,101 @@
+"""ctypes binding of libkten_hip.so: the same entry points a Kotlin host would bind.
+
+Every function of include/kten_hip.h is declared here with its C signature; `check`
+turns a negative status into the Python exception that corresponds to what the
+reference throws for that class of error (IllegalArgumentException -> ValueError,
+IllegalStateException / device failures -> RuntimeError).
+
+There is no CPU fallback: if the shared library is missing this module raises.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_size_t, c_uint64
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libkten_hip.so")
+
+KTH_MAX_DIMS = 10
+KTH_OK, KTH_E_NOT_INIT, KTH_E_HANDLE, KTH_E_ARGUMENT, KTH_E_SHAPE, KTH_E_MEMORY, KTH_E_DEVICE = 0, -1, -2, -3, -4, -5, -6
+
+
+class Op:
+    """Operation codes (OCLKernelConstant.kt:5-43 numbering, plus NEG)."""
+    PLUS, MINUS, TIMES, DIV, POW, RECIPROCAL, LOG = 0, 1, 2, 3, 4, 5, 6
+    SUM, MEAN, MAX, MIN, ARG_MAX, ARG_MIN = 7, 8, 9, 10, 11, 12
+    LT, LTE, GT, GTE, EQ, NEQ = 13, 14, 15, 16, 17, 18
+    EXP, TANH, SIGMOID, SINH, COSH, ABS, SIGN, SQRT = 19, 20, 21, 22, 23, 24, 25, 26
+    SIN, COS, TAN, ASIN, ACOS, ATAN, FLOOR, CEIL, ROUND, TRUNC, RSQRT = 27, 28, 29, 30, 31, 32, 33, 34, 35, 36, 37
+    NEG = 40
+
+
+# name -> (restype, argtypes): exactly the declarations of include/kten_hip.h
+SIGNATURES = {
+    "kth_init": (c_int, [c_int]),
+    "kth_shutdown": (c_int, []),
+    "kth_last_error": (c_char_p, []),
+    "kth_device_info": (c_int, [ctypes.c_char_p, c_size_t, POINTER(c_uint64), POINTER(c_int), POINTER(c_int)]),
+    "kth_set_epsilon": (c_int, [c_float]),
+    "kth_set_memory_scale_hint": (c_int, [c_double]),
+    "kth_alloc": (c_int, [c_uint64, POINTER(c_uint64)]),
+    "kth_retain": (c_int, [c_uint64]),
+    "kth_release": (c_int, [c_uint64]),
+    "kth_upload": (c_int, [c_uint64, c_uint64, ctypes.c_void_p, c_uint64]),
+    "kth_download": (c_int, [ctypes.c_void_p, c_uint64, c_uint64, c_uint64]),
+    "kth_read_scalar": (c_int, [c_uint64, c_uint64, POINTER(c_float)]),
+    "kth_copy": (c_int, [c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
+    "kth_fill": (c_int, [c_uint64, c_uint64, c_uint64, c_float]),
+    "kth_contains_nan": (c_int, [c_uint64, c_uint64, POINTER(c_int)]),
+    "kth_binary": (c_int, [c_int, c_uint64, POINTER(c_int32), c_int, c_uint64, POINTER(c_int32), c_int,
+                           c_uint64, POINTER(c_int32), c_int]),
+    "kth_binary_inplace": (c_int, [c_int, c_uint64, c_uint64, c_uint64]),
+    "kth_scalar": (c_int, [c_int, c_uint64, c_float, c_int, c_uint64, c_uint64]),
+    "kth_unary": (c_int, [c_int, c_uint64, c_uint64, c_uint64]),
+    "kth_clamp": (c_int, [c_uint64, c_uint64, c_uint64, c_float, c_float]),
+    "kth_broadcast_to": (c_int, [c_uint64, POINTER(c_int32), c_int, c_uint64, POINTER(c_int32), c_int]),
+    "kth_reduce_axis": (c_int, [c_int, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
+    "kth_reduce_all": (c_int, [c_int, c_uint64, c_uint64, c_uint64]),
+    "kth_sync": (c_int, []),
+    "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
+    "kth_timer_begin": (c_int, []),
+    "kth_timer_end": (c_int, [POINTER(c_float)]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads libkten_hip.so (once) and declares every entry point. Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `make -C kten_amd/csrc`. There is no CPU fallback for the HIP backend.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError here means the .so is stale
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return load().kth_last_error().decode("utf-8", "replace")
+
+
+def check(status):
+    """Maps a status code to the exception class the reference would throw."""
+    if status == KTH_OK:
+        return
+    msg = last_error()
+    if status in (KTH_E_ARGUMENT, KTH_E_SHAPE):
+        raise ValueError(msg)              # IllegalArgumentException
+    if status == KTH_E_MEMORY:
+        raise MemoryError(msg)
+    raise RuntimeError(f"[kth status {status}] {msg}")   # IllegalStateException / device error
+
+
+def shape_array(shape):
+    return (c_int32 * max(len(shape), 1))(*shape)

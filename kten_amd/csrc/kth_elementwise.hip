@@ -1,0 +1,591 @@
+// Elementwise kernels: unary maps, tensor-scalar maps, same-shape and broadcast binary
+// ops, fill, materialised broadcast, NaN scan. All are HBM-streaming kernels: every
+// thread moves float4s, loads of a tile are issued before any arithmetic, and a
+// workgroup of 256 threads (4 wave64s) covers a contiguous 16 KiB span per operand.
+#include "kth_internal.h"
+#include "kth_ops.h"
+
+using namespace kth;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;                       // float4s per thread
+constexpr uint32_t kTile = kBlock * kUnroll;     // float4s per workgroup
+
+__device__ __forceinline__ float4 ld4(const float* p, uint32_t i4) {
+    return reinterpret_cast<const float4*>(p)[i4];
+}
+__device__ __forceinline__ void st4(float* p, uint32_t i4, float4 v) {
+    reinterpret_cast<float4*>(p)[i4] = v;
+}
+
+// ---------------------------------------------------------------- contiguous maps
+
+// out[i] = Op(a[i], p, q). out may alias a.
+template <class Op>
+__global__ __launch_bounds__(kBlock) void unary_kernel(const float* a, float* out, uint32_t n, float p, float q) {
+    const uint32_t n4 = n >> 2;
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+    float4 v[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) v[k] = ld4(a, i);
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            r.x = Op::apply(v[k].x, p, q); r.y = Op::apply(v[k].y, p, q);
+            r.z = Op::apply(v[k].z, p, q); r.w = Op::apply(v[k].w, p, q);
+            st4(out, i, r);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        uint32_t i = (n4 << 2) + threadIdx.x;
+        out[i] = Op::apply(a[i], p, q);
+    }
+}
+
+// out[i] = REV ? Op(c, a[i]) : Op(a[i], c). out may alias a.
+template <class Op, bool REV>
+__global__ __launch_bounds__(kBlock) void scalar_kernel(const float* a, float* out, uint32_t n, float c, float eps) {
+    const uint32_t n4 = n >> 2;
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+    float4 v[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) v[k] = ld4(a, i);
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            if (REV) {
+                r.x = Op::apply(c, v[k].x, eps); r.y = Op::apply(c, v[k].y, eps);
+                r.z = Op::apply(c, v[k].z, eps); r.w = Op::apply(c, v[k].w, eps);
+            } else {
+                r.x = Op::apply(v[k].x, c, eps); r.y = Op::apply(v[k].y, c, eps);
+                r.z = Op::apply(v[k].z, c, eps); r.w = Op::apply(v[k].w, c, eps);
+            }
+            st4(out, i, r);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        uint32_t i = (n4 << 2) + threadIdx.x;
+        out[i] = REV ? Op::apply(c, a[i], eps) : Op::apply(a[i], c, eps);
+    }
+}
+
+// out[i] = Op(a[i], b[i]). out may alias a or b.
+template <class Op>
+__global__ __launch_bounds__(kBlock) void binary_same_kernel(const float* a, const float* b, float* out, uint32_t n, float eps) {
+    const uint32_t n4 = n >> 2;
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+    float4 va[kUnroll], vb[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) { va[k] = ld4(a, i); vb[k] = ld4(b, i); }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            r.x = Op::apply(va[k].x, vb[k].x, eps); r.y = Op::apply(va[k].y, vb[k].y, eps);
+            r.z = Op::apply(va[k].z, vb[k].z, eps); r.w = Op::apply(va[k].w, vb[k].w, eps);
+            st4(out, i, r);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        uint32_t i = (n4 << 2) + threadIdx.x;
+        out[i] = Op::apply(a[i], b[i], eps);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void fill_kernel(float* out, uint32_t n, float v) {
+    // `out` may start at any element offset, so the float4 body begins at the first
+    // 16-byte aligned element.
+    const uint32_t head = static_cast<uint32_t>((4u - ((reinterpret_cast<uintptr_t>(out) >> 2) & 3u)) & 3u);
+    const uint32_t h = head < n ? head : n;
+    float* body = out + h;
+    const uint32_t nb = n - h;
+    const uint32_t n4 = nb >> 2;
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+    const float4 v4 = make_float4(v, v, v, v);
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) st4(body, i, v4);
+    }
+    if (blockIdx.x == 0) {
+        if (threadIdx.x < h) out[threadIdx.x] = v;
+        if (threadIdx.x < (nb & 3u)) body[(n4 << 2) + threadIdx.x] = v;
+    }
+}
+
+// ---------------------------------------------------------------- broadcast
+
+// Division by a launch-constant divisor d for numerators below 2^31:
+// q = (mulhi(n, mul) + n) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
+struct FastDiv { uint32_t mul, shift; };
+
+// The broadcast plan travels by value in the kernel arguments. Dim 0 is the innermost
+// coalesced dim. For the vector kernels dim 0 is counted in float4s and an operand's
+// dim-0 stride is 4 (contiguous) or 0 (broadcast along it); all strides are in floats.
+struct BcastPlan {
+    int      ndim;
+    uint32_t size[KTH_MAX_DIMS];
+    FastDiv  div[KTH_MAX_DIMS];
+    uint32_t astride[KTH_MAX_DIMS];
+    uint32_t bstride[KTH_MAX_DIMS];
+};
+
+__device__ __forceinline__ void decompose(const BcastPlan& pl, uint32_t idx, uint32_t& aoff, uint32_t& boff) {
+    aoff = 0; boff = 0;
+    for (int d = 0; d < pl.ndim - 1; d++) {
+        uint32_t q = (__umulhi(idx, pl.div[d].mul) + idx) >> pl.div[d].shift;
+        uint32_t r = idx - q * pl.size[d];
+        aoff += r * pl.astride[d];
+        boff += r * pl.bstride[d];
+        idx = q;
+    }
+    aoff += idx * pl.astride[pl.ndim - 1];
+    boff += idx * pl.bstride[pl.ndim - 1];
+}
+
+template <bool VEC>
+__device__ __forceinline__ float4 ld_operand(const float* p, uint32_t off) {
+    if (VEC) return *reinterpret_cast<const float4*>(p + off);
+    float s = p[off];
+    return make_float4(s, s, s, s);
+}
+
+// out[o] = Op(a[map_a(o)], b[map_b(o)]) over n4 float4s of the output, innermost dim
+// a multiple of 4. AV / BV: the operand is contiguous along the innermost dim (float4
+// load) or broadcast along it (one scalar load per float4, served by L2).
+template <class Op, bool AV, bool BV>
+__global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                  float* __restrict__ out, uint32_t n4, float eps, BcastPlan pl) {
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+    float4 va[kUnroll], vb[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            uint32_t ao, bo;
+            decompose(pl, i, ao, bo);
+            va[k] = ld_operand<AV>(a, ao);
+            vb[k] = ld_operand<BV>(b, bo);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            r.x = Op::apply(va[k].x, vb[k].x, eps); r.y = Op::apply(va[k].y, vb[k].y, eps);
+            r.z = Op::apply(va[k].z, vb[k].z, eps); r.w = Op::apply(va[k].w, vb[k].w, eps);
+            st4(out, i, r);
+        }
+    }
+}
+
+// Any shapes: one output element per (thread, k); strides in floats, dim 0 in elements.
+template <class Op>
+__global__ __launch_bounds__(kBlock) void binary_bcast_scalar_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                     float* __restrict__ out, uint32_t n, float eps, BcastPlan pl) {
+    const uint32_t base = blockIdx.x * kTile + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < kUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n) {
+            uint32_t ao, bo;
+            decompose(pl, i, ao, bo);
+            out[i] = Op::apply(a[ao], b[bo], eps);
+        }
+    }
+}
+
+struct OpFirst { static __device__ __forceinline__ float apply(float a, float, float) { return a; } };
+
+// ---------------------------------------------------------------- NaN scan
+
+__global__ __launch_bounds__(kBlock) void contains_nan_kernel(const float* __restrict__ a, uint32_t n, int* flag) {
+    const uint32_t n4 = n >> 2;
+    int found = 0;
+    for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n4; i += gridDim.x * kBlock) {
+        float4 v = ld4(a, i);
+        found |= (v.x != v.x) | (v.y != v.y) | (v.z != v.z) | (v.w != v.w);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        float v = a[(n4 << 2) + threadIdx.x];
+        found |= (v != v);
+    }
+    // Every writer stores the same value, so plain stores need no atomics.
+    if (__syncthreads_or(found) && threadIdx.x == 0) *flag = 1;
+}
+
+__global__ void clear_flag_kernel(int* flag) { *flag = 0; }
+
+// ---------------------------------------------------------------- host side
+
+inline uint32_t blocks_for(uint64_t vec_count) {
+    uint64_t b = (vec_count + kTile - 1) / kTile;
+    return static_cast<uint32_t>(b == 0 ? 1 : b);
+}
+
+FastDiv make_div(uint32_t d) {
+    FastDiv f;
+    uint32_t shift = 0;
+    while ((1ull << shift) < d) shift++;
+    f.shift = shift;
+    f.mul = static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1);
+    return f;
+}
+
+// Builds the coalesced broadcast plan for out = a (op) b. Returns false when an operand
+// does not broadcast to oshape (ShapeFunctions.kt:187-201).
+// On return plan.size[0] is in elements; *vec_ok says whether the float4 kernels apply.
+bool build_plan(const int32_t* ashape, int adims, const int32_t* bshape, int bdims,
+                const int32_t* oshape, int odims, BcastPlan* plan, bool* vec_ok, bool* a_vec, bool* b_vec) {
+    if (adims > odims || bdims > odims) return false;
+    // Right-aligned, left-padded shapes and row-major strides with 0 on broadcast dims.
+    int64_t osz[KTH_MAX_DIMS], ast[KTH_MAX_DIMS], bst[KTH_MAX_DIMS];
+    int64_t arun = 1, brun = 1;
+    for (int d = odims - 1; d >= 0; d--) {
+        int ad = d - (odims - adims), bd = d - (odims - bdims);
+        int64_t as = ad >= 0 ? ashape[ad] : 1, bs = bd >= 0 ? bshape[bd] : 1, os = oshape[d];
+        if (!(as == os || as == 1) || !(bs == os || bs == 1)) return false;
+        osz[d] = os;
+        ast[d] = (as == 1 && os != 1) ? 0 : arun;
+        bst[d] = (bs == 1 && os != 1) ? 0 : brun;
+        arun *= as; brun *= bs;
+    }
+    // Innermost-first list without size-1 dims, then merge a dim into the one inside
+    // it when both operands step through them as through one longer dim.
+    int n = 0;
+    int64_t sz[KTH_MAX_DIMS], sa[KTH_MAX_DIMS], sb[KTH_MAX_DIMS];
+    for (int d = odims - 1; d >= 0; d--) {
+        if (osz[d] == 1) continue;
+        if (n > 0 && ast[d] == sa[n - 1] * sz[n - 1] && bst[d] == sb[n - 1] * sz[n - 1]) {
+            sz[n - 1] *= osz[d];
+        } else {
+            sz[n] = osz[d]; sa[n] = ast[d]; sb[n] = bst[d]; n++;
+        }
+    }
+    if (n == 0) { sz[0] = 1; sa[0] = 1; sb[0] = 1; n = 1; }
+    plan->ndim = n;
+    for (int d = 0; d < n; d++) {
+        plan->size[d] = static_cast<uint32_t>(sz[d]);
+        plan->astride[d] = static_cast<uint32_t>(sa[d]);
+        plan->bstride[d] = static_cast<uint32_t>(sb[d]);
+        plan->div[d] = make_div(plan->size[d]);
+    }
+    *a_vec = (sa[0] == 1);
+    *b_vec = (sb[0] == 1);
+    *vec_ok = (sz[0] % 4 == 0) && (sa[0] <= 1) && (sb[0] <= 1);
+    return true;
+}
+
+void to_vector_units(BcastPlan* plan) {
+    plan->size[0] /= 4;
+    plan->div[0] = make_div(plan->size[0]);
+    plan->astride[0] *= 4;
+    plan->bstride[0] *= 4;
+}
+
+int check_shape(const int32_t* shape, int dims, const char* what, uint64_t* count) {
+    if (dims < 0 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "%s: %d dims (max %d)", what, dims, KTH_MAX_DIMS);
+    if (dims > 0 && !shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
+    uint64_t n = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0) return fail(KTH_E_ARGUMENT, "%s: negative dim %d", what, shape[i]);
+        n *= static_cast<uint64_t>(shape[i]);
+        if (n > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: more than 2^31-1 elements", what);
+    }
+    *count = n;
+    return KTH_OK;
+}
+
+template <class Op>
+void launch_unary(const float* a, float* out, uint32_t n, float p, float q) {
+    hipLaunchKernelGGL((unary_kernel<Op>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, p, q);
+}
+
+template <class Op>
+void launch_scalar(bool rev, const float* a, float* out, uint32_t n, float c, float eps) {
+    if (rev) hipLaunchKernelGGL((scalar_kernel<Op, true>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
+    else     hipLaunchKernelGGL((scalar_kernel<Op, false>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
+}
+
+template <class Op>
+void launch_binary_same(const float* a, const float* b, float* out, uint32_t n, float eps) {
+    hipLaunchKernelGGL((binary_same_kernel<Op>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, b, out, n, eps);
+}
+
+template <class Op>
+void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n, float eps,
+                         BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec) {
+    hipStream_t st = state().stream;
+    if (vec_ok) {
+        to_vector_units(&plan);
+        uint32_t n4 = n >> 2;
+        dim3 grid(blocks_for(n4)), block(kBlock);
+        if (a_vec && b_vec)  hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, true, true>), grid, block, 0, st, a, b, out, n4, eps, plan);
+        else if (a_vec)      hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, true, false>), grid, block, 0, st, a, b, out, n4, eps, plan);
+        else if (b_vec)      hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n4, eps, plan);
+        else                 hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n4, eps, plan);
+    } else {
+        hipLaunchKernelGGL((binary_bcast_scalar_kernel<Op>), dim3(blocks_for(n)), dim3(kBlock), 0, st, a, b, out, n, eps, plan);
+    }
+}
+
+#define KTH_BINARY_DISPATCH(op, CALL)                          \
+    switch (op) {                                              \
+    case KTH_PLUS:  CALL(OpPlus);  break;                      \
+    case KTH_MINUS: CALL(OpMinus); break;                      \
+    case KTH_TIMES: CALL(OpTimes); break;                      \
+    case KTH_DIV:   CALL(OpDiv);   break;                      \
+    case KTH_POW:   CALL(OpPow);   break;                      \
+    case KTH_LT:    CALL(OpLt);    break;                      \
+    case KTH_LTE:   CALL(OpLte);   break;                      \
+    case KTH_GT:    CALL(OpGt);    break;                      \
+    case KTH_GTE:   CALL(OpGte);   break;                      \
+    case KTH_EQ:    CALL(OpEq);    break;                      \
+    case KTH_NEQ:   CALL(OpNeq);   break;                      \
+    default: break;                                            \
+    }
+
+bool is_binary_op(int op) {
+    return (op >= KTH_PLUS && op <= KTH_POW) || (op >= KTH_LT && op <= KTH_NEQ);
+}
+
+}  // namespace
+
+extern "C" {
+
+int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* st = lookup(handle, "kth_fill");
+    if (!st) return KTH_E_HANDLE;
+    if (offset > st->n_floats || n > st->n_floats - offset)
+        return fail(KTH_E_ARGUMENT, "kth_fill: range [%llu, +%llu) outside a store of %llu floats",
+                    (unsigned long long)offset, (unsigned long long)n, (unsigned long long)st->n_floats);
+    if (n == 0) return KTH_OK;
+    uint32_t n32 = static_cast<uint32_t>(n);
+    hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(n32 >> 2)), dim3(kBlock), 0, state().stream, st->ptr + offset, n32, value);
+    KTH_LAUNCH_CHECK("fill");
+    count_launch(n * 4);
+    return KTH_OK;
+}
+
+int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* sa = lookup(a, "kth_unary(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_unary(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (n > sa->n_floats || n > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_unary: n=%llu exceeds a store (%llu in, %llu out)", (unsigned long long)n,
+                    (unsigned long long)sa->n_floats, (unsigned long long)so->n_floats);
+    const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
+#define U(OP) if (n32) launch_unary<OP>(pa, po, n32, 0.0f, 0.0f)
+    switch (op) {
+    case KTH_NEG: U(OpNeg); break;           case KTH_RECIPROCAL: U(OpReciprocal); break;
+    case KTH_LOG: U(OpLog); break;           case KTH_EXP: U(OpExp); break;
+    case KTH_TANH: U(OpTanh); break;         case KTH_SIGMOID: U(OpSigmoid); break;
+    case KTH_SINH: U(OpSinh); break;         case KTH_COSH: U(OpCosh); break;
+    case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
+    case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSin); break;
+    case KTH_COS: U(OpCos); break;           case KTH_TAN: U(OpTan); break;
+    case KTH_ASIN: U(OpAsin); break;         case KTH_ACOS: U(OpAcos); break;
+    case KTH_ATAN: U(OpAtan); break;         case KTH_FLOOR: U(OpFloor); break;
+    case KTH_CEIL: U(OpCeil); break;         case KTH_ROUND: U(OpRound); break;
+    case KTH_TRUNC: U(OpTrunc); break;       case KTH_RSQRT: U(OpRsqrt); break;
+    default: return fail(KTH_E_ARGUMENT, "kth_unary: op %d is not a unary map", op);
+    }
+#undef U
+    if (n == 0) return KTH_OK;
+    KTH_LAUNCH_CHECK("unary");
+    count_launch(n * 8);
+    return KTH_OK;
+}
+
+int kth_clamp(uint64_t a, uint64_t out, uint64_t n, float lo, float hi) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* sa = lookup(a, "kth_clamp(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_clamp(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (n > sa->n_floats || n > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_clamp: n=%llu exceeds a store", (unsigned long long)n);
+    if (n == 0) return KTH_OK;
+    launch_unary<OpClamp>(sa->ptr, so->ptr, static_cast<uint32_t>(n), lo, hi);
+    KTH_LAUNCH_CHECK("clamp");
+    count_launch(n * 8);
+    return KTH_OK;
+}
+
+int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_scalar: op %d is not a binary op", op);
+    Store* sa = lookup(a, "kth_scalar(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_scalar(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (n > sa->n_floats || n > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_scalar: n=%llu exceeds a store", (unsigned long long)n);
+    if (n == 0) return KTH_OK;
+    const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
+    const float eps = state().epsilon;
+    const bool rev = reverse != 0;
+    // pow with an exponent whose f64 result is exact needs no transcendental:
+    // pow(x, 2) is the exact product x*x (48 bits fit a double), pow(x, 1) is x.
+    if (op == KTH_POW && !rev && c == 2.0f)      launch_unary<OpSquare>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == 1.0f) launch_unary<OpIdentity>(pa, po, n32, 0.0f, 0.0f);
+    else {
+#define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
+        KTH_BINARY_DISPATCH(op, S)
+#undef S
+    }
+    KTH_LAUNCH_CHECK("scalar");
+    count_launch(n * 8);
+    return KTH_OK;
+}
+
+int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_binary_inplace: op %d is not a binary op", op);
+    Store* sa = lookup(a, "kth_binary_inplace(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* sb = lookup(b, "kth_binary_inplace(b)");
+    if (!sb) return KTH_E_HANDLE;
+    if (n > sa->n_floats || n > sb->n_floats)
+        return fail(KTH_E_SHAPE, "kth_binary_inplace: n=%llu exceeds a store (%llu, %llu)", (unsigned long long)n,
+                    (unsigned long long)sa->n_floats, (unsigned long long)sb->n_floats);
+    if (n == 0) return KTH_OK;
+    float* pa = sa->ptr; const float* pb = sb->ptr; uint32_t n32 = static_cast<uint32_t>(n);
+    const float eps = state().epsilon;
+#define B(OP) launch_binary_same<OP>(pa, pb, pa, n32, eps)
+    KTH_BINARY_DISPATCH(op, B)
+#undef B
+    KTH_LAUNCH_CHECK("binary_inplace");
+    count_launch(n * 12);
+    return KTH_OK;
+}
+
+int kth_binary(int op,
+               uint64_t a, const int32_t* ashape, int adims,
+               uint64_t b, const int32_t* bshape, int bdims,
+               uint64_t out, const int32_t* oshape, int odims) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_binary: op %d is not a binary op", op);
+    uint64_t an, bn, on;
+    if (int rc = check_shape(ashape, adims, "kth_binary(a)", &an)) return rc;
+    if (int rc = check_shape(bshape, bdims, "kth_binary(b)", &bn)) return rc;
+    if (int rc = check_shape(oshape, odims, "kth_binary(out)", &on)) return rc;
+    Store* sa = lookup(a, "kth_binary(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* sb = lookup(b, "kth_binary(b)");
+    if (!sb) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_binary(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (an > sa->n_floats || bn > sb->n_floats || on > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_binary: a shape needs more elements than its store holds");
+    BcastPlan plan;
+    bool vec_ok, a_vec, b_vec;
+    if (!build_plan(ashape, adims, bshape, bdims, oshape, odims, &plan, &vec_ok, &a_vec, &b_vec))
+        return fail(KTH_E_SHAPE, "kth_binary: operand shapes do not broadcast to the output shape");
+    const bool all_same = (an == on && bn == on);
+    if (!all_same && (so->ptr == sa->ptr || so->ptr == sb->ptr))
+        return fail(KTH_E_ARGUMENT, "kth_binary: output aliases a broadcast operand");
+    if (on == 0) return KTH_OK;
+    const float* pa = sa->ptr; const float* pb = sb->ptr; float* po = so->ptr;
+    const uint32_t n32 = static_cast<uint32_t>(on);
+    const float eps = state().epsilon;
+    if (all_same) {
+#define B(OP) launch_binary_same<OP>(pa, pb, po, n32, eps)
+        KTH_BINARY_DISPATCH(op, B)
+#undef B
+    } else {
+#define B(OP) launch_binary_bcast<OP>(pa, pb, po, n32, eps, plan, vec_ok, a_vec, b_vec)
+        KTH_BINARY_DISPATCH(op, B)
+#undef B
+    }
+    KTH_LAUNCH_CHECK("binary");
+    count_launch((an + bn + on) * 4);
+    return KTH_OK;
+}
+
+int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
+                     uint64_t dst, const int32_t* dshape, int ddims) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    uint64_t sn, dn;
+    if (int rc = check_shape(sshape, sdims, "kth_broadcast_to(src)", &sn)) return rc;
+    if (int rc = check_shape(dshape, ddims, "kth_broadcast_to(dst)", &dn)) return rc;
+    Store* ss = lookup(src, "kth_broadcast_to(src)");
+    if (!ss) return KTH_E_HANDLE;
+    Store* sd = lookup(dst, "kth_broadcast_to(dst)");
+    if (!sd) return KTH_E_HANDLE;
+    if (sn > ss->n_floats || dn > sd->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_broadcast_to: a shape needs more elements than its store holds");
+    BcastPlan plan;
+    bool vec_ok, a_vec, b_vec;
+    // Planned as the binary op first(src, src): both operand maps are the source's.
+    if (!build_plan(sshape, sdims, sshape, sdims, dshape, ddims, &plan, &vec_ok, &a_vec, &b_vec))
+        return fail(KTH_E_SHAPE, "kth_broadcast_to: source shape does not broadcast to the target shape");
+    if (ss->ptr == sd->ptr) return fail(KTH_E_ARGUMENT, "kth_broadcast_to: source and target are the same store");
+    if (dn == 0) return KTH_OK;
+    if (sn == dn) {
+        KTH_HIP(hipMemcpyAsync(sd->ptr, ss->ptr, dn * 4, hipMemcpyDeviceToDevice, state().stream));
+    } else {
+        launch_binary_bcast<OpFirst>(ss->ptr, ss->ptr, sd->ptr, static_cast<uint32_t>(dn), 0.0f, plan, vec_ok, a_vec, b_vec);
+        KTH_LAUNCH_CHECK("broadcast_to");
+    }
+    count_launch((sn + dn) * 4);
+    return KTH_OK;
+}
+
+int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!out) return fail(KTH_E_ARGUMENT, "kth_contains_nan: null output");
+    Store* st = lookup(handle, "kth_contains_nan");
+    if (!st) return KTH_E_HANDLE;
+    if (n > st->n_floats) return fail(KTH_E_ARGUMENT, "kth_contains_nan: n=%llu exceeds the store", (unsigned long long)n);
+    *out = 0;
+    if (n == 0) return KTH_OK;
+    uint64_t cap;
+    int* flag = reinterpret_cast<int*>(workspace_acquire(4, &cap));
+    if (!flag) return fail(KTH_E_MEMORY, "kth_contains_nan: no workspace");
+    State& s = state();
+    hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, s.stream, flag);
+    uint32_t n32 = static_cast<uint32_t>(n);
+    uint32_t blocks = blocks_for(n32 >> 2);
+    uint32_t cap_blocks = static_cast<uint32_t>(s.compute_units) * 8u;
+    if (blocks > cap_blocks) blocks = cap_blocks;
+    hipLaunchKernelGGL(contains_nan_kernel, dim3(blocks), dim3(kBlock), 0, s.stream, st->ptr, n32, flag);
+    int host_flag = 0;
+    hipError_t e = hipMemcpyAsync(&host_flag, flag, 4, hipMemcpyDeviceToHost, s.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
+    workspace_release(reinterpret_cast<float*>(flag), cap);
+    if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_contains_nan: %s", hipGetErrorString(e));
+    *out = host_flag;
+    count_launch(n * 4);
+    return KTH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,90 @@
+// Shared host-side state and helpers of libkten_hip.so (not part of the public ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "../../include/kten_hip.h"
+
+namespace kth {
+
+// One device-resident fp32 store. `cap_bytes` is the pool size class it was cut from.
+struct Store {
+    float*   ptr = nullptr;
+    uint64_t n_floats = 0;
+    uint64_t cap_bytes = 0;
+    uint32_t refs = 0;
+    uint32_t generation = 0;   // bumped on release so stale handles are detected
+};
+
+struct State {
+    bool        ready = false;
+    int         device = -1;
+    hipStream_t stream = nullptr;
+    hipEvent_t  ev_begin = nullptr, ev_end = nullptr;
+    bool        timer_open = false;
+
+    char     name[256] = {0};
+    uint64_t total_mem = 0;
+    int      compute_units = 0;
+    int      wave_size = 0;
+
+    float  epsilon = 1e-7f;
+    double mem_hint = 0.85;
+
+    std::vector<Store>    table;       // handle index -> store
+    std::vector<uint32_t> free_slots;
+    std::map<uint64_t, std::vector<float*>> pool;   // size class (bytes) -> idle buffers
+
+    uint64_t live_bytes = 0, pool_bytes = 0, launches = 0, bytes_moved = 0;
+};
+
+State&      state();
+std::mutex& lock();
+
+// Records the message for kth_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+
+// Handle -> store, or nullptr (with the error recorded).
+Store* lookup(uint64_t handle, const char* what);
+
+// Pool-backed raw device memory for kernels' own workspaces (partials of two-pass
+// reductions). Stream-ordered: a workspace returned to the pool may be reused by a
+// later launch because every launch is on the one in-order stream.
+float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
+void   workspace_release(float* p, uint64_t cap_bytes);
+
+inline void count_launch(uint64_t algorithmic_bytes) {
+    state().launches += 1;
+    state().bytes_moved += algorithmic_bytes;
+}
+
+#define KTH_REQUIRE_INIT()                                                         \
+    do {                                                                           \
+        if (!kth::state().ready) return kth::fail(KTH_E_NOT_INIT, "kth_init has not been called"); \
+    } while (0)
+
+#define KTH_HIP(call)                                                              \
+    do {                                                                           \
+        hipError_t e__ = (call);                                                   \
+        if (e__ != hipSuccess)                                                     \
+            return kth::fail(KTH_E_DEVICE, "%s failed: %s", #call, hipGetErrorString(e__)); \
+    } while (0)
+
+// After a kernel launch: surface launch-configuration errors immediately.
+#define KTH_LAUNCH_CHECK(name)                                                     \
+    do {                                                                           \
+        hipError_t e__ = hipGetLastError();                                        \
+        if (e__ != hipSuccess)                                                     \
+            return kth::fail(KTH_E_DEVICE, "launch of %s failed: %s", name, hipGetErrorString(e__)); \
+    } while (0)
+
+constexpr uint64_t kMaxElements = 0x7fffffffull;   // store size is a Kotlin Int
+
+}  // namespace kth

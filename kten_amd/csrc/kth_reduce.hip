@@ -1,0 +1,398 @@
+// Axis and full reductions over a row-major tensor seen as [outer, axis, inner].
+//
+// Three first-pass kernels cover the layouts:
+//   rows    (inner == 1): G lanes of a wave64 (or a whole 256-thread workgroup) walk one
+//           contiguous row with float4 loads, combine by xor shuffles (+ LDS across waves);
+//   columns (inner >= 64): a wave owns 64 float4-wide (or scalar) columns so every load
+//           instruction is a contiguous 1 KiB (256 B) span; the waves of a workgroup
+//           take different rows and combine through LDS;
+//   strided (small inner): one thread per output element, serial walk down the axis.
+// When the output alone gives too few workgroups to fill 256 CUs, the axis is cut into
+// S segments; each (output, segment) writes a partial and a second kernel combines the
+// S partials in a fixed order. No atomics anywhere: the same input always gives the
+// same bits.
+//
+// Sums accumulate in f64 from the first add (f64 adds are full rate on CDNA), so SUM and
+// MEAN land within an ulp of the float64 reference; kten-jvm's serial float accumulation
+// order (JVMRawTensor.kt:146-148,185-207) is not reproduced bit-for-bit, only bounded.
+// MAX/MIN/ARG_MAX/ARG_MIN are order-independent and bit-exact (JVMRawTensor.kt:159-184).
+#include "kth_internal.h"
+#include "kth_ops.h"
+
+using namespace kth;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- reducers
+
+struct ArgAcc { float v; uint32_t i; };
+
+__device__ __forceinline__ double shfl_xor_acc(double a, int m) { return __shfl_xor(a, m); }
+__device__ __forceinline__ float  shfl_xor_acc(float a, int m)  { return __shfl_xor(a, m); }
+__device__ __forceinline__ ArgAcc shfl_xor_acc(ArgAcc a, int m) {
+    ArgAcc r;
+    r.v = __shfl_xor(a.v, m);
+    r.i = static_cast<uint32_t>(__shfl_xor(static_cast<int>(a.i), m));
+    return r;
+}
+
+template <bool MEAN>
+struct RedSumT {
+    using Acc = double;
+    static __device__ __forceinline__ Acc init() { return 0.0; }
+    static __device__ __forceinline__ void step(Acc& a, float x, uint32_t) { a += static_cast<double>(x); }
+    static __device__ __forceinline__ Acc merge(Acc a, Acc b) { return a + b; }
+    // MEAN divides once in f64 and rounds once (FloatArray.average, JVMRawTensor.kt:150-152).
+    static __device__ __forceinline__ float finish(Acc a, uint32_t n) {
+        return MEAN ? static_cast<float>(a / static_cast<double>(n)) : static_cast<float>(a);
+    }
+};
+using RedSum = RedSumT<false>;
+using RedMean = RedSumT<true>;
+
+template <bool MAX>
+struct RedExtT {
+    using Acc = float;
+    static __device__ __forceinline__ Acc init() { return MAX ? -INFINITY : INFINITY; }
+    static __device__ __forceinline__ void step(Acc& a, float x, uint32_t) { a = MAX ? jmax(a, x) : jmin(a, x); }
+    static __device__ __forceinline__ Acc merge(Acc a, Acc b) { return MAX ? jmax(a, b) : jmin(a, b); }
+    static __device__ __forceinline__ float finish(Acc a, uint32_t) { return a; }
+};
+using RedMax = RedExtT<true>;
+using RedMin = RedExtT<false>;
+
+// temp starts at -/+inf, index at 0, update on strict compare only: ties keep the lowest
+// index, NaNs never win, a lane with nothing strictly better yields 0 (JVMRawTensor.kt:167-184).
+template <bool MAX>
+struct RedArgT {
+    using Acc = ArgAcc;
+    static __device__ __forceinline__ Acc init() { Acc a; a.v = MAX ? -INFINITY : INFINITY; a.i = 0; return a; }
+    static __device__ __forceinline__ void step(Acc& a, float x, uint32_t idx) {
+        if (MAX ? (x > a.v) : (x < a.v)) { a.v = x; a.i = idx; }
+    }
+    static __device__ __forceinline__ Acc merge(Acc a, Acc b) {
+        bool take_b = (MAX ? (b.v > a.v) : (b.v < a.v)) || (b.v == a.v && b.i < a.i);
+        return take_b ? b : a;
+    }
+    static __device__ __forceinline__ float finish(Acc a, uint32_t) { return static_cast<float>(a.i); }
+};
+using RedArgMax = RedArgT<true>;
+using RedArgMin = RedArgT<false>;
+
+// ---------------------------------------------------------------- geometry
+
+// One launch's view of the tensor. Segment s covers axis positions
+// [s * seg_len, min((s + 1) * seg_len, axis)). With segments > 1 results go to
+// `partial` laid out [outer][segments][inner].
+struct Geom {
+    uint32_t outer, axis, inner;
+    uint32_t segments, seg_len;
+};
+
+template <class R>
+__device__ __forceinline__ void emit(const Geom& g, uint32_t o, uint32_t s, uint32_t i, typename R::Acc acc,
+                                     float* out, typename R::Acc* partial) {
+    if (g.segments == 1) out[static_cast<size_t>(o) * g.inner + i] = R::finish(acc, g.axis);
+    else partial[(static_cast<size_t>(o) * g.segments + s) * g.inner + i] = acc;
+}
+
+// ---------------------------------------------------------------- rows: inner == 1
+
+// G lanes per row (G in 1..64 a power of two, or 256 = the whole workgroup).
+// VEC = 4 requires axis % 4 == 0 and seg_len % 4 == 0 so every row segment is 16-byte aligned.
+template <class R, int G, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                            typename R::Acc* __restrict__ partial, Geom g) {
+    using Acc = typename R::Acc;
+    constexpr int kRows = kBlock / G;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t s = bid % g.segments;
+    const uint32_t row = (bid / g.segments) * kRows + threadIdx.x / G;
+    const uint32_t lane = threadIdx.x % G;
+    Acc acc = R::init();
+    if (row < g.outer) {
+        const float* base = in + static_cast<size_t>(row) * g.axis;
+        const uint32_t begin = s * g.seg_len;
+        const uint32_t end = min(begin + g.seg_len, g.axis);
+        if (VEC == 4) {
+#pragma unroll 4
+            for (uint32_t j = begin + lane * 4; j < end; j += G * 4) {
+                float4 v = *reinterpret_cast<const float4*>(base + j);
+                R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
+            }
+        } else {
+#pragma unroll 4
+            for (uint32_t j = begin + lane; j < end; j += G) R::step(acc, base[j], j);
+        }
+    }
+    constexpr int kLanes = G < kWave ? G : kWave;
+#pragma unroll
+    for (int m = kLanes / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
+    if (G == kBlock) {
+        __shared__ Acc lds[kBlock / kWave];
+        if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            Acc t = lds[0];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; w++) t = R::merge(t, lds[w]);
+            emit<R>(g, row, s, 0, t, out, partial);
+        }
+    } else {
+        if (lane == 0 && row < g.outer) emit<R>(g, row, s, 0, acc, out, partial);
+    }
+}
+
+// ---------------------------------------------------------------- columns: inner >= 64
+
+// Workgroup = 64 x WY threads: lane x owns VEC adjacent columns of a 64*VEC-column tile,
+// wave y takes rows y, y + WY, ... of the segment.
+template <class R, int VEC, int WY>
+__global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                 typename R::Acc* __restrict__ partial, Geom g, uint32_t tiles) {
+    using Acc = typename R::Acc;
+    const uint32_t bid = blockIdx.x;
+    const uint32_t tile = bid % tiles;
+    const uint32_t rest = bid / tiles;
+    const uint32_t s = rest % g.segments;
+    const uint32_t o = rest / g.segments;
+    const uint32_t tx = threadIdx.x, ty = threadIdx.y;
+    const uint32_t col = (tile * kWave + tx) * VEC;
+    const bool active = col < g.inner;          // inner % VEC == 0, so a float4 is all in or all out
+    Acc acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = R::init();
+    if (active) {
+        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
+        const uint32_t begin = s * g.seg_len;
+        const uint32_t end = min(begin + g.seg_len, g.axis);
+#pragma unroll 4
+        for (uint32_t r = begin + ty; r < end; r += WY) {
+            const float* p = base + static_cast<size_t>(r) * g.inner;
+            if (VEC == 4) {
+                float4 v = *reinterpret_cast<const float4*>(p);
+                R::step(acc[0], v.x, r); R::step(acc[1 % VEC], v.y, r);
+                R::step(acc[2 % VEC], v.z, r); R::step(acc[3 % VEC], v.w, r);
+            } else {
+                R::step(acc[0], *p, r);
+            }
+        }
+    }
+    __shared__ Acc lds[WY][kWave * VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) lds[ty][tx * VEC + v] = acc[v];
+    __syncthreads();
+    if (ty == 0 && active) {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            Acc t = lds[0][tx * VEC + v];
+            for (int w = 1; w < WY; w++) t = R::merge(t, lds[w][tx * VEC + v]);
+            emit<R>(g, o, s, col + v, t, out, partial);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- strided: small inner
+
+template <class R>
+__global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                               typename R::Acc* __restrict__ partial, Geom g) {
+    const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const uint64_t n_out = static_cast<uint64_t>(g.outer) * g.inner;
+    if (t >= n_out * g.segments) return;
+    const uint32_t i = static_cast<uint32_t>(t % g.inner);
+    const uint64_t rest = t / g.inner;
+    const uint32_t s = static_cast<uint32_t>(rest % g.segments);
+    const uint32_t o = static_cast<uint32_t>(rest / g.segments);
+    const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + i;
+    const uint32_t begin = s * g.seg_len;
+    const uint32_t end = min(begin + g.seg_len, g.axis);
+    typename R::Acc acc = R::init();
+#pragma unroll 4
+    for (uint32_t r = begin; r < end; r++) R::step(acc, base[static_cast<size_t>(r) * g.inner], r);
+    emit<R>(g, o, s, i, acc, out, partial);
+}
+
+// ---------------------------------------------------------------- second pass
+
+// Combines the `segments` partials of each output in ascending segment order.
+// WAVE = false: one thread per output. WAVE = true: one wave64 per output, for few
+// outputs with many partials (full reductions).
+template <class R, bool WAVE>
+__global__ __launch_bounds__(kBlock) void reduce_finalize_kernel(const typename R::Acc* __restrict__ partial,
+                                                                float* __restrict__ out, Geom g) {
+    using Acc = typename R::Acc;
+    const uint64_t n_out = static_cast<uint64_t>(g.outer) * g.inner;
+    if (WAVE) {
+        const uint64_t idx = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+        const uint32_t lane = threadIdx.x & (kWave - 1);
+        Acc acc = R::init();
+        if (idx < n_out) {
+            const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
+            for (uint32_t s = lane; s < g.segments; s += kWave)
+                acc = R::merge(acc, partial[(static_cast<size_t>(o) * g.segments + s) * g.inner + i]);
+        }
+#pragma unroll
+        for (int m = kWave / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
+        if (lane == 0 && idx < n_out) out[idx] = R::finish(acc, g.axis);
+    } else {
+        const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+        if (idx >= n_out) return;
+        const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
+        Acc acc = partial[(static_cast<size_t>(o) * g.segments) * g.inner + i];
+        for (uint32_t s = 1; s < g.segments; s++)
+            acc = R::merge(acc, partial[(static_cast<size_t>(o) * g.segments + s) * g.inner + i]);
+        out[idx] = R::finish(acc, g.axis);
+    }
+}
+
+// ---------------------------------------------------------------- host planning
+
+uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
+
+// Cuts the axis into segments so that `base_blocks * segments` reaches `target` blocks,
+// while every segment keeps at least `min_len` positions and is a multiple of `quantum`.
+void plan_segments(Geom* g, uint64_t base_blocks, uint64_t target, uint32_t quantum, uint32_t min_len) {
+    uint32_t want = base_blocks >= target ? 1u : ceil_div(target, base_blocks);
+    uint32_t max_seg = g->axis / min_len;
+    if (max_seg < 1) max_seg = 1;
+    if (want > max_seg) want = max_seg;
+    uint32_t len = ceil_div(g->axis, want);
+    len = ceil_div(len, quantum) * quantum;
+    g->seg_len = len;
+    g->segments = ceil_div(g->axis, len);
+}
+
+template <class R>
+int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
+    using Acc = typename R::Acc;
+    State& st = state();
+    hipStream_t stream = st.stream;
+    const uint64_t target = static_cast<uint64_t>(st.compute_units) * 8;
+    Geom g{outer, axis, inner, 1, axis};
+    const uint64_t n_out = static_cast<uint64_t>(outer) * inner;
+
+    enum { ROWS, COLS, STRIDED } kind;
+    int G = 1, VEC = 1;
+    uint32_t tiles = 0;
+    uint64_t blocks = 0;
+    if (inner == 1) {
+        kind = ROWS;
+        VEC = (axis % 4 == 0) ? 4 : 1;
+        const uint32_t per_lane = axis / VEC;          // loads per row
+        G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : 1;
+        const uint64_t base_blocks = ceil_div(outer, kBlock / G);
+        plan_segments(&g, base_blocks, target, G * VEC, G * VEC * 8);
+        blocks = base_blocks * g.segments;
+    } else if (inner >= 64) {
+        kind = COLS;
+        VEC = (inner % 4 == 0) ? 4 : 1;
+        tiles = ceil_div(inner, kWave * VEC);
+        const uint64_t base_blocks = static_cast<uint64_t>(tiles) * outer;
+        plan_segments(&g, base_blocks, target, 4, 4 * 8);
+        blocks = base_blocks * g.segments;
+    } else {
+        kind = STRIDED;
+        const uint64_t base_blocks = ceil_div(n_out, kBlock);
+        plan_segments(&g, base_blocks, target / 2, 1, 64);
+        blocks = ceil_div(n_out * g.segments, kBlock);
+    }
+    if (blocks > 0x7fffffffull) return fail(KTH_E_ARGUMENT, "kth_reduce: grid too large");
+
+    Acc* partial = nullptr;
+    uint64_t cap = 0;
+    if (g.segments > 1) {
+        partial = reinterpret_cast<Acc*>(workspace_acquire(n_out * g.segments * sizeof(Acc), &cap));
+        if (!partial) return fail(KTH_E_MEMORY, "kth_reduce: no workspace for %llu partials",
+                                  (unsigned long long)(n_out * g.segments));
+    }
+    const dim3 grid(static_cast<uint32_t>(blocks));
+    if (kind == ROWS) {
+#define ROWS_LAUNCH(GG, VV) hipLaunchKernelGGL((reduce_rows_kernel<R, GG, VV>), grid, dim3(kBlock), 0, stream, in, out, partial, g)
+        if (VEC == 4) {
+            switch (G) { case 256: ROWS_LAUNCH(256, 4); break; case 64: ROWS_LAUNCH(64, 4); break;
+                         case 16: ROWS_LAUNCH(16, 4); break; case 4: ROWS_LAUNCH(4, 4); break; default: ROWS_LAUNCH(1, 4); }
+        } else {
+            switch (G) { case 256: ROWS_LAUNCH(256, 1); break; case 64: ROWS_LAUNCH(64, 1); break;
+                         case 16: ROWS_LAUNCH(16, 1); break; case 4: ROWS_LAUNCH(4, 1); break; default: ROWS_LAUNCH(1, 1); }
+        }
+#undef ROWS_LAUNCH
+    } else if (kind == COLS) {
+        if (VEC == 4) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+        else          hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+    } else {
+        hipLaunchKernelGGL((reduce_strided_kernel<R>), grid, dim3(kBlock), 0, stream, in, out, partial, g);
+    }
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess && g.segments > 1) {
+        if (n_out < 4096 && g.segments > 16)
+            hipLaunchKernelGGL((reduce_finalize_kernel<R, true>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
+                               partial, out, g);
+        else
+            hipLaunchKernelGGL((reduce_finalize_kernel<R, false>), dim3(ceil_div(n_out, kBlock)), dim3(kBlock), 0, stream,
+                               partial, out, g);
+        e = hipGetLastError();
+    }
+    if (partial) workspace_release(reinterpret_cast<float*>(partial), cap);
+    if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+    count_launch((static_cast<uint64_t>(outer) * axis * inner + n_out) * 4);
+    return KTH_OK;
+}
+
+int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
+    switch (op) {
+    case KTH_SUM:     return run_reduce<RedSum>(in, out, outer, axis, inner);
+    case KTH_MEAN:    return run_reduce<RedMean>(in, out, outer, axis, inner);
+    case KTH_MAX:     return run_reduce<RedMax>(in, out, outer, axis, inner);
+    case KTH_MIN:     return run_reduce<RedMin>(in, out, outer, axis, inner);
+    case KTH_ARG_MAX: return run_reduce<RedArgMax>(in, out, outer, axis, inner);
+    case KTH_ARG_MIN: return run_reduce<RedArgMin>(in, out, outer, axis, inner);
+    default:          return fail(KTH_E_ARGUMENT, "kth_reduce: op %d is not an aggregating operation", op);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: op %d is not an aggregating operation", op);
+    Store* si = lookup(in, "kth_reduce_axis(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_reduce_axis(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (axis == 0) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: empty axis");
+    if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
+        outer * axis > kMaxElements || outer * axis * inner > kMaxElements)
+        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: more than 2^31-1 elements");
+    if ((op == KTH_ARG_MAX || op == KTH_ARG_MIN) && axis > (1ull << 24))
+        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: axis %llu too long for an index stored as float", (unsigned long long)axis);
+    if (outer * axis * inner > si->n_floats || outer * inner > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: [%llu,%llu,%llu] exceeds a store", (unsigned long long)outer,
+                    (unsigned long long)axis, (unsigned long long)inner);
+    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: output aliases the input");
+    if (outer * inner == 0) return KTH_OK;
+    return dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
+                           static_cast<uint32_t>(inner));
+}
+
+int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (op != KTH_SUM && op != KTH_MEAN) return fail(KTH_E_ARGUMENT, "kth_reduce_all: op %d is not SUM or MEAN", op);
+    Store* si = lookup(in, "kth_reduce_all(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_reduce_all(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (n == 0) return fail(KTH_E_ARGUMENT, "kth_reduce_all: empty input");
+    if (n > si->n_floats || so->n_floats < 1) return fail(KTH_E_ARGUMENT, "kth_reduce_all: n=%llu exceeds the store", (unsigned long long)n);
+    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "kth_reduce_all: output aliases the input");
+    return dispatch_reduce(op, si->ptr, so->ptr, 1u, static_cast<uint32_t>(n), 1u);
+}
+
+}  // extern "C"

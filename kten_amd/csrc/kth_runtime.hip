@@ -1,0 +1,336 @@
+// Platform bring-up, the store table, the reuse pool, host<->device transfers.
+#include "kth_internal.h"
+
+#include <cstring>
+
+namespace kth {
+
+State& state() { static State s; return s; }
+std::mutex& lock() { static std::mutex m; return m; }
+
+static thread_local char tl_error[512] = {0};
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(tl_error, sizeof(tl_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static inline uint64_t make_handle(uint32_t index, uint32_t generation) {
+    return (static_cast<uint64_t>(generation) << 32) | static_cast<uint64_t>(index + 1);
+}
+
+Store* lookup(uint64_t handle, const char* what) {
+    State& s = state();
+    uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
+    uint32_t gen = static_cast<uint32_t>(handle >> 32);
+    if (low == 0 || low > s.table.size()) {
+        fail(KTH_E_HANDLE, "%s: unknown handle 0x%llx", what, (unsigned long long)handle);
+        return nullptr;
+    }
+    Store& st = s.table[low - 1];
+    if (st.refs == 0 || st.generation != gen) {
+        fail(KTH_E_HANDLE, "%s: handle 0x%llx was released", what, (unsigned long long)handle);
+        return nullptr;
+    }
+    return &st;
+}
+
+// Size classes: 512-byte granules up to 1 MiB, then 1/8-octave steps (at most 12.5 %
+// slack), so the differently-sized tensors of one graph reuse each other's buffers.
+static uint64_t size_class(uint64_t bytes) {
+    if (bytes == 0) bytes = 4;
+    if (bytes <= (1ull << 20)) return (bytes + 511) & ~511ull;
+    int top = 63 - __builtin_clzll(bytes);
+    uint64_t step = 1ull << (top - 3);
+    return (bytes + step - 1) & ~(step - 1);
+}
+
+static void trim_pool() {
+    State& s = state();
+    for (auto& kv : s.pool) {
+        for (float* p : kv.second) {
+            (void)hipFree(p);
+            s.pool_bytes -= kv.first;
+        }
+        kv.second.clear();
+    }
+    s.pool.clear();
+}
+
+static float* pool_take(uint64_t cap) {
+    State& s = state();
+    auto it = s.pool.find(cap);
+    if (it != s.pool.end() && !it->second.empty()) {
+        float* p = it->second.back();
+        it->second.pop_back();
+        s.pool_bytes -= cap;
+        return p;
+    }
+    uint64_t budget = static_cast<uint64_t>(s.mem_hint * static_cast<double>(s.total_mem));
+    if (s.live_bytes + s.pool_bytes + cap > budget) {
+        // Freeing must not race with kernels still using pooled buffers' old contents.
+        (void)hipStreamSynchronize(s.stream);
+        trim_pool();
+        if (s.live_bytes + cap > budget) return nullptr;
+    }
+    void* p = nullptr;
+    if (hipMalloc(&p, cap) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipStreamSynchronize(s.stream);
+        trim_pool();
+        if (hipMalloc(&p, cap) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
+    return static_cast<float*>(p);
+}
+
+float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes) {
+    uint64_t cap = size_class(bytes);
+    float* p = pool_take(cap);
+    if (p) { *cap_bytes = cap; state().live_bytes += cap; }
+    return p;
+}
+
+void workspace_release(float* p, uint64_t cap_bytes) {
+    State& s = state();
+    s.pool[cap_bytes].push_back(p);
+    s.live_bytes -= cap_bytes;
+    s.pool_bytes += cap_bytes;
+}
+
+}  // namespace kth
+
+using namespace kth;
+
+extern "C" {
+
+const char* kth_last_error(void) { return tl_error; }
+
+int kth_init(int device) {
+    std::lock_guard<std::mutex> g(lock());
+    State& s = state();
+    if (s.ready) {
+        if (s.device == device) return KTH_OK;
+        return fail(KTH_E_ARGUMENT, "already initialised on device %d", s.device);
+    }
+    int count = 0;
+    KTH_HIP(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count)
+        return fail(KTH_E_ARGUMENT, "device %d out of range (%d visible)", device, count);
+    KTH_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    KTH_HIP(hipGetDeviceProperties(&prop, device));
+    snprintf(s.name, sizeof(s.name), "%s (%s)", prop.name, prop.gcnArchName);
+    s.total_mem = prop.totalGlobalMem;
+    s.compute_units = prop.multiProcessorCount;
+    s.wave_size = prop.warpSize;
+    if (s.wave_size != 64)
+        return fail(KTH_E_DEVICE, "kernels are written for wave64; device reports wave %d", s.wave_size);
+    KTH_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+    KTH_HIP(hipEventCreate(&s.ev_begin));
+    KTH_HIP(hipEventCreate(&s.ev_end));
+    s.device = device;
+    s.ready = true;
+    return KTH_OK;
+}
+
+int kth_shutdown(void) {
+    std::lock_guard<std::mutex> g(lock());
+    State& s = state();
+    if (!s.ready) return KTH_OK;
+    (void)hipStreamSynchronize(s.stream);
+    for (Store& st : s.table)
+        if (st.refs > 0 && st.ptr) (void)hipFree(st.ptr);
+    s.table.clear();
+    s.free_slots.clear();
+    trim_pool();
+    (void)hipEventDestroy(s.ev_begin);
+    (void)hipEventDestroy(s.ev_end);
+    (void)hipStreamDestroy(s.stream);
+    s = State();
+    return KTH_OK;
+}
+
+int kth_device_info(char* name, size_t cap, uint64_t* total_mem, int* compute_units, int* wave_size) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    if (name && cap > 0) { strncpy(name, s.name, cap - 1); name[cap - 1] = 0; }
+    if (total_mem) *total_mem = s.total_mem;
+    if (compute_units) *compute_units = s.compute_units;
+    if (wave_size) *wave_size = s.wave_size;
+    return KTH_OK;
+}
+
+int kth_set_epsilon(float eps) {
+    std::lock_guard<std::mutex> g(lock());
+    state().epsilon = eps;
+    return KTH_OK;
+}
+
+int kth_set_memory_scale_hint(double fraction) {
+    std::lock_guard<std::mutex> g(lock());
+    if (!(fraction > 0.0 && fraction <= 1.0))
+        return fail(KTH_E_ARGUMENT, "memory scale hint %g outside (0, 1]", fraction);
+    state().mem_hint = fraction;
+    return KTH_OK;
+}
+
+int kth_alloc(uint64_t n_floats, uint64_t* handle) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!handle) return fail(KTH_E_ARGUMENT, "kth_alloc: null handle pointer");
+    if (n_floats > kMaxElements)
+        return fail(KTH_E_ARGUMENT, "kth_alloc: %llu elements exceed the 2^31-1 store limit",
+                    (unsigned long long)n_floats);
+    State& s = state();
+    uint64_t cap = size_class(n_floats * 4);
+    float* p = pool_take(cap);
+    if (!p)
+        return fail(KTH_E_MEMORY, "kth_alloc: cannot allocate %llu bytes (live %llu, hint %.2f of %llu)",
+                    (unsigned long long)cap, (unsigned long long)s.live_bytes, s.mem_hint,
+                    (unsigned long long)s.total_mem);
+    uint32_t idx;
+    if (!s.free_slots.empty()) { idx = s.free_slots.back(); s.free_slots.pop_back(); }
+    else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); }
+    Store& st = s.table[idx];
+    st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1;
+    s.live_bytes += cap;
+    *handle = make_handle(idx, st.generation);
+    return KTH_OK;
+}
+
+int kth_retain(uint64_t handle) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* st = lookup(handle, "kth_retain");
+    if (!st) return KTH_E_HANDLE;
+    st->refs += 1;
+    return KTH_OK;
+}
+
+int kth_release(uint64_t handle) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* st = lookup(handle, "kth_release");
+    if (!st) return KTH_E_HANDLE;
+    st->refs -= 1;
+    if (st->refs == 0) {
+        State& s = state();
+        s.pool[st->cap_bytes].push_back(st->ptr);
+        s.live_bytes -= st->cap_bytes;
+        s.pool_bytes += st->cap_bytes;
+        st->ptr = nullptr;
+        st->generation += 1;
+        s.free_slots.push_back(static_cast<uint32_t>((handle & 0xffffffffu) - 1));
+    }
+    return KTH_OK;
+}
+
+static int check_range(const Store* st, uint64_t off, uint64_t n, const char* what) {
+    if (off > st->n_floats || n > st->n_floats - off)
+        return fail(KTH_E_ARGUMENT, "%s: range [%llu, +%llu) outside a store of %llu floats", what,
+                    (unsigned long long)off, (unsigned long long)n, (unsigned long long)st->n_floats);
+    return KTH_OK;
+}
+
+int kth_upload(uint64_t handle, uint64_t offset, const float* src, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* st = lookup(handle, "kth_upload");
+    if (!st) return KTH_E_HANDLE;
+    if (int rc = check_range(st, offset, n, "kth_upload")) return rc;
+    if (n == 0) return KTH_OK;
+    if (!src) return fail(KTH_E_ARGUMENT, "kth_upload: null source");
+    State& s = state();
+    KTH_HIP(hipMemcpyAsync(st->ptr + offset, src, n * 4, hipMemcpyHostToDevice, s.stream));
+    KTH_HIP(hipStreamSynchronize(s.stream));
+    return KTH_OK;
+}
+
+int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* st = lookup(handle, "kth_download");
+    if (!st) return KTH_E_HANDLE;
+    if (int rc = check_range(st, offset, n, "kth_download")) return rc;
+    if (n == 0) return KTH_OK;
+    if (!dst) return fail(KTH_E_ARGUMENT, "kth_download: null destination");
+    State& s = state();
+    KTH_HIP(hipMemcpyAsync(dst, st->ptr + offset, n * 4, hipMemcpyDeviceToHost, s.stream));
+    KTH_HIP(hipStreamSynchronize(s.stream));
+    return KTH_OK;
+}
+
+int kth_read_scalar(uint64_t handle, uint64_t index, float* out) {
+    if (!out) return fail(KTH_E_ARGUMENT, "kth_read_scalar: null output");
+    return kth_download(out, handle, index, 1);
+}
+
+int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    Store* d = lookup(dst, "kth_copy(dst)");
+    if (!d) return KTH_E_HANDLE;
+    Store* sst = lookup(src, "kth_copy(src)");
+    if (!sst) return KTH_E_HANDLE;
+    if (int rc = check_range(d, dst_offset, n, "kth_copy(dst)")) return rc;
+    if (int rc = check_range(sst, src_offset, n, "kth_copy(src)")) return rc;
+    if (n == 0) return KTH_OK;
+    if (d->ptr == sst->ptr) {
+        uint64_t lo = dst_offset < src_offset ? dst_offset : src_offset;
+        uint64_t hi = dst_offset < src_offset ? src_offset : dst_offset;
+        if (hi - lo < n) return fail(KTH_E_ARGUMENT, "kth_copy: overlapping ranges in one store");
+    }
+    State& s = state();
+    KTH_HIP(hipMemcpyAsync(d->ptr + dst_offset, sst->ptr + src_offset, n * 4, hipMemcpyDeviceToDevice, s.stream));
+    count_launch(n * 8);
+    return KTH_OK;
+}
+
+int kth_sync(void) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    KTH_HIP(hipStreamSynchronize(state().stream));
+    return KTH_OK;
+}
+
+int kth_metrics(uint64_t* live_bytes, uint64_t* pool_bytes, uint64_t* launches, uint64_t* bytes_moved) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    if (live_bytes) *live_bytes = s.live_bytes;
+    if (pool_bytes) *pool_bytes = s.pool_bytes;
+    if (launches) *launches = s.launches;
+    if (bytes_moved) *bytes_moved = s.bytes_moved;
+    return KTH_OK;
+}
+
+int kth_timer_begin(void) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    KTH_HIP(hipEventRecord(s.ev_begin, s.stream));
+    s.timer_open = true;
+    return KTH_OK;
+}
+
+int kth_timer_end(float* milliseconds) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    if (!milliseconds) return fail(KTH_E_ARGUMENT, "kth_timer_end: null output");
+    if (!s.timer_open) return fail(KTH_E_ARGUMENT, "kth_timer_end without kth_timer_begin");
+    KTH_HIP(hipEventRecord(s.ev_end, s.stream));
+    KTH_HIP(hipEventSynchronize(s.ev_end));
+    KTH_HIP(hipEventElapsedTime(milliseconds, s.ev_begin, s.ev_end));
+    s.timer_open = false;
+    return KTH_OK;
+}
+
+}  // extern "C"

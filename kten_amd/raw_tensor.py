@@ -1,0 +1,232 @@
+"""The raw-tensor side of the backend contract, for the broadcast / reduction path.
+
+`AbstractRawTensor` mirrors the reference's
+kten-api/src/main/kotlin/eu/redbean/kten/api/tensor/store/AbstractRawTensor.kt: the same
+member names, argument meaning and error behaviour, with the concrete helpers of the
+base class (axis normalisation, keep-dims handling, reshape / squeeze / unsqueeze,
+common-shape calculation) restated once here so that every backend shares them, as in
+the reference. Kotlin's overloads on (tensor | Float) become one Python method that
+dispatches on the argument type; Kotlin operators are also exposed as Python operators.
+
+Members of the contract that lie outside the accelerated path (indexed get/set,
+gather/scatter, transpose/permute, BLAS, nn) are not part of this mirror.
+"""
+from enum import Enum
+from typing import List, Sequence
+
+from . import shape_functions as sf
+
+
+class AggregatingOperation(Enum):
+    """kten-api/.../tensor/store/AggregatingOperation.kt:3-5"""
+    SUM = "SUM"
+    MEAN = "MEAN"
+    MAX = "MAX"
+    MIN = "MIN"
+    ARG_MAX = "ARG_MAX"
+    ARG_MIN = "ARG_MIN"
+
+
+def _is_number(x) -> bool:
+    return isinstance(x, (int, float)) and not isinstance(x, bool)
+
+
+class AbstractRawTensor:
+    """AbstractRawTensor.kt:5-23 — a shape plus a backend-owned store."""
+
+    def __init__(self, shape: Sequence[int]):
+        self._shape = list(shape)
+
+    # --- shape -------------------------------------------------------------------------
+    @property
+    def shape(self) -> List[int]:
+        return self._shape
+
+    @shape.setter
+    def shape(self, value: Sequence[int]):
+        self._shape = list(value)
+
+    @property
+    def dimensions(self) -> int:
+        return len(self._shape)
+
+    # --- abstract: what a backend supplies (AbstractRawTensor.kt:25-75,121-122,164-246) ---
+    def broadcastTo(self, shape): raise NotImplementedError
+    def _binary(self, op: str, other): raise NotImplementedError             # tensor (op) tensor, broadcasting
+    def _binary_assign(self, op: str, other): raise NotImplementedError      # in place, equal shapes
+    def _scalar(self, op: str, constant: float, reverse=False): raise NotImplementedError
+    def _scalar_assign(self, op: str, constant: float): raise NotImplementedError
+    def _compare(self, op: str, other): raise NotImplementedError            # tensor or float
+    def _unary(self, op: str): raise NotImplementedError
+    def clamp(self, min: float, max: float): raise NotImplementedError
+    def aggregateOverAxis(self, axis: int, resShape, aggregatingOperation): raise NotImplementedError
+    def _sum_all(self): raise NotImplementedError
+    def _mean_all(self): raise NotImplementedError
+    def view(self, shape): raise NotImplementedError
+    def copy(self, shallow: bool = False): raise NotImplementedError
+    def getSingleValue(self, indexes) -> float: raise NotImplementedError
+    def containsNan(self) -> bool: raise NotImplementedError
+    def inplaceFill(self, value: float): raise NotImplementedError
+    def toList(self): raise NotImplementedError                              # flat host copy (serializable data)
+
+    # --- arithmetic (AbstractRawTensor.kt:39-73) ---------------------------------------
+    def plus(self, other):
+        return self._scalar("plus", float(other)) if _is_number(other) else self._binary("plus", other)
+
+    def plusAssign(self, other):
+        if _is_number(other): self._scalar_assign("plus", float(other))
+        else: self._binary_assign("plus", other)
+
+    def minus(self, other):
+        return self._scalar("minus", float(other)) if _is_number(other) else self._binary("minus", other)
+
+    def unaryMinus(self):
+        return self._unary("neg")
+
+    def times(self, other):
+        return self._scalar("times", float(other)) if _is_number(other) else self._binary("times", other)
+
+    def timesAssign(self, other):
+        if _is_number(other): self._scalar_assign("times", float(other))
+        else: self._binary_assign("times", other)
+
+    def div(self, other):
+        return self._scalar("div", float(other)) if _is_number(other) else self._binary("div", other)
+
+    def divAssign(self, constant):
+        self._scalar_assign("div", float(constant))
+
+    def pow(self, other):
+        return self._scalar("pow", float(other)) if _is_number(other) else self._binary("pow", other)
+
+    def reciprocal(self): return self._unary("reciprocal")
+    def log(self): return self._unary("log")
+
+    __add__ = plus
+    __sub__ = minus
+    __mul__ = times
+    __truediv__ = div
+    __pow__ = pow
+    __neg__ = unaryMinus
+
+    def __iadd__(self, other):
+        self.plusAssign(other)
+        return self
+
+    def __imul__(self, other):
+        self.timesAssign(other)
+        return self
+
+    def __itruediv__(self, other):
+        self.divAssign(other)
+        return self
+
+    # --- comparisons (AbstractRawTensor.kt:194-206) ------------------------------------
+    def lt(self, other): return self._compare("lt", other)
+    def lte(self, other): return self._compare("lte", other)
+    def gt(self, other): return self._compare("gt", other)
+    def gte(self, other): return self._compare("gte", other)
+    def eq(self, other): return self._compare("eq", other)
+    def neq(self, other): return self._compare("neq", other)
+
+    # --- pointwise maths (AbstractRawTensor.kt:208-227) --------------------------------
+    def exp(self): return self._unary("exp")
+    def tanh(self): return self._unary("tanh")
+    def sigmoid(self): return self._unary("sigmoid")
+    def sinh(self): return self._unary("sinh")
+    def cosh(self): return self._unary("cosh")
+    def abs(self): return self._unary("abs")
+    def sign(self): return self._unary("sign")
+    def sqrt(self): return self._unary("sqrt")
+    def sin(self): return self._unary("sin")
+    def cos(self): return self._unary("cos")
+    def tan(self): return self._unary("tan")
+    def asin(self): return self._unary("asin")
+    def acos(self): return self._unary("acos")
+    def atan(self): return self._unary("atan")
+    def floor(self): return self._unary("floor")
+    def ceil(self): return self._unary("ceil")
+    def round(self): return self._unary("round")
+    def trunc(self): return self._unary("trunc")
+    def rsqrt(self): return self._unary("rsqrt")
+
+    # --- reshaping helpers (AbstractRawTensor.kt:77-88,124-144) ------------------------
+    def reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (list, tuple)):
+            shape = shape[0]
+        new_shape = sf.reshape(self.shape, shape)
+        res = self.copy()
+        res.shape = new_shape
+        return res
+
+    def inplaceReshape(self, shape):
+        self.shape = sf.reshape(self.shape, shape)
+
+    def inplaceSqueeze(self, axis: int):
+        new_shape = list(self.shape)
+        del new_shape[sf.normalize_axis(self.shape, axis)]
+        self.shape = new_shape
+
+    def squeeze(self, axis: int):
+        res = self.copy()
+        res.inplaceSqueeze(axis)
+        return res
+
+    def inplaceUnsqueeze(self, axis: int):
+        self.shape = sf.unsqueeze(self.shape, axis)
+
+    def unsqueeze(self, axis: int):
+        res = self.copy()
+        res.inplaceUnsqueeze(axis)
+        return res
+
+    # --- reductions (AbstractRawTensor.kt:92-122) --------------------------------------
+    def _aggregatingOpOverAxis(self, axis: int, keepDims: bool, op: AggregatingOperation):
+        """AbstractRawTensor.kt:92-108: normalise the axis, reduce to the keep-dims shape,
+        then drop the dim unless kept or the result would become 0-D."""
+        normalized = sf.normalize_axis(self.shape, axis)
+        res_shape = sf.aggregate_over(self.shape, normalized, True)
+        res = self.aggregateOverAxis(normalized, res_shape, op)
+        if not keepDims and len(res_shape) > 1:
+            without = list(res_shape)
+            del without[normalized]
+            res.shape = without
+        return res
+
+    def sum(self, axis=None, keepDimensions: bool = False):
+        if axis is None:
+            return self._sum_all()
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.SUM)
+
+    def mean(self, axis=None, keepDimensions: bool = False):
+        if axis is None:
+            return self._mean_all()
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.MEAN)
+
+    def max(self, axis: int, keepDimensions: bool = False):
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.MAX)
+
+    def min(self, axis: int, keepDimensions: bool = False):
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.MIN)
+
+    def argMax(self, axis: int = 0, keepDimensions: bool = False):
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.ARG_MAX)
+
+    def argMin(self, axis: int = 0, keepDimensions: bool = False):
+        return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.ARG_MIN)
+
+    # --- broadcasting (AbstractRawTensor.kt:170-192) -----------------------------------
+    def calculateCommonShapeWith(self, other) -> List[int]:
+        """Right-align, keep the longer operand's extra leading dims, per-dim max.
+        Validity is only checked later, by broadcastTo's rule."""
+        if self.shape == other.shape:
+            return list(self.shape)
+        a, b = list(self.shape), list(other.shape)
+        res: List[int] = []
+        diff = len(a) - len(b)
+        if diff > 0:
+            res.extend(a[:diff]); a = a[diff:]
+        elif diff < 0:
+            res.extend(b[:-diff]); b = b[-diff:]
+        res.extend(max(x, y) for x, y in zip(a, b))
+        return res

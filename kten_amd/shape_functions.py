@@ -1,0 +1,142 @@
+"""Shape algebra used on both sides of the raw-tensor contract.
+
+Host-side restatement of the part of the reference's
+kten-api/src/main/kotlin/eu/redbean/kten/api/autograd/utils/ShapeFunctions.kt that the
+broadcast / reduction path uses. Shapes are Python lists of ints; every function raises
+ValueError where the reference throws IllegalArgumentException, before anything is
+launched on the device.
+"""
+from typing import List, Sequence
+
+
+def to_store_size(shape: Sequence[int]) -> int:
+    """ShapeFunctions.kt:344 — element count of a row-major store."""
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def normalize_axis(shape: Sequence[int], axis: int) -> int:
+    """ShapeFunctions.kt:41-48 — negative axes count from the end; out of range throws."""
+    res = len(shape) + axis if axis < 0 else axis
+    if res < 0 or res >= len(shape):
+        raise ValueError(f"Cannot address axis: {axis} in tensor with dimensions: {len(shape)}")
+    return res
+
+
+def reshape(shape: Sequence[int], new_shape: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:11-39 — at most one -1 is inferred; element counts must match."""
+    new_shape = list(new_shape)
+    if any(d < -1 for d in new_shape):
+        raise ValueError(f"Invalid shape: {new_shape}")
+    inferred = [i for i, d in enumerate(new_shape) if d == -1]
+    if len(inferred) > 1:
+        raise ValueError(f"Cannot reshape to {new_shape}. Only one dimension can be inferred")
+    res = list(new_shape)
+    elements = to_store_size(shape)
+    if inferred:
+        res[inferred[0]] = 1
+        known = to_store_size(res)
+        res[inferred[0]] = elements // known if known else 0
+    if elements != to_store_size(res):
+        raise ValueError(f"Cannot reshape tensor with shape: {list(shape)} to shape: {new_shape}")
+    return res
+
+
+def squeeze(shape: Sequence[int], axis: int) -> List[int]:
+    """ShapeFunctions.kt:50-59."""
+    a = normalize_axis(shape, axis)
+    if shape[a] != 1:
+        raise ValueError(f"Cannot squeeze tensor with shape: {list(shape)} at axis: {axis}")
+    res = list(shape)
+    del res[a]
+    return res
+
+
+def unsqueeze(shape: Sequence[int], axis: int) -> List[int]:
+    """ShapeFunctions.kt:61-71 — axis == len appends; a negative axis inserts after the
+    dim it names, except -(len+1) which inserts in front."""
+    n = len(shape)
+    if axis == n:
+        a = axis
+    elif axis < 0:
+        a = 0 if axis == -(n + 1) else normalize_axis(shape, axis) + 1
+    else:
+        a = normalize_axis(shape, axis)
+    res = list(shape)
+    res.insert(a, 1)
+    return res
+
+
+def aggregate_over(shape: Sequence[int], axis: int, keep_dimensions: bool) -> List[int]:
+    """ShapeFunctions.kt:73-83 — the reduced dim becomes 1 and is dropped unless kept or
+    the result would be 0-D."""
+    a = normalize_axis(shape, axis)
+    res = list(shape)
+    res[a] = 1
+    if not keep_dimensions and len(res) > 1:
+        del res[a]
+    return res
+
+
+def infer_implicit_broadcast_shape(shape1: Sequence[int], shape2: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:168-185 — right-align, pad with leading 1s, each pair must be
+    equal or contain a 1."""
+    dims = max(len(shape1), len(shape2))
+    s1 = [1] * (dims - len(shape1)) + list(shape1)
+    s2 = [1] * (dims - len(shape2)) + list(shape2)
+    out = []
+    for a, b in zip(s1, s2):
+        if a == b or a == 1 or b == 1:
+            out.append(max(a, b))
+        else:
+            raise ValueError(
+                f"Shape {s1} must match {s2} for every non-singleton dimensions (missing dimensions count as "
+                "singleton dimension at the beginning of the shapes)")
+    return out
+
+
+def infer_explicit_broadcast_shape(shape: Sequence[int], target: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:187-201 — one-directional: `shape` must expand to `target`."""
+    if len(shape) > len(target):
+        raise ValueError(f"Tensor with shape: {list(shape)} cannot be broadcasted to shape: {list(target)}")
+    padded = [1] * (len(target) - len(shape)) + list(shape)
+    out = []
+    for a, b in zip(padded, target):
+        if a == b or a == 1:
+            out.append(max(a, b))
+        else:
+            raise ValueError(
+                f"Shape {list(shape)} must match {list(target)} for every non-singleton dimensions (missing "
+                "dimensions count as singleton dimension at the beginning of the shapes)")
+    return out
+
+
+def normalize_index(shape: Sequence[int], index: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:203-215 — per-dim negative wrap and bounds check."""
+    if len(index) > len(shape):
+        raise ValueError(f"Cannot index tensor with shape: {list(shape)} with index: {list(index)}")
+    out = []
+    for size, item in zip(shape, index):
+        n = size + item if item < 0 else item
+        if n < 0 or n >= size:
+            raise ValueError(f"Cannot index tensor with shape: {list(shape)} with index: {list(index)}")
+        out.append(n)
+    return out
+
+
+def store_index(shape: Sequence[int], index: Sequence[int]) -> int:
+    """Row-major offset of a full index (AbstractIndexing.kt:7-11,107-109)."""
+    idx = normalize_index(shape, index)
+    if len(idx) != len(shape):
+        raise ValueError(f"Index {list(index)} does not address a single element of shape {list(shape)}")
+    off = 0
+    for size, i in zip(shape, idx):
+        off = off * size + i
+    return off
+
+
+def outer_axis_inner(shape: Sequence[int], axis: int):
+    """The [outer, axis, inner] view of a row-major tensor around a normalised axis."""
+    return to_store_size(shape[:axis]), shape[axis], to_store_size(shape[axis + 1:])

@@ -1,0 +1,159 @@
+"""The five benchmark / parity workloads, written against the `Tensor` API exactly as a
+kten user would write them, so that the backend sees the raw-op sequences the reference's
+autograd layer emits. Each workload has: its input shapes, the seeded inputs, the
+computation, and the algorithmic bytes of the raw-op sequence (every operand counted once
+at its un-broadcast size plus the output, 4 bytes each, op at a time; in-place targets
+are counted as read + write).
+
+`dims` lets tests run the same workload at a size a CPU checker finishes in seconds.
+"""
+from dataclasses import dataclass
+from typing import Callable, Dict, List
+
+import numpy as np
+
+from .inputs import SplitMix64
+
+
+@dataclass
+class Workload:
+    name: str
+    description: str
+    full_dims: Dict[str, int]
+    make_inputs: Callable[[Dict[str, int]], Dict[str, np.ndarray]]
+    run: Callable            # (ops, inputs) -> dict name -> Tensor
+    algorithmic_bytes: Callable[[Dict[str, int]], int]
+
+
+# ---- 1: broadcast + full reduction ------------------------------------------------------
+
+def _in1(d):
+    g = SplitMix64(0)
+    return {"x": g.uniform([d["rows"], d["cols"]], -1.0, 1.0), "b": g.uniform([d["cols"]], -1.0, 1.0)}
+
+
+def _run1(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    b = ops.create(list(inp["b"].shape), False, inp["b"])
+    y = (x + b) * x
+    s = y.sum()
+    return {"y": y, "s": s}
+
+
+def _bytes1(d):
+    n, k = d["rows"] * d["cols"], d["cols"]
+    return 4 * (6 * n + k + 1)
+
+
+# ---- 2: unary chain -----------------------------------------------------------------------
+
+def _in2(d):
+    return {"x": SplitMix64(1).normal([d["n"]])}
+
+
+def _run2(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    z = (-(x ** 2)).exp() + (x.abs() + 1e-3).log()
+    return {"z": z}
+
+
+def _bytes2(d):
+    return 4 * 17 * d["n"]
+
+
+# ---- 3: axis reductions -------------------------------------------------------------------
+
+def _in3(d):
+    return {"x": SplitMix64(2).normal([d["rows"], d["cols"]])}
+
+
+def _run3(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    return {"sum0": x.sum(0), "sum1": x.sum(1), "mean0": x.mean(0), "mean1": x.mean(1),
+            "max1": x.max(1), "argmax1": x.argMax(1)}
+
+
+def _bytes3(d):
+    n = d["rows"] * d["cols"]
+    return 4 * (2 * (n + d["cols"]) + 4 * (n + d["rows"]))
+
+
+# ---- 4: channel broadcast + reduce over (0, 2, 3) ------------------------------------------
+
+def _in4(d):
+    g = SplitMix64(3)
+    n, c, h, w = d["n"], d["c"], d["h"], d["w"]
+    return {"act": g.uniform([n, c, h, w], -2.0, 2.0), "scale": g.uniform([1, c, 1, 1], 0.5, 1.5),
+            "bias": g.uniform([1, c, 1, 1], -0.1, 0.1)}
+
+
+def _run4(ops, inp):
+    act = ops.create(list(inp["act"].shape), False, inp["act"])
+    scale = ops.create(list(inp["scale"].shape), False, inp["scale"])
+    bias = ops.create(list(inp["bias"].shape), False, inp["bias"])
+    out = act * scale + bias
+    # the axis order in which the reference reduces a gradient to a [1,C,1,1] operand
+    s = out.sum(0, True).sum(2, True).sum(3, True)
+    m = out.mean(0, True).mean(2, True).mean(3, True)
+    return {"out": out, "sum": s, "mean": m}
+
+
+def _bytes4(d):
+    n, c, h, w = d["n"], d["c"], d["h"], d["w"]
+    full = n * c * h * w
+    chain = (full + c * h * w) + (c * h * w + c * w) + (c * w + c)
+    return 4 * (4 * full + 2 * c + 2 * chain)
+
+
+# ---- 5: autograd forward + backward --------------------------------------------------------
+
+def _in5(d):
+    g = SplitMix64(4)
+    return {"x": g.normal([d["rows"], d["cols"]]), "w": g.uniform([d["cols"]], -0.05, 0.05),
+            "b": g.uniform([1], -0.05, 0.05)}
+
+
+def cfg5_setup(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    w = ops.create(list(inp["w"].shape), True, inp["w"])
+    b = ops.create(list(inp["b"].shape), True, inp["b"])
+    return x, w, b
+
+
+def cfg5_step(x, w, b):
+    loss = (((x * w) + b) ** 2).sum()
+    loss.backward()
+    return loss
+
+
+def _run5(ops, inp):
+    x, w, b = cfg5_setup(ops, inp)
+    loss = cfg5_step(x, w, b)
+    return {"loss": loss, "grad_w": w.grad(), "grad_b": b.grad()}
+
+
+def _bytes5(d):
+    m, c = d["rows"] * d["cols"], d["cols"]
+    big = 22 * m                      # F1-F4, B1-B8: the passes over [rows, cols]
+    small = (2 * c                    # w read by x*w and g*w
+             + 1                      # b read by +b
+             + 1 + 1                  # sum() output, the [1] seed gradient read by broadcastTo
+             + c + (c + 1)            # sum(0) -> [cols] for b, then sum(0, keep) -> [1]
+             + c                      # sum(0) -> [cols] for w
+             + 3 * c + 3)             # gradient += g on w and b (read, read, write)
+    return 4 * (big + small)
+
+
+WORKLOADS: Dict[str, Workload] = {
+    "cfg1": Workload("cfg1", "y=(x+b)*x; sum(y): x[2048,1024], b[1024], U(-1,1), seed 0",
+                     {"rows": 2048, "cols": 1024}, _in1, _run1, _bytes1),
+    "cfg2": Workload("cfg2", "z=exp(-(x pow 2))+log(abs(x)+1e-3): x[2^26], N(0,1), seed 1",
+                     {"n": 1 << 26}, _in2, _run2, _bytes2),
+    "cfg3": Workload("cfg3", "sum/mean over axis 0 and 1, max and argmax over axis 1: x[8192,8192], N(0,1), seed 2",
+                     {"rows": 8192, "cols": 8192}, _in3, _run3, _bytes3),
+    "cfg4": Workload("cfg4", "act*scale+bias on NCHW [64,128,56,56] with [1,128,1,1] operands, then sum and mean "
+                             "over axes (0,2,3); seed 3",
+                     {"n": 64, "c": 128, "h": 56, "w": 56}, _in4, _run4, _bytes4),
+    "cfg5": Workload("cfg5", "loss=sum(((x*w)+b) pow 2); backward(): x[16384,4096], w[4096], b[1], seed 4",
+                     {"rows": 16384, "cols": 4096}, _in5, _run5, _bytes5),
+}

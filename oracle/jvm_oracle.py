@@ -1,0 +1,319 @@
+"""Python face of the CPU checker (test infrastructure; never imported by the library).
+
+`lib()` loads oracle/libkten_jvm_oracle.so (the C restatement of kten-jvm's arithmetic,
+kten_jvm_oracle.c) and `JvmOracleRawTensor` / `JvmOracleOperations` wrap it behind the
+same raw-tensor contract the HIP backend implements, so one graph written against the
+`Tensor` API can run on both and be compared. Only tests, the smoke check and the
+benchmark's CPU-baseline leg may import this module.
+"""
+import ctypes
+import os
+import subprocess
+from contextlib import contextmanager
+from ctypes import POINTER, c_double, c_float, c_int, c_int32, c_int64, c_void_p
+
+import numpy as np
+
+from kten_amd import shape_functions as sf
+from kten_amd.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libkten_jvm_oracle.so")
+_lib = None
+
+OPS = {"plus": 0, "minus": 1, "times": 2, "div": 3, "pow": 4, "reciprocal": 5, "log": 6,
+       "sum": 7, "mean": 8, "max": 9, "min": 10, "arg_max": 11, "arg_min": 12,
+       "lt": 13, "lte": 14, "gt": 15, "gte": 16, "eq": 17, "neq": 18,
+       "exp": 19, "tanh": 20, "sigmoid": 21, "sinh": 22, "cosh": 23, "abs": 24, "sign": 25, "sqrt": 26,
+       "sin": 27, "cos": 28, "tan": 29, "asin": 30, "acos": 31, "atan": 32, "floor": 33, "ceil": 34,
+       "round": 35, "trunc": 36, "rsqrt": 37, "neg": 40}
+_AGG = {AggregatingOperation.SUM: 7, AggregatingOperation.MEAN: 8, AggregatingOperation.MAX: 9,
+        AggregatingOperation.MIN: 10, AggregatingOperation.ARG_MAX: 11, AggregatingOperation.ARG_MIN: 12}
+
+
+def build():
+    subprocess.run(["make", "-C", _HERE], check=True, stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        build()
+    L = ctypes.CDLL(_SO)
+    fp, ip = c_void_p, POINTER(c_int32)
+    L.kjo_set_threads.argtypes = [c_int]
+    L.kjo_get_threads.restype = c_int
+    L.kjo_common_shape.argtypes = [ip, c_int, ip, c_int, ip]
+    L.kjo_common_shape.restype = c_int
+    L.kjo_broadcast_to.argtypes = [fp, ip, c_int, fp, ip, c_int]
+    L.kjo_broadcast_to.restype = c_int
+    L.kjo_binary_same.argtypes = [c_int, fp, fp, fp, c_int64, c_float]
+    L.kjo_binary.argtypes = [c_int, fp, ip, c_int, fp, ip, c_int, fp, ip, c_float]
+    L.kjo_binary.restype = c_int
+    L.kjo_binary_inplace.argtypes = [c_int, fp, fp, c_int64, c_float]
+    L.kjo_scalar.argtypes = [c_int, fp, c_float, c_int, fp, c_int64, c_float]
+    L.kjo_scalar_inplace.argtypes = [c_int, fp, c_float, c_int64]
+    L.kjo_unary.argtypes = [c_int, fp, fp, c_int64]
+    L.kjo_clamp.argtypes = [fp, fp, c_int64, c_float, c_float]
+    L.kjo_fill.argtypes = [fp, c_int64, c_float]
+    L.kjo_contains_nan.argtypes = [fp, c_int64]
+    L.kjo_contains_nan.restype = c_int
+    L.kjo_sum_all.argtypes = [fp, c_int64]
+    L.kjo_sum_all.restype = c_float
+    L.kjo_mean_all.argtypes = [fp, c_int64]
+    L.kjo_mean_all.restype = c_float
+    L.kjo_aggregate_over_axis.argtypes = [c_int, fp, fp, c_int64, c_int64, c_int64]
+    L.kjo_sum_all_f64.argtypes = [fp, c_int64]
+    L.kjo_sum_all_f64.restype = c_double
+    L.kjo_axis_sum_f64.argtypes = [fp, fp, fp, c_int64, c_int64, c_int64]
+    L.kjo_unary_f64.argtypes = [c_int, c_float]
+    L.kjo_unary_f64.restype = c_double
+    _lib = L
+    return L
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(c_void_p)
+
+
+def _sh(shape):
+    return (c_int32 * max(len(shape), 1))(*shape)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+# ---------------------------------------------------------------- array-level helpers
+
+def set_threads(n: int):
+    lib().kjo_set_threads(int(n))
+
+
+def unary(op: str, a) -> np.ndarray:
+    a = _f32(a); out = np.empty_like(a)
+    lib().kjo_unary(OPS[op], _p(a), _p(out), a.size)
+    return out
+
+
+def scalar(op: str, a, c: float, reverse=False, eps=1e-7) -> np.ndarray:
+    a = _f32(a); out = np.empty_like(a)
+    lib().kjo_scalar(OPS[op], _p(a), c, 1 if reverse else 0, _p(out), a.size, eps)
+    return out
+
+
+def clamp(a, lo: float, hi: float) -> np.ndarray:
+    a = _f32(a); out = np.empty_like(a)
+    lib().kjo_clamp(_p(a), _p(out), a.size, lo, hi)
+    return out
+
+
+def binary(op: str, a, b, eps=1e-7) -> np.ndarray:
+    """Broadcasting binary op; raises ValueError where the reference throws."""
+    a, b = _f32(a), _f32(b)
+    oshape = (c_int32 * 10)()
+    odims = lib().kjo_common_shape(_sh(a.shape), a.ndim, _sh(b.shape), b.ndim, oshape)
+    shape = [oshape[i] for i in range(odims)]
+    out = np.empty(shape, dtype=np.float32)
+    rc = lib().kjo_binary(OPS[op], _p(a), _sh(a.shape), a.ndim, _p(b), _sh(b.shape), b.ndim, _p(out), oshape, eps)
+    if rc < 0:
+        raise ValueError(f"Shapes {list(a.shape)} and {list(b.shape)} do not broadcast")
+    return out
+
+
+def broadcast_to(a, shape) -> np.ndarray:
+    a = _f32(a); out = np.empty(list(shape), dtype=np.float32)
+    if lib().kjo_broadcast_to(_p(a), _sh(a.shape), a.ndim, _p(out), _sh(shape), len(shape)) != 0:
+        raise ValueError(f"Tensor with shape: {list(a.shape)} cannot be broadcasted to shape: {list(shape)}")
+    return out
+
+
+def aggregate(op: str, a, axis: int) -> np.ndarray:
+    """aggregateOverAxis with keep-dims result shape."""
+    a = _f32(a)
+    outer, length, inner = sf.outer_axis_inner(list(a.shape), axis)
+    res_shape = list(a.shape); res_shape[axis] = 1
+    out = np.empty(res_shape, dtype=np.float32)
+    lib().kjo_aggregate_over_axis(OPS[op], _p(a), _p(out), outer, length, inner)
+    return out
+
+
+def sum_all(a) -> np.float32:
+    a = _f32(a)
+    return np.float32(lib().kjo_sum_all(_p(a), a.size))
+
+
+def mean_all(a) -> np.float32:
+    a = _f32(a)
+    return np.float32(lib().kjo_mean_all(_p(a), a.size))
+
+
+def sum_all_f64(a) -> float:
+    a = _f32(a)
+    return lib().kjo_sum_all_f64(_p(a), a.size)
+
+
+def axis_sum_f64(a, axis: int):
+    """(sum, sum of |x|) per lane in extended precision, keep-dims shape."""
+    a = _f32(a)
+    outer, length, inner = sf.outer_axis_inner(list(a.shape), axis)
+    res_shape = list(a.shape); res_shape[axis] = 1
+    out = np.empty(res_shape, dtype=np.float64); ab = np.empty(res_shape, dtype=np.float64)
+    lib().kjo_axis_sum_f64(_p(a), _p(out), _p(ab), outer, length, inner)
+    return out, ab
+
+
+def unary_f64(op: str, x: float) -> float:
+    return lib().kjo_unary_f64(OPS[op], x)
+
+
+# ---------------------------------------------------------------- the contract on the CPU
+
+class JvmOracleRawTensor(AbstractRawTensor):
+    """A FloatArray-backed raw tensor computing through the C restatement."""
+
+    def __init__(self, shape, store: np.ndarray, ops):
+        super().__init__(shape)
+        self.storeReference = store           # flat float32 array
+        self.ops = ops
+
+    def _wrap(self, arr: np.ndarray, shape=None):
+        return JvmOracleRawTensor(list(arr.shape) if shape is None else shape, arr.reshape(-1), self.ops)
+
+    def _nd(self) -> np.ndarray:
+        return self.storeReference.reshape(self.shape)
+
+    def broadcastTo(self, shape):
+        shape = list(shape)
+        if self.shape == shape:
+            return self
+        return self._wrap(broadcast_to(self._nd(), shape))
+
+    def _binary(self, op, other):
+        return self._wrap(binary(op, self._nd(), other._nd(), self.ops.epsilon))
+
+    def _binary_assign(self, op, other):
+        if self.shape != other.shape:
+            raise ValueError(
+                f"Shapes does not match for inplace operation on tensors with shapes: {self.shape} and {other.shape}.")
+        lib().kjo_binary_inplace(OPS[op], _p(self.storeReference), _p(other.storeReference),
+                                 self.storeReference.size, self.ops.epsilon)
+
+    def _scalar(self, op, constant, reverse=False):
+        return self._wrap(scalar(op, self.storeReference, constant, reverse, self.ops.epsilon), list(self.shape))
+
+    def _scalar_assign(self, op, constant):
+        lib().kjo_scalar_inplace(OPS[op], _p(self.storeReference), constant, self.storeReference.size)
+
+    def _compare(self, op, other):
+        if _is_number(other):
+            return self._scalar(op, float(other))
+        if self.storeReference.size != other.storeReference.size:
+            raise ValueError("Comparison needs equally sized tensors")
+        out = np.empty_like(self.storeReference)
+        lib().kjo_binary_same(OPS[op], _p(self.storeReference), _p(other.storeReference), _p(out), out.size,
+                              self.ops.epsilon)
+        return self._wrap(out, list(self.shape))
+
+    def _unary(self, op):
+        return self._wrap(unary(op, self.storeReference), list(self.shape))
+
+    def clamp(self, min, max):
+        return self._wrap(clamp(self.storeReference, min, max), list(self.shape))
+
+    def aggregateOverAxis(self, axis, resShape, aggregatingOperation):
+        outer, length, inner = sf.outer_axis_inner(self.shape, axis)
+        out = np.empty(sf.to_store_size(resShape), dtype=np.float32)
+        lib().kjo_aggregate_over_axis(_AGG[aggregatingOperation], _p(self.storeReference), _p(out), outer, length, inner)
+        return self._wrap(out, list(resShape))
+
+    def _sum_all(self):
+        return self._wrap(np.array([sum_all(self.storeReference)], dtype=np.float32))
+
+    def _mean_all(self):
+        return self._wrap(np.array([mean_all(self.storeReference)], dtype=np.float32))
+
+    def copy(self, shallow=False):
+        if shallow:
+            return JvmOracleRawTensor(list(self.shape), self.storeReference, self.ops)
+        return JvmOracleRawTensor(list(self.shape), self.storeReference.copy(), self.ops)
+
+    def view(self, shape):
+        return JvmOracleRawTensor(sf.reshape(self.shape, shape), self.storeReference, self.ops)
+
+    def getSingleValue(self, indexes):
+        return float(self.storeReference[sf.store_index(self.shape, list(indexes))])
+
+    def containsNan(self):
+        return bool(lib().kjo_contains_nan(_p(self.storeReference), self.storeReference.size))
+
+    def inplaceFill(self, value):
+        lib().kjo_fill(_p(self.storeReference), self.storeReference.size, value)
+
+    def toArray(self):
+        return self.storeReference.reshape(self.shape).copy()
+
+    def toList(self):
+        return self.storeReference.tolist()
+
+
+class JvmOracleOperations:
+    """The operations object of the CPU checker. Lifetime calls are no-ops, as on the
+    JVM backend (AbstractJVMTensorOperations.kt:73-79,90-92)."""
+
+    platformKey = "JVM-oracle"
+
+    def __init__(self):
+        lib()
+        self.epsilon = 1e-7
+
+    @contextmanager
+    def garbageCollector(self):
+        yield
+
+    def release(self, *rawTensors): pass
+    def incrementRef(self, rawTensor): pass
+    def markSurviveGC(self, rawTensor): pass
+    def markReleasableInGC(self, rawTensor): pass
+
+    def createRaw(self, shape, init=None):
+        shape = list(shape)
+        n = sf.to_store_size(shape)
+        if init is None:
+            store = np.zeros(n, dtype=np.float32)
+        elif callable(init):
+            store = np.fromiter((init(i) for i in range(n)), dtype=np.float32, count=n)
+        else:
+            store = np.array(init, dtype=np.float32).reshape(-1)
+            if store.size != n:
+                raise ValueError(f"init holds {store.size} values, shape {shape} needs {n}")
+        return JvmOracleRawTensor(shape, store, self)
+
+    def createRawFill(self, shape, constant):
+        return JvmOracleRawTensor(list(shape), np.full(sf.to_store_size(shape), constant, dtype=np.float32), self)
+
+    def zerosLike(self, rawTensor):
+        return self.createRawFill(rawTensor.shape, 0.0)
+
+    def zeroOut(self, rawTensor):
+        rawTensor.inplaceFill(0.0)
+
+    def pow(self, constant, rawTensor):
+        return rawTensor._scalar("pow", float(constant), reverse=True)
+
+    def create(self, shape, requiresGrad=False, init=None):
+        from kten_amd.autograd import NoGradVariable, Variable
+        raw = self.createRaw(shape, init)
+        return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
+
+    def createFillConst(self, shape, requiresGrad=False, constant=0.0):
+        from kten_amd.autograd import NoGradVariable, Variable
+        raw = self.createRawFill(shape, constant)
+        return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
+
+    def setEpsilon(self, eps):
+        self.epsilon = float(eps)
+
+    def sync(self): pass

@@ -1,0 +1,410 @@
+/*
+ * kten_jvm_oracle.c — CPU restatement of the kten-jvm backend's arithmetic for the
+ * broadcast-elementwise / reduction hot path.
+ *
+ * THIS IS TEST INFRASTRUCTURE. It is a checker: only tests, the smoke check and the
+ * CPU-baseline leg of the benchmark may load it. Nothing the library ships routes
+ * through it. It is written from the text of the reference's Kotlin sources (it is not
+ * the reference's code, and no JVM was run to produce it); every function cites the
+ * reference lines it follows, relative to the reference root:
+ *
+ *   JVM  = backend/kten-jvm/src/main/kotlin/eu/redbean/kten/jvm/tensor/store/JVMRawTensor.kt
+ *   OPS  = backend/kten-jvm/src/main/kotlin/eu/redbean/kten/jvm/tensor/operations/AbstractJVMTensorOperations.kt
+ *   RAW  = kten-api/src/main/kotlin/eu/redbean/kten/api/tensor/store/AbstractRawTensor.kt
+ *   IDX  = kten-api/src/main/kotlin/eu/redbean/kten/api/tensor/store/AbstractIndexing.kt
+ *
+ * Third-party arithmetic the reference delegates to (not under the reference tree):
+ * kotlin-stdlib 1.4.21 (FloatArray.sum/average, kotlin.math Float overloads) on top of
+ * java.lang.Math (JVM target 12). Their documented behaviour is restated here:
+ *   - kotlin.math.f(Float) = Math.f(x.toDouble()).toFloat()  -> f64 libm, round once to f32
+ *   - Float.pow(Float)     = Math.pow(double,double).toFloat() (Java special cases below)
+ *   - Math.max/min(float)  : NaN propagates, -0 < +0
+ *   - Math.round(float)    : floor(x + 1/2), NaN -> 0, saturating int, then int -> float
+ *   - Math.signum          : +-0 -> +-0, NaN -> NaN
+ *   - kotlin truncate      : NaN/inf pass, x > 0 ? floor : ceil
+ *
+ * Pinning status (what checks each group, see tests/test_oracle_*.py):
+ *   - index map, + - * / sqrt, compare, max/min/argmax/argmin, round/sign/trunc/floor/ceil:
+ *     pinned by the reference's own known-answer tests (tests/golden/known_answers.json)
+ *     and by brute-force / IEEE closed forms.
+ *   - exp log pow tanh sinh cosh sin cos tan asin acos atan at ULP granularity:
+ *     "parity unpinned" by the reference (its tests check six points at 1e-4 absolute);
+ *     pinned here only to the closed form (float)libm_f64((double)x) and those six points.
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -fopenmp).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+#include <stdlib.h>
+
+#define KJO_MAX_DIMS 10
+
+/* Operation codes: the numbering of the reference's OpenCL backend
+ * (backend/kten-opencl/.../platform/kernels/OCLKernelConstant.kt:4-43), plus NEG. */
+enum {
+    KJO_PLUS = 0, KJO_MINUS = 1, KJO_TIMES = 2, KJO_DIV = 3, KJO_POW = 4,
+    KJO_RECIPROCAL = 5, KJO_LOG = 6,
+    KJO_SUM = 7, KJO_MEAN = 8, KJO_MAX = 9, KJO_MIN = 10, KJO_ARG_MAX = 11, KJO_ARG_MIN = 12,
+    KJO_LT = 13, KJO_LTE = 14, KJO_GT = 15, KJO_GTE = 16, KJO_EQ = 17, KJO_NEQ = 18,
+    KJO_EXP = 19, KJO_TANH = 20, KJO_SIGMOID = 21, KJO_SINH = 22, KJO_COSH = 23, KJO_ABS = 24,
+    KJO_SIGN = 25, KJO_SQRT = 26, KJO_SIN = 27, KJO_COS = 28, KJO_TAN = 29, KJO_ASIN = 30,
+    KJO_ACOS = 31, KJO_ATAN = 32, KJO_FLOOR = 33, KJO_CEIL = 34, KJO_ROUND = 35, KJO_TRUNC = 36,
+    KJO_RSQRT = 37,
+    KJO_NEG = 40
+};
+
+static int g_threads = 1;
+
+/* Number of worker threads used by the operations the reference runs on a parallel
+ * stream (in-place maps JVM:95,106; axis aggregation JVM:219; zeroOut OPS:86-88).
+ * Copy-producing maps and full sum()/mean() are single-threaded in the reference
+ * (JVM:75-79,99-103,146-152) and stay so here regardless of this value. */
+void kjo_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+int kjo_get_threads(void) { return g_threads; }
+
+/* ---------------------------------------------------------------- Java scalar semantics */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+/* java.lang.Math.max(float,float): NaN if either is NaN; max(-0,+0) = +0. JVM:159 */
+static inline float jmax(float a, float b) {
+    if (a != a) return a;
+    if (a == 0.0f && b == 0.0f && f2u(a) == 0x80000000u) return b;
+    return (a >= b) ? a : b;
+}
+
+/* java.lang.Math.min(float,float): NaN if either is NaN; min(+0,-0) = -0. JVM:160 */
+static inline float jmin(float a, float b) {
+    if (a != a) return a;
+    if (a == 0.0f && b == 0.0f && f2u(b) == 0x80000000u) return b;
+    return (a <= b) ? a : b;
+}
+
+/* java.lang.Math.pow(double,double), then .toFloat(). JVM:138-140, OPS:94-96.
+ * Java differs from C99 pow in two documented cases: pow(x, NaN) is NaN even for
+ * x == 1, and pow(+-1, +-inf) is NaN. pow(x, +-0) is 1 in both. */
+static inline float jpow(float a, float b) {
+    double x = (double)a, y = (double)b;
+    if (y == 0.0) return 1.0f;
+    if (y != y) return (float)y;
+    if (isinf(y) && fabs(x) == 1.0) return NAN;
+    return (float)pow(x, y);
+}
+
+/* java.lang.Math.round(float) then Int.toFloat(). JVM:431.
+ * Spec: floor(a + 1/2) computed without intermediate rounding, NaN -> 0, results
+ * outside int range saturate. (double)a + 0.5 is exact for |a| < 2^23, and every
+ * |a| >= 2^23 is already an integer. */
+static inline float jround(float a) {
+    if (a != a) return 0.0f;
+    double r = floor((double)a + 0.5);
+    int32_t i;
+    if (r >= 2147483647.0) i = INT32_MAX;
+    else if (r <= -2147483648.0) i = INT32_MIN;
+    else i = (int32_t)r;
+    return (float)i;
+}
+
+/* java.lang.Math.signum(float). JVM:407 */
+static inline float jsignum(float a) {
+    if (a != a || a == 0.0f) return a;
+    return a > 0.0f ? 1.0f : -1.0f;
+}
+
+/* kotlin.math.truncate(Float). JVM:433 */
+static inline float ktruncate(float a) {
+    if (a != a || isinf(a)) return a;
+    return a > 0.0f ? (float)floor((double)a) : (float)ceil((double)a);
+}
+
+/* JVM:110-144 (binary lambdas), JVM:355-377 (comparisons; eq/neq use
+ * |a-b| < PlatformProvider.epsilon). */
+static inline float binary_op(int op, float a, float b, float eps) {
+    switch (op) {
+    case KJO_PLUS:  return a + b;
+    case KJO_MINUS: return a - b;
+    case KJO_TIMES: return a * b;
+    case KJO_DIV:   return a / b;
+    case KJO_POW:   return jpow(a, b);
+    case KJO_LT:    return a <  b ? 1.0f : 0.0f;
+    case KJO_LTE:   return a <= b ? 1.0f : 0.0f;
+    case KJO_GT:    return a >  b ? 1.0f : 0.0f;
+    case KJO_GTE:   return a >= b ? 1.0f : 0.0f;
+    case KJO_EQ:    return fabsf(a - b) < eps ? 1.0f : 0.0f;
+    case KJO_NEQ:   return fabsf(a - b) < eps ? 0.0f : 1.0f;
+    default:        return NAN;
+    }
+}
+
+/* JVM:122,142,144,395-435. Every kotlin.math Float overload is f64 libm rounded once. */
+static inline float unary_op(int op, float x) {
+    switch (op) {
+    case KJO_NEG:        return -x;                                   /* JVM:122 */
+    case KJO_RECIPROCAL: return 1.0f / x;                             /* JVM:142 */
+    case KJO_LOG:        return (float)log((double)x);                /* JVM:144 */
+    case KJO_EXP:        return (float)exp((double)x);                /* JVM:395 */
+    case KJO_TANH:       return (float)tanh((double)x);               /* JVM:397 */
+    case KJO_SIGMOID: {                                               /* JVM:399 */
+        float m = -1.0f * x;
+        float e = (float)exp((double)m);
+        float d = 1.0f + e;
+        return 1.0f / d;
+    }
+    case KJO_SINH:       return (float)sinh((double)x);               /* JVM:401 */
+    case KJO_COSH:       return (float)cosh((double)x);               /* JVM:403 */
+    case KJO_ABS:        return fabsf(x);                             /* JVM:405 */
+    case KJO_SIGN:       return jsignum(x);                           /* JVM:407 */
+    case KJO_SQRT:       return (float)sqrt((double)x);               /* JVM:413 */
+    case KJO_SIN:        return (float)sin((double)x);                /* JVM:415 */
+    case KJO_COS:        return (float)cos((double)x);                /* JVM:417 */
+    case KJO_TAN:        return (float)tan((double)x);                /* JVM:419 */
+    case KJO_ASIN:       return (float)asin((double)x);               /* JVM:421 */
+    case KJO_ACOS:       return (float)acos((double)x);               /* JVM:423 */
+    case KJO_ATAN:       return (float)atan((double)x);               /* JVM:425 */
+    case KJO_FLOOR:      return (float)floor((double)x);              /* JVM:427 */
+    case KJO_CEIL:       return (float)ceil((double)x);               /* JVM:429 */
+    case KJO_ROUND:      return jround(x);                            /* JVM:431 */
+    case KJO_TRUNC:      return ktruncate(x);                         /* JVM:433 */
+    case KJO_RSQRT: {                                                 /* JVM:435 */
+        float s = (float)sqrt((double)x);
+        return 1.0f / s;
+    }
+    default:             return NAN;
+    }
+}
+
+/* ---------------------------------------------------------------- shapes and broadcast */
+
+static int64_t store_size(const int32_t* shape, int dims) {          /* ShapeFunctions.kt:344 */
+    int64_t n = 1;
+    for (int i = 0; i < dims; i++) n *= shape[i];
+    return n;
+}
+
+/* RAW:170-192 calculateCommonShapeWith: right-align, copy the longer operand's extra
+ * leading dims, then per-dim max. No validity check happens here (it happens in
+ * broadcastTo). Returns the number of dims written to `out`. */
+int kjo_common_shape(const int32_t* a, int adims, const int32_t* b, int bdims, int32_t* out) {
+    int n = 0, diff = adims - bdims;
+    if (diff > 0) { for (int i = 0; i < diff; i++) out[n++] = a[i]; a += diff; adims -= diff; }
+    else if (diff < 0) { for (int i = 0; i < -diff; i++) out[n++] = b[i]; b += -diff; bdims += diff; }
+    for (int i = 0; i < adims; i++) out[n++] = a[i] > b[i] ? a[i] : b[i];
+    return n;
+}
+
+/* JVM:51-73 broadcastTo. Validity rule of ShapeFunctions.kt:187-201
+ * (inferExplicitBroadcastShape): source must not have more dims; after left-padding
+ * with 1s each dim must equal the target or be 1. Index rule JVM:62-70: target store
+ * index -> tensor index (IDX:111-121), each component taken modulo the padded source
+ * dim, then row-major offset in the padded source shape.
+ * Returns 0 on success, -1 if the shapes cannot broadcast (the reference throws
+ * IllegalArgumentException). */
+int kjo_broadcast_to(const float* src, const int32_t* sshape, int sdims,
+                     float* dst, const int32_t* dshape, int ddims) {
+    if (sdims > ddims || ddims > KJO_MAX_DIMS) return -1;
+    int32_t padded[KJO_MAX_DIMS];
+    int pad = ddims - sdims;
+    for (int i = 0; i < pad; i++) padded[i] = 1;
+    for (int i = 0; i < sdims; i++) padded[pad + i] = sshape[i];
+    for (int i = 0; i < ddims; i++)
+        if (!(padded[i] == dshape[i] || padded[i] == 1)) return -1;
+    int64_t n = store_size(dshape, ddims);
+    for (int64_t it = 0; it < n; it++) {
+        int64_t i = it, off = 0, stride = 1;
+        for (int d = ddims - 1; d >= 0; d--) {
+            int32_t idx = (int32_t)(i % dshape[d]);
+            i /= dshape[d];
+            off += (int64_t)(idx % padded[d]) * stride;
+            stride *= padded[d];
+        }
+        dst[it] = src[off];
+    }
+    return 0;
+}
+
+/* JVM:75-79 elementwiseOpOnCommonShapedTensors: same-size buffers, index order,
+ * single-threaded. */
+void kjo_binary_same(int op, const float* a, const float* b, float* out, int64_t n, float eps) {
+    for (int64_t i = 0; i < n; i++) out[i] = binary_op(op, a[i], b[i], eps);
+}
+
+/* JVM:81-87 elementwiseOpOnTensors: common shape, materialise both broadcasts, then
+ * the same-shape loop. `out` must hold the common shape's element count; the common
+ * shape is written to `oshape` and its dim count returned (or -1 when the operands do
+ * not broadcast). */
+int kjo_binary(int op, const float* a, const int32_t* ashape, int adims,
+               const float* b, const int32_t* bshape, int bdims,
+               float* out, int32_t* oshape, float eps) {
+    int odims = kjo_common_shape(ashape, adims, bshape, bdims, oshape);
+    int64_t n = store_size(oshape, odims);
+    float* ta = (float*)malloc(sizeof(float) * (size_t)(n ? n : 1));
+    float* tb = (float*)malloc(sizeof(float) * (size_t)(n ? n : 1));
+    int rc = -1;
+    if (ta && tb &&
+        kjo_broadcast_to(a, ashape, adims, ta, oshape, odims) == 0 &&
+        kjo_broadcast_to(b, bshape, bdims, tb, oshape, odims) == 0) {
+        kjo_binary_same(op, ta, tb, out, n, eps);
+        rc = odims;
+    }
+    free(ta); free(tb);
+    return rc;
+}
+
+/* JVM:89-97 inplaceElementwiseOpOnTensors (plusAssign JVM:114, timesAssign JVM:126).
+ * The caller has already checked the shapes are equal. Parallel stream in the
+ * reference; elements are independent so the result does not depend on threading. */
+void kjo_binary_inplace(int op, float* a, const float* b, int64_t n, float eps) {
+    #pragma omp parallel for num_threads(g_threads) if (g_threads > 1 && n > 65536)
+    for (int64_t i = 0; i < n; i++) a[i] = binary_op(op, a[i], b[i], eps);
+}
+
+/* JVM:99-103 mapElementsCopy with a constant: plus JVM:112, minus :120, times :128,
+ * div :134, pow :140, comparisons :379-393. reverse != 0 is constant-first, which the
+ * reference only has for pow (OPS:94-96). Single-threaded. */
+void kjo_scalar(int op, const float* a, float c, int reverse, float* out, int64_t n, float eps) {
+    if (reverse) for (int64_t i = 0; i < n; i++) out[i] = binary_op(op, c, a[i], eps);
+    else         for (int64_t i = 0; i < n; i++) out[i] = binary_op(op, a[i], c, eps);
+}
+
+/* JVM:105-108 inplaceMapElements: plusAssign(c) JVM:116, timesAssign(c) :130,
+ * divAssign(c) :136. Parallel stream in the reference. */
+void kjo_scalar_inplace(int op, float* a, float c, int64_t n) {
+    #pragma omp parallel for num_threads(g_threads) if (g_threads > 1 && n > 65536)
+    for (int64_t i = 0; i < n; i++) a[i] = binary_op(op, a[i], c, 0.0f);
+}
+
+/* JVM:99-103 mapElementsCopy with the unary lambdas of JVM:122,142,144,395-435. */
+void kjo_unary(int op, const float* a, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = unary_op(op, a[i]);
+}
+
+/* JVM:409-411 clamp = Math.min(Math.max(x, lo), hi). */
+void kjo_clamp(const float* a, float* out, int64_t n, float lo, float hi) {
+    for (int64_t i = 0; i < n; i++) out[i] = jmin(jmax(a[i], lo), hi);
+}
+
+/* JVM:533-535 inplaceFill; OPS:81-88 zerosLike / zeroOut are fills with 0. */
+void kjo_fill(float* a, int64_t n, float v) {
+    for (int64_t i = 0; i < n; i++) a[i] = v;
+}
+
+/* JVM:520-522 containsNan. */
+int kjo_contains_nan(const float* a, int64_t n) {
+    for (int64_t i = 0; i < n; i++) if (a[i] != a[i]) return 1;
+    return 0;
+}
+
+/* ---------------------------------------------------------------- reductions */
+
+/* JVM:146-148 sum() = kotlin FloatArray.sum(): float accumulator from 0f, index order. */
+float kjo_sum_all(const float* a, int64_t n) {
+    float acc = 0.0f;   /* built without -ffast-math: the adds stay in index order */
+    for (int64_t i = 0; i < n; i++) acc = acc + a[i];
+    return acc;
+}
+
+/* JVM:150-152 mean() = FloatArray.average().toFloat(): double accumulator, index
+ * order, divided by the count, rounded once. Empty array gives NaN. */
+float kjo_mean_all(const float* a, int64_t n) {
+    if (n == 0) return NAN;
+    double acc = 0.0;
+    for (int64_t i = 0; i < n; i++) acc = acc + (double)a[i];
+    return (float)(acc / (double)n);
+}
+
+/* One output lane of JVM:154-209 mapAggregatingOp: element j of the lane lives at
+ * base + j*inner. */
+static float aggregate_lane(int op, const float* base, int64_t axis, int64_t inner) {
+    switch (op) {
+    case KJO_ARG_MAX: case KJO_ARG_MIN: {                              /* JVM:167-184 */
+        float temp = (op == KJO_ARG_MAX) ? -INFINITY : INFINITY;
+        float agg = 0.0f;
+        for (int64_t j = 0; j < axis; j++) {
+            float cur = base[j * inner];
+            if ((op == KJO_ARG_MAX && cur > temp) || (op == KJO_ARG_MIN && cur < temp)) {
+                temp = cur;
+                agg = (float)(int32_t)j;
+            }
+        }
+        return agg;
+    }
+    case KJO_MEAN: {                                                   /* JVM:185-192 */
+        float agg = 0.0f;
+        for (int64_t j = 0; j < axis; j++) agg = agg + base[j * inner];
+        return agg / (float)(int32_t)axis;
+    }
+    case KJO_MAX: {                                                    /* JVM:193-207 */
+        float agg = -INFINITY;
+        for (int64_t j = 0; j < axis; j++) agg = jmax(agg, base[j * inner]);
+        return agg;
+    }
+    case KJO_MIN: {
+        float agg = INFINITY;
+        for (int64_t j = 0; j < axis; j++) agg = jmin(agg, base[j * inner]);
+        return agg;
+    }
+    case KJO_SUM: {
+        float agg = 0.0f;
+        for (int64_t j = 0; j < axis; j++) agg = agg + base[j * inner];
+        return agg;
+    }
+    default: return NAN;
+    }
+}
+
+/* JVM:211-225 aggregateOverAxis on a row-major tensor seen as [outer, axis, inner]
+ * (outer = product of dims before the axis, inner = product after); the result is
+ * [outer, 1, inner]. Parallel over outputs in the reference. */
+void kjo_aggregate_over_axis(int op, const float* in, float* out,
+                             int64_t outer, int64_t axis, int64_t inner) {
+    int64_t n_out = outer * inner;
+    #pragma omp parallel for num_threads(g_threads) if (g_threads > 1 && n_out > 1) schedule(static)
+    for (int64_t o = 0; o < n_out; o++) {
+        int64_t oi = o / inner, ii = o % inner;
+        out[o] = aggregate_lane(op, in + oi * axis * inner + ii, axis, inner);
+    }
+}
+
+/* ---------------------------------------------------------------- float64 references
+ * Not a restatement of anything in the reference: the yardstick the reduction
+ * tolerance is defined against (sum and mean in extended precision, per lane). */
+
+double kjo_sum_all_f64(const float* a, int64_t n) {
+    long double acc = 0.0L;
+    for (int64_t i = 0; i < n; i++) acc += (long double)a[i];
+    return (double)acc;
+}
+
+/* Also returns sum |x| per lane in abs_out (may be NULL) for error normalisation. */
+void kjo_axis_sum_f64(const float* in, double* out, double* abs_out,
+                      int64_t outer, int64_t axis, int64_t inner) {
+    int64_t n_out = outer * inner;
+    #pragma omp parallel for num_threads(g_threads) if (g_threads > 1 && n_out > 1) schedule(static)
+    for (int64_t o = 0; o < n_out; o++) {
+        int64_t oi = o / inner, ii = o % inner;
+        const float* base = in + oi * axis * inner + ii;
+        long double acc = 0.0L, aacc = 0.0L;
+        for (int64_t j = 0; j < axis; j++) {
+            long double v = (long double)base[j * inner];
+            acc += v;
+            aacc += v < 0 ? -v : v;
+        }
+        out[o] = (double)acc;
+        if (abs_out) abs_out[o] = (double)aacc;
+    }
+}
+
+/* Correctly-rounded-in-double reference value of a unary op at x, before the final
+ * rounding to float: used to measure ULP distance of device results. Ops whose float
+ * result is exact by construction return that float widened. */
+double kjo_unary_f64(int op, float x) {
+    double d = (double)x;
+    switch (op) {
+    case KJO_LOG: return log(d);   case KJO_EXP: return exp(d);   case KJO_TANH: return tanh(d);
+    case KJO_SINH: return sinh(d); case KJO_COSH: return cosh(d); case KJO_SIN: return sin(d);
+    case KJO_COS: return cos(d);   case KJO_TAN: return tan(d);   case KJO_ASIN: return asin(d);
+    case KJO_ACOS: return acos(d); case KJO_ATAN: return atan(d);
+    default: return (double)unary_op(op, x);
+    }
+}
