@@ -1,0 +1,276 @@
+"""The reference's own known-answer tests for the hot path, written once against the
+`Tensor` API and run on any backend (`ops`): the CPU checker in the CPU suite, the HIP
+backend in the GPU suite. Each case follows the reference test named in the fixture's
+`cite` field (tests/golden/known_answers.json); expected values and tolerances are the
+reference's.
+"""
+import json
+import os
+
+import numpy as np
+
+from kten_amd.autograd import ones, tensorOf
+
+with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
+    K = json.load(f)
+
+
+def T(ops, spec, requiresGrad=False):
+    t = tensorOf(ops, *spec["values"]).reshape(spec["shape"])
+    return t.asVariable(requiresGrad=True) if requiresGrad else t
+
+
+def filled(ops, value, shape, requiresGrad=True):
+    return tensorOf(ops, value).expand(shape).asVariable(requiresGrad=requiresGrad)
+
+
+def assertTensorEquals(expected, actual, tolerance=1e-6, shape=None):
+    """TestUtils.kt:9-29 — equal shapes, elementwise absolute tolerance."""
+    a = actual.toArray() if hasattr(actual, "toArray") else np.asarray(actual, dtype=np.float32)
+    if isinstance(expected, dict):
+        shape, expected = expected["shape"], expected["values"]
+    e = np.asarray(expected, dtype=np.float32)
+    if e.ndim == 0:
+        e = np.full(a.shape, e, dtype=np.float32)
+    if shape is not None:
+        assert list(a.shape) == list(shape), f"shape {list(a.shape)} != {list(shape)}"
+    e = e.reshape(a.shape)
+    assert np.all(np.abs(e - a) <= np.float32(tolerance)), f"expected {e.tolist()} but was {a.tolist()}"
+
+
+def case_addition(ops):
+    c = K["addition"]
+    assertTensorEquals(c["expected"], T(ops, c["t1"]) + T(ops, c["t2"]), c["tol"])
+
+
+def case_mse_and_grads(ops):
+    c = K["mse_and_grads"]
+    t1, t2 = T(ops, c["t1"], True), T(ops, c["t2"], True)
+    error = ((t1 - t2) ** 2.0).mean()
+    error.backward()
+    assertTensorEquals(c["error"], error, c["tol"], [1])
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], [2, 3])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], [2, 3])
+
+
+def case_max_last_axis_4d(ops):
+    c = K["max_last_axis_4d"]
+    assertTensorEquals(c["expected"], T(ops, c["t1"]).max(axis=-1), c["tol"])
+
+
+def case_broadcasting_addition_with_grads(ops):
+    c = K["broadcasting_addition_with_grads"]
+    t1, t2 = filled(ops, c["t1_fill"], c["t1_shape"]), filled(ops, c["t2_fill"], c["t2_shape"])
+    summary = ((t1 + t2) ** 2).sum()
+    assert summary.item() == c["summary"]
+    summary.backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_shape"])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], c["t2_shape"])
+
+
+def case_broadcasting_minus_with_grads(ops):
+    c = K["broadcasting_minus_with_grads"]
+    t1 = filled(ops, c["t1_fill"], c["t1_shape"])
+    t2 = tensorOf(ops, c["t2_value"], requiresGrad=True)
+    res = (t1 - t2).sum()
+    assert res.item() == c["res"]
+    res.backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_shape"])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], [1])
+
+
+def case_tensor_constant_addition(ops):
+    c = K["tensor_constant_addition"]
+    t1 = T(ops, c["t1"], True)
+    tc, ct = t1 + c["constant"], c["constant"] + t1
+    assertTensorEquals(c["expected"], tc, c["tol"], c["t1"]["shape"])
+    assertTensorEquals(c["expected"], ct, c["tol"], c["t1"]["shape"])
+    tc.sum().backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"])
+    t1.zeroGrad()
+    ct.sum().backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"])
+
+
+def case_tensor_constant_minus(ops):
+    c = K["tensor_constant_minus"]
+    t1 = T(ops, c["t1"], True)
+    tc, ct = t1 - c["constant"], c["constant"] - t1
+    assertTensorEquals(c["expected_tc"], tc, c["tol"], c["t1"]["shape"])
+    assertTensorEquals(c["expected_ct"], ct, c["tol"], c["t1"]["shape"])
+    tc.sum().backward()
+    assertTensorEquals(c["grad_tc"], t1.grad(), c["tol"])
+    t1.zeroGrad()
+    ct.sum().backward()
+    assertTensorEquals(c["grad_ct"], t1.grad(), c["tol"])
+
+
+def case_tensor_times_tensor(ops):
+    c = K["tensor_times_tensor"]
+    t1, t2 = filled(ops, c["t1_fill"], c["t1_shape"]), filled(ops, c["t2_fill"], c["t2_shape"])
+    res = (t1 * t2).sum()
+    assert res.item() == c["res"]
+    res.backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_shape"])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], c["t2_shape"])
+
+
+def case_tensor_div_tensor(ops):
+    c = K["tensor_div_tensor"]
+    t1, t2 = filled(ops, c["t1_fill"], c["t1_shape"]), filled(ops, c["t2_fill"], c["t2_shape"])
+    res = (t1 / t2).sum()
+    assert res.item() == c["res"]
+    res.backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_shape"])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], c["t2_shape"])
+
+
+def case_tensor_constant_times(ops):
+    c = K["tensor_constant_times"]
+    t1 = T(ops, c["t1"], True)
+    tc, ct = t1 * c["constant"], c["constant"] * t1
+    assertTensorEquals(c["expected"], tc, c["tol"], c["t1"]["shape"])
+    assertTensorEquals(c["expected"], ct, c["tol"], c["t1"]["shape"])
+    tc.sum().backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"])
+    t1.zeroGrad()
+    ct.sum().backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"])
+
+
+def case_tensor_constant_div(ops):
+    c = K["tensor_constant_div"]
+    t1 = T(ops, c["t1"], True)
+    tc, ct = t1 / c["constant"], c["constant"] / t1
+    assertTensorEquals(c["expected_tc"], tc, c["tol"], c["t1"]["shape"])
+    assertTensorEquals(c["expected_ct"], ct, c["tol"], c["t1"]["shape"])
+    tc.sum().backward()
+    assertTensorEquals(c["grad_tc"], t1.grad(), c["tol"])
+    t1.zeroGrad()
+    ct.sum().backward()
+    assertTensorEquals(c["grad_ct"], t1.grad(), c["tol"])
+
+
+def case_tensor_pow_tensor(ops):
+    c = K["tensor_pow_tensor"]
+    t1, t2 = T(ops, c["t1"], True), T(ops, c["t2"], True)
+    res = (t1 ** t2).sum()
+    assert res.item() == c["res"]
+    res.backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1"]["shape"])
+    # The expected values are near 15 and 89, where an fp32 ulp is 1e-6 and 8e-6: the
+    # reference's 1e-6 absolute tolerance admits only the exact float.
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], c["t2"]["shape"])
+
+
+def case_constant_tensor_pow(ops):
+    c = K["constant_tensor_pow"]
+    t1 = T(ops, c["t1"], True)
+    res = c["constant"] ** t1
+    assertTensorEquals(c["expected"], res, c["tol"], c["t1"]["shape"])
+    res.sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["grad_tol"], c["t1"]["shape"])
+
+
+def _axis_case(ops, name, method):
+    c = K[name]
+    t1 = T(ops, c["t1"], True)
+    res = getattr(t1, method)(axis=c["axis"], keepDimensions=c["keep"])
+    assertTensorEquals(c["expected"], res, c["tol"])
+    res.backward(tensorOf(ops, c["backward_fill"]).expand(c["expected"]["shape"]))
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"], c["t1"]["shape"])
+
+
+def case_sum_over_axis(ops): _axis_case(ops, "sum_over_axis", "sum")
+def case_sum_over_axis_keep_dims(ops): _axis_case(ops, "sum_over_axis_keep_dims", "sum")
+def case_mean_over_axis(ops): _axis_case(ops, "mean_over_axis", "mean")
+def case_mean_over_axis_keep_dims(ops): _axis_case(ops, "mean_over_axis_keep_dims", "mean")
+
+
+def case_max_min_over_axis(ops):
+    # Forward values only: the gradients of Max/Min go through inplaceScatter, which is
+    # outside this backend's accelerated path.
+    c = K["max_min_over_axis"]
+    t1 = T(ops, c["t1"])
+    assertTensorEquals(c["max_last"], t1.max(axis=-1), c["tol"])
+    assertTensorEquals(c["max_0_keep"], t1.max(axis=0, keepDimensions=True), c["tol"])
+    assertTensorEquals(c["min_last"], t1.min(axis=-1), c["tol"])
+    assertTensorEquals(c["min_0_keep"], t1.min(axis=0, keepDimensions=True), c["tol"])
+    # What the scatter of Max.doBackward would produce follows from argMax alone: a one
+    # at the arg index of every lane. This pins ties -> lowest index.
+    for key, idx, axis in (("max_0_keep_grad", t1.argMax(0, True), 0), ("max_last_grad", t1.argMax(-1, True), 1),
+                           ("min_0_keep_grad", t1.argMin(0, True), 0), ("min_last_grad", t1.argMin(-1, True), 1)):
+        grad = np.zeros((3, 3), dtype=np.float32)
+        np.put_along_axis(grad, idx.toArray().astype(np.int64), 1.0, axis=axis)
+        assertTensorEquals(c[key], grad, c["tol"], [3, 3])
+
+
+def case_argmax_argmin(ops):
+    c = K["argmax_argmin"]
+    t1 = T(ops, c["t1"])
+    assertTensorEquals(c["argmax_last"], t1.argMax(axis=-1), c["tol"])
+    assertTensorEquals(c["argmax_0_keep"], t1.argMax(axis=0, keepDimensions=True), c["tol"])
+    assertTensorEquals(c["argmin_last"], t1.argMin(axis=-1), c["tol"])
+    assertTensorEquals(c["argmin_0_keep"], t1.argMin(axis=0, keepDimensions=True), c["tol"])
+
+
+def case_exp_with_grads(ops):
+    c = K["exp_with_grads"]
+    t1 = tensorOf(ops, *c["input"]).reshape(2, 3).asVariable(requiresGrad=True)
+    res = t1.exp()
+    assertTensorEquals(c["expected"], res, c["tol"], [2, 3])
+    res.mean().backward()
+    assertTensorEquals(c["grads_after_mean_backward"], t1.grad(), c["tol"], [2, 3])
+
+
+def _elementwise(ops, name):
+    e = K["elementwise"]
+    c = e["ops"][name]
+    t1 = tensorOf(ops, *c["input"]).reshape(2, 3).asVariable(requiresGrad=True)
+    if name == "clamp":
+        res = t1.clamp(*c["args"])
+    elif name.startswith("reciprocal_"):
+        res = getattr(t1.reciprocal(), name.split("_", 1)[1])()
+    else:
+        res = getattr(t1, name)()
+    assertTensorEquals(c["expected"], res, e["tol"], e["shape"])
+    res.sum().backward()
+    assertTensorEquals(c["grads"], t1.grad(), e["tol"], e["shape"])
+
+
+ELEMENTWISE_NAMES = sorted(K["elementwise"]["ops"].keys())
+
+
+def case_expand_with_grad(ops):
+    c = K["expand_with_grad"]
+    t1 = tensorOf(ops, c["value"], requiresGrad=True)
+    t1.expand(*c["shape"]).sum().backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"], [1])
+
+
+def case_long_graph_output_reuse(ops):
+    c = K["long_graph_output_reuse"]
+    t1 = ones(ops, *c["shape"]).asVariable(requiresGrad=True)
+    t2 = ones(ops, *c["shape"]).asVariable(requiresGrad=True)
+    a, b, cc = t1 + 2.0, t2 + 2.0, t1 + 2.0
+    add1 = a + b
+    add2 = add1 + cc
+    for _ in range(4):
+        a = a * 2.0
+        b = b * 2.0
+        cc = cc * 2.0
+    branch = a + b + cc
+    out = add2 + branch
+    out.backward(ones(ops, *c["shape"]))
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["shape"])
+    assertTensorEquals(c["t2_grad"], t2.grad(), c["tol"], c["shape"])
+
+
+def case_readme_sum_of_squares(ops):
+    c = K["readme_sum_of_squares"]
+    t = T(ops, c["t1"], True)
+    (t ** 2).sum().backward()
+    assertTensorEquals(c["grad"], t.grad(), c["tol"], c["t1"]["shape"])
+
+
+CASES = [v for k, v in sorted(globals().items()) if k.startswith("case_")]

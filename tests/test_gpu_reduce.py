@@ -1,0 +1,125 @@
+"""Parity of the reduction kernels with the CPU checker, through the C ABI.
+MAX / MIN / ARG_MAX / ARG_MIN: bit-exact. SUM / MEAN: the two-clause tolerance of
+parity.py against the extended-precision sum, with the checker's own serial-float
+error as the second clause."""
+import numpy as np
+import pytest
+
+from oracle import jvm_oracle as jo
+from parity import assert_bits_equal, assert_reduction_close
+
+pytestmark = pytest.mark.gpu
+
+# [shape, axis]: chosen to hit every kernel variant — rows with 1/4/16/64/256 lanes per
+# row, aligned and unaligned; columns with float4 and scalar lanes, with and without
+# axis segmentation; the strided kernel for small inner sizes.
+GEOMETRIES = [
+    ([7], 0), ([1000], 0), ([4099], 0), ([300000], 0), ([1 << 21], 0),
+    ([5, 3], 1), ([100, 7], 1), ([64, 40], 1), ([50, 200], 1), ([9, 1000], 1), ([3, 5000], 1), ([2, 100001], 1),
+    ([2, 70000], 1), ([3000, 16], 1), ([1000, 33], 1),
+    ([8, 64], 0), ([100, 256], 0), ([5000, 128], 0), ([70000, 64], 0), ([333, 1000], 0), ([40000, 65], 0),
+    ([4, 50, 64], 1), ([3, 2000, 68], 1), ([2, 3, 4], 0), ([2, 3, 4], 1), ([6, 30000, 5], 1), ([10, 56, 56], 1),
+    ([128, 56, 56], 1), ([64, 16, 49], 0), ([3, 17, 1, 9], 1), ([2, 2, 2, 2, 2, 2, 2, 2, 2, 5], 4),
+]
+OPS = ["sum", "mean", "max", "min", "argMax", "argMin"]
+CODE = {"sum": "sum", "mean": "mean", "max": "max", "min": "min", "argMax": "arg_max", "argMin": "arg_min"}
+
+
+def raw(gc, a):
+    return gc.createRaw(list(a.shape), a)
+
+
+@pytest.mark.parametrize("shape,axis", GEOMETRIES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_axis_reductions(shape, axis, gc):
+    rng = np.random.default_rng(len(shape) * 1000 + shape[0] + axis)
+    x = rng.standard_normal(shape).astype(np.float32)
+    # ties for the arg ops: quantise a slice
+    flat = x.reshape(-1)
+    flat[::3] = np.round(flat[::3] * 2) / 2
+    t = raw(gc, x)
+    ref64, _ = jo.axis_sum_f64(x, axis)
+    for op in OPS:
+        for keep in (False, True):
+            res = getattr(t, op)(axis, keep)
+            want_shape = list(shape); want_shape[axis] = 1
+            if not keep and len(shape) > 1:
+                del want_shape[axis]
+            assert res.shape == want_shape
+            got = res.toArray().reshape(-1)
+            want = jo.aggregate(CODE[op], x, axis).reshape(-1)
+            if op == "sum":
+                assert_reduction_close(got, ref64, want, f"sum {shape} axis {axis}")
+            elif op == "mean":
+                assert_reduction_close(got, ref64 / shape[axis], want, f"mean {shape} axis {axis}")
+            else:
+                assert_bits_equal(got, want, f"{op} {shape} axis {axis}")
+
+
+@pytest.mark.parametrize("shape,axis", [([64, 40], 1), ([9, 1000], 1), ([3, 5000], 1), ([333, 1000], 0), ([4, 50, 64], 1),
+                                        ([6, 3000, 5], 1), ([2, 70000], 1), ([70000, 64], 0)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_special_values_in_reductions(shape, axis, gc):
+    """NaN propagation in max/min, NaN skipping in arg ops, signed zeros, lanes of -inf / +inf, ties."""
+    rng = np.random.default_rng(7)
+    lanes = int(np.prod(shape)) // shape[axis]
+    m = rng.integers(-2, 3, size=(shape[axis], lanes)).astype(np.float32)     # [axis, lane]: heavy ties, many zeros
+    flat = m.reshape(-1)
+    idx = rng.choice(flat.size, size=max(4, flat.size // 50), replace=False)
+    flat[idx[0::4]] = np.nan
+    flat[idx[1::4]] = -0.0
+    flat[idx[2::4]] = np.inf
+    flat[idx[3::4]] = -np.inf
+    m[:, 0] = -np.inf                                                          # a lane with nothing > -inf
+    m[:, -1] = np.where(np.arange(shape[axis]) % 2 == 0, 0.0, -0.0)            # a lane of signed zeros only
+    m[:, lanes // 2] = np.nan                                                  # a lane of NaNs only
+    rest = [d for i, d in enumerate(shape) if i != axis]
+    x = np.ascontiguousarray(np.moveaxis(m.reshape([shape[axis]] + rest), 0, axis))
+    t = raw(gc, x)
+    for op in ("max", "min", "argMax", "argMin"):
+        assert_bits_equal(getattr(t, op)(axis).toArray().reshape(-1), jo.aggregate(CODE[op], x, axis).reshape(-1),
+                          f"{op} {shape} axis {axis}")
+
+
+@pytest.mark.parametrize("n", [1, 2, 5, 1000, 4099, 300001, 1 << 22])
+def test_full_sum_and_mean(n, gc):
+    x = (np.random.default_rng(n).standard_normal(n) * 10 + 0.5).astype(np.float32)
+    t = raw(gc, x)
+    ref = jo.sum_all_f64(x)
+    s, m = t.sum(), t.mean()
+    assert s.shape == [1] and m.shape == [1]
+    assert_reduction_close(s.toArray(), [ref], [jo.sum_all(x)], f"sum() n={n}")
+    assert_reduction_close(m.toArray(), [ref / n], [jo.mean_all(x)], f"mean() n={n}")
+    # mean() accumulates in f64 on both sides: it should be the correctly rounded mean
+    assert abs(float(m.toArray()[0]) - ref / n) <= abs(ref / n) * 2 ** -23
+
+
+def test_sum_of_cancelling_terms_is_exact_in_f64(gc):
+    # kten-jvm's serial float sum returns 0 here; the true sum is 1 and f64 accumulation finds it.
+    x = np.array([1e8, 1.0, -1e8], np.float32)
+    assert raw(gc, x).sum().toArray()[0] == 1.0
+    y = np.array([16777216.0] + [1.0] * 64, np.float32)
+    assert raw(gc, y).sum().toArray()[0] == np.float32(16777216.0 + 64.0)
+    assert raw(gc, y).mean().toArray()[0] == jo.mean_all(y)
+
+
+def test_reductions_are_deterministic(gc):
+    x = np.random.default_rng(11).standard_normal((3000, 700)).astype(np.float32)
+    t = raw(gc, x)
+    for axis in (0, 1):
+        a = t.sum(axis).toArray(); b = t.sum(axis).toArray()
+        assert_bits_equal(a, b, f"sum axis {axis} twice")
+    a = t.sum().toArray(); b = t.sum().toArray()
+    assert_bits_equal(a, b, "sum() twice")
+
+
+def test_reduce_to_shape_matches_numpy(gc):
+    """mayUnexpand = numpy.sum over the broadcast axes with keepdims, reshaped to the operand."""
+    from kten_amd.autograd import mayUnexpand
+    rng = np.random.default_rng(13)
+    for gshape, oshape, axes in [([6, 40, 7, 9], [1, 40, 1, 1], (0, 2, 3)), ([50, 30], [30], (0,)), ([50, 30], [1], (0, 1)),
+                                 ([4, 5, 6], [5, 1], (0, 2)), ([3, 3], [3, 1], (1,))]:
+        g = rng.standard_normal(gshape).astype(np.float32)
+        res = mayUnexpand(raw(gc, g), oshape, gc)
+        assert res.shape == oshape
+        ref = g.astype(np.float64).sum(axes, keepdims=True).reshape(oshape)
+        np.testing.assert_allclose(res.toArray(), ref, rtol=1e-5, atol=1e-5)

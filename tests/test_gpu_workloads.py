@@ -1,0 +1,209 @@
+"""The five benchmark configurations through the `Tensor` API on the HIP backend.
+
+Scaled-down shapes are compared with the CPU checker running the very same graph.
+Full BASELINE shapes are checked through what does not need the serial CPU restatement
+of every pass: numpy closed forms for single-rounding ops, float64 references for the
+reductions (plus the checker's own error on the reductions, which it can do in seconds),
+argmax against numpy on tie-free data."""
+import numpy as np
+import pytest
+
+from kten_amd.workloads import WORKLOADS
+from oracle import jvm_oracle as jo
+from parity import assert_bits_equal, assert_reduction_close, assert_ulp_close, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+SMALL = {"cfg1": {"rows": 96, "cols": 200}, "cfg2": {"n": 100003}, "cfg3": {"rows": 300, "cols": 520},
+         "cfg4": {"n": 6, "c": 16, "h": 12, "w": 20}, "cfg5": {"rows": 512, "cols": 384}}
+
+
+def run_both(name, dims, gc):
+    wl = WORKLOADS[name]
+    inputs = wl.make_inputs(dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inputs).items()}
+    want = {k: v.toArray() for k, v in wl.run(jo.JvmOracleOperations(), inputs).items()}
+    return inputs, got, want
+
+
+def test_cfg1_small(gc):
+    inp, got, want = run_both("cfg1", SMALL["cfg1"], gc)
+    assert_bits_equal(got["y"], want["y"], "y")
+    assert_reduction_close(got["s"], [jo.sum_all_f64(want["y"])], want["s"], "s")
+
+
+def test_cfg2_small(gc):
+    inp, got, want = run_both("cfg2", SMALL["cfg2"], gc)
+    # z = e + l: each addend is within 2 ulp of the checker's, so z is within a few ulp of
+    # the larger addend; the per-op bars are checked in test_gpu_elementwise.
+    assert_ulp_close(got["z"], want["z"], 2, "z")
+
+
+def test_cfg3_small(gc):
+    inp, got, want = run_both("cfg3", SMALL["cfg3"], gc)
+    x = inp["x"]
+    for axis in (0, 1):
+        ref, _ = jo.axis_sum_f64(x, axis)
+        assert_reduction_close(got[f"sum{axis}"], ref, want[f"sum{axis}"], f"sum{axis}")
+        assert_reduction_close(got[f"mean{axis}"], ref / x.shape[axis], want[f"mean{axis}"], f"mean{axis}")
+    assert_bits_equal(got["max1"], want["max1"], "max1")
+    assert_bits_equal(got["argmax1"], want["argmax1"], "argmax1")
+
+
+def test_cfg4_small(gc):
+    inp, got, want = run_both("cfg4", SMALL["cfg4"], gc)
+    assert_bits_equal(got["out"], want["out"], "out")
+    ref = want["out"].astype(np.float64).sum((0, 2, 3), keepdims=True)
+    n = want["out"].size // want["out"].shape[1]
+    assert got["sum"].shape == (1, SMALL["cfg4"]["c"], 1, 1)
+    assert_reduction_close(got["sum"], ref, want["sum"], "sum(0,2,3)")
+    assert_reduction_close(got["mean"], ref / n, want["mean"], "mean(0,2,3)")
+
+
+def test_cfg5_small(gc):
+    inp, got, want = run_both("cfg5", SMALL["cfg5"], gc)
+    x, w, b = (inp[k].astype(np.float64) for k in ("x", "w", "b"))
+    # the reference values follow the fp32 intermediates the graph really produces
+    t32 = (inp["x"] * inp["w"]) + inp["b"]
+    g32 = (np.float32(2.0) * np.ones_like(t32)) * t32
+    assert_reduction_close(got["loss"], [(t32 * t32).astype(np.float64).sum()], want["loss"], "loss")
+    assert_reduction_close(got["grad_w"], (g32 * inp["x"]).astype(np.float64).sum(0), want["grad_w"], "grad w")
+    assert_reduction_close(got["grad_b"], [g32.astype(np.float64).sum()], want["grad_b"], "grad b")
+    # and are close to the exact mathematics
+    t = x * w + b
+    np.testing.assert_allclose(got["loss"], [(t * t).sum()], rtol=1e-5)
+    np.testing.assert_allclose(got["grad_w"], (2 * t * x).sum(0), rtol=1e-4, atol=1e-4)
+
+
+def test_cfg5_raw_op_sequence_intermediates_bit_exact(gc):
+    """The elementwise passes of the forward and backward graph, op by op (bit-exact)."""
+    inp = WORKLOADS["cfg5"].make_inputs(SMALL["cfg5"])
+    cpu = jo.JvmOracleOperations()
+    outs = []
+    for ops in (gc, cpu):
+        x = ops.createRaw(list(inp["x"].shape), inp["x"]); w = ops.createRaw(list(inp["w"].shape), inp["w"])
+        b = ops.createRaw([1], inp["b"])
+        t1 = x * w; t2 = t1 + b; t3 = t2.pow(2.0)
+        g = ops.createRaw([1], [1.0]).broadcastTo(t3.shape)
+        ig = g * 2.0
+        ig *= t2.pow(1.0)
+        gw = ig * x; gx = ig * w
+        outs.append([t.toArray() for t in (t1, t2, t3, g, ig, gw, gx)])
+    for name, a, c in zip(("x*w", "+b", "pow 2", "broadcast", "*2 *= pow1", "g*x", "g*w"), *outs):
+        assert_bits_equal(a, c, name)
+
+
+def test_cfg5_gradient_accumulates_over_two_backward_passes(gc):
+    from kten_amd.workloads import cfg5_setup, cfg5_step
+    inp = WORKLOADS["cfg5"].make_inputs({"rows": 64, "cols": 128})
+    x, w, b = cfg5_setup(gc, inp)
+    cfg5_step(x, w, b)
+    g1 = w.grad().toArray().copy()
+    cfg5_step(x, w, b)
+    np.testing.assert_allclose(w.grad().toArray(), 2 * g1, rtol=1e-6)
+    w.zeroGrad()
+    assert not w.grad().toArray().any()
+
+
+# ---------------------------------------------------------------- full BASELINE shapes
+
+def test_cfg1_full(gc):
+    wl = WORKLOADS["cfg1"]
+    inp, got, want = run_both("cfg1", wl.full_dims, gc)
+    assert_bits_equal(got["y"], want["y"], "y")
+    assert_bits_equal(got["y"], (inp["x"] + inp["b"]) * inp["x"], "y vs numpy")
+    ref = jo.sum_all_f64(want["y"])
+    assert_reduction_close(got["s"], [ref], want["s"], "s")
+    assert abs(float(got["s"][0]) - ref) <= 1e-5 * abs(ref)
+
+
+def test_cfg2_full(gc):
+    wl = WORKLOADS["cfg2"]
+    inp = wl.make_inputs(wl.full_dims)
+    x = inp["x"]
+    xt = gc.create([x.size], False, x)
+    sq = xt ** 2
+    assert_bits_equal(sq.toArray(), x * x, "pow 2")
+    neg = -sq
+    assert_bits_equal(neg.toArray(), (-(x * x)) + np.float32(0.0), "-(x pow 2)")
+    ab = xt.abs() + 1e-3
+    assert_bits_equal(ab.toArray(), np.abs(x) + np.float32(1e-3), "abs + 1e-3")
+    e, l = neg.exp(), ab.log()
+    z = (e + l).toArray()
+    ea, la = e.toArray(), l.toArray()
+    assert_bits_equal(z, ea + la, "e + l")
+    # exp / log against f64 numpy on the whole tensor (numpy's f64 routines agree with the
+    # checker's libm to the last f64 bit or nearly so), and against the checker itself on a slice
+    e_ref = np.exp((-(x * x)).astype(np.float64)).astype(np.float32)
+    l_ref = np.log((np.abs(x) + np.float32(1e-3)).astype(np.float64)).astype(np.float32)
+    assert ulp_distance(ea, e_ref).max() <= 2 and ulp_distance(la, l_ref).max() <= 2
+    sl = slice(12345, 12345 + (1 << 20))
+    assert_ulp_close(ea[sl], jo.unary("exp", (-(x[sl] * x[sl])) + np.float32(0.0)), 2, "exp slice")
+    assert_ulp_close(la[sl], jo.unary("log", np.abs(x[sl]) + np.float32(1e-3)), 2, "log slice")
+
+
+def test_cfg3_full(gc):
+    wl = WORKLOADS["cfg3"]
+    inp = wl.make_inputs(wl.full_dims)
+    x = inp["x"]
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    jo.set_threads(16)
+    try:
+        for axis in (0, 1):
+            ref, _ = jo.axis_sum_f64(x, axis)
+            jvm_sum = jo.aggregate("sum", x, axis); jvm_mean = jo.aggregate("mean", x, axis)
+            e, je = assert_reduction_close(got[f"sum{axis}"], ref, jvm_sum, f"sum{axis}")
+            print(f"sum axis {axis}: max |err| {e:.3e} (kten-jvm restatement {je:.3e})")
+            assert_reduction_close(got[f"mean{axis}"], ref / x.shape[axis], jvm_mean, f"mean{axis}")
+        assert_bits_equal(got["max1"], jo.aggregate("max", x, 1).reshape(-1), "max1")
+        assert_bits_equal(got["argmax1"], jo.aggregate("arg_max", x, 1).reshape(-1), "argmax1")
+    finally:
+        jo.set_threads(1)
+    assert_bits_equal(got["max1"], x.max(1), "max1 vs numpy")
+    assert (got["argmax1"] == np.argmax(x, 1)).all()
+
+
+def test_cfg4_full(gc):
+    wl = WORKLOADS["cfg4"]
+    inp = wl.make_inputs(wl.full_dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    out = inp["act"] * inp["scale"] + inp["bias"]            # numpy: one rounding per op, like the JVM
+    assert_bits_equal(got["out"], out, "out")
+    ref = out.astype(np.float64).sum((0, 2, 3), keepdims=True)
+    cpu = jo.JvmOracleOperations()
+    jo.set_threads(16)
+    try:
+        o = cpu.createRaw(list(out.shape), out)
+        jvm_sum = o.sum(0, True).sum(2, True).sum(3, True).toArray()
+        jvm_mean = o.mean(0, True).mean(2, True).mean(3, True).toArray()
+    finally:
+        jo.set_threads(1)
+    assert got["sum"].shape == (1, 128, 1, 1)
+    assert_reduction_close(got["sum"], ref, jvm_sum, "sum(0,2,3)")
+    assert_reduction_close(got["mean"], ref / (64 * 56 * 56), jvm_mean, "mean(0,2,3)")
+
+
+def test_cfg5_full(gc):
+    wl = WORKLOADS["cfg5"]
+    inp = wl.make_inputs(wl.full_dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    x32, w32, b32 = inp["x"], inp["w"], inp["b"]
+    t32 = (x32 * w32) + b32                                    # fp32 intermediates as the graph makes them
+    g32 = np.float32(2.0) * t32                                # (1 * 2f) * (t pow 1f)
+    loss_ref = np.square(t32).astype(np.float64).sum()
+    gw_ref = np.einsum("ij,ij->j", g32.astype(np.float64), x32.astype(np.float64))
+    gb_ref = g32.astype(np.float64).sum()
+    # kten-jvm's own serial-float results for the same reductions
+    jo.set_threads(16)
+    try:
+        jvm_loss = jo.sum_all(np.square(t32))
+        gx = g32 * x32
+        jvm_gw = jo.aggregate("sum", gx, 0).reshape(-1)
+        jvm_gb = jo.aggregate("sum", jo.aggregate("sum", g32, 0).reshape(-1), 0)
+    finally:
+        jo.set_threads(1)
+    e, je = assert_reduction_close(got["loss"], [loss_ref], [jvm_loss], "loss")
+    print(f"loss {got['loss'][0]!r}: |err| {e:.3e} (kten-jvm restatement {je:.3e})")
+    assert_reduction_close(got["grad_w"], gw_ref, jvm_gw, "grad w")
+    assert_reduction_close(got["grad_b"], [gb_ref], jvm_gb, "grad b")
+    assert abs(float(got["loss"][0]) - loss_ref) <= 1e-5 * loss_ref

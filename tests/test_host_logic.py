@@ -1,0 +1,213 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports every symbol
+the header declares, entry points refuse to run before kth_init, the shape algebra and
+error behaviour of the contract mirror, the seeded generator, the workloads' byte counts.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from kten_amd import abi, shape_functions as sf
+from kten_amd.inputs import SplitMix64
+from kten_amd.workloads import WORKLOADS
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "kten_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kth_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = abi.load()
+    names = header_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/kten_hip.h but not exported"
+    assert sorted(abi.SIGNATURES) == names, "abi.SIGNATURES and include/kten_hip.h declare different entry points"
+
+
+def test_entry_points_refuse_to_run_before_init():
+    import subprocess, sys
+    # A fresh process, so that an initialised library elsewhere in this session cannot interfere.
+    code = ("import ctypes, sys; sys.path.insert(0, %r); from kten_amd import abi; L = abi.load(); h = ctypes.c_uint64();"
+            "rc = L.kth_alloc(16, ctypes.byref(h)); print(rc, abi.last_error())" % ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, check=True).stdout
+    assert out.startswith(f"{abi.KTH_E_NOT_INIT} "), out
+    assert "kth_init" in out
+
+
+def test_status_codes_map_to_reference_exception_classes(monkeypatch):
+    monkeypatch.setattr(abi, "last_error", lambda: "msg")
+    with pytest.raises(ValueError):
+        abi.check(abi.KTH_E_SHAPE)          # IllegalArgumentException
+    with pytest.raises(ValueError):
+        abi.check(abi.KTH_E_ARGUMENT)
+    with pytest.raises(MemoryError):
+        abi.check(abi.KTH_E_MEMORY)
+    with pytest.raises(RuntimeError):
+        abi.check(abi.KTH_E_DEVICE)
+    abi.check(abi.KTH_OK)
+
+
+# ---------------------------------------------------------------- shape algebra
+
+def test_normalize_axis():
+    assert sf.normalize_axis([2, 3, 4], -1) == 2 and sf.normalize_axis([2, 3, 4], 0) == 0
+    for bad in (3, -4):
+        with pytest.raises(ValueError):
+            sf.normalize_axis([2, 3, 4], bad)
+
+
+def test_aggregate_over_never_goes_0d():
+    assert sf.aggregate_over([3, 4], 0, False) == [4]
+    assert sf.aggregate_over([3, 4], 1, True) == [3, 1]
+    assert sf.aggregate_over([5], 0, False) == [1]          # stays [1]
+
+
+def test_broadcast_shape_inference():
+    assert sf.infer_implicit_broadcast_shape([3, 1], [1, 3]) == [3, 3]
+    assert sf.infer_implicit_broadcast_shape([4], [2, 3, 4]) == [2, 3, 4]
+    assert sf.infer_explicit_broadcast_shape([1], [3, 3]) == [3, 3]
+    with pytest.raises(ValueError):
+        sf.infer_implicit_broadcast_shape([3], [4])
+    with pytest.raises(ValueError):
+        sf.infer_explicit_broadcast_shape([2, 3], [3])       # explicit broadcast never drops dims
+    with pytest.raises(ValueError):
+        sf.infer_explicit_broadcast_shape([3, 3], [3, 1])    # nor shrinks them
+
+
+def test_reshape_squeeze_unsqueeze():
+    assert sf.reshape([2, 3, 4], [-1, 4]) == [6, 4]
+    with pytest.raises(ValueError):
+        sf.reshape([2, 3], [4, -1, -1])
+    with pytest.raises(ValueError):
+        sf.reshape([2, 3], [4, 2])
+    assert sf.squeeze([2, 1, 3], 1) == [2, 3]
+    with pytest.raises(ValueError):
+        sf.squeeze([2, 1, 3], 0)
+    assert sf.unsqueeze([2, 3], 0) == [1, 2, 3]
+    assert sf.unsqueeze([2, 3], 2) == [2, 3, 1]
+    assert sf.unsqueeze([2, 3], -1) == [2, 3, 1]
+    assert sf.unsqueeze([2, 3], -3) == [1, 2, 3]
+
+
+def test_store_index_row_major_and_bounds():
+    assert sf.store_index([2, 3, 4], [1, 2, 3]) == 23
+    assert sf.store_index([2, 3, 4], [-1, 0, 0]) == 12
+    with pytest.raises(ValueError):
+        sf.store_index([2, 3], [0, 3])
+
+
+def test_contract_error_behaviour_on_the_host(oracle_ops):
+    # The same checks guard the HIP backend before any launch; exercised here on the CPU
+    # implementation of the contract.
+    a = oracle_ops.createRaw([2, 3], [1, 2, 3, 4, 5, 6])
+    b = oracle_ops.createRaw([3, 2], [1, 2, 3, 4, 5, 6])
+    with pytest.raises(ValueError):
+        a.plusAssign(b)                                       # in-place needs equal shapes
+    with pytest.raises(ValueError):
+        a.plus(b)                                             # [2,3] and [3,2] do not broadcast
+    with pytest.raises(ValueError):
+        a.sum(2)
+    assert a.sum(0).shape == [3] and a.sum(-1, True).shape == [2, 1]
+    v = oracle_ops.createRaw([4], [1, 2, 3, 4])
+    assert v.sum(0).shape == [1] and v.argMax(0).shape == [1]
+    assert a.broadcastTo([2, 3]) is a                         # equal shape returns this
+    assert a.calculateCommonShapeWith(oracle_ops.createRaw([4, 1, 3])) == [4, 2, 3]
+
+
+def test_may_unexpand_axis_order(oracle_ops):
+    from kten_amd.autograd import mayUnexpand
+    calls = []
+    g = oracle_ops.createRaw([2, 3, 4, 5], np.arange(120, dtype=np.float32))
+    orig = type(g).sum
+    def spy(self, axis=None, keepDimensions=False):
+        calls.append((axis, keepDimensions, list(self.shape)))
+        return orig(self, axis, keepDimensions)
+    type(g).sum = spy
+    try:
+        res = mayUnexpand(g, [1, 3, 1, 1], oracle_ops)
+        assert calls == [(0, True, [2, 3, 4, 5]), (2, True, [1, 3, 4, 5]), (3, True, [1, 3, 1, 5])]
+        assert res.shape == [1, 3, 1, 1]
+        np.testing.assert_array_equal(res.toArray(), np.arange(120, dtype=np.float32).reshape(2, 3, 4, 5).sum((0, 2, 3), keepdims=True))
+        calls.clear()
+        res = mayUnexpand(oracle_ops.createRaw([6, 4], np.ones(24, np.float32)), [1], oracle_ops)
+        assert calls == [(0, False, [6, 4]), (0, True, [4])] and res.shape == [1] and res.toArray()[0] == 24
+    finally:
+        type(g).sum = orig
+
+
+# ---------------------------------------------------------------- generator and workloads
+
+def test_splitmix64_published_vectors():
+    # First outputs of the reference SplitMix64 implementation for seed 1234567.
+    assert SplitMix64(1234567).next_u64(5).tolist() == [6457827717110365317, 3203168211198807973, 9817491932198370423,
+                                                         4593380528125082431, 16408922859458223821]
+    g = SplitMix64(7)
+    a = g.next_u64(3); b = g.next_u64(4)
+    assert np.concatenate([a, b]).tolist() == SplitMix64(7).next_u64(7).tolist()      # one stream, any chunking
+
+
+def test_generator_distributions_and_determinism():
+    u = SplitMix64(0).uniform([100000], -1.0, 1.0)
+    assert u.dtype == np.float32 and u.min() >= -1.0 and u.max() < 1.0 and abs(u.mean()) < 0.01
+    assert u[:2].view(np.uint32).tolist() == [1061437776, 3188472592]
+    n = SplitMix64(1).normal([100001])
+    assert n.shape == (100001,) and abs(n.mean()) < 0.02 and abs(n.std() - 1) < 0.02
+    assert np.array_equal(n[:1000], SplitMix64(1).normal([1000]))
+    assert np.isfinite(n).all()
+
+
+def test_algorithmic_bytes_match_the_published_plan():
+    want = {"cfg1": 50335748, "cfg2": 4563402752, "cfg3": 1610809344, "cfg4": 623101952}
+    for name, b in want.items():
+        wl = WORKLOADS[name]
+        assert wl.algorithmic_bytes(wl.full_dims) == b
+    wl = WORKLOADS["cfg5"]
+    m = 16384 * 4096
+    got = wl.algorithmic_bytes(wl.full_dims)
+    assert 22 * m * 4 <= got <= 22 * m * 4 + 200000
+
+
+def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
+    # Count bytes op by op on the CPU implementation of the contract (operands at their
+    # true size + output; in-place: target twice + other) and compare with the formula.
+    import contextlib
+    from oracle.jvm_oracle import JvmOracleRawTensor as R
+    counted = [0]
+    saved = {}
+
+    def wrap(name, cost):
+        orig = getattr(R, name)
+        saved[name] = orig
+        def f(self, *a, **k):
+            res = orig(self, *a, **k)
+            counted[0] += cost(self, a, res)
+            return res
+        setattr(R, name, f)
+
+    size = lambda t: int(np.prod(t.shape))
+    wrap("_binary", lambda s, a, r: size(s) + size(a[1]) + size(r))
+    wrap("_binary_assign", lambda s, a, r: 2 * size(s) + size(a[1]))
+    wrap("_scalar", lambda s, a, r: size(s) + size(r))
+    wrap("_scalar_assign", lambda s, a, r: 2 * size(s))
+    wrap("_unary", lambda s, a, r: size(s) + size(r))
+    wrap("aggregateOverAxis", lambda s, a, r: size(s) + size(r))
+    wrap("_sum_all", lambda s, a, r: size(s) + 1)
+    wrap("broadcastTo", lambda s, a, r: 0 if r is s else size(s) + size(r))
+    try:
+        small = {"cfg1": {"rows": 8, "cols": 12}, "cfg2": {"n": 100}, "cfg3": {"rows": 6, "cols": 10},
+                 "cfg4": {"n": 2, "c": 3, "h": 4, "w": 5}, "cfg5": {"rows": 8, "cols": 12}}
+        for name, dims in small.items():
+            wl = WORKLOADS[name]
+            counted[0] = 0
+            wl.run(oracle_ops, wl.make_inputs(dims))
+            assert counted[0] * 4 == wl.algorithmic_bytes(dims), name
+    finally:
+        for name, orig in saved.items():
+            setattr(R, name, orig)
