@@ -20,7 +20,7 @@
  *   - Shapes travel by value inside the kernel arguments; nothing is uploaded per launch.
  *   - All launches are asynchronous on one internal in-order stream. The only blocking
  *     calls are kth_upload, kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
- *     kth_timer_end and kth_shutdown.
+ *     kth_timer_end, kth_profile_end and kth_shutdown.
  *   - Shape / argument errors are reported before anything is launched, as the
  *     reference throws IllegalArgumentException host-side before computing
  *     (JVM:89-93, ShapeFunctions.kt:187-201).
@@ -186,6 +186,17 @@ int kth_metrics(uint64_t* live_bytes, uint64_t* pool_bytes, uint64_t* launches, 
  * no timing facility. kth_timer_end blocks until the second event completes. */
 int kth_timer_begin(void);
 int kth_timer_end(float* milliseconds);
+
+/* Per-kernel device timing, for benchmarks that must attribute the time of a region to
+ * the kernels in it. No counterpart in the reference. Between kth_profile_begin and
+ * kth_profile_end every kernel launch is bracketed by a HIP event pair on the internal
+ * stream; kth_profile_end blocks until those launches have finished. Afterwards
+ * kth_profile_count gives the number of distinct kernels seen and kth_profile_entry the
+ * name ("family<Op>"), launch count, algorithmic bytes and summed duration of one. */
+int kth_profile_begin(void);
+int kth_profile_end(void);
+int kth_profile_count(int* count);
+int kth_profile_entry(int index, char* name, size_t cap, uint64_t* launches, uint64_t* bytes, double* total_ms);
 
 #ifdef __cplusplus
 }

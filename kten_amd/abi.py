@@ -58,6 +58,10 @@ SIGNATURES = {
     "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
     "kth_timer_begin": (c_int, []),
     "kth_timer_end": (c_int, [POINTER(c_float)]),
+    "kth_profile_begin": (c_int, []),
+    "kth_profile_end": (c_int, []),
+    "kth_profile_count": (c_int, [POINTER(c_int)]),
+    "kth_profile_entry": (c_int, [c_int, ctypes.c_char_p, c_size_t, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_double)]),
 }
 
 _lib = None

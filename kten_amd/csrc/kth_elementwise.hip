@@ -212,7 +212,7 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_scalar_kernel(const float
     }
 }
 
-struct OpFirst { static __device__ __forceinline__ float apply(float a, float, float) { return a; } };
+struct OpFirst { static constexpr const char* name = "OpFirst"; static __device__ __forceinline__ float apply(float a, float, float) { return a; } };
 
 // ---------------------------------------------------------------- NaN scan
 
@@ -315,24 +315,30 @@ int check_shape(const int32_t* shape, int dims, const char* what, uint64_t* coun
 
 template <class Op>
 void launch_unary(const float* a, float* out, uint32_t n, float p, float q) {
+    LaunchScope scope("unary_kernel", Op::name, static_cast<uint64_t>(n) * 8);
     hipLaunchKernelGGL((unary_kernel<Op>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, p, q);
 }
 
 template <class Op>
 void launch_scalar(bool rev, const float* a, float* out, uint32_t n, float c, float eps) {
+    LaunchScope scope(rev ? "scalar_kernel_rev" : "scalar_kernel", Op::name, static_cast<uint64_t>(n) * 8);
     if (rev) hipLaunchKernelGGL((scalar_kernel<Op, true>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
     else     hipLaunchKernelGGL((scalar_kernel<Op, false>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
 }
 
 template <class Op>
 void launch_binary_same(const float* a, const float* b, float* out, uint32_t n, float eps) {
+    LaunchScope scope("binary_same_kernel", Op::name, static_cast<uint64_t>(n) * 12);
     hipLaunchKernelGGL((binary_same_kernel<Op>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, b, out, n, eps);
 }
 
 template <class Op>
 void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n, float eps,
-                         BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec) {
+                         BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec, uint64_t bytes) {
     hipStream_t st = state().stream;
+    LaunchScope scope(!vec_ok ? "binary_bcast_scalar_kernel" : (a_vec && b_vec) ? "binary_bcast_vec_kernel_vv"
+                      : a_vec ? "binary_bcast_vec_kernel_vs" : b_vec ? "binary_bcast_vec_kernel_sv"
+                      : "binary_bcast_vec_kernel_ss", Op::name, bytes);
     if (vec_ok) {
         to_vector_units(&plan);
         uint32_t n4 = n >> 2;
@@ -380,9 +386,11 @@ int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value) {
                     (unsigned long long)offset, (unsigned long long)n, (unsigned long long)st->n_floats);
     if (n == 0) return KTH_OK;
     uint32_t n32 = static_cast<uint32_t>(n);
-    hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(n32 >> 2)), dim3(kBlock), 0, state().stream, st->ptr + offset, n32, value);
+    {
+        LaunchScope scope("fill_kernel", "", n * 4);
+        hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(n32 >> 2)), dim3(kBlock), 0, state().stream, st->ptr + offset, n32, value);
+    }
     KTH_LAUNCH_CHECK("fill");
-    count_launch(n * 4);
     return KTH_OK;
 }
 
@@ -415,7 +423,6 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
 #undef U
     if (n == 0) return KTH_OK;
     KTH_LAUNCH_CHECK("unary");
-    count_launch(n * 8);
     return KTH_OK;
 }
 
@@ -431,7 +438,6 @@ int kth_clamp(uint64_t a, uint64_t out, uint64_t n, float lo, float hi) {
     if (n == 0) return KTH_OK;
     launch_unary<OpClamp>(sa->ptr, so->ptr, static_cast<uint32_t>(n), lo, hi);
     KTH_LAUNCH_CHECK("clamp");
-    count_launch(n * 8);
     return KTH_OK;
 }
 
@@ -459,7 +465,6 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
 #undef S
     }
     KTH_LAUNCH_CHECK("scalar");
-    count_launch(n * 8);
     return KTH_OK;
 }
 
@@ -481,7 +486,6 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
     KTH_BINARY_DISPATCH(op, B)
 #undef B
     KTH_LAUNCH_CHECK("binary_inplace");
-    count_launch(n * 12);
     return KTH_OK;
 }
 
@@ -520,12 +524,11 @@ int kth_binary(int op,
         KTH_BINARY_DISPATCH(op, B)
 #undef B
     } else {
-#define B(OP) launch_binary_bcast<OP>(pa, pb, po, n32, eps, plan, vec_ok, a_vec, b_vec)
+#define B(OP) launch_binary_bcast<OP>(pa, pb, po, n32, eps, plan, vec_ok, a_vec, b_vec, (an + bn + on) * 4)
         KTH_BINARY_DISPATCH(op, B)
 #undef B
     }
     KTH_LAUNCH_CHECK("binary");
-    count_launch((an + bn + on) * 4);
     return KTH_OK;
 }
 
@@ -550,12 +553,13 @@ int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
     if (ss->ptr == sd->ptr) return fail(KTH_E_ARGUMENT, "kth_broadcast_to: source and target are the same store");
     if (dn == 0) return KTH_OK;
     if (sn == dn) {
+        LaunchScope scope("memcpy_d2d", "", dn * 8);
         KTH_HIP(hipMemcpyAsync(sd->ptr, ss->ptr, dn * 4, hipMemcpyDeviceToDevice, state().stream));
     } else {
-        launch_binary_bcast<OpFirst>(ss->ptr, ss->ptr, sd->ptr, static_cast<uint32_t>(dn), 0.0f, plan, vec_ok, a_vec, b_vec);
+        launch_binary_bcast<OpFirst>(ss->ptr, ss->ptr, sd->ptr, static_cast<uint32_t>(dn), 0.0f, plan, vec_ok, a_vec, b_vec,
+                                     (sn + dn) * 4);
         KTH_LAUNCH_CHECK("broadcast_to");
     }
-    count_launch((sn + dn) * 4);
     return KTH_OK;
 }
 
@@ -577,14 +581,16 @@ int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
     uint32_t blocks = blocks_for(n32 >> 2);
     uint32_t cap_blocks = static_cast<uint32_t>(s.compute_units) * 8u;
     if (blocks > cap_blocks) blocks = cap_blocks;
-    hipLaunchKernelGGL(contains_nan_kernel, dim3(blocks), dim3(kBlock), 0, s.stream, st->ptr, n32, flag);
+    {
+        LaunchScope scope("contains_nan_kernel", "", n * 4);
+        hipLaunchKernelGGL(contains_nan_kernel, dim3(blocks), dim3(kBlock), 0, s.stream, st->ptr, n32, flag);
+    }
     int host_flag = 0;
     hipError_t e = hipMemcpyAsync(&host_flag, flag, 4, hipMemcpyDeviceToHost, s.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
     workspace_release(reinterpret_cast<float*>(flag), cap);
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_contains_nan: %s", hipGetErrorString(e));
     *out = host_flag;
-    count_launch(n * 4);
     return KTH_OK;
 }
 

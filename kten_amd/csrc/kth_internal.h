@@ -23,6 +23,14 @@ struct Store {
     uint32_t generation = 0;   // bumped on release so stale handles are detected
 };
 
+// One profiled launch: which kernel, the algorithmic bytes it moved, its event pair.
+struct LaunchRecord {
+    const char* family;
+    const char* op;
+    uint64_t    bytes;
+    hipEvent_t  begin, end;
+};
+
 struct State {
     bool        ready = false;
     int         device = -1;
@@ -43,6 +51,10 @@ struct State {
     std::map<uint64_t, std::vector<float*>> pool;   // size class (bytes) -> idle buffers
 
     uint64_t live_bytes = 0, pool_bytes = 0, launches = 0, bytes_moved = 0;
+
+    bool profiling = false;
+    std::vector<LaunchRecord> records;      // launches of the current / last profile
+    std::vector<hipEvent_t>   event_pool;   // idle events, reused across profiles
 };
 
 State&      state();
@@ -60,10 +72,17 @@ Store* lookup(uint64_t handle, const char* what);
 float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
 void   workspace_release(float* p, uint64_t cap_bytes);
 
-inline void count_launch(uint64_t algorithmic_bytes) {
-    state().launches += 1;
-    state().bytes_moved += algorithmic_bytes;
-}
+// Brackets the launch of one kernel: counts it for kth_metrics and, while a profile is
+// being recorded, puts a HIP event before and after it on the library's stream.
+class LaunchScope {
+public:
+    LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes);
+    ~LaunchScope();
+    LaunchScope(const LaunchScope&) = delete;
+    LaunchScope& operator=(const LaunchScope&) = delete;
+private:
+    int record_ = -1;
+};
 
 #define KTH_REQUIRE_INIT()                                                         \
     do {                                                                           \

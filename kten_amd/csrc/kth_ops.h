@@ -37,22 +37,23 @@ __device__ __forceinline__ float jpow(float a, float b) {
 }
 
 // ---- binary functors: apply(a, b, p) where p carries PlatformProvider.epsilon for eq/neq.
-struct OpPlus  { static __device__ __forceinline__ float apply(float a, float b, float) { return a + b; } };
-struct OpMinus { static __device__ __forceinline__ float apply(float a, float b, float) { return a - b; } };
-struct OpTimes { static __device__ __forceinline__ float apply(float a, float b, float) { return a * b; } };
-struct OpDiv   { static __device__ __forceinline__ float apply(float a, float b, float) { return a / b; } };
-struct OpPow   { static __device__ __forceinline__ float apply(float a, float b, float) { return jpow(a, b); } };
+struct OpPlus  { static constexpr const char* name = "OpPlus"; static __device__ __forceinline__ float apply(float a, float b, float) { return a + b; } };
+struct OpMinus { static constexpr const char* name = "OpMinus"; static __device__ __forceinline__ float apply(float a, float b, float) { return a - b; } };
+struct OpTimes { static constexpr const char* name = "OpTimes"; static __device__ __forceinline__ float apply(float a, float b, float) { return a * b; } };
+struct OpDiv   { static constexpr const char* name = "OpDiv"; static __device__ __forceinline__ float apply(float a, float b, float) { return a / b; } };
+struct OpPow   { static constexpr const char* name = "OpPow"; static __device__ __forceinline__ float apply(float a, float b, float) { return jpow(a, b); } };
 // JVMRawTensor.kt:355-377
-struct OpLt    { static __device__ __forceinline__ float apply(float a, float b, float) { return a <  b ? 1.0f : 0.0f; } };
-struct OpLte   { static __device__ __forceinline__ float apply(float a, float b, float) { return a <= b ? 1.0f : 0.0f; } };
-struct OpGt    { static __device__ __forceinline__ float apply(float a, float b, float) { return a >  b ? 1.0f : 0.0f; } };
-struct OpGte   { static __device__ __forceinline__ float apply(float a, float b, float) { return a >= b ? 1.0f : 0.0f; } };
-struct OpEq    { static __device__ __forceinline__ float apply(float a, float b, float eps) { return fabsf(a - b) < eps ? 1.0f : 0.0f; } };
-struct OpNeq   { static __device__ __forceinline__ float apply(float a, float b, float eps) { return fabsf(a - b) < eps ? 0.0f : 1.0f; } };
+struct OpLt    { static constexpr const char* name = "OpLt"; static __device__ __forceinline__ float apply(float a, float b, float) { return a <  b ? 1.0f : 0.0f; } };
+struct OpLte   { static constexpr const char* name = "OpLte"; static __device__ __forceinline__ float apply(float a, float b, float) { return a <= b ? 1.0f : 0.0f; } };
+struct OpGt    { static constexpr const char* name = "OpGt"; static __device__ __forceinline__ float apply(float a, float b, float) { return a >  b ? 1.0f : 0.0f; } };
+struct OpGte   { static constexpr const char* name = "OpGte"; static __device__ __forceinline__ float apply(float a, float b, float) { return a >= b ? 1.0f : 0.0f; } };
+struct OpEq    { static constexpr const char* name = "OpEq"; static __device__ __forceinline__ float apply(float a, float b, float eps) { return fabsf(a - b) < eps ? 1.0f : 0.0f; } };
+struct OpNeq   { static constexpr const char* name = "OpNeq"; static __device__ __forceinline__ float apply(float a, float b, float eps) { return fabsf(a - b) < eps ? 0.0f : 1.0f; } };
 
 // ---- unary functors: apply(x, p, q); p, q are only used by clamp.
 #define KTH_UNARY(NAME, EXPR)                                                             \
-    struct NAME { static __device__ __forceinline__ float apply(float x, float p, float q) { \
+    struct NAME { static constexpr const char* name = #NAME;                              \
+        static __device__ __forceinline__ float apply(float x, float p, float q) {       \
         (void)p; (void)q; return (EXPR); } };
 
 KTH_UNARY(OpNeg,        -x)                                             // :122
@@ -80,6 +81,7 @@ KTH_UNARY(OpIdentity,   x)                                              // pow(x
 
 // sigmoid = 1f / (1f + exp(-1f * x)) with exp rounded to float first. (:399)
 struct OpSigmoid {
+    static constexpr const char* name = "OpSigmoid";
     static __device__ __forceinline__ float apply(float x, float, float) {
         float m = -1.0f * x;
         float e = static_cast<float>(exp(static_cast<double>(m)));
@@ -90,6 +92,7 @@ struct OpSigmoid {
 
 // Math.signum. (:407)
 struct OpSign {
+    static constexpr const char* name = "OpSign";
     static __device__ __forceinline__ float apply(float x, float, float) {
         if (x != x || x == 0.0f) return x;
         return x > 0.0f ? 1.0f : -1.0f;
@@ -99,6 +102,7 @@ struct OpSign {
 // Math.round(float).toFloat() (:431): floor(x + 1/2) without the rounding error of
 // x + 0.5f, NaN -> 0, saturation at the Int range, zero results are +0.
 struct OpRound {
+    static constexpr const char* name = "OpRound";
     static __device__ __forceinline__ float apply(float x, float, float) {
         if (x != x) return 0.0f;
         float r = floorf(x);
@@ -111,6 +115,7 @@ struct OpRound {
 
 // clamp = Math.min(Math.max(x, lo), hi). (:409-411)
 struct OpClamp {
+    static constexpr const char* name = "OpClamp";
     static __device__ __forceinline__ float apply(float x, float lo, float hi) {
         return jmin(jmax(x, lo), hi);
     }

@@ -41,6 +41,7 @@ __device__ __forceinline__ ArgAcc shfl_xor_acc(ArgAcc a, int m) {
 
 template <bool MEAN>
 struct RedSumT {
+    static constexpr const char* name = MEAN ? "RedMean" : "RedSum";
     using Acc = double;
     static __device__ __forceinline__ Acc init() { return 0.0; }
     static __device__ __forceinline__ void step(Acc& a, float x, uint32_t) { a += static_cast<double>(x); }
@@ -55,6 +56,7 @@ using RedMean = RedSumT<true>;
 
 template <bool MAX>
 struct RedExtT {
+    static constexpr const char* name = MAX ? "RedMax" : "RedMin";
     using Acc = float;
     static __device__ __forceinline__ Acc init() { return MAX ? -INFINITY : INFINITY; }
     static __device__ __forceinline__ void step(Acc& a, float x, uint32_t) { a = MAX ? jmax(a, x) : jmin(a, x); }
@@ -68,6 +70,7 @@ using RedMin = RedExtT<false>;
 // index, NaNs never win, a lane with nothing strictly better yields 0 (JVMRawTensor.kt:167-184).
 template <bool MAX>
 struct RedArgT {
+    static constexpr const char* name = MAX ? "RedArgMax" : "RedArgMin";
     using Acc = ArgAcc;
     static __device__ __forceinline__ Acc init() { Acc a; a.v = MAX ? -INFINITY : INFINITY; a.i = 0; return a; }
     static __device__ __forceinline__ void step(Acc& a, float x, uint32_t idx) {
@@ -310,24 +313,31 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
                                   (unsigned long long)(n_out * g.segments));
     }
     const dim3 grid(static_cast<uint32_t>(blocks));
-    if (kind == ROWS) {
+    const uint64_t bytes = (static_cast<uint64_t>(outer) * axis * inner + n_out) * 4;
+    hipError_t e;
+    {
+        LaunchScope scope(kind == ROWS ? "reduce_rows_kernel" : kind == COLS ? "reduce_cols_kernel" : "reduce_strided_kernel",
+                          R::name, bytes);
+        if (kind == ROWS) {
 #define ROWS_LAUNCH(GG, VV) hipLaunchKernelGGL((reduce_rows_kernel<R, GG, VV>), grid, dim3(kBlock), 0, stream, in, out, partial, g)
-        if (VEC == 4) {
-            switch (G) { case 256: ROWS_LAUNCH(256, 4); break; case 64: ROWS_LAUNCH(64, 4); break;
-                         case 16: ROWS_LAUNCH(16, 4); break; case 4: ROWS_LAUNCH(4, 4); break; default: ROWS_LAUNCH(1, 4); }
-        } else {
-            switch (G) { case 256: ROWS_LAUNCH(256, 1); break; case 64: ROWS_LAUNCH(64, 1); break;
-                         case 16: ROWS_LAUNCH(16, 1); break; case 4: ROWS_LAUNCH(4, 1); break; default: ROWS_LAUNCH(1, 1); }
-        }
+            if (VEC == 4) {
+                switch (G) { case 256: ROWS_LAUNCH(256, 4); break; case 64: ROWS_LAUNCH(64, 4); break;
+                             case 16: ROWS_LAUNCH(16, 4); break; case 4: ROWS_LAUNCH(4, 4); break; default: ROWS_LAUNCH(1, 4); }
+            } else {
+                switch (G) { case 256: ROWS_LAUNCH(256, 1); break; case 64: ROWS_LAUNCH(64, 1); break;
+                             case 16: ROWS_LAUNCH(16, 1); break; case 4: ROWS_LAUNCH(4, 1); break; default: ROWS_LAUNCH(1, 1); }
+            }
 #undef ROWS_LAUNCH
-    } else if (kind == COLS) {
-        if (VEC == 4) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
-        else          hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
-    } else {
-        hipLaunchKernelGGL((reduce_strided_kernel<R>), grid, dim3(kBlock), 0, stream, in, out, partial, g);
+        } else if (kind == COLS) {
+            if (VEC == 4) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+            else          hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+        } else {
+            hipLaunchKernelGGL((reduce_strided_kernel<R>), grid, dim3(kBlock), 0, stream, in, out, partial, g);
+        }
+        e = hipGetLastError();
     }
-    hipError_t e = hipGetLastError();
     if (e == hipSuccess && g.segments > 1) {
+        LaunchScope scope("reduce_finalize_kernel", R::name, 0);
         if (n_out < 4096 && g.segments > 16)
             hipLaunchKernelGGL((reduce_finalize_kernel<R, true>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
                                partial, out, g);
@@ -338,7 +348,6 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     }
     if (partial) workspace_release(reinterpret_cast<float*>(partial), cap);
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
-    count_launch((static_cast<uint64_t>(outer) * axis * inner + n_out) * 4);
     return KTH_OK;
 }
 

@@ -103,6 +103,32 @@ void workspace_release(float* p, uint64_t cap_bytes) {
     s.pool_bytes += cap_bytes;
 }
 
+static hipEvent_t take_event() {
+    State& s = state();
+    if (!s.event_pool.empty()) { hipEvent_t e = s.event_pool.back(); s.event_pool.pop_back(); return e; }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    return e;
+}
+
+LaunchScope::LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes) {
+    State& s = state();
+    s.launches += 1;
+    s.bytes_moved += algorithmic_bytes;
+    if (!s.profiling) return;
+    LaunchRecord r{family, op, algorithmic_bytes, take_event(), take_event()};
+    if (!r.begin || !r.end) return;
+    (void)hipEventRecord(r.begin, s.stream);
+    s.records.push_back(r);
+    record_ = static_cast<int>(s.records.size()) - 1;
+}
+
+LaunchScope::~LaunchScope() {
+    if (record_ < 0) return;
+    State& s = state();
+    (void)hipEventRecord(s.records[record_].end, s.stream);
+}
+
 }  // namespace kth
 
 using namespace kth;
@@ -149,6 +175,8 @@ int kth_shutdown(void) {
     s.table.clear();
     s.free_slots.clear();
     trim_pool();
+    for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
+    for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(s.ev_begin);
     (void)hipEventDestroy(s.ev_end);
     (void)hipStreamDestroy(s.stream);
@@ -288,8 +316,8 @@ int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offse
         if (hi - lo < n) return fail(KTH_E_ARGUMENT, "kth_copy: overlapping ranges in one store");
     }
     State& s = state();
+    LaunchScope scope("memcpy_d2d", "", n * 8);
     KTH_HIP(hipMemcpyAsync(d->ptr + dst_offset, sst->ptr + src_offset, n * 4, hipMemcpyDeviceToDevice, s.stream));
-    count_launch(n * 8);
     return KTH_OK;
 }
 
@@ -330,6 +358,70 @@ int kth_timer_end(float* milliseconds) {
     KTH_HIP(hipEventSynchronize(s.ev_end));
     KTH_HIP(hipEventElapsedTime(milliseconds, s.ev_begin, s.ev_end));
     s.timer_open = false;
+    return KTH_OK;
+}
+
+int kth_profile_begin(void) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    for (LaunchRecord& r : s.records) { s.event_pool.push_back(r.begin); s.event_pool.push_back(r.end); }
+    s.records.clear();
+    s.profiling = true;
+    return KTH_OK;
+}
+
+int kth_profile_end(void) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    s.profiling = false;
+    KTH_HIP(hipStreamSynchronize(s.stream));
+    return KTH_OK;
+}
+
+// Aggregates the recorded launches by (kernel family, op) in first-seen order.
+static int profile_aggregate(std::vector<LaunchRecord>* keys, std::vector<uint64_t>* launches,
+                             std::vector<uint64_t>* bytes, std::vector<double>* ms) {
+    State& s = state();
+    for (const LaunchRecord& r : s.records) {
+        size_t k = 0;
+        for (; k < keys->size(); k++)
+            if (!strcmp((*keys)[k].family, r.family) && !strcmp((*keys)[k].op, r.op)) break;
+        if (k == keys->size()) { keys->push_back(r); launches->push_back(0); bytes->push_back(0); ms->push_back(0.0); }
+        float t = 0.0f;
+        KTH_HIP(hipEventElapsedTime(&t, r.begin, r.end));
+        (*launches)[k] += 1; (*bytes)[k] += r.bytes; (*ms)[k] += t;
+    }
+    return KTH_OK;
+}
+
+int kth_profile_count(int* count) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!count) return fail(KTH_E_ARGUMENT, "kth_profile_count: null output");
+    if (state().profiling) return fail(KTH_E_ARGUMENT, "kth_profile_count: a profile is still being recorded");
+    std::vector<LaunchRecord> keys; std::vector<uint64_t> l, b; std::vector<double> ms;
+    if (int rc = profile_aggregate(&keys, &l, &b, &ms)) return rc;
+    *count = static_cast<int>(keys.size());
+    return KTH_OK;
+}
+
+int kth_profile_entry(int index, char* name, size_t cap, uint64_t* launches, uint64_t* bytes, double* total_ms) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (state().profiling) return fail(KTH_E_ARGUMENT, "kth_profile_entry: a profile is still being recorded");
+    std::vector<LaunchRecord> keys; std::vector<uint64_t> l, b; std::vector<double> ms;
+    if (int rc = profile_aggregate(&keys, &l, &b, &ms)) return rc;
+    if (index < 0 || index >= static_cast<int>(keys.size()))
+        return fail(KTH_E_ARGUMENT, "kth_profile_entry: index %d of %zu", index, keys.size());
+    if (name && cap > 0) {
+        if (keys[index].op[0]) snprintf(name, cap, "%s<%s>", keys[index].family, keys[index].op);
+        else snprintf(name, cap, "%s", keys[index].family);
+    }
+    if (launches) *launches = l[index];
+    if (bytes) *bytes = b[index];
+    if (total_ms) *total_ms = ms[index];
     return KTH_OK;
 }
 

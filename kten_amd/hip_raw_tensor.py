@@ -365,6 +365,22 @@ class HipTensorOperations:
         check(self.lib.kth_timer_end(ctypes.byref(ms)))
         return ms.value
 
+    def profileBegin(self):
+        check(self.lib.kth_profile_begin())
+
+    def profileEnd(self):
+        """Stops recording and returns {kernel name: (launches, algorithmic bytes, total ms)}."""
+        check(self.lib.kth_profile_end())
+        n = ctypes.c_int()
+        check(self.lib.kth_profile_count(ctypes.byref(n)))
+        out = {}
+        for i in range(n.value):
+            name = ctypes.create_string_buffer(128)
+            launches, nbytes, ms = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_double()
+            check(self.lib.kth_profile_entry(i, name, 128, ctypes.byref(launches), ctypes.byref(nbytes), ctypes.byref(ms)))
+            out[name.value.decode()] = (launches.value, nbytes.value, ms.value)
+        return out
+
     def shutdown(self):
         if self.alive:
             self.alive = False
