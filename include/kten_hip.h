@@ -19,7 +19,7 @@
  *     (kten-api/.../autograd/utils/ShapeFunctions.kt:344).
  *   - Shapes travel by value inside the kernel arguments; nothing is uploaded per launch.
  *   - All launches are asynchronous on one internal in-order stream. The only blocking
- *     calls are kth_upload, kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
+ *     calls are kth_upload (above 1 MiB), kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
  *     kth_timer_end, kth_profile_end and kth_shutdown.
  *   - Shape / argument errors are reported before anything is launched, as the
  *     reference throws IllegalArgumentException host-side before computing
@@ -103,7 +103,10 @@ int kth_retain(uint64_t handle);
 int kth_release(uint64_t handle);
 
 /* Host -> device. Serves createRaw(shape, init) (OPS:11), fromCommonSerializable
- * (OPS:135) and the JVM -> device platform transformer. Blocking. */
+ * (OPS:135) and the JVM -> device platform transformer. `src` may be reused as soon as
+ * the call returns. Uploads of up to 1 MiB do not wait for the stream (they are staged
+ * through pinned memory or, for a few values, carried in kernel arguments); larger ones
+ * block until the copy is done. */
 int kth_upload(uint64_t handle, uint64_t offset, const float* src, uint64_t n);
 
 /* Device -> host after draining the stream. Serves toSerializableData (OPS:133) and

@@ -52,6 +52,15 @@ struct State {
 
     uint64_t live_bytes = 0, pool_bytes = 0, launches = 0, bytes_moved = 0;
 
+    // Pinned staging slots for asynchronous small uploads; slot i may be refilled once
+    // stage_done[i] has completed.
+    static constexpr int kStageSlots = 8;
+    static constexpr uint64_t kStageBytes = 1ull << 20;
+    char*      stage[kStageSlots] = {nullptr};
+    hipEvent_t stage_done[kStageSlots] = {nullptr};
+    bool       stage_used[kStageSlots] = {false};
+    int        stage_next = 0;
+
     bool profiling = false;
     std::vector<LaunchRecord> records;      // launches of the current / last profile
     std::vector<hipEvent_t>   event_pool;   // idle events, reused across profiles

@@ -26,6 +26,16 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWave = 64;
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// The input of a reduction is read exactly once: non-temporal loads, so the stream does
+// not displace other tensors from the memory-side cache.
+__device__ __forceinline__ float4 ld4_stream(const float* p) {
+    v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float ld1_stream(const float* p) { return __builtin_nontemporal_load(p); }
+
 // ---------------------------------------------------------------- reducers
 
 struct ArgAcc { float v; uint32_t i; };
@@ -123,12 +133,12 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
         if (VEC == 4) {
 #pragma unroll 4
             for (uint32_t j = begin + lane * 4; j < end; j += G * 4) {
-                float4 v = *reinterpret_cast<const float4*>(base + j);
+                float4 v = ld4_stream(base + j);
                 R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
             }
         } else {
 #pragma unroll 4
-            for (uint32_t j = begin + lane; j < end; j += G) R::step(acc, base[j], j);
+            for (uint32_t j = begin + lane; j < end; j += G) R::step(acc, ld1_stream(base + j), j);
         }
     }
     constexpr int kLanes = G < kWave ? G : kWave;
@@ -176,11 +186,11 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
         for (uint32_t r = begin + ty; r < end; r += WY) {
             const float* p = base + static_cast<size_t>(r) * g.inner;
             if (VEC == 4) {
-                float4 v = *reinterpret_cast<const float4*>(p);
+                float4 v = ld4_stream(p);
                 R::step(acc[0], v.x, r); R::step(acc[1 % VEC], v.y, r);
                 R::step(acc[2 % VEC], v.z, r); R::step(acc[3 % VEC], v.w, r);
             } else {
-                R::step(acc[0], *p, r);
+                R::step(acc[0], ld1_stream(p), r);
             }
         }
     }
@@ -215,41 +225,59 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __r
     const uint32_t end = min(begin + g.seg_len, g.axis);
     typename R::Acc acc = R::init();
 #pragma unroll 4
-    for (uint32_t r = begin; r < end; r++) R::step(acc, base[static_cast<size_t>(r) * g.inner], r);
+    for (uint32_t r = begin; r < end; r++) R::step(acc, ld1_stream(base + static_cast<size_t>(r) * g.inner), r);
     emit<R>(g, o, s, i, acc, out, partial);
 }
 
 // ---------------------------------------------------------------- second pass
 
-// Combines the `segments` partials of each output in ascending segment order.
-// WAVE = false: one thread per output. WAVE = true: one wave64 per output, for few
-// outputs with many partials (full reductions).
-template <class R, bool WAVE>
-__global__ __launch_bounds__(kBlock) void reduce_finalize_kernel(const typename R::Acc* __restrict__ partial,
-                                                                float* __restrict__ out, Geom g) {
+// Combines the `segments` partials of each output, always in the same order.
+// One wave64 per output: for a handful of outputs with many partials (full reductions).
+template <class R>
+__global__ __launch_bounds__(kBlock) void reduce_finalize_wave_kernel(const typename R::Acc* __restrict__ partial,
+                                                                     float* __restrict__ out, Geom g) {
     using Acc = typename R::Acc;
     const uint64_t n_out = static_cast<uint64_t>(g.outer) * g.inner;
-    if (WAVE) {
-        const uint64_t idx = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
-        const uint32_t lane = threadIdx.x & (kWave - 1);
-        Acc acc = R::init();
-        if (idx < n_out) {
-            const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
-            for (uint32_t s = lane; s < g.segments; s += kWave)
-                acc = R::merge(acc, partial[(static_cast<size_t>(o) * g.segments + s) * g.inner + i]);
-        }
-#pragma unroll
-        for (int m = kWave / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
-        if (lane == 0 && idx < n_out) out[idx] = R::finish(acc, g.axis);
-    } else {
-        const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-        if (idx >= n_out) return;
+    const uint64_t idx = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    Acc acc = R::init();
+    if (idx < n_out) {
         const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
-        Acc acc = partial[(static_cast<size_t>(o) * g.segments) * g.inner + i];
-        for (uint32_t s = 1; s < g.segments; s++)
-            acc = R::merge(acc, partial[(static_cast<size_t>(o) * g.segments + s) * g.inner + i]);
-        out[idx] = R::finish(acc, g.axis);
+        const Acc* p = partial + (static_cast<size_t>(o) * g.segments) * g.inner + i;
+#pragma unroll 8
+        for (uint32_t s = lane; s < g.segments; s += kWave) acc = R::merge(acc, p[static_cast<size_t>(s) * g.inner]);
     }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
+    if (lane == 0 && idx < n_out) out[idx] = R::finish(acc, g.axis);
+}
+
+// 64 adjacent outputs x TY segment groups per workgroup: loads are coalesced along the
+// outputs, group y folds segments y, y + TY, ..., and LDS folds the TY groups in order.
+template <class R, int TY>
+__global__ __launch_bounds__(kWave * TY) void reduce_finalize_tile_kernel(const typename R::Acc* __restrict__ partial,
+                                                                          float* __restrict__ out, Geom g) {
+    using Acc = typename R::Acc;
+    const uint64_t n_out = static_cast<uint64_t>(g.outer) * g.inner;
+    const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kWave + threadIdx.x;
+    const uint32_t ty = threadIdx.y;
+    Acc acc = R::init();
+    if (idx < n_out) {
+        const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
+        const Acc* p = partial + (static_cast<size_t>(o) * g.segments) * g.inner + i;
+#pragma unroll 8
+        for (uint32_t s = ty; s < g.segments; s += TY) acc = R::merge(acc, p[static_cast<size_t>(s) * g.inner]);
+    }
+    if (TY > 1) {
+        __shared__ Acc lds[TY][kWave];
+        lds[ty][threadIdx.x] = acc;
+        __syncthreads();
+        if (ty == 0) {
+#pragma unroll
+            for (int w = 1; w < TY; w++) acc = R::merge(acc, lds[w][threadIdx.x]);
+        }
+    }
+    if (ty == 0 && idx < n_out) out[idx] = R::finish(acc, g.axis);
 }
 
 // ---------------------------------------------------------------- host planning
@@ -279,7 +307,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     const uint64_t n_out = static_cast<uint64_t>(outer) * inner;
 
     enum { ROWS, COLS, STRIDED } kind;
-    int G = 1, VEC = 1;
+    int G = 1, VEC = 1, WY = 4;
     uint32_t tiles = 0;
     uint64_t blocks = 0;
     if (inner == 1) {
@@ -288,14 +316,17 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         const uint32_t per_lane = axis / VEC;          // loads per row
         G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : 1;
         const uint64_t base_blocks = ceil_div(outer, kBlock / G);
-        plan_segments(&g, base_blocks, target, G * VEC, G * VEC * 8);
+        plan_segments(&g, base_blocks, target / 2, G * VEC, G * VEC * 16);
         blocks = base_blocks * g.segments;
     } else if (inner >= 64) {
         kind = COLS;
         VEC = (inner % 4 == 0) ? 4 : 1;
         tiles = ceil_div(inner, kWave * VEC);
         const uint64_t base_blocks = static_cast<uint64_t>(tiles) * outer;
-        plan_segments(&g, base_blocks, target, 4, 4 * 8);
+        // Few column tiles and a long axis: 16 waves per workgroup fold 16 rows at a time
+        // through LDS, which cuts the number of partials per output by four.
+        WY = (base_blocks * 4 < target && axis >= 2048) ? 16 : 4;
+        plan_segments(&g, base_blocks, WY == 16 ? target / 4 : target, WY, WY * 8);
         blocks = base_blocks * g.segments;
     } else {
         kind = STRIDED;
@@ -329,8 +360,10 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
             }
 #undef ROWS_LAUNCH
         } else if (kind == COLS) {
-            if (VEC == 4) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
-            else          hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+            if (VEC == 4 && WY == 16) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 16>), grid, dim3(kWave, 16), 0, stream, in, out, partial, g, tiles);
+            else if (VEC == 4)        hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+            else if (WY == 16)        hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 16>), grid, dim3(kWave, 16), 0, stream, in, out, partial, g, tiles);
+            else                      hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
         } else {
             hipLaunchKernelGGL((reduce_strided_kernel<R>), grid, dim3(kBlock), 0, stream, in, out, partial, g);
         }
@@ -338,11 +371,14 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     }
     if (e == hipSuccess && g.segments > 1) {
         LaunchScope scope("reduce_finalize_kernel", R::name, 0);
-        if (n_out < 4096 && g.segments > 16)
-            hipLaunchKernelGGL((reduce_finalize_kernel<R, true>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
+        if (n_out < 64)
+            hipLaunchKernelGGL((reduce_finalize_wave_kernel<R>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
+                               partial, out, g);
+        else if (g.segments >= 8)
+            hipLaunchKernelGGL((reduce_finalize_tile_kernel<R, 4>), dim3(ceil_div(n_out, kWave)), dim3(kWave, 4), 0, stream,
                                partial, out, g);
         else
-            hipLaunchKernelGGL((reduce_finalize_kernel<R, false>), dim3(ceil_div(n_out, kBlock)), dim3(kBlock), 0, stream,
+            hipLaunchKernelGGL((reduce_finalize_tile_kernel<R, 1>), dim3(ceil_div(n_out, kWave)), dim3(kWave, 1), 0, stream,
                                partial, out, g);
         e = hipGetLastError();
     }

@@ -137,7 +137,7 @@ def _bytes5(d):
     big = 22 * m                      # F1-F4, B1-B8: the passes over [rows, cols]
     small = (2 * c                    # w read by x*w and g*w
              + 1                      # b read by +b
-             + 1 + 1                  # sum() output, the [1] seed gradient read by broadcastTo
+             + 1 + 1 + 1              # sum() output, the [1] seed gradient written, then read by broadcastTo
              + c + (c + 1)            # sum(0) -> [cols] for b, then sum(0, keep) -> [1]
              + c                      # sum(0) -> [cols] for w
              + 3 * c + 3)             # gradient += g on w and b (read, read, write)
