@@ -130,15 +130,35 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
         const float* base = in + static_cast<size_t>(row) * g.axis;
         const uint32_t begin = s * g.seg_len;
         const uint32_t end = min(begin + g.seg_len, g.axis);
+        // Loads are issued kBatch at a time before any of them is consumed, so every
+        // thread keeps kBatch requests in flight.
+        constexpr uint32_t kBatch = 8;
         if (VEC == 4) {
-#pragma unroll 4
-            for (uint32_t j = begin + lane * 4; j < end; j += G * 4) {
+            uint32_t j = begin + lane * 4;
+            for (; j + (kBatch - 1) * G * 4 < end; j += kBatch * G * 4) {
+                float4 v[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + j + k * G * 4);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) {
+                    const uint32_t jj = j + k * G * 4;
+                    R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3);
+                }
+            }
+            for (; j < end; j += G * 4) {
                 float4 v = ld4_stream(base + j);
                 R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
             }
         } else {
-#pragma unroll 4
-            for (uint32_t j = begin + lane; j < end; j += G) R::step(acc, ld1_stream(base + j), j);
+            uint32_t j = begin + lane;
+            for (; j + (kBatch - 1) * G < end; j += kBatch * G) {
+                float v[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + j + k * G);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) R::step(acc, v[k], j + k * G);
+            }
+            for (; j < end; j += G) R::step(acc, ld1_stream(base + j), j);
         }
     }
     constexpr int kLanes = G < kWave ? G : kWave;
@@ -182,8 +202,28 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
         const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
         const uint32_t begin = s * g.seg_len;
         const uint32_t end = min(begin + g.seg_len, g.axis);
-#pragma unroll 4
-        for (uint32_t r = begin + ty; r < end; r += WY) {
+        constexpr uint32_t kBatch = 8;          // loads in flight per thread
+        uint32_t r = begin + ty;
+        for (; r + (kBatch - 1) * WY < end; r += kBatch * WY) {
+            if (VEC == 4) {
+                float4 v[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WY) * g.inner);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) {
+                    const uint32_t rr = r + k * WY;
+                    R::step(acc[0], v[k].x, rr); R::step(acc[1 % VEC], v[k].y, rr);
+                    R::step(acc[2 % VEC], v[k].z, rr); R::step(acc[3 % VEC], v[k].w, rr);
+                }
+            } else {
+                float v[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + static_cast<size_t>(r + k * WY) * g.inner);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], v[k], r + k * WY);
+            }
+        }
+        for (; r < end; r += WY) {
             const float* p = base + static_cast<size_t>(r) * g.inner;
             if (VEC == 4) {
                 float4 v = ld4_stream(p);
@@ -224,8 +264,16 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __r
     const uint32_t begin = s * g.seg_len;
     const uint32_t end = min(begin + g.seg_len, g.axis);
     typename R::Acc acc = R::init();
-#pragma unroll 4
-    for (uint32_t r = begin; r < end; r++) R::step(acc, ld1_stream(base + static_cast<size_t>(r) * g.inner), r);
+    constexpr uint32_t kBatch = 8;
+    uint32_t r = begin;
+    for (; r + kBatch <= end; r += kBatch) {
+        float v[kBatch];
+#pragma unroll
+        for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + static_cast<size_t>(r + k) * g.inner);
+#pragma unroll
+        for (uint32_t k = 0; k < kBatch; k++) R::step(acc, v[k], r + k);
+    }
+    for (; r < end; r++) R::step(acc, ld1_stream(base + static_cast<size_t>(r) * g.inner), r);
     emit<R>(g, o, s, i, acc, out, partial);
 }
 
