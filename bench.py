@@ -25,6 +25,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
+# scaled by what the same counter reads for the plain copy kernel unary_kernel<OpIdentity>
+# of 262 144 KiB (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.000). Source: profiles/*.md.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg5", "binary_same_kernel<OpTimes>"): int((262151 * 1.9998 + 262144) * 1024),
+}
 METRIC = "achieved HBM GB/s (% of MI355X peak) for broadcast binary ops and axis sum"
 
 
@@ -163,7 +170,8 @@ def main():
         dom, (n, b, ms) = max(kernels.items(), key=lambda kv: kv[1][2])
         achieved = b / ms / 1e6
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
                     "bytes_per_launch": b // n, "avg_launch_us": round(ms / n * 1e3, 3), "launches": n,
                     "kernel_time_share": round(ms / tot, 4)}
 
