@@ -4,6 +4,10 @@
 // workgroup of 256 threads (4 wave64s) covers a contiguous 8 KiB span per operand.
 #include "kth_internal.h"
 #include "kth_ops.h"
+#include "kth_tables.h"
+
+#include <cmath>
+#include <cstring>
 
 using namespace kth;
 
@@ -54,6 +58,71 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const float* a, float* ou
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
         uint32_t i = (n4 << 2) + threadIdx.x;
         out[i] = Op::apply(a[i], p, q);
+    }
+}
+
+// ---------------------------------------------------------------- table-driven exp / log
+
+__device__ LogEntry g_log_table[kLogTableEntries];
+__device__ double   g_exp_table[kExpTableEntries];
+
+struct OpLogT {
+    static constexpr const char* name = "OpLog";
+    static constexpr int kTableDoubles = 2 * kLogTableEntries;
+    static __device__ __forceinline__ const double* table() { return reinterpret_cast<const double*>(g_log_table); }
+    static __device__ __forceinline__ float apply(float x, const double* lds) {
+        return table_log(x, reinterpret_cast<const LogEntry*>(lds));
+    }
+};
+struct OpExpT {
+    static constexpr const char* name = "OpExp";
+    static constexpr int kTableDoubles = kExpTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_exp(x, lds); }
+};
+// sigmoid = 1f / (1f + exp(-1f * x)), exp rounded to float first (JVMRawTensor.kt:399).
+struct OpSigmoidT {
+    static constexpr const char* name = "OpSigmoid";
+    static constexpr int kTableDoubles = kExpTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) {
+        float m = -1.0f * x;
+        float e = table_exp(m, lds);
+        float d = 1.0f + e;
+        return 1.0f / d;
+    }
+};
+
+// Unary map whose op reads a small f64 table through LDS. The data loads of the tile are
+// issued first, the table copy overlaps them. Four float4 per thread, so the 1-2 KiB
+// table is amortised over a 16 KiB tile.
+constexpr int kLdsUnroll = 4;
+template <class Op>
+__global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float* out, uint32_t n) {
+    __shared__ double tab[Op::kTableDoubles];
+    const uint32_t n4 = n >> 2;
+    const uint32_t base = blockIdx.x * (kBlock * kLdsUnroll) + threadIdx.x;
+    float4 v[kLdsUnroll];
+#pragma unroll
+    for (int k = 0; k < kLdsUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) v[k] = ld4(a, i);
+    }
+    for (int i = threadIdx.x; i < Op::kTableDoubles; i += kBlock) tab[i] = Op::table()[i];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kLdsUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            r.x = Op::apply(v[k].x, tab); r.y = Op::apply(v[k].y, tab);
+            r.z = Op::apply(v[k].z, tab); r.w = Op::apply(v[k].w, tab);
+            st4(out, i, r);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        uint32_t i = (n4 << 2) + threadIdx.x;
+        out[i] = Op::apply(a[i], tab);
     }
 }
 
@@ -334,6 +403,14 @@ void launch_unary(const float* a, float* out, uint32_t n, float p, float q) {
 }
 
 template <class Op>
+void launch_unary_lds(const float* a, float* out, uint32_t n) {
+    LaunchScope scope("unary_lds_kernel", Op::name, static_cast<uint64_t>(n) * 8);
+    const uint64_t tile = static_cast<uint64_t>(kBlock) * kLdsUnroll;
+    const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + tile - 1) / tile);
+    hipLaunchKernelGGL((unary_lds_kernel<Op>), dim3(blocks == 0 ? 1 : blocks), dim3(kBlock), 0, state().stream, a, out, n);
+}
+
+template <class Op>
 void launch_scalar(bool rev, const float* a, float* out, uint32_t n, float c, float eps) {
     LaunchScope scope(rev ? "scalar_kernel_rev" : "scalar_kernel", Op::name, static_cast<uint64_t>(n) * 8);
     if (rev) hipLaunchKernelGGL((scalar_kernel<Op, true>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
@@ -422,8 +499,10 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
 #define U(OP) if (n32) launch_unary<OP>(pa, po, n32, 0.0f, 0.0f)
     switch (op) {
     case KTH_NEG: U(OpNeg); break;           case KTH_RECIPROCAL: U(OpReciprocal); break;
-    case KTH_LOG: U(OpLog); break;           case KTH_EXP: U(OpExp); break;
-    case KTH_TANH: U(OpTanh); break;         case KTH_SIGMOID: U(OpSigmoid); break;
+    case KTH_LOG: if (n32) launch_unary_lds<OpLogT>(pa, po, n32); break;
+    case KTH_EXP: if (n32) launch_unary_lds<OpExpT>(pa, po, n32); break;
+    case KTH_TANH: U(OpTanh); break;
+    case KTH_SIGMOID: if (n32) launch_unary_lds<OpSigmoidT>(pa, po, n32); break;
     case KTH_SINH: U(OpSinh); break;         case KTH_COSH: U(OpCosh); break;
     case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
     case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSin); break;
@@ -612,3 +691,31 @@ int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
 }
 
 }  // extern "C"
+
+namespace kth {
+
+hipError_t init_math_tables() {
+    LogEntry log_tab[kLogTableEntries];
+    double exp_tab[kExpTableEntries];
+    for (int i = 0; i < kLogTableEntries; i++) {
+        // The z values with index i have bit patterns kLogOff + (i << 45) + [0, 2^45).
+        uint64_t lo_bits = kLogOff + (static_cast<uint64_t>(i) << 45), hi_bits = lo_bits + (1ull << 45);
+        double lo, hi;
+        memcpy(&lo, &lo_bits, 8); memcpy(&hi, &hi_bits, 8);
+        if (lo == 1.0) {                       // the interval that starts at 1: exact, no cancellation near 1
+            log_tab[i].invc = 1.0; log_tab[i].logc = 0.0;
+            continue;
+        }
+        const long double c = (static_cast<long double>(lo) + static_cast<long double>(hi)) / 2.0L;
+        const double invc = static_cast<double>(1.0L / c);
+        log_tab[i].invc = invc;
+        log_tab[i].logc = static_cast<double>(-logl(static_cast<long double>(invc)));
+    }
+    for (int i = 0; i < kExpTableEntries; i++)
+        exp_tab[i] = static_cast<double>(exp2l(static_cast<long double>(i) / kExpTableEntries));
+    hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_log_table), log_tab, sizeof(log_tab));
+    if (e != hipSuccess) return e;
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_exp_table), exp_tab, sizeof(exp_tab));
+}
+
+}  // namespace kth

@@ -81,6 +81,10 @@ Store* lookup(uint64_t handle, const char* what);
 float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
 void   workspace_release(float* p, uint64_t cap_bytes);
 
+// Computes the exp / log tables on the host (extended precision) and copies them into the
+// device symbols of the elementwise kernels. Called once from kth_init.
+hipError_t init_math_tables();
+
 // Brackets the launch of one kernel: counts it for kth_metrics and, while a profile is
 // being recorded, puts a HIP event before and after it on the library's stream.
 class LaunchScope {

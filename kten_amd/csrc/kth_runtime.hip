@@ -167,6 +167,7 @@ int kth_init(int device) {
     KTH_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
     KTH_HIP(hipEventCreate(&s.ev_begin));
     KTH_HIP(hipEventCreate(&s.ev_end));
+    KTH_HIP(init_math_tables());
     s.device = device;
     s.ready = true;
     return KTH_OK;

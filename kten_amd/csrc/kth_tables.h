@@ -1,0 +1,75 @@
+// Table-driven exp and log for the "f64 libm, round once to f32" rule of kotlin.math
+// (JVMRawTensor.kt:144,395,399). Both evaluate in f64 to about 1e-16 relative error, so
+// after the single rounding to fp32 they return the correctly rounded float for all but a
+// vanishing fraction of inputs, while costing about twenty f64 operations, which keeps
+// the elementwise kernels HBM-bound. The tables are computed on the host in extended
+// precision when the library is initialised and read through LDS.
+//
+//   log: x = z * 2^k with z in [0.6875, 1.375); the top 7 mantissa bits of z pick a
+//        centre c with invc ~ 1/c and logc = -log(invc); r = z * invc - 1 (one fma, so
+//        exact up to its own rounding), |r| < 2^-7;
+//        log x = k ln2 + logc + log1p(r), log1p by its Taylor series to r^7.
+//        The interval starting at 1.0 has invc = 1, logc = 0: no cancellation near 1.
+//   exp: k = round(x * 128 / ln2), r = x - k ln2 / 128 (two fmas with a split constant),
+//        |r| <= ln2 / 256; e^x = 2^(k >> 7) * T[k & 127] * e^r, T[i] = 2^(i/128),
+//        e^r by its Taylor series to r^6, scaling by ldexp (handles overflow to inf and
+//        gradual underflow).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace kth {
+
+constexpr int kLogTableEntries = 128;     // {invc, logc} pairs
+constexpr int kExpTableEntries = 128;
+
+struct LogEntry { double invc, logc; };
+
+constexpr uint64_t kLogOff = 0x3fe6000000000000ull;   // 0.6875
+
+__device__ __forceinline__ float table_log(float x, const LogEntry* tab) {
+    const double d = static_cast<double>(x);                 // exact; fp32 denormals become normal doubles
+    const uint64_t ix = static_cast<uint64_t>(__double_as_longlong(d));
+    const uint64_t tmp = ix - kLogOff;
+    const int i = static_cast<int>(tmp >> 45) & (kLogTableEntries - 1);
+    const int k = static_cast<int>(static_cast<int64_t>(tmp) >> 52);
+    const double z = __longlong_as_double(static_cast<long long>(ix - (tmp & 0xfff0000000000000ull)));
+    const LogEntry e = tab[i];
+    const double r = fma(z, e.invc, -1.0);
+    double p = fma(r, 1.0 / 7.0, -1.0 / 6.0);
+    p = fma(r, p, 1.0 / 5.0);
+    p = fma(r, p, -1.0 / 4.0);
+    p = fma(r, p, 1.0 / 3.0);
+    p = fma(r, p, -1.0 / 2.0);
+    const double l1p = fma(r * r, p, r);
+    const double y = fma(static_cast<double>(k), 0.693147180559945309417232121458, e.logc) + l1p;
+    float res = static_cast<float>(y);
+    // Math.log: NaN or negative -> NaN, +-0 -> -inf, +inf -> +inf.
+    if (x == 0.0f) res = -INFINITY;
+    if (x < 0.0f) res = __uint_as_float(0x7fc00000u);
+    if (!(x < INFINITY)) res = x;                            // +inf and NaN pass through
+    return res;
+}
+
+__device__ __forceinline__ float table_exp(float x, const double* tab) {
+    // Outside [-120, 100] the fp32 result is already 0 or inf; clamping keeps k in int range.
+    const double d = fmin(fmax(static_cast<double>(x), -120.0), 100.0);
+    const double kd = rint(d * 184.664965233787316142070359168242182);   // 128 / ln2
+    const int k = static_cast<int>(kd);
+    // ln2 / 128 split so that kd * hi is exact for |kd| < 2^16.
+    double r = fma(kd, -0x1.62e42fefa0000p-8, d);
+    r = fma(kd, -0x1.cf79abc9e3b3ap-47, r);
+    const double s = tab[k & (kExpTableEntries - 1)];
+    double p = fma(r, 1.0 / 720.0, 1.0 / 120.0);
+    p = fma(r, p, 1.0 / 24.0);
+    p = fma(r, p, 1.0 / 6.0);
+    p = fma(r, p, 0.5);
+    p = fma(r * r, p, r);                                    // e^r - 1
+    const double y = ldexp(fma(s, p, s), k >> 7);
+    float res = static_cast<float>(y);
+    if (x != x) res = x;
+    return res;
+}
+
+}  // namespace kth

@@ -1,0 +1,55 @@
+"""Unary ops over the whole fp32 input space, against the CPU checker.
+
+By default every 509th bit pattern of the 2^32 (8.4 M inputs per op, every exponent and
+sign, all specials) is checked. With KTEN_ALL_FLOATS=1 all 2^32 patterns are checked,
+64 Mi at a time (about a minute of CPU time per op for the checker): run by hand, results
+recorded in the design notes.
+Bars: exact ops bit-exact; f64-libm-then-round ops at most 2 ulp (NaN matches NaN)."""
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import pytest
+
+from oracle import jvm_oracle as jo
+from parity import ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+EXACT = ["neg", "reciprocal", "abs", "sign", "sqrt", "floor", "ceil", "round", "trunc", "rsqrt"]
+LIBM = ["log", "exp", "sigmoid", "tanh", "sinh", "cosh", "sin", "cos", "tan", "asin", "acos", "atan"]
+FULL = os.environ.get("KTEN_ALL_FLOATS") == "1"
+CHUNK = 1 << 26
+
+
+def chunks():
+    if FULL:
+        for start in range(0, 1 << 32, CHUNK):
+            yield np.arange(start, start + CHUNK, dtype=np.uint64).astype(np.uint32)
+    else:
+        yield np.arange(0, 1 << 32, 509, dtype=np.uint64).astype(np.uint32)
+
+
+def checker(op, x):
+    """The single-threaded checker on 16 slices at once (ctypes releases the GIL)."""
+    parts = np.array_split(x, 16)
+    with ThreadPoolExecutor(16) as pool:
+        return np.concatenate(list(pool.map(lambda p: jo.unary(op, p), parts)))
+
+
+@pytest.mark.parametrize("op", EXACT + LIBM)
+def test_unary_over_the_float_space(op, hip):
+    worst, differing, total = 0, 0, 0
+    for bits in chunks():
+        x = bits.view(np.float32)
+        with hip.garbageCollector():
+            got = hip.createRaw([x.size], x)._unary(op).toArray()
+        want = checker(op, x)
+        d = ulp_distance(got, want)
+        if op in EXACT:
+            # +0 and -0 are one "ulp step" apart in this metric and must not be confused
+            bad = np.flatnonzero(d)
+            assert bad.size == 0, f"{op}: {bad.size} mismatches, first x={x[bad[0]]!r} got {got[bad[0]]!r} want {want[bad[0]]!r}"
+        worst = max(worst, int(d.max())); differing += int(np.count_nonzero(d)); total += x.size
+    print(f"{op}: {total} inputs, {differing} differ from the checker, max distance {worst} ulp")
+    assert worst <= 2
