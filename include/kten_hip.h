@@ -20,7 +20,8 @@
  *   - Shapes travel by value inside the kernel arguments; nothing is uploaded per launch.
  *   - All launches are asynchronous on one internal in-order stream. The only blocking
  *     calls are kth_upload (above 1 MiB), kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
- *     kth_timer_end, kth_profile_end and kth_shutdown.
+ *     kth_gather / kth_scatter / kth_scatter_fill (they report bad index values), kth_timer_end,
+ *     kth_profile_end and kth_shutdown.
  *   - Shape / argument errors are reported before anything is launched, as the
  *     reference throws IllegalArgumentException host-side before computing
  *     (JVM:89-93, ShapeFunctions.kt:187-201).
@@ -172,6 +173,28 @@ int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t 
 
 /* sum() / mean() (RAW:121-122; JVM:146-152) of n values into out[0]. op: KTH_SUM, KTH_MEAN. */
 int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
+
+/* ------------------------------------------------------------------ indexed moves along an axis */
+
+/* gather (RAW:164; JVM:334-353). in and index have `dims` dims; out has index's shape:
+ * out[p, i] = in[p, (int) index[p, i]] for every position p of index's shape without the
+ * axis. index dims other than the axis must not exceed in's. Blocking: an index value
+ * outside [0, in_shape[axis]) returns KTH_E_ARGUMENT, as the reference throws
+ * IllegalArgumentException (JVM:345-346). */
+int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32_t* index_shape,
+               int dims, int axis, uint64_t out);
+
+/* inplaceScatter / inplaceScatterAdd(axis, index, src) (RAW:146-148; JVM:227-255):
+ * target[p, (int) index[p, i]] = (or +=, when add != 0) src[p, i], i ascending, so
+ * duplicate indices inside one position resolve as on the JVM. Shape rule of
+ * kten-api/.../autograd/utils/ShapeFunctions.kt:346-371 (else KTH_E_SHAPE). Blocking:
+ * an out-of-range index returns KTH_E_ARGUMENT (JVM:238-239). */
+int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
+                uint64_t src, const int32_t* src_shape, int dims, int axis);
+
+/* inplaceScatter(axis, index, Float) (RAW:150; JVM:317-332). */
+int kth_scatter_fill(uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
+                     int dims, int axis, float value);
 
 /* ------------------------------------------------------------------ control and metrics */
 

@@ -54,6 +54,10 @@ SIGNATURES = {
     "kth_broadcast_to": (c_int, [c_uint64, POINTER(c_int32), c_int, c_uint64, POINTER(c_int32), c_int]),
     "kth_reduce_axis": (c_int, [c_int, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
     "kth_reduce_all": (c_int, [c_int, c_uint64, c_uint64, c_uint64]),
+    "kth_gather": (c_int, [c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_int, c_int, c_uint64]),
+    "kth_scatter": (c_int, [c_int, c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32),
+                            c_int, c_int]),
+    "kth_scatter_fill": (c_int, [c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_int, c_int, c_float]),
     "kth_sync": (c_int, []),
     "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
     "kth_timer_begin": (c_int, []),

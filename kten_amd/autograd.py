@@ -133,6 +133,15 @@ class AGTensor(Tensor):
     def sum(self, axis=_NO_AXIS, keepDimensions=False): return Sum(self.ops)(self, axis, keepDimensions)
     def mean(self, axis=_NO_AXIS, keepDimensions=False): return Mean(self.ops)(self, axis, keepDimensions)
 
+    def max(self, axis, keepDimensions=False): return Max(self.ops)(self, axis, keepDimensions)
+    def min(self, axis, keepDimensions=False): return Min(self.ops)(self, axis, keepDimensions)
+    def gather(self, axis, index): return Gather(self.ops)(self, axis, index)
+    def scatter(self, axis, index, source): return Scatter(self.ops)(self, axis, index, source)
+
+    def softmaxCrossEntropy(self, targets):
+        """functions/nn/TensorExtensions.kt: logits.softmaxCrossEntropy(targets)."""
+        return SoftmaxCrossEntropy(self.ops)(self, targets)
+
     def argMax(self, axis=0, keepDimensions=False):
         return NoGradVariable(self.ops, self._forwarded().getRawValue().argMax(axis, keepDimensions))
 
@@ -228,6 +237,13 @@ class NoGradVariable(AGTensor):
 
     def max(self, axis, keepDimensions=False): return self._new(self.rawValue.max(axis, keepDimensions))
     def min(self, axis, keepDimensions=False): return self._new(self.rawValue.min(axis, keepDimensions))
+    def gather(self, axis, index): return self._new(self.rawValue.gather(axis, index.getRawValue()))          # :196
+
+    def scatter(self, axis, index, source):                                                                   # :198-202
+        if source.requiresGrad:
+            return AGTensor.scatter(self, axis, index, source)
+        return self._new(self.rawValue.scatter(axis, index.getRawValue(), source.getRawValue()))
+
     def clamp(self, min, max): return self._new(self.rawValue.clamp(float(min), float(max)))
     def _reshape(self, newShape): return self._new(self.rawValue.reshape(newShape))
     def _expand(self, newShape): return self._new(self.rawValue.broadcastTo(newShape))
@@ -830,6 +846,35 @@ class Mean(AggregatorFunction):                                                 
         return [gradInput]
 
 
+class SelectionFunction(AggregatorFunction):                                          # :56-81
+    """Max / Min: the forward keeps the arg indices; the backward scatters the gradient
+    into zeros at those indices."""
+    def select(self, tensor, axis, keepDimensions): raise NotImplementedError
+
+    def doForward(self, input):
+        self.inputShape = list(input.shape)
+        res, indices = self.select(input, self.axis, self.keepDimensions)
+        self.saveForBackward(input, indices)
+        self.output = res
+
+    def doBackward(self, gradient):
+        input, indices = self.valuesSaved
+        gradInput = self.ops.zerosLike(input)
+        if not self.keepDimensions and len(self.inputShape) != 1:
+            gradient.inplaceUnsqueeze(self.axis)
+            indices.inplaceUnsqueeze(self.axis)
+        gradInput.inplaceScatter(self.axis, indices, gradient)
+        return [gradInput]
+
+
+class Max(SelectionFunction):                                                         # :83-87
+    def select(self, t, axis, keep): return t.max(axis, keep), t.argMax(axis, keep)
+
+
+class Min(SelectionFunction):                                                         # :89-93
+    def select(self, t, axis, keep): return t.min(axis, keep), t.argMin(axis, keep)
+
+
 # ------------------------------------------------------------------ TensorFunctions.kt
 
 class Reshape(UnaryTensorFunction):                                                   # :200-231
@@ -877,6 +922,105 @@ class Expand(UnaryTensorFunction):                                              
             if i > 0:
                 self.ops.release(to_release)
         return [g]
+
+
+class Gather(UnaryTensorFunction):                                                    # :444-479
+    modifiesShape = True
+
+    def __call__(self, tensor, axis, index):
+        if index.requiresGrad:
+            raise ValueError("Gather cannot differentiate the index. The index tensor passed to gather should never "
+                             "require gradients.")
+        super().__call__(tensor)
+        self.axis, self.index = axis, index
+        return self
+
+    def doForward(self, input):
+        self.inputShape = list(input.shape)
+        indexRaw = self.index.getRawValue()
+        self.saveForBackward(indexRaw)
+        self.output = input.gather(self.axis, indexRaw)
+
+    def doBackward(self, gradient):
+        gradInput = self.ops.createRawFill(self.inputShape, 0.0)
+        (index,) = self.valuesSaved
+        gradInput.inplaceScatterAdd(self.axis, index, gradient)
+        return [gradInput]
+
+
+class Scatter(BiTensorFunction):                                                      # :481-527
+    broadcastingOperation = False
+
+    def __call__(self, tensor, axis, index, source):
+        if index.requiresGrad:
+            raise ValueError("Scatter cannot differentiate the index. The index tensor passed to scatter should never "
+                             "require gradients.")
+        super().__call__(tensor, source)
+        self.cachedShape = list(tensor.shape)
+        self.axis, self.index = axis, index
+        return self
+
+    def doForward(self, tensor, source):
+        indexRaw = self.index.getRawValue()
+        self.saveForBackward(indexRaw)
+        self.output = tensor.scatter(self.axis, indexRaw, source)
+
+    def doBackward(self, gradient):
+        (index,) = self.valuesSaved
+        if index.shape != self.bShape:
+            raise ValueError(f"Index shape: {index.shape} is not compatible with source shape: {self.bShape}")
+        first, second = self.inputs
+        gradInput = gradient.scatter(self.axis, index, 0.0) if first.requiresGrad else None
+        gradSource = gradient.gather(self.axis, index) if second.requiresGrad else None
+        return [gradInput, gradSource]
+
+
+class SoftmaxCrossEntropy(UnaryTensorFunction):
+    """functions/nn/SoftmaxCrossEntropy.kt:10-69 — composed entirely of raw ops on the
+    path: max, minus, exp, sum, div, clamp, log, gather, neg, mean; the backward is
+    zerosLike, scatter of -1, plusAssign, divAssign (and, as in the reference, does not
+    use the incoming gradient)."""
+    modifiesShape = True
+    epsilon = 1e-7          # PlatformProvider.epsilon
+
+    def __call__(self, logits, targets):
+        super().__call__(logits)
+        self.cachedShape = [1]
+        if targets.requiresGrad:
+            raise ValueError("SoftmaxCrossEntropy only accept targets that don't require gradients")
+        if logits.dimensions != 2:
+            raise ValueError(f"SoftmaxCrossEntropy requires 2D logits, but got tensor with shape {logits.shape}")
+        if targets.dimensions != 1:
+            raise ValueError(f"SoftmaxCrossEntropy requires 1D targets, but got tensor with shape {targets.shape}")
+        if logits.shape[0] != targets.shape[0]:
+            raise ValueError("Logits must have the same size at the first dimension as targets, but got tensors with "
+                             f"shape: logits: {logits.shape}, targets: {targets.shape}")
+        self.targets = targets.unsqueeze(-1)
+        return self
+
+    def doForward(self, input):
+        maxVal = input.max(-1, keepDimensions=True)
+        inputMinusMax = input - maxVal
+        expVal = inputMinusMax.exp()
+        expValSum = expVal.sum(-1, keepDimensions=True)
+        softmaxRes = expVal / expValSum
+        self.saveForBackward(softmaxRes)
+        softmaxSum = softmaxRes.sum(-1, keepDimensions=True)
+        softmaxNorm = softmaxRes / softmaxSum
+        softmaxNormClip = softmaxNorm.clamp(_f32(self.epsilon), _f32(1.0 - _f32(self.epsilon)))
+        logSoftmax = softmaxNormClip.log()
+        logSoftmaxAtTargets = logSoftmax.gather(-1, self.targets.getRawValue())
+        negativeLogLikelihood = -logSoftmaxAtTargets
+        self.output = negativeLogLikelihood.mean()
+        self.ops.release(maxVal, inputMinusMax, expVal, expValSum, softmaxSum, softmaxNorm, softmaxNormClip, logSoftmax,
+                         logSoftmaxAtTargets, negativeLogLikelihood)
+
+    def doBackward(self, gradient):
+        gradIn = self.ops.zerosLike(self.valuesSaved[0])
+        gradIn.inplaceScatter(-1, self.targets.getRawValue(), -1.0)
+        gradIn += self.valuesSaved[0]
+        gradIn /= float(self.targets.shape[0])
+        return [gradIn]
 
 
 # ------------------------------------------------------------------ companion factories

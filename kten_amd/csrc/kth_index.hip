@@ -1,0 +1,247 @@
+// gather / inplaceScatter / inplaceScatterAdd / inplaceScatter(Float) along an axis
+// (reference: JVMRawTensor.kt:227-255,317-353 with StoreIndexing.applyAt,
+// AbstractIndexing.kt:123-146). Positions run over the index tensor's shape without the
+// axis; one thread owns one position and walks the axis in ascending order, so within a
+// position duplicates resolve exactly as on the JVM ("last write wins", "added in order"),
+// and different positions never touch the same target element.
+// Index values are floats: Kotlin's toInt() (truncate, NaN -> 0, saturate) is what
+// v_cvt_i32_f32 does. An index outside [0, axis length) is skipped and reported: the host
+// turns the report into the reference's IllegalArgumentException.
+#include "kth_internal.h"
+
+using namespace kth;
+
+namespace {
+
+constexpr int kBlock = 256;
+
+struct FastDiv { uint32_t mul, shift; };
+
+// Dim 0 is the innermost of the position dims (index shape without the axis).
+struct IndexPlan {
+    int      ndim;
+    uint32_t size[KTH_MAX_DIMS];
+    FastDiv  div[KTH_MAX_DIMS];
+    uint32_t i_stride[KTH_MAX_DIMS];   // index tensor (and, for gather, the result)
+    uint32_t a_stride[KTH_MAX_DIMS];   // gather: input; scatter: target
+    uint32_t b_stride[KTH_MAX_DIMS];   // scatter: source
+    uint32_t i_axis_stride, a_axis_stride, b_axis_stride;
+    uint32_t i_axis_len, a_axis_len;
+};
+
+__device__ __forceinline__ void locate(const IndexPlan& pl, uint32_t pos, uint32_t& io, uint32_t& ao, uint32_t& bo) {
+    io = ao = bo = 0;
+    for (int d = 0; d < pl.ndim; d++) {
+        uint32_t q = (__umulhi(pos, pl.div[d].mul) + pos) >> pl.div[d].shift;
+        uint32_t r = pos - q * pl.size[d];
+        io += r * pl.i_stride[d]; ao += r * pl.a_stride[d]; bo += r * pl.b_stride[d];
+        pos = q;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict__ in, const float* __restrict__ index,
+                                                       float* __restrict__ out, uint32_t positions, IndexPlan pl, int* bad) {
+    const uint32_t pos = blockIdx.x * kBlock + threadIdx.x;
+    if (pos >= positions) return;
+    uint32_t io, ao, bo;
+    locate(pl, pos, io, ao, bo);
+    for (uint32_t i = 0; i < pl.i_axis_len; i++) {
+        const uint32_t at = io + i * pl.i_axis_stride;
+        const int sel = static_cast<int>(index[at]);
+        if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
+        out[at] = in[ao + static_cast<uint32_t>(sel) * pl.a_axis_stride];
+    }
+}
+
+// MODE 0: assign from src, 1: add from src, 2: assign the constant.
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ target, const float* __restrict__ index,
+                                                        const float* __restrict__ src, float value, uint32_t positions,
+                                                        IndexPlan pl, int* bad) {
+    const uint32_t pos = blockIdx.x * kBlock + threadIdx.x;
+    if (pos >= positions) return;
+    uint32_t io, ao, bo;
+    locate(pl, pos, io, ao, bo);
+    for (uint32_t i = 0; i < pl.i_axis_len; i++) {
+        const int sel = static_cast<int>(index[io + i * pl.i_axis_stride]);
+        if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
+        float* to = target + ao + static_cast<uint32_t>(sel) * pl.a_axis_stride;
+        if (MODE == 2) *to = value;
+        else {
+            const float v = src[bo + i * pl.b_axis_stride];
+            if (MODE == 1) *to = *to + v; else *to = v;
+        }
+    }
+}
+
+__global__ void clear_int_kernel(int* p) { *p = 0; }
+
+FastDiv make_div(uint32_t d) {
+    FastDiv f;
+    uint32_t shift = 0;
+    while ((1ull << shift) < d) shift++;
+    f.shift = shift;
+    f.mul = static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1);
+    return f;
+}
+
+int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
+    if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
+    uint64_t n = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0) return fail(KTH_E_ARGUMENT, "%s: negative dim %d", what, shape[i]);
+        n *= static_cast<uint64_t>(shape[i]);
+        if (n > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: more than 2^31-1 elements", what);
+    }
+    *count = n;
+    return KTH_OK;
+}
+
+// Strides of `shape` for the position dims (all dims but the axis, innermost first) and for the axis.
+void strides_without_axis(const int32_t* shape, int dims, int axis, uint32_t* pos_strides, uint32_t* axis_stride) {
+    uint64_t run = 1;
+    int n = 0;
+    for (int d = dims - 1; d >= 0; d--) {
+        if (d == axis) *axis_stride = static_cast<uint32_t>(run);
+        else pos_strides[n++] = static_cast<uint32_t>(run);
+        run *= static_cast<uint64_t>(shape[d]);
+    }
+}
+
+// Runs `launch(flag)` with a cleared device flag and reports a set flag as an argument error.
+template <class F>
+int with_index_check(const char* what, F launch) {
+    State& s = state();
+    uint64_t cap;
+    int* flag = reinterpret_cast<int*>(workspace_acquire(4, &cap));
+    if (!flag) return fail(KTH_E_MEMORY, "%s: no workspace", what);
+    hipLaunchKernelGGL(clear_int_kernel, dim3(1), dim3(1), 0, s.stream, flag);
+    launch(flag);
+    hipError_t e = hipGetLastError();
+    int host_flag = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&host_flag, flag, 4, hipMemcpyDeviceToHost, s.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
+    workspace_release(reinterpret_cast<float*>(flag), cap);
+    if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    if (host_flag) return fail(KTH_E_ARGUMENT, "%s got invalid index, an index value is out of bounds at the axis", what);
+    return KTH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32_t* index_shape,
+               int dims, int axis, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "kth_gather: %d dims", dims);
+    if (axis < 0 || axis >= dims) return fail(KTH_E_ARGUMENT, "kth_gather: axis %d of %d dims", axis, dims);
+    uint64_t in_n, idx_n;
+    if (int rc = shape_count(in_shape, dims, "kth_gather(in)", &in_n)) return rc;
+    if (int rc = shape_count(index_shape, dims, "kth_gather(index)", &idx_n)) return rc;
+    for (int d = 0; d < dims; d++)
+        if (d != axis && index_shape[d] > in_shape[d])
+            return fail(KTH_E_SHAPE, "kth_gather: index dim %d (%d) exceeds the input's (%d)", d, index_shape[d], in_shape[d]);
+    Store* si = lookup(in, "kth_gather(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* sx = lookup(index, "kth_gather(index)");
+    if (!sx) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_gather(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (in_n > si->n_floats || idx_n > sx->n_floats || idx_n > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_gather: a shape needs more elements than its store holds");
+    if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_gather: output aliases an input");
+    if (idx_n == 0) return KTH_OK;
+    IndexPlan pl{};
+    pl.ndim = dims - 1;
+    uint64_t positions = 1;
+    int n = 0;
+    for (int d = dims - 1; d >= 0; d--) {
+        if (d == axis) continue;
+        pl.size[n] = static_cast<uint32_t>(index_shape[d]);
+        pl.div[n] = make_div(pl.size[n]);
+        positions *= pl.size[n];
+        n++;
+    }
+    strides_without_axis(index_shape, dims, axis, pl.i_stride, &pl.i_axis_stride);
+    strides_without_axis(in_shape, dims, axis, pl.a_stride, &pl.a_axis_stride);
+    pl.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
+    pl.a_axis_len = static_cast<uint32_t>(in_shape[axis]);
+    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+    return with_index_check("Gather", [&](int* flag) {
+        LaunchScope scope("gather_kernel", "", (2 * idx_n + idx_n) * 4);
+        hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, state().stream, si->ptr, sx->ptr, so->ptr,
+                           static_cast<uint32_t>(positions), pl, flag);
+    });
+}
+
+static int scatter_common(int mode, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
+                          uint64_t src, const int32_t* src_shape, int dims, int axis, float value) {
+    KTH_REQUIRE_INIT();
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "kth_scatter: %d dims", dims);
+    if (axis < 0 || axis >= dims) return fail(KTH_E_ARGUMENT, "kth_scatter: axis %d of %d dims", axis, dims);
+    uint64_t t_n, idx_n, src_n = 0;
+    if (int rc = shape_count(target_shape, dims, "kth_scatter(target)", &t_n)) return rc;
+    if (int rc = shape_count(index_shape, dims, "kth_scatter(index)", &idx_n)) return rc;
+    if (mode != 2) { if (int rc = shape_count(src_shape, dims, "kth_scatter(src)", &src_n)) return rc; }
+    // ShapeFunctions.kt:346-371: index must fit the source everywhere and the target off the axis.
+    for (int d = 0; d < dims; d++) {
+        if (mode != 2 && index_shape[d] > src_shape[d])
+            return fail(KTH_E_SHAPE, "Scatter requires that index.shape[a] <= src.shape[a] for all axis 'a'");
+        if (d != axis && index_shape[d] > target_shape[d])
+            return fail(KTH_E_SHAPE, "Scatter requires that index.shape[a] <= target.shape[a] for all axis 'a' except the specified axis");
+    }
+    Store* st = lookup(target, "kth_scatter(target)");
+    if (!st) return KTH_E_HANDLE;
+    Store* sx = lookup(index, "kth_scatter(index)");
+    if (!sx) return KTH_E_HANDLE;
+    Store* ss = nullptr;
+    if (mode != 2) { ss = lookup(src, "kth_scatter(src)"); if (!ss) return KTH_E_HANDLE; }
+    if (t_n > st->n_floats || idx_n > sx->n_floats || (ss && src_n > ss->n_floats))
+        return fail(KTH_E_ARGUMENT, "kth_scatter: a shape needs more elements than its store holds");
+    if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
+    if (idx_n == 0) return KTH_OK;
+    IndexPlan pl{};
+    pl.ndim = dims - 1;
+    uint64_t positions = 1;
+    int n = 0;
+    for (int d = dims - 1; d >= 0; d--) {
+        if (d == axis) continue;
+        pl.size[n] = static_cast<uint32_t>(index_shape[d]);
+        pl.div[n] = make_div(pl.size[n]);
+        positions *= pl.size[n];
+        n++;
+    }
+    strides_without_axis(index_shape, dims, axis, pl.i_stride, &pl.i_axis_stride);
+    strides_without_axis(target_shape, dims, axis, pl.a_stride, &pl.a_axis_stride);
+    if (mode != 2) strides_without_axis(src_shape, dims, axis, pl.b_stride, &pl.b_axis_stride);
+    pl.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
+    pl.a_axis_len = static_cast<uint32_t>(target_shape[axis]);
+    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+    const float* psrc = ss ? ss->ptr : nullptr;
+    const uint64_t bytes = (mode == 2 ? 2 : mode == 1 ? 4 : 3) * idx_n * 4;
+    return with_index_check("Scatter", [&](int* flag) {
+        LaunchScope scope("scatter_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
+        const dim3 grid(blocks), block(kBlock);
+        const uint32_t p32 = static_cast<uint32_t>(positions);
+        hipStream_t stream = state().stream;
+        if (mode == 0)      hipLaunchKernelGGL((scatter_kernel<0>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
+        else if (mode == 1) hipLaunchKernelGGL((scatter_kernel<1>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
+        else                hipLaunchKernelGGL((scatter_kernel<2>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
+    });
+}
+
+int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
+                uint64_t src, const int32_t* src_shape, int dims, int axis) {
+    std::lock_guard<std::mutex> g(lock());
+    return scatter_common(add ? 1 : 0, target, target_shape, index, index_shape, src, src_shape, dims, axis, 0.0f);
+}
+
+int kth_scatter_fill(uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
+                     int dims, int axis, float value) {
+    std::lock_guard<std::mutex> g(lock());
+    return scatter_common(2, target, target_shape, index, index_shape, 0, nullptr, dims, axis, value);
+}
+
+}  // extern "C"

@@ -185,6 +185,33 @@ class HipRawTensor(AbstractRawTensor):
         check(self.ops.lib.kth_reduce_all(Op.MEAN, self.storeReference, self.size, res.storeReference))
         return res
 
+    def gather(self, axis, index):
+        """JVMRawTensor.kt:334-353: the result has index's shape."""
+        self._require_live(); index._require_live()
+        a = sf.normalize_axis(self.shape, axis)
+        if index.dimensions != self.dimensions:
+            raise ValueError(f"Gather expects index with {self.dimensions} dimensions, got shape {index.shape}")
+        res = self._new(index.shape)
+        check(self.ops.lib.kth_gather(self.storeReference, abi.shape_array(self.shape), index.storeReference,
+                                      abi.shape_array(index.shape), self.dimensions, a, res.storeReference))
+        return res
+
+    def _scatter(self, axis, index, src, add):
+        """JVMRawTensor.kt:227-255 (tensor source) and 317-332 (constant)."""
+        self._require_live(); index._require_live()
+        if _is_number(src):
+            a = sf.normalize_axis(self.shape, axis)
+            if index.dimensions != self.dimensions:
+                raise ValueError(f"Scatter expects index with {self.dimensions} dimensions, got shape {index.shape}")
+            check(self.ops.lib.kth_scatter_fill(self.storeReference, abi.shape_array(self.shape), index.storeReference,
+                                                abi.shape_array(index.shape), self.dimensions, a, float(src)))
+            return
+        src._require_live()
+        a = sf.normalized_axis_scatter(self.shape, axis, index.shape, src.shape)
+        check(self.ops.lib.kth_scatter(1 if add else 0, self.storeReference, abi.shape_array(self.shape),
+                                       index.storeReference, abi.shape_array(index.shape), src.storeReference,
+                                       abi.shape_array(src.shape), self.dimensions, a))
+
     def copy(self, shallow: bool = False):
         """JVMRawTensor.kt:257-262; a shallow copy shares the store (OCLRawTensor.kt:252-258)."""
         self._require_live()

@@ -9,7 +9,7 @@ the reference. Kotlin's overloads on (tensor | Float) become one Python method t
 dispatches on the argument type; Kotlin operators are also exposed as Python operators.
 
 Members of the contract that lie outside the accelerated path (indexed get/set,
-gather/scatter, transpose/permute, BLAS, nn) are not part of this mirror.
+transpose/permute, indexSelect/indexAdd, BLAS, nn) are not part of this mirror.
 """
 from enum import Enum
 from typing import List, Sequence
@@ -214,6 +214,22 @@ class AbstractRawTensor:
 
     def argMin(self, axis: int = 0, keepDimensions: bool = False):
         return self._aggregatingOpOverAxis(axis, keepDimensions, AggregatingOperation.ARG_MIN)
+
+    # --- indexed moves along an axis (AbstractRawTensor.kt:146-164) --------------------
+    def gather(self, axis: int, index): raise NotImplementedError
+    def _scatter(self, axis: int, index, src, add: bool): raise NotImplementedError   # src: tensor or float
+
+    def inplaceScatter(self, axis: int, index, src):
+        self._scatter(axis, index, src, False)
+
+    def inplaceScatterAdd(self, axis: int, index, src):
+        self._scatter(axis, index, src, True)
+
+    def scatter(self, axis: int, index, src):
+        """AbstractRawTensor.kt:152-162: copy, then scatter into the copy."""
+        res = self.copy()
+        res.inplaceScatter(axis, index, src)
+        return res
 
     # --- broadcasting (AbstractRawTensor.kt:170-192) -----------------------------------
     def calculateCommonShapeWith(self, other) -> List[int]:

@@ -140,3 +140,20 @@ def store_index(shape: Sequence[int], index: Sequence[int]) -> int:
 def outer_axis_inner(shape: Sequence[int], axis: int):
     """The [outer, axis, inner] view of a row-major tensor around a normalised axis."""
     return to_store_size(shape[:axis]), shape[axis], to_store_size(shape[axis + 1:])
+
+
+def normalized_axis_scatter(shape: Sequence[int], axis: int, index_shape: Sequence[int], src_shape: Sequence[int]) -> int:
+    """ShapeFunctions.kt:346-371 — target, index and source have equal dim counts; the index
+    fits the source everywhere and the target everywhere but along the axis."""
+    if len(shape) != len(index_shape) or len(shape) != len(src_shape):
+        raise ValueError("Scatter expects tensors (target, index, source) to have the same dimensions, but got tensors "
+                         f"with shapes: target: {list(shape)}, index: {list(index_shape)}, source: {list(src_shape)}")
+    a = normalize_axis(shape, axis)
+    for d in range(len(shape)):
+        if index_shape[d] > src_shape[d]:
+            raise ValueError("Scatter requires that index.shape[a] <= src.shape[a] for all axis 'a', but got tensors with "
+                             f"shapes: index: {list(index_shape)}, src: {list(src_shape)}")
+        if d != a and index_shape[d] > shape[d]:
+            raise ValueError("Scatter requires that index.shape[a] <= target.shape[a] for all axis 'a', except the specified "
+                             f"'axis' of the operation, but got tensors with shapes: index: {list(index_shape)}, target: {list(shape)}")
+    return a

@@ -68,6 +68,12 @@ def lib():
     L.kjo_sum_all_f64.argtypes = [fp, c_int64]
     L.kjo_sum_all_f64.restype = c_double
     L.kjo_axis_sum_f64.argtypes = [fp, fp, fp, c_int64, c_int64, c_int64]
+    L.kjo_gather.argtypes = [fp, ip, fp, ip, c_int, c_int, fp]
+    L.kjo_gather.restype = c_int
+    L.kjo_scatter.argtypes = [c_int, fp, ip, fp, ip, fp, ip, c_int, c_int]
+    L.kjo_scatter.restype = c_int
+    L.kjo_scatter_fill.argtypes = [fp, ip, fp, ip, c_int, c_int, c_float]
+    L.kjo_scatter_fill.restype = c_int
     L.kjo_unary_f64.argtypes = [c_int, c_float]
     L.kjo_unary_f64.restype = c_double
     _lib = L
@@ -234,6 +240,28 @@ class JvmOracleRawTensor(AbstractRawTensor):
 
     def _mean_all(self):
         return self._wrap(np.array([mean_all(self.storeReference)], dtype=np.float32))
+
+    def gather(self, axis, index):
+        a = sf.normalize_axis(self.shape, axis)
+        if index.dimensions != self.dimensions:
+            raise ValueError(f"Gather expects index with {self.dimensions} dimensions, got shape {index.shape}")
+        out = np.zeros(sf.to_store_size(index.shape), dtype=np.float32)
+        if lib().kjo_gather(_p(self.storeReference), _sh(self.shape), _p(index.storeReference), _sh(index.shape),
+                            self.dimensions, a, _p(out)) != 0:
+            raise ValueError("Gather got invalid index, an index value is out of bounds at the axis")
+        return self._wrap(out, list(index.shape))
+
+    def _scatter(self, axis, index, src, add):
+        if _is_number(src):
+            a = sf.normalize_axis(self.shape, axis)
+            rc = lib().kjo_scatter_fill(_p(self.storeReference), _sh(self.shape), _p(index.storeReference),
+                                        _sh(index.shape), self.dimensions, a, float(src))
+        else:
+            a = sf.normalized_axis_scatter(self.shape, axis, index.shape, src.shape)
+            rc = lib().kjo_scatter(1 if add else 0, _p(self.storeReference), _sh(self.shape), _p(index.storeReference),
+                                   _sh(index.shape), _p(src.storeReference), _sh(src.shape), self.dimensions, a)
+        if rc != 0:
+            raise ValueError("Scatter got invalid index, an index value is out of bounds at the axis")
 
     def copy(self, shallow=False):
         if shallow:

@@ -295,6 +295,97 @@ int kjo_contains_nan(const float* a, int64_t n) {
     return 0;
 }
 
+/* ---------------------------------------------------------------- gather / scatter */
+
+/* Row-major offset of a multi-index inside `shape` (IDX:7-11 calcIndexBase). */
+static int64_t index_base(const int32_t* idx, const int32_t* shape, int dims) {
+    int64_t a = 0;
+    for (int d = 0; d < dims; d++) a = a * shape[d] + idx[d];
+    return a;
+}
+
+/* Walks every position of `walk_shape` with the axis removed, in store order
+ * (IDX:123-146 StoreIndexing.applyAt): `idx` holds the full multi-index with idx[axis]
+ * left for the caller to set. Returns 0 when the walk is finished. */
+static int next_position(int32_t* idx, const int32_t* walk_shape, int dims, int axis, int64_t it) {
+    int64_t elements = 1;
+    for (int d = 0; d < dims; d++) if (d != axis) elements *= walk_shape[d];
+    if (it >= elements) return 0;
+    int64_t i = it;
+    for (int d = dims - 1; d >= 0; d--) {
+        if (d == axis) continue;
+        idx[d] = (int32_t)(i % walk_shape[d]);
+        i /= walk_shape[d];
+    }
+    return 1;
+}
+
+/* Kotlin Float.toInt(): truncation toward zero, NaN -> 0, saturating. (JVM:236) */
+static inline int32_t f2i(float f) {
+    if (f != f) return 0;
+    if (f >= 2147483648.0f) return INT32_MAX;
+    if (f <= -2147483648.0f) return INT32_MIN;
+    return (int32_t)f;
+}
+
+/* JVM:334-353 gather: res has index's shape; res[p, i] = this[p, index[p, i]] where p runs
+ * over res's positions without the axis and is applied to each tensor's own shape.
+ * Returns 0, or -1 at the first index outside [0, this.shape[axis]) (the reference throws
+ * IllegalArgumentException there). */
+int kjo_gather(const float* in, const int32_t* in_shape, const float* index, const int32_t* index_shape,
+               int dims, int axis, float* out) {
+    int32_t idx[KJO_MAX_DIMS];
+    for (int64_t it = 0; next_position(idx, index_shape, dims, axis, it); it++) {
+        for (int32_t i = 0; i < index_shape[axis]; i++) {
+            idx[axis] = i;
+            int64_t at = index_base(idx, index_shape, dims);
+            int32_t sel = f2i(index[at]);
+            if (sel < 0 || sel >= in_shape[axis]) return -1;
+            idx[axis] = sel;
+            out[at] = in[index_base(idx, in_shape, dims)];
+        }
+    }
+    return 0;
+}
+
+/* JVM:227-255 internalInplaceScatter: positions run over index's shape without the axis;
+ * target[p, index[p, i]] (= | +=) src[p, i], i ascending, positions in store order, so
+ * duplicates resolve as "last write wins" / "added in i order". add != 0 is
+ * inplaceScatterAdd. Returns -1 at the first bad index (earlier writes stay, as on the JVM). */
+int kjo_scatter(int add, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
+                const float* src, const int32_t* src_shape, int dims, int axis) {
+    int32_t idx[KJO_MAX_DIMS];
+    for (int64_t it = 0; next_position(idx, index_shape, dims, axis, it); it++) {
+        for (int32_t i = 0; i < index_shape[axis]; i++) {
+            idx[axis] = i;
+            int32_t sel = f2i(index[index_base(idx, index_shape, dims)]);
+            if (sel < 0 || sel >= target_shape[axis]) return -1;
+            float v = src[index_base(idx, src_shape, dims)];
+            idx[axis] = sel;
+            int64_t to = index_base(idx, target_shape, dims);
+            if (add) target[to] = target[to] + v;
+            else target[to] = v;
+        }
+    }
+    return 0;
+}
+
+/* JVM:317-332 inplaceScatter(axis, index, Float). */
+int kjo_scatter_fill(float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
+                     int dims, int axis, float value) {
+    int32_t idx[KJO_MAX_DIMS];
+    for (int64_t it = 0; next_position(idx, index_shape, dims, axis, it); it++) {
+        for (int32_t i = 0; i < index_shape[axis]; i++) {
+            idx[axis] = i;
+            int32_t sel = f2i(index[index_base(idx, index_shape, dims)]);
+            if (sel < 0 || sel >= target_shape[axis]) return -1;
+            idx[axis] = sel;
+            target[index_base(idx, target_shape, dims)] = value;
+        }
+    }
+    return 0;
+}
+
 /* ---------------------------------------------------------------- reductions */
 
 /* JVM:146-148 sum() = kotlin FloatArray.sum(): float accumulator from 0f, index order. */

@@ -55,7 +55,11 @@ def case_mse_and_grads(ops):
 
 def case_max_last_axis_4d(ops):
     c = K["max_last_axis_4d"]
-    assertTensorEquals(c["expected"], T(ops, c["t1"]).max(axis=-1), c["tol"])
+    t1 = T(ops, c["t1"], True)
+    res = t1.max(axis=-1)
+    assertTensorEquals(c["expected"], res, c["tol"])
+    res.sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"])
 
 
 def case_broadcasting_addition_with_grads(ops):
@@ -188,21 +192,77 @@ def case_mean_over_axis_keep_dims(ops): _axis_case(ops, "mean_over_axis_keep_dim
 
 
 def case_max_min_over_axis(ops):
-    # Forward values only: the gradients of Max/Min go through inplaceScatter, which is
-    # outside this backend's accelerated path.
     c = K["max_min_over_axis"]
+    for name, method, axis, keep in (("max_last", "max", -1, False), ("max_0_keep", "max", 0, True),
+                                     ("min_last", "min", -1, False), ("min_0_keep", "min", 0, True)):
+        t1 = T(ops, c["t1"], True)
+        res = getattr(t1, method)(axis=axis, keepDimensions=keep)
+        assertTensorEquals(c[name], res, c["tol"])
+        res.sum().backward()                       # Max/Min.doBackward: zerosLike + inplaceScatter at the arg indices
+        assertTensorEquals(c[name + "_grad"], t1.grad(), c["tol"], [3, 3])
+
+
+def case_gather_with_grads(ops):
+    c = K["gather_with_grads"]
+    t1 = T(ops, c["t1"], True)
+    res = t1.gather(c["axis"], T(ops, c["index"]))
+    assertTensorEquals(c["expected"], res, c["tol"])
+    res.sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"])
+
+
+def case_scatter(ops):
+    from kten_amd.autograd import zeros
+    c = K["scatter"]
     t1 = T(ops, c["t1"])
-    assertTensorEquals(c["max_last"], t1.max(axis=-1), c["tol"])
-    assertTensorEquals(c["max_0_keep"], t1.max(axis=0, keepDimensions=True), c["tol"])
-    assertTensorEquals(c["min_last"], t1.min(axis=-1), c["tol"])
-    assertTensorEquals(c["min_0_keep"], t1.min(axis=0, keepDimensions=True), c["tol"])
-    # What the scatter of Max.doBackward would produce follows from argMax alone: a one
-    # at the arg index of every lane. This pins ties -> lowest index.
-    for key, idx, axis in (("max_0_keep_grad", t1.argMax(0, True), 0), ("max_last_grad", t1.argMax(-1, True), 1),
-                           ("min_0_keep_grad", t1.argMin(0, True), 0), ("min_last_grad", t1.argMin(-1, True), 1)):
-        grad = np.zeros((3, 3), dtype=np.float32)
-        np.put_along_axis(grad, idx.toArray().astype(np.int64), 1.0, axis=axis)
-        assertTensorEquals(c[key], grad, c["tol"], [3, 3])
+    res1 = zeros(ops, *c["target_shape"]).scatter(c["axis1"], T(ops, c["index1"]), t1)
+    res2 = zeros(ops, *c["target_shape"]).scatter(c["axis2"], T(ops, c["index2"]), t1)
+    assertTensorEquals(c["expected1"], res1, c["tol"])
+    assertTensorEquals(c["expected2"], res2, c["tol"])
+
+
+def case_scatter_with_grads(ops):
+    from kten_amd.autograd import zeros
+    c = K["scatter_with_grads"]
+    t1 = T(ops, c["t1"], True)
+    target = zeros(ops, *c["target_shape"]).asVariable(requiresGrad=True)
+    res = (target + 1.0).scatter(c["axis"], T(ops, c["index"]), t1) ** 2
+    assertTensorEquals(c["expected"], res, c["res_tol"])
+    res.sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"])
+    assertTensorEquals(c["target_grad"], target.grad(), c["tol"])
+
+
+def case_softmax_cross_entropy_two_formulations(ops):
+    """TensorTestsBase.kt:2205-2225: the fused function against the same loss composed from
+    tensor ops (exp, max with its scatter backward, sum, div, clamp, log, mean), values and
+    gradients, at the reference's 1e-6 tolerance. Inputs are seeded here (the reference
+    draws them unseeded); the one-hot targets are built on the host."""
+    import numpy as np
+    from kten_amd.inputs import SplitMix64
+    g = SplitMix64(11)
+    n, classes = 64, 200
+    logits = g.normal([n, classes])
+    labels = (g.uniform([n], 0.0, 1.0) * classes).astype(np.int64).clip(0, classes - 1)
+    onehot = np.zeros((n, classes), np.float32); onehot[np.arange(n), labels] = 1.0
+    tensor = ops.create([n, classes], True, logits)
+    tensor2 = ops.create([n, classes], True, logits)
+    targets = ops.create([n], False, labels.astype(np.float32))
+    targetsOneHot = ops.create([n, classes], False, onehot)
+    res = tensor.softmaxCrossEntropy(targets)
+    res.backward()
+    expVal = (tensor2 - tensor2.max(-1, keepDimensions=True)).exp()
+    softmax = expVal / expVal.sum(-1, keepDimensions=True)
+    eps = float(np.float32(1e-7))
+    softmaxNorm = (softmax / softmax.sum(-1, keepDimensions=True)).clamp(eps, float(np.float32(1.0) - np.float32(eps)))
+    res2 = (-(targetsOneHot * softmaxNorm.log()).sum(-1)).mean()
+    res2.backward()
+    assertTensorEquals(res2.toArray(), res, 1e-6)
+    assertTensorEquals(tensor2.grad().toArray(), tensor.grad(), 1e-6)
+    # and against the closed form: mean of -log softmax at the label
+    z = logits.astype(np.float64); z -= z.max(1, keepdims=True)
+    ref = -(z[np.arange(n), labels] - np.log(np.exp(z).sum(1))).mean()
+    assert abs(float(res.toArray()[0]) - ref) < 1e-5
 
 
 def case_argmax_argmin(ops):

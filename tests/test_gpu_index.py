@@ -1,0 +1,78 @@
+"""gather / inplaceScatter / inplaceScatterAdd / inplaceScatter(Float) on the device against
+the CPU checker: bit-exact, including duplicate indices inside a position (assignment:
+last write wins; add: summed in ascending order) and the error behaviour."""
+import numpy as np
+import pytest
+
+from oracle import jvm_oracle as jo
+from parity import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([3, 4, 5], [2, 4, 2], 2), ([6], [9], 0),
+         ([2, 3, 4, 5], [2, 3, 7, 5], 2), ([1000, 300], [1000, 1], 1), ([1000, 300], [1, 300], 0), ([64, 2048], [64, 1], 1),
+         ([70000, 7], [70000, 3], 1), ([5, 3, 2, 2, 3, 2, 2, 2, 3, 4], [5, 3, 2, 2, 6, 2, 2, 2, 3, 4], 4)]
+
+
+def both(gc, shape, array):
+    cpu = jo.JvmOracleOperations()
+    return gc.createRaw(shape, array), cpu.createRaw(shape, array)
+
+
+@pytest.mark.parametrize("shape,ishape,axis", CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_gather_scatter_parity(shape, ishape, axis, gc):
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = rng.integers(0, shape[axis], size=ishape).astype(np.float32)
+    src = rng.standard_normal(ishape).astype(np.float32)
+    gx, cx = both(gc, shape, x); gi, ci = both(gc, ishape, idx); gs, cs = both(gc, ishape, src)
+    assert_bits_equal(gx.gather(axis, gi).toArray(), cx.gather(axis, ci).toArray(), "gather")
+    for name in ("inplaceScatter", "inplaceScatterAdd"):
+        gt, ct = both(gc, shape, x)
+        getattr(gt, name)(axis, gi, gs); getattr(ct, name)(axis, ci, cs)
+        assert_bits_equal(gt.toArray(), ct.toArray(), name)
+    gt, ct = both(gc, shape, x)
+    gt.inplaceScatter(axis, gi, -1.0); ct.inplaceScatter(axis, ci, -1.0)
+    assert_bits_equal(gt.toArray(), ct.toArray(), "inplaceScatter(Float)")
+    assert_bits_equal(gx.scatter(axis, gi, gs).toArray(), cx.scatter(axis, ci, cs).toArray(), "scatter (copy)")
+    assert_bits_equal(gx.toArray(), x, "scatter must not touch its receiver")
+
+
+def test_bad_indices_raise_like_the_reference(gc):
+    x = gc.createRaw([2, 3], np.arange(6, dtype=np.float32))
+    for bad in (3.0, -1.0, 1e10):
+        with pytest.raises(ValueError):
+            x.gather(1, gc.createRaw([2, 1], [0.0, bad]))
+        with pytest.raises(ValueError):
+            x.inplaceScatter(1, gc.createRaw([2, 1], [0.0, bad]), gc.createRaw([2, 1], [1.0, 1.0]))
+        with pytest.raises(ValueError):
+            x.inplaceScatter(1, gc.createRaw([2, 1], [0.0, bad]), 5.0)
+    got = x.gather(1, gc.createRaw([2, 1], [2.9, float("nan")])).toArray()         # Float.toInt(): 2 and 0
+    assert got.tolist() == [[2.0], [3.0]]
+    with pytest.raises(ValueError):
+        x.inplaceScatter(1, gc.createRaw([2, 2], [0, 1, 0, 1]), gc.createRaw([2, 1], [1.0, 1.0]))
+    with pytest.raises(ValueError):
+        x.inplaceScatter(1, gc.createRaw([2], [0, 1]), gc.createRaw([2], [1.0, 1.0]))
+    with pytest.raises(ValueError):
+        x.gather(2, gc.createRaw([2, 1], [0.0, 0.0]))
+
+
+def test_max_backward_at_scale_matches_checker(gc):
+    """Max over the last axis with its scatter backward, and a softmax-cross-entropy step,
+    on [512, 1000]: device against the checker running the same graph."""
+    from kten_amd.inputs import SplitMix64
+    g = SplitMix64(5)
+    x = g.normal([512, 1000])
+    labels = (g.uniform([512], 0.0, 1.0) * 1000).astype(np.int64).clip(0, 999).astype(np.float32)
+    out = []
+    for ops in (gc, jo.JvmOracleOperations()):
+        t = ops.create([512, 1000], True, x)
+        t.max(-1).sum().backward()
+        g_max = t.grad().toArray().copy()
+        t2 = ops.create([512, 1000], True, x)
+        loss = t2.softmaxCrossEntropy(ops.create([512], False, labels))
+        loss.backward()
+        out.append((g_max, loss.toArray(), t2.grad().toArray()))
+    assert_bits_equal(out[0][0], out[1][0], "grad of max")
+    assert abs(float(out[0][1][0]) - float(out[1][1][0])) <= 1e-6 * abs(float(out[1][1][0]))
+    np.testing.assert_allclose(out[0][2], out[1][2], rtol=0, atol=1e-9)

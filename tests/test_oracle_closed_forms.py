@@ -348,3 +348,55 @@ def test_contains_nan_and_fill(oracle_ops):
     assert not t.containsNan()
     t.inplaceFill(float("nan"))
     assert t.containsNan()
+
+
+# ------------------------------------------------------------------ gather / scatter
+
+INDEX_CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([3, 4, 5], [2, 4, 2], 2),
+               ([6], [9], 0), ([2, 3, 4, 5], [2, 3, 7, 5], 2)]
+
+
+@pytest.mark.parametrize("shape,ishape,axis", INDEX_CASES)
+def test_gather_matches_numpy_take_along_axis(shape, ishape, axis, oracle_ops):
+    x = RNG.standard_normal(shape).astype(np.float32)
+    idx = RNG.integers(0, shape[axis], size=ishape)
+    got = oracle_ops.createRaw(shape, x).gather(axis, oracle_ops.createRaw(ishape, idx.astype(np.float32))).toArray()
+    # numpy needs equal non-axis dims: compare on the corner of x that index addresses
+    corner = x[tuple(slice(0, ishape[d]) if d != axis else slice(None) for d in range(len(shape)))]
+    assert_bits_equal(got, np.take_along_axis(corner, idx, axis))
+
+
+@pytest.mark.parametrize("shape,ishape,axis", INDEX_CASES)
+def test_scatter_and_scatter_add_brute_force(shape, ishape, axis, oracle_ops):
+    idx = RNG.integers(0, shape[axis], size=ishape)                      # duplicates along the axis are likely
+    src = RNG.standard_normal(ishape).astype(np.float32)
+    base = RNG.standard_normal(shape).astype(np.float32)
+    want_set, want_add, want_fill = base.copy(), base.copy(), base.copy()
+    for pos in np.ndindex(*ishape):                                      # store order: last write wins, adds in order
+        to = list(pos); to[axis] = idx[pos]
+        want_set[tuple(to)] = src[pos]
+        want_add[tuple(to)] = np.float32(want_add[tuple(to)] + src[pos])
+        want_fill[tuple(to)] = 7.5
+    ri = oracle_ops.createRaw(ishape, idx.astype(np.float32))
+    t = oracle_ops.createRaw(shape, base); t.inplaceScatter(axis, ri, oracle_ops.createRaw(ishape, src))
+    assert_bits_equal(t.toArray(), want_set)
+    t = oracle_ops.createRaw(shape, base); t.inplaceScatterAdd(axis, ri, oracle_ops.createRaw(ishape, src))
+    assert_bits_equal(t.toArray(), want_add)
+    t = oracle_ops.createRaw(shape, base); t.inplaceScatter(axis, ri, 7.5)
+    assert_bits_equal(t.toArray(), want_fill)
+    copy = oracle_ops.createRaw(shape, base).scatter(axis, ri, oracle_ops.createRaw(ishape, src))
+    assert_bits_equal(copy.toArray(), want_set)
+
+
+def test_gather_scatter_reject_bad_indices_and_shapes(oracle_ops):
+    x = oracle_ops.createRaw([2, 3], np.arange(6, dtype=np.float32))
+    for bad in (3.0, -1.0):
+        with pytest.raises(ValueError):
+            x.gather(1, oracle_ops.createRaw([2, 1], [0.0, bad]))
+        with pytest.raises(ValueError):
+            x.inplaceScatter(1, oracle_ops.createRaw([2, 1], [0.0, bad]), oracle_ops.createRaw([2, 1], [1.0, 1.0]))
+    assert x.gather(1, oracle_ops.createRaw([2, 1], [2.9, float("nan")])).toArray().tolist() == [[2.0], [3.0]]   # toInt(): 2, 0
+    with pytest.raises(ValueError):      # index wider than the source
+        x.inplaceScatter(1, oracle_ops.createRaw([2, 2], [0, 1, 0, 1]), oracle_ops.createRaw([2, 1], [1.0, 1.0]))
+    with pytest.raises(ValueError):      # dim count mismatch
+        x.inplaceScatter(1, oracle_ops.createRaw([2], [0, 1]), oracle_ops.createRaw([2], [1.0, 1.0]))
