@@ -51,6 +51,17 @@ def make_step(name, ops, inputs):
         def step():
             return cfg5_step(x, w, b)          # backward() opens its own garbage-collector scope
         return step
+    if name in ("max_backward", "softmax_ce"):
+        # Leaves are created once; the step is graph + backward, gradients zeroed in between.
+        first = "x" if name == "max_backward" else "logits"
+        leaf = ops.create(list(inputs[first].shape), True, inputs[first])
+        other = None if name == "max_backward" else ops.create(list(inputs["targets"].shape), False, inputs["targets"])
+
+        def step():
+            out = leaf.max(-1).sum() if other is None else leaf.softmaxCrossEntropy(other)
+            out.backward()
+            return out
+        return step
     resident = {k: ops.createRaw(list(v.shape), v) for k, v in inputs.items()}
     for r in resident.values():
         r.incrementRef()
@@ -82,7 +93,8 @@ def cpu_baseline(name, threads):
     from oracle import jvm_oracle as jo
     wl = WORKLOADS[name]
     sample = {"cfg1": dict(wl.full_dims), "cfg2": dict(wl.full_dims), "cfg3": dict(wl.full_dims),
-              "cfg4": dict(wl.full_dims), "cfg5": {"rows": 8192, "cols": 4096}}[name]
+              "cfg4": dict(wl.full_dims), "cfg5": {"rows": 8192, "cols": 4096},
+              "max_backward": dict(wl.full_dims), "softmax_ce": {"batch": 8192, "classes": 2048}}[name]
     inputs = wl.make_inputs(sample)
     jo.set_threads(threads)
     try:
@@ -104,7 +116,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="cfg5", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--config", default="cfg5",
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce"])
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,

@@ -39,18 +39,19 @@ __device__ __forceinline__ void locate(const IndexPlan& pl, uint32_t pos, uint32
     }
 }
 
+// One thread per element of the index tensor (= per element of the result, which has
+// the same contiguous layout): gather has no ordering constraint. The plan's dims are all
+// dims of the index shape, the input stride of the axis dim is 0 and the selected
+// position along the axis is added separately.
 __global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict__ in, const float* __restrict__ index,
-                                                       float* __restrict__ out, uint32_t positions, IndexPlan pl, int* bad) {
-    const uint32_t pos = blockIdx.x * kBlock + threadIdx.x;
-    if (pos >= positions) return;
+                                                       float* __restrict__ out, uint32_t elements, IndexPlan pl, int* bad) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= elements) return;
     uint32_t io, ao, bo;
-    locate(pl, pos, io, ao, bo);
-    for (uint32_t i = 0; i < pl.i_axis_len; i++) {
-        const uint32_t at = io + i * pl.i_axis_stride;
-        const int sel = static_cast<int>(index[at]);
-        if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
-        out[at] = in[ao + static_cast<uint32_t>(sel) * pl.a_axis_stride];
-    }
+    locate(pl, e, io, ao, bo);
+    const int sel = static_cast<int>(index[e]);
+    if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; return; }
+    out[e] = in[ao + static_cast<uint32_t>(sel) * pl.a_axis_stride];
 }
 
 // MODE 0: assign from src, 1: add from src, 2: assign the constant.
@@ -154,25 +155,21 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_gather: output aliases an input");
     if (idx_n == 0) return KTH_OK;
     IndexPlan pl{};
-    pl.ndim = dims - 1;
-    uint64_t positions = 1;
-    int n = 0;
-    for (int d = dims - 1; d >= 0; d--) {
-        if (d == axis) continue;
+    pl.ndim = dims;
+    uint64_t in_run = 1;
+    for (int d = dims - 1, n = 0; d >= 0; d--, n++) {
         pl.size[n] = static_cast<uint32_t>(index_shape[d]);
         pl.div[n] = make_div(pl.size[n]);
-        positions *= pl.size[n];
-        n++;
+        pl.a_stride[n] = d == axis ? 0u : static_cast<uint32_t>(in_run);
+        if (d == axis) pl.a_axis_stride = static_cast<uint32_t>(in_run);
+        in_run *= static_cast<uint64_t>(in_shape[d]);
     }
-    strides_without_axis(index_shape, dims, axis, pl.i_stride, &pl.i_axis_stride);
-    strides_without_axis(in_shape, dims, axis, pl.a_stride, &pl.a_axis_stride);
-    pl.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
     pl.a_axis_len = static_cast<uint32_t>(in_shape[axis]);
-    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+    const uint32_t blocks = static_cast<uint32_t>((idx_n + kBlock - 1) / kBlock);
     return with_index_check("Gather", [&](int* flag) {
-        LaunchScope scope("gather_kernel", "", (2 * idx_n + idx_n) * 4);
+        LaunchScope scope("gather_kernel", "", 3 * idx_n * 4);
         hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, state().stream, si->ptr, sx->ptr, so->ptr,
-                           static_cast<uint32_t>(positions), pl, flag);
+                           static_cast<uint32_t>(idx_n), pl, flag);
     });
 }
 

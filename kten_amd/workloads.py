@@ -144,7 +144,53 @@ def _bytes5(d):
     return 4 * (big + small)
 
 
+# ---- next rows: Max with its scatter backward, softmax cross entropy --------------------------
+
+def _in_max(d):
+    return {"x": SplitMix64(5).normal([d["rows"], d["cols"]])}
+
+
+def _run_max(ops, inp):
+    x = ops.create(list(inp["x"].shape), True, inp["x"])
+    m = x.max(-1)
+    m.sum().backward()
+    return {"max": m, "grad_x": x.grad()}
+
+
+def _bytes_max(d):
+    n, r = d["rows"] * d["cols"], d["rows"]
+    # max + argMax (2(N+R)), sum() (R+1), seed (1), broadcastTo (1+R), zerosLike (N), scatter (3R), gradient += (3N)
+    return 4 * (6 * n + 7 * r + 3)
+
+
+def _in_sce(d):
+    g = SplitMix64(6)
+    logits = g.normal([d["batch"], d["classes"]])
+    labels = np.floor(g.uniform([d["batch"]], 0.0, 1.0) * np.float32(d["classes"])).clip(0, d["classes"] - 1)
+    return {"logits": logits, "targets": labels.astype(np.float32)}
+
+
+def _run_sce(ops, inp):
+    logits = ops.create(list(inp["logits"].shape), True, inp["logits"])
+    targets = ops.create(list(inp["targets"].shape), False, inp["targets"])
+    loss = logits.softmaxCrossEntropy(targets)
+    loss.backward()
+    return {"loss": loss, "grad_logits": logits.grad()}
+
+
+def _bytes_sce(d):
+    n, b = d["batch"] * d["classes"], d["batch"]
+    # 15N + 12B + 1 forward, 9N + 2B + 1 backward, 2B for the copy made by targets.unsqueeze(-1)
+    return 4 * (24 * n + 16 * b + 2)
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "max_backward": Workload("max_backward", "x.max(-1).sum().backward(): x[8192,8192], N(0,1), seed 5 "
+                                             "(max, argMax, zerosLike, inplaceScatter, gradient +=)",
+                             {"rows": 8192, "cols": 8192}, _in_max, _run_max, _bytes_max),
+    "softmax_ce": Workload("softmax_ce", "logits.softmaxCrossEntropy(targets).backward(): logits[32768,2048], seed 6 "
+                                         "(max, minus, exp, sum, div, clamp, log, gather, mean; scatter, +=, /=)",
+                           {"batch": 32768, "classes": 2048}, _in_sce, _run_sce, _bytes_sce),
     "cfg1": Workload("cfg1", "y=(x+b)*x; sum(y): x[2048,1024], b[1024], U(-1,1), seed 0",
                      {"rows": 2048, "cols": 1024}, _in1, _run1, _bytes1),
     "cfg2": Workload("cfg2", "z=exp(-(x pow 2))+log(abs(x)+1e-3): x[2^26], N(0,1), seed 1",

@@ -187,7 +187,7 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
         saved[name] = orig
         def f(self, *a, **k):
             res = orig(self, *a, **k)
-            counted[0] += cost(self, a, res)
+            counted[0] += cost(self, a + tuple(k.values()), res)
             return res
         setattr(R, name, f)
 
@@ -200,15 +200,37 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
     wrap("aggregateOverAxis", lambda s, a, r: size(s) + size(r))
     wrap("_sum_all", lambda s, a, r: size(s) + 1)
     wrap("broadcastTo", lambda s, a, r: 0 if r is s else size(s) + size(r))
+    wrap("_mean_all", lambda s, a, r: size(s) + 1)
+    wrap("clamp", lambda s, a, r: size(s) + size(r))
+    wrap("gather", lambda s, a, r: 3 * size(r))
+    wrap("_scatter", lambda s, a, r: size(a[1]) * (2 if isinstance(a[2], float) else 4 if a[3] else 3))
+    wrap("inplaceFill", lambda s, a, r: size(s))
+    wrap("copy", lambda s, a, r: 0 if (a and a[0]) else 2 * size(s))        # deep copies only
     orig_create = type(oracle_ops).createRaw
     def counting_create(self, shape, init=None):
         if callable(init):                      # the [1] seed gradient of backward(): one store
             counted[0] += int(np.prod(shape))
         return orig_create(self, shape, init)
     type(oracle_ops).createRaw = counting_create
+    orig_fill = type(oracle_ops).createRawFill
+    setting_up = [False]
+    def counting_fill(self, shape, constant):     # zerosLike / createRawFill: one store per element
+        if not setting_up[0]:
+            counted[0] += int(np.prod(shape))
+        return orig_fill(self, shape, constant)
+    type(oracle_ops).createRawFill = counting_fill
+    orig_tensor_create = type(oracle_ops).create
+    def quiet_create(self, shape, requiresGrad=False, init=None):   # creating the leaves is set-up, not part of a step
+        setting_up[0] = True
+        try:
+            return orig_tensor_create(self, shape, requiresGrad, init)
+        finally:
+            setting_up[0] = False
+    type(oracle_ops).create = quiet_create
     try:
         small = {"cfg1": {"rows": 8, "cols": 12}, "cfg2": {"n": 100}, "cfg3": {"rows": 6, "cols": 10},
-                 "cfg4": {"n": 2, "c": 3, "h": 4, "w": 5}, "cfg5": {"rows": 8, "cols": 12}}
+                 "cfg4": {"n": 2, "c": 3, "h": 4, "w": 5}, "cfg5": {"rows": 8, "cols": 12},
+                 "max_backward": {"rows": 6, "cols": 10}, "softmax_ce": {"batch": 6, "classes": 10}}
         for name, dims in small.items():
             wl = WORKLOADS[name]
             counted[0] = 0
@@ -216,5 +238,7 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
             assert counted[0] * 4 == wl.algorithmic_bytes(dims), name
     finally:
         type(oracle_ops).createRaw = orig_create
+        type(oracle_ops).createRawFill = orig_fill
+        type(oracle_ops).create = orig_tensor_create
         for name, orig in saved.items():
             setattr(R, name, orig)
