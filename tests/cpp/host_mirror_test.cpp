@@ -1,0 +1,130 @@
+// Drives libkten_hip.so through the C++ host mirror (include/kten_hip.hpp) on the known
+// answers the reference asserts in its own suite (file:line beside each case) and on the
+// error behaviour of the raw-tensor contract. Exit status 0 means every check held.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <initializer_list>
+
+#include "kten_hip.hpp"
+
+using namespace kten::hip;
+
+static int g_checks = 0, g_failed = 0;
+
+static void expect(bool ok, const char* what) {
+    g_checks++;
+    if (!ok) { g_failed++; std::printf("FAILED: %s\n", what); std::fflush(stdout); }
+}
+
+static void expect_values(const Raw& t, const Shape& shape, std::initializer_list<float> values, float tol, const char* what) {
+    bool ok = t->shape == shape;
+    const std::vector<float> got = t->toVector();
+    ok = ok && got.size() == values.size();
+    size_t i = 0;
+    for (float v : values) { if (ok && !(std::fabs(got[i] - v) <= tol)) ok = false; i++; }
+    expect(ok, what);
+}
+
+template <class F>
+static void expect_illegal_argument(F&& f, const char* what) {
+    bool thrown = false;
+    try { f(); } catch (const std::invalid_argument&) { thrown = true; }
+    expect(thrown, what);
+}
+
+static Raw tensor(HipTensorOperations& ops, const Shape& shape, std::initializer_list<float> values) {
+    std::vector<float> v(values);
+    return ops.createRaw(shape, [&](int i) { return v[static_cast<size_t>(i)]; });
+}
+
+int main() {
+    HipTensorOperations ops(0);
+    std::printf("platform: %s, %d compute units\n", ops.platformKey.c_str(), ops.computeUnits);
+    std::fflush(stdout);
+    {
+        auto gc = ops.garbageCollector();
+
+        // kten-testing/.../tests/TensorTestsBase.kt:33-53  [2,4] + [2,1]
+        Raw t1 = tensor(ops, {2, 4}, {1, 2, 3, 4, 5, 6, 7, 8});
+        Raw t2 = tensor(ops, {2, 1}, {1, 2});
+        expect_values(t1->plus(t2), {2, 4}, {2, 3, 4, 5, 7, 8, 9, 10}, 0.0f, "addition with broadcast");
+
+        // TensorTestsBase.kt:319-350  tensor - constant and constant - tensor ((-t) + c)
+        Raw t3 = tensor(ops, {2, 3}, {1, 2, 3, 4, 5, 6});
+        expect_values(t3->minus(2.0f), {2, 3}, {-1, 0, 1, 2, 3, 4}, 0.0f, "tensor minus constant");
+        expect_values(t3->unaryMinus()->plus(2.0f), {2, 3}, {1, 0, -1, -2, -3, -4}, 0.0f, "constant minus tensor");
+
+        // TensorTestsBase.kt:469-497  [3,3] pow [1,3]
+        Raw p1 = tensor(ops, {3, 3}, {2, 3, 2, 3, 3, 3, 2, 3, 2});
+        Raw p2 = tensor(ops, {1, 3}, {2, 3, 2});
+        expect_values(p1->pow(p2), {3, 3}, {4, 27, 4, 9, 27, 9, 4, 27, 4}, 0.0f, "tensor pow tensor");
+        // TensorTestsBase.kt:500-529  constant pow tensor
+        expect_values(ops.pow(2.0f, p1), {3, 3}, {4, 8, 4, 8, 8, 8, 4, 8, 4}, 0.0f, "constant pow tensor");
+
+        // TensorTestsBase.kt:532-609  sum / mean over an axis, with and without keepDimensions
+        Raw s = tensor(ops, {3, 3}, {1, 1, 1, 2, 2, 2, 3, 3, 3});
+        expect_values(s->sum(-1), {3}, {3, 6, 9}, 0.0f, "sum(axis=-1)");
+        expect_values(s->sum(0, true), {1, 3}, {6, 6, 6}, 0.0f, "sum(axis=0, keepDimensions)");
+        expect_values(s->mean(0), {3}, {2, 2, 2}, 0.0f, "mean(axis=0)");
+        expect_values(s->mean(-1, true), {3, 1}, {1, 2, 3}, 0.0f, "mean(axis=-1, keepDimensions)");
+        expect_values(s->sum(), {1}, {18}, 0.0f, "sum()");
+        expect_values(s->mean(), {1}, {2}, 0.0f, "mean()");
+
+        // TensorTestsBase.kt:612-757  max / min / argMax / argMin
+        Raw m = tensor(ops, {3, 3}, {3, 2, 1, 1, 3, 2, 3, 1, 2});
+        expect_values(m->max(-1), {3}, {3, 3, 3}, 0.0f, "max(axis=-1)");
+        expect_values(m->min(0), {3}, {1, 1, 1}, 0.0f, "min(axis=0)");
+        expect_values(m->argMax(-1), {3}, {0, 1, 0}, 0.0f, "argMax(axis=-1): ties resolve to the lowest index");
+        expect_values(m->argMin(0), {3}, {1, 2, 0}, 0.0f, "argMin(axis=0)");
+
+        // TensorTestsBase.kt:760-784  exp
+        Raw e = tensor(ops, {2, 3}, {0.1f, 0.2f, 0.3f, 0.4f, 0.5f, 0.6f});
+        expect_values(e->exp(), {2, 3}, {1.1052f, 1.2214f, 1.3499f, 1.4918f, 1.6487f, 1.8221f}, 1e-4f, "exp");
+
+        // TensorTestsBase.kt:1320-1349  gather along axis 1
+        Raw g = tensor(ops, {2, 2}, {1, 2, 3, 4});
+        Raw gi = tensor(ops, {2, 2}, {0, 0, 1, 0});
+        expect_values(g->gather(1, gi), {2, 2}, {1, 1, 4, 3}, 0.0f, "gather");
+
+        // kten-api/.../autograd/functions/Utils.kt:14-41  reduce-to-shape of an incoming gradient
+        Raw grad = ops.createRawFill({4, 3, 5}, 1.0f);
+        expect_values(mayUnexpand(grad, {3, 1}, ops), {3, 1}, {20, 20, 20}, 0.0f, "mayUnexpand [4,3,5] -> [3,1]");
+        expect_values(mayUnexpand(grad, {5}, ops), {5}, {12, 12, 12, 12, 12}, 0.0f, "mayUnexpand [4,3,5] -> [5]");
+        Raw same = mayUnexpand(grad, {4, 3, 5}, ops);
+        expect(same.get() == grad.get(), "mayUnexpand returns its argument when nothing was expanded");
+
+        // shapes: view shares the store, reshape copies (AbstractRawTensor.kt:77-90)
+        Raw v = t1->view({4, -1});
+        expect(v->shape == Shape({4, 2}) && v->storeReference == t1->storeReference, "view infers -1 and shares the store");
+        Raw r = t1->reshape({8});
+        expect(r->shape == Shape({8}) && r->storeReference != t1->storeReference, "reshape copies");
+        expect(std::fabs(t1->getSingleValue({1, -1}) - 8.0f) == 0.0f, "getSingleValue with a negative index");
+
+        // error behaviour: IllegalArgumentException on the host side of the call
+        expect_illegal_argument([&] { t1->plusAssign(t2); }, "plusAssign refuses unequal shapes (JVMRawTensor.kt:89-93)");
+        expect_illegal_argument([&] { t1->plus(tensor(ops, {3}, {1, 2, 3})); }, "plus refuses shapes that do not broadcast");
+        expect_illegal_argument([&] { t1->sum(2); }, "axis out of range (ShapeFunctions.kt:41-48)");
+        expect_illegal_argument([&] { t1->broadcastTo({4}); }, "broadcastTo a lower rank (ShapeFunctions.kt:187-201)");
+        expect_illegal_argument([&] { t1->view({3, -1, -1}); }, "view with two inferred dimensions");
+        expect_illegal_argument([&] { g->gather(1, tensor(ops, {2, 2}, {0, 2, 0, 0})); }, "gather index out of range (JVMRawTensor.kt:345-346)");
+
+        // in-place arithmetic and NaN detection
+        Raw acc = ops.zerosLike(t1);
+        acc->plusAssign(t1);
+        acc->timesAssign(2.0f);
+        acc->plusAssign(1.0f);
+        expect_values(acc, {2, 4}, {3, 5, 7, 9, 11, 13, 15, 17}, 0.0f, "plusAssign / timesAssign");
+        expect(!acc->containsNan(), "containsNan on finite values");
+        expect(tensor(ops, {2}, {1.0f, NAN})->containsNan(), "containsNan finds a NaN");
+
+        // survive the scope
+        ops.markSurviveGC(t1);
+        gc.close();
+        expect(t1->referenced() && !t2->referenced(), "garbage collector scope releases all but the survivors");
+        ops.markReleasableInGC(t1);
+        t1->release();
+    }
+    std::printf("%d checks, %d failed\n", g_checks, g_failed);
+    return g_failed == 0 ? 0 : 1;
+}

@@ -1,0 +1,41 @@
+"""The C++ host mirror (include/kten_hip.hpp): compiles on its own with a host compiler,
+and its test program, which replays known answers of the reference's suite and the
+contract's error behaviour through the C ABI, passes on the GPU."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BINARY = os.path.join(ROOT, "tests", "cpp", "host_mirror_test")
+
+
+def test_header_is_self_contained(tmp_path):
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no host C++ compiler")
+    src = tmp_path / "tu.cpp"
+    src.write_text('#include "kten_hip.hpp"\nint main() { return 0; }\n')
+    subprocess.run([gxx, "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                    "-I", os.path.join(ROOT, "include"), str(src)], check=True)
+
+
+def test_header_is_plain_c_too(tmp_path):
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no host C compiler")
+    src = tmp_path / "tu.c"
+    src.write_text('#include "kten_hip.h"\nint main(void) { return KTH_OK; }\n')
+    subprocess.run([gcc, "-std=c11", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                    "-I", os.path.join(ROOT, "include"), str(src)], check=True)
+
+
+@pytest.mark.gpu
+def test_cpp_host_mirror_known_answers():
+    assert os.path.exists(BINARY), "tests/cpp/host_mirror_test is not built (python __graft_entry__.py build)"
+    done = subprocess.run([BINARY], capture_output=True, text=True, timeout=120)
+    print(done.stdout)
+    print(done.stderr)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "0 failed" in done.stdout
