@@ -196,6 +196,51 @@ int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t 
 int kth_scatter_fill(uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
                      int dims, int axis, float value);
 
+/* ------------------------------------------------------------------ layout movers */
+
+/* get(Array<IntRange>) (RAW:29; JVM:276-280) and narrow (RAW:232; JVM:468-473): copies the
+ * box first[d]..last[d] (inclusive, already normalised by the host as
+ * kten-api/.../autograd/utils/ShapeFunctions.kt:240-259 does, one range per dim, unindexed
+ * trailing dims given as 0..shape[d]-1) of `in` into `out` in row-major order, which is the
+ * order in which the reference concatenates its sparse store ranges
+ * (kten-api/.../tensor/store/AbstractIndexing.kt:65-88). A range outside its dim returns
+ * KTH_E_ARGUMENT. get(IntArray) (RAW:27; JVM:270-274) selects one contiguous store range:
+ * the host uses kth_copy for it. */
+int kth_get_range(uint64_t in, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, uint64_t out);
+
+/* set(Array<IntRange>, tensor) (RAW:33; JVM:291-304) and, called once per input, concat
+ * (kten-api/.../tensor/operations/TensorOperations.kt:41;
+ * backend/kten-jvm/.../operations/AbstractJVMTensorOperations.kt:106-120): the first value_n
+ * floats of `value` fill the box in row-major order. As in the reference only the element
+ * count is compared (JVM:295-296): a different count returns KTH_E_SHAPE. set(IntArray,
+ * tensor) (RAW:31; JVM:282-289) is one contiguous range: the host uses kth_copy. */
+int kth_set_range(uint64_t target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
+                  uint64_t value, uint64_t value_n);
+
+/* set(Array<IntRange>, Float) (RAW:37; JVM:311-315). set(IntArray, Float) (RAW:35;
+ * JVM:306-309) is one contiguous range: the host uses kth_fill. */
+int kth_fill_range(uint64_t target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, float value);
+
+/* transpose (RAW:228; JVM:437-451): out has `shape` with dims axis1 and axis2 (already
+ * normalised, different) exchanged, out[.., i at axis1, .., j at axis2, ..] =
+ * in[.., j at axis1, .., i at axis2, ..]: the axis swap the contract documents
+ * (kten-api/.../tensor/Tensor.kt:1028-1058) and the reference's OpenCL backend computes
+ * (backend/kten-opencl/src/main/resources/kernels.cl:263-287). kten-jvm's slab copy gives
+ * the same result when the axes are adjacent or every dim between them has size 1, and a
+ * different element order otherwise. */
+int kth_transpose(uint64_t in, const int32_t* shape, int dims, int axis1, int axis2, uint64_t out);
+
+/* permute (RAW:230; JVM:453-466): out.shape[d] = shape[axes[d]] and the element at
+ * multi-index t of `in` lands at (t[axes[0]], t[axes[1]], ..) of out. axes must name every
+ * dim once (ShapeFunctions.kt:106-113), else KTH_E_ARGUMENT. */
+int kth_permute(uint64_t in, const int32_t* shape, int dims, const int32_t* axes, uint64_t out);
+
+/* maskedFill (RAW:246; JVM:537-540): out[i] = mask'[i] == 1f ? value : a[i] where mask' is
+ * the mask broadcast to a's shape inside the kernel (JVM:538 materialises it). A mask that
+ * does not broadcast to a's shape returns KTH_E_SHAPE. out may be a. */
+int kth_masked_fill(uint64_t a, const int32_t* ashape, int adims, uint64_t mask, const int32_t* mshape, int mdims,
+                    float value, uint64_t out);
+
 /* ------------------------------------------------------------------ control and metrics */
 
 /* Wait for everything launched so far. */

@@ -28,6 +28,23 @@ def _is_number(x) -> bool:
     return isinstance(x, (int, float)) and not isinstance(x, bool)
 
 
+def _safe(t):
+    """AGTensor.kt:26-30."""
+    return t.inplaceSafe() if isinstance(t, AGTensor) else t
+
+
+def _as_list(args):
+    return list(args[0]) if len(args) == 1 and isinstance(args[0], (list, tuple)) else list(args)
+
+
+def _as_index(index):
+    """`t[1, 1]` -> [1, 1]; `t[(1, 1), ALL, (1, -1)]` -> three ranges; `t[2]` -> [2];
+    `t[ALL]` -> one range."""
+    if isinstance(index, sf.IntRange) or not isinstance(index, (tuple, list)):
+        return [index]
+    return list(index)
+
+
 def mayUnexpand(rawTensor, oldShape: Sequence[int], ops):
     """Reduce a gradient back to the shape an operand had before broadcasting
     (functions/Utils.kt:14-41): sum(0) without keepDims once per extra leading dim, then
@@ -92,20 +109,49 @@ class Tensor:
 
     def toArray(self):
         """Host copy of the values (forwards a pending graph first)."""
-        if self.requiresGrad:
-            self.forward()
-        return self.getRawValue().toArray()
+        t = self.inplaceSafe() if isinstance(self, AGTensor) else self
+        if t.requiresGrad:
+            t.forward()
+        return t.getRawValue().toArray()
 
 
 class AGTensor(Tensor):
     """autograd/tensor/AGTensor.kt — every method builds a graph node."""
 
     requiresGrad = True
+    inplaceSafeThis = None
+
+    def inplaceSafe(self):
+        """AGTensor.kt:24-34: after an indexed set the tensor stands for the function that
+        performed it, so later uses see the modified value in the graph."""
+        return self.inplaceSafeThis if self.inplaceSafeThis is not None else self
 
     def _forwarded(self):
-        if isinstance(self, Function) and not self.hasValue():
-            self.forward()
-        return self
+        """AGTensor.kt:52-59 inplaceSafeForwarded."""
+        t = self.inplaceSafe()
+        if isinstance(t, Function) and not t.hasValue():
+            t.forward()
+        return t
+
+    # AGTensor.kt:61-83. An index is all ints (Kotlin `t[1, 1]`) or all ranges: IntRange,
+    # (first, last) pairs with both ends inclusive, or ALL (Kotlin `t[1..1, all, 1..-1]`).
+    def __getitem__(self, index):
+        return Index(self.ops)(_safe(self), _as_index(index))
+
+    def __setitem__(self, index, value):
+        index = _as_index(index)
+        if _is_number(value):
+            self.inplaceSafeThis = IndexSetConstant(self.ops)(_safe(self), index, float(value))
+        else:
+            self.inplaceSafeThis = IndexSetTensor(self.ops)(_safe(self), index, _safe(value))
+
+    def transpose(self, axis1, axis2): return Transpose(self.ops)(self, axis1, axis2)          # AGTensor.kt:265-267
+    def permute(self, *axes): return Permute(self.ops)(self, _as_list(axes))                  # AGTensor.kt:277-279
+    def concat(self, axis, tensors): return Concat(self.ops)(axis, [_safe(t) for t in tensors])   # AGTensor.kt:281-283
+    def maskedFill(self, mask, value): return MaskedFill(self.ops)(self, mask, float(value))  # AGTensor.kt:525-527
+    def copy(self): return Copy(self.ops)(self)
+    def squeeze(self, axis): return Squeeze(self.ops)(self, axis)
+    def unsqueeze(self, axis): return Unsqueeze(self.ops)(self, axis)
 
     def item(self) -> float:
         """AGTensor.kt:36-46."""
@@ -247,8 +293,29 @@ class NoGradVariable(AGTensor):
     def clamp(self, min, max): return self._new(self.rawValue.clamp(float(min), float(max)))
     def _reshape(self, newShape): return self._new(self.rawValue.reshape(newShape))
     def _expand(self, newShape): return self._new(self.rawValue.broadcastTo(newShape))
-    def view(self, *newShape): return self._new(self.rawValue.view(list(newShape)))
+    def view(self, *newShape): return self._new(self.rawValue.view(_as_list(newShape)))
     def copy(self): return self._new(self.rawValue.copy())
+
+    def __getitem__(self, index): return self._new(self.rawValue.get(_as_index(index)))       # :42-44
+
+    def __setitem__(self, index, value):                                                      # :46-64
+        if _is_number(value):
+            self.rawValue.set(_as_index(index), float(value))
+            return
+        if value.requiresGrad:
+            value.forward()
+        self.rawValue.set(_as_index(index), _safe(value).getRawValue())
+
+    def transpose(self, axis1, axis2): return self._new(self.rawValue.transpose(axis1, axis2))    # :172
+    def permute(self, *axes): return self._new(self.rawValue.permute(_as_list(axes)))         # :180
+
+    def concat(self, axis, tensors):                                                          # :182-186
+        if any(t.requiresGrad for t in tensors):
+            return super().concat(axis, tensors)
+        return self._new(self.ops.concat(axis, [t.getRawValue() for t in tensors]))
+
+    def maskedFill(self, mask, value):                                                        # :282
+        return self._new(self.rawValue.maskedFill(mask.getRawValue(), float(value)))
     def squeeze(self, axis): return self._new(self.rawValue.squeeze(axis))
     def unsqueeze(self, axis): return self._new(self.rawValue.unsqueeze(axis))
     def lt(self, o): return self._new(self.rawValue.lt(o if _is_number(o) else o.getRawValue()))
@@ -442,6 +509,7 @@ class BiTensorFunction(Function):
     broadcastingOperation = True
 
     def __call__(self, a, b):
+        a, b = _safe(a), _safe(b)
         if self.broadcastingOperation:
             self.cachedShape = sf.infer_implicit_broadcast_shape(a.shape, b.shape)
         self.inputs = (a, b)
@@ -469,6 +537,7 @@ class UnaryTensorFunction(Function):
     modifiesShape = False
 
     def __call__(self, tensor):
+        tensor = _safe(tensor)
         if not self.modifiesShape:
             self.cachedShape = list(tensor.shape)
         self.tensor = tensor
@@ -975,6 +1044,207 @@ class Scatter(BiTensorFunction):                                                
         return [gradInput, gradSource]
 
 
+class AnyTensorFunction(Function):
+    """functions/AnyTensorFunction.kt — a node over a list of inputs."""
+
+    def getInputsAsList(self): return list(self.inputTensors)
+
+    def internalForward(self):
+        super().internalForward()
+        if self.hasValue():
+            return
+        fns = [t for t in self.inputTensors if isinstance(t, Function)]
+        for f in fns:
+            f.internalForward()
+        if not self.hasValue():
+            self.doForward([t.getRawValue() for t in self.inputTensors])
+        for f in fns:
+            f.mayFreeOutput()
+
+
+class AbstractIndexingFunction(UnaryTensorFunction):                                  # TensorFunctions.kt:33-61
+    def __call__(self, tensor, index):
+        ranged = sf.is_range_index(index)
+        if ranged:
+            self.index, indexedShape = sf.normalized_range_indexed_shape(tensor.shape, index)
+        else:
+            self.index, indexedShape = sf.normalized_indexed_shape(tensor.shape, index)
+        super().__call__(tensor)
+        if ranged or self.modifiesShape:
+            self.cachedShape = indexedShape
+        return self
+
+    def doForward(self, input):
+        self.inputShape = list(input.shape)
+
+
+class Index(AbstractIndexingFunction):                                                # :63-82
+    modifiesShape = True
+
+    def doForward(self, input):
+        super().doForward(input)
+        self.output = input.get(self.index)
+
+    def doBackward(self, gradient):
+        gradInput = self.ops.createRawFill(self.inputShape, 0.0)
+        gradInput.set(self.index, gradient)
+        return [gradInput]
+
+
+class IndexSetTensor(BiTensorFunction):                                               # :84-131
+    broadcastingOperation = False
+
+    def __call__(self, tensor, index, value):
+        if sf.is_range_index(index):
+            normalized, indexedShape = sf.normalized_range_indexed_shape(tensor.shape, index)
+        else:
+            normalized, indexedShape = sf.normalized_indexed_shape(tensor.shape, index)
+        self.valueShape = list(value.shape)
+        if self.valueShape != indexedShape:
+            raise ValueError(f"Cannot set value with shape: {self.valueShape} at index: {list(index)} on tensor with "
+                             f"shape: {tensor.shape}")
+        super().__call__(tensor, value)
+        self.cachedShape = list(tensor.shape)
+        self.index = normalized
+        return self
+
+    def doForward(self, a, b):
+        self.ops.incrementRef(a)        # not to be freed after forward
+        a.set(self.index, b)
+        self.output = a
+
+    def doBackward(self, gradient):
+        gradInput = gradient.copy()
+        gradInput.set(self.index, 0.0)
+        gradValue = gradient.get(self.index).view(self.valueShape)
+        return [gradInput, gradValue]
+
+
+class IndexSetConstant(AbstractIndexingFunction):                                     # :133-177
+    def __call__(self, tensor, index, value):
+        super().__call__(tensor, index)
+        self.cachedShape = list(tensor.shape)
+        if len(index) != len(tensor.shape):
+            raise ValueError(f"Cannot set value at index: {list(index)} on tensor with shape: {tensor.shape} "
+                             "(All tensor dimensions must be indexed to set a constant value)")
+        self.value = float(value)
+        return self
+
+    def doForward(self, input):
+        super().doForward(input)
+        self.ops.incrementRef(input)
+        input.set(self.index, self.value)
+        self.output = input
+
+    def doBackward(self, gradient):
+        gradInput = gradient.copy()
+        gradInput.set(self.index, 0.0)
+        return [gradInput]
+
+
+class Transpose(UnaryTensorFunction):                                                 # :179-198
+    modifiesShape = True
+
+    def __call__(self, tensor, axis1, axis2):
+        super().__call__(tensor)
+        self.cachedShape = sf.transpose_normalize_axes(tensor.shape, axis1, axis2)[0]
+        self.axis1, self.axis2 = axis1, axis2
+        return self
+
+    def doForward(self, input):
+        self.output = input.transpose(self.axis1, self.axis2)
+
+    def doBackward(self, gradient):
+        return [gradient.transpose(self.axis1, self.axis2)]
+
+
+class Permute(UnaryTensorFunction):                                                   # :286-312
+    modifiesShape = True
+
+    def __call__(self, tensor, axes):
+        super().__call__(tensor)
+        self.cachedShape = sf.permute(tensor.shape, axes)
+        self.axes = list(axes)
+        return self
+
+    def doForward(self, input):
+        self.reverseShapeIndices = [self.axes.index(d) for d in range(len(self.axes))]
+        self.output = input.permute(self.axes)
+
+    def doBackward(self, gradient):
+        return [gradient.permute(self.reverseShapeIndices)]
+
+
+class Concat(AnyTensorFunction):                                                      # :349-378
+    def __call__(self, axis, inputTensors):
+        self.cachedShape = sf.concat_shapes([t.shape for t in inputTensors], axis)
+        self.inputTensors = list(inputTensors)
+        self.axis = sf.normalize_axis(self.cachedShape, axis)
+        return self
+
+    def doForward(self, inputs):
+        self.inputSizes = [t.shape[self.axis] for t in inputs]
+        self.output = self.ops.concat(self.axis, inputs)
+
+    def doBackward(self, gradient):
+        grads, end = [], 0
+        for size in self.inputSizes:
+            end += size
+            grads.append(gradient.narrow(self.axis, end - size, size))
+        return grads
+
+
+class Copy(UnaryTensorFunction):                                                      # :380-392
+    def doForward(self, input): self.output = input.copy()
+    def doBackward(self, gradient): return [gradient.copy(shallow=True)]
+
+
+class Squeeze(UnaryTensorFunction):                                                   # :394-420
+    modifiesShape = True
+
+    def __call__(self, tensor, axis):
+        super().__call__(tensor)
+        self.cachedShape = sf.squeeze(tensor.shape, axis)
+        self.axis = axis
+        return self
+
+    def doForward(self, input):
+        self.inputShape = list(input.shape)
+        self.output = input.squeeze(self.axis)
+
+    def doBackward(self, gradient):
+        return [gradient.reshape(self.inputShape)]
+
+
+class Unsqueeze(UnaryTensorFunction):                                                 # :422-442
+    modifiesShape = True
+
+    def __call__(self, tensor, axis):
+        super().__call__(tensor)
+        self.cachedShape = sf.unsqueeze(tensor.shape, axis)
+        self.axis = axis
+        return self
+
+    def doForward(self, input): self.output = input.unsqueeze(self.axis)
+    def doBackward(self, gradient): return [gradient.squeeze(self.axis)]
+
+
+class MaskedFill(UnaryTensorFunction):                                                # :561-584
+    def __call__(self, tensor, mask, value):
+        super().__call__(tensor)
+        if mask.requiresGrad:
+            raise ValueError("Masked fill only accepts mask that doesn't require gradients")
+        self.mask = mask.getRawValue()
+        self.value = float(value)
+        return self
+
+    def doForward(self, input):
+        self.output = input.maskedFill(self.mask, self.value)
+
+    def doBackward(self, gradient):
+        return [gradient.maskedFill(self.mask, 0.0)]
+
+
 class SoftmaxCrossEntropy(UnaryTensorFunction):
     """functions/nn/SoftmaxCrossEntropy.kt:10-69 — composed entirely of raw ops on the
     path: max, minus, exp, sum, div, clamp, log, gather, neg, mean; the backward is
@@ -1029,6 +1299,17 @@ def tensorOf(ops, *values, requiresGrad=False):
     """Tensor.tensorOf (Tensor.kt:1645-1655): a 1-D tensor of the given values."""
     vals = [float(v) for v in values]
     return ops.create([len(vals)], requiresGrad, vals)
+
+
+def concat(*tensors, axis=0):
+    """Tensor.concat (Tensor.kt:1774-1784)."""
+    tensors = _as_list(tensors)
+    if len(tensors) == 0:
+        raise ValueError("No tensors were passed to concat")
+    if len(tensors) == 1:
+        return tensors[0]
+    owner = next((t for t in tensors if t.requiresGrad), tensors[0])
+    return owner.concat(axis, tensors)
 
 
 def ones(ops, *shape, requiresGrad=False):

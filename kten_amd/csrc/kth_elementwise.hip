@@ -213,10 +213,6 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(float* out, uint32_t n, fl
 
 // ---------------------------------------------------------------- broadcast
 
-// Division by a launch-constant divisor d for numerators below 2^31:
-// q = (mulhi(n, mul) + n) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
-struct FastDiv { uint32_t mul, shift; };
-
 // The broadcast plan travels by value in the kernel arguments. Dim 0 is the innermost
 // coalesced dim. For the vector kernels dim 0 is counted in float4s and an operand's
 // dim-0 stride is 4 (contiguous) or 0 (broadcast along it); all strides are in floats.
@@ -301,6 +297,8 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_scalar_kernel(const float
 }
 
 struct OpFirst { static constexpr const char* name = "OpFirst"; static __device__ __forceinline__ float apply(float a, float, float) { return a; } };
+// maskedFill (JVMRawTensor.kt:537-540): the fill value rides in the third argument.
+struct OpMaskedFill { static constexpr const char* name = "OpMaskedFill"; static __device__ __forceinline__ float apply(float a, float m, float value) { return m == 1.0f ? value : a; } };
 
 // ---------------------------------------------------------------- NaN scan
 
@@ -326,15 +324,6 @@ __global__ void clear_flag_kernel(int* flag) { *flag = 0; }
 inline uint32_t blocks_for(uint64_t vec_count) {
     uint64_t b = (vec_count + kTile - 1) / kTile;
     return static_cast<uint32_t>(b == 0 ? 1 : b);
-}
-
-FastDiv make_div(uint32_t d) {
-    FastDiv f;
-    uint32_t shift = 0;
-    while ((1ull << shift) < d) shift++;
-    f.shift = shift;
-    f.mul = static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1);
-    return f;
 }
 
 // Builds the coalesced broadcast plan for out = a (op) b. Returns false when an operand
@@ -630,6 +619,36 @@ int kth_binary(int op,
 #undef B
     }
     KTH_LAUNCH_CHECK("binary");
+    return KTH_OK;
+}
+
+int kth_masked_fill(uint64_t a, const int32_t* ashape, int adims, uint64_t mask, const int32_t* mshape, int mdims,
+                    float value, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    uint64_t an, mn;
+    if (int rc = check_shape(ashape, adims, "kth_masked_fill(a)", &an)) return rc;
+    if (int rc = check_shape(mshape, mdims, "kth_masked_fill(mask)", &mn)) return rc;
+    Store* sa = lookup(a, "kth_masked_fill(a)");
+    if (!sa) return KTH_E_HANDLE;
+    Store* sm = lookup(mask, "kth_masked_fill(mask)");
+    if (!sm) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_masked_fill(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (an > sa->n_floats || mn > sm->n_floats || an > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_masked_fill: a shape needs more elements than its store holds");
+    BcastPlan plan;
+    bool vec_ok, a_vec, b_vec;
+    if (!build_plan(ashape, adims, mshape, mdims, ashape, adims, &plan, &vec_ok, &a_vec, &b_vec))
+        return fail(KTH_E_SHAPE, "kth_masked_fill: the mask does not broadcast to the tensor's shape");
+    if (mn != an && (so->ptr == sm->ptr)) return fail(KTH_E_ARGUMENT, "kth_masked_fill: output aliases the broadcast mask");
+    if (an == 0) return KTH_OK;
+    plan.a_stream = true;
+    plan.b_stream = (mn == an);
+    const uint32_t n32 = static_cast<uint32_t>(an);
+    if (mn == an) launch_binary_same<OpMaskedFill>(sa->ptr, sm->ptr, so->ptr, n32, value);
+    else launch_binary_bcast<OpMaskedFill>(sa->ptr, sm->ptr, so->ptr, n32, value, plan, vec_ok, a_vec, b_vec, (2 * an + mn) * 4);
+    KTH_LAUNCH_CHECK("masked_fill");
     return KTH_OK;
 }
 

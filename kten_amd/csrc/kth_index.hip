@@ -15,8 +15,6 @@ namespace {
 
 constexpr int kBlock = 256;
 
-struct FastDiv { uint32_t mul, shift; };
-
 // Dim 0 is the innermost of the position dims (index shape without the axis).
 struct IndexPlan {
     int      ndim;
@@ -76,15 +74,6 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 }
 
 __global__ void clear_int_kernel(int* p) { *p = 0; }
-
-FastDiv make_div(uint32_t d) {
-    FastDiv f;
-    uint32_t shift = 0;
-    while ((1ull << shift) < d) shift++;
-    f.shift = shift;
-    f.mul = static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1);
-    return f;
-}
 
 int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
     if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);

@@ -1,0 +1,369 @@
+// Layout movers: get / set / fill by index ranges, transpose, permute
+// (reference: JVMRawTensor.kt:270-315,437-466 with RangeTensorIndexing.sparseStoreRanges,
+// AbstractIndexing.kt:65-88; narrow JVM:468-473 and concat
+// AbstractJVMTensorOperations.kt:106-120 are range get / set on the host side).
+//
+// All of them are copies between a dense row-major tensor and a strided view of another:
+//   - a range index selects a box of the tensor; the reference concatenates the box's store
+//     ranges in order, which is the box read in row-major order;
+//   - permute reads the input through permuted strides.
+// When the innermost dim of the dense side is also contiguous on the strided side the copy
+// is a plain coalesced move (move_kernel, float4 when offsets allow). When the permutation
+// changes the innermost dim, 64x64 tiles go through LDS so that both the loads and the
+// stores are coalesced (permute_tile_kernel).
+#include "kth_internal.h"
+
+using namespace kth;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMoveUnroll = 2;
+constexpr int kTileDim = 64;
+constexpr int kTileRows = kBlock / kTileDim;          // rows of a tile one pass of the block covers
+constexpr int kTilePasses = kTileDim / kTileRows;
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// The strided side of a move. Dim 0 is the innermost dim of the dense side; for the float4
+// kernel size[0] is counted in float4s and stride[0] is 4. Strides and base are in floats.
+struct MovePlan {
+    int      ndim;
+    uint32_t size[KTH_MAX_DIMS];
+    FastDiv  div[KTH_MAX_DIMS];
+    uint32_t stride[KTH_MAX_DIMS];
+    uint32_t base;
+};
+
+__device__ __forceinline__ uint32_t strided_offset(const MovePlan& pl, uint32_t idx) {
+    uint32_t off = pl.base;
+    for (int d = 0; d < pl.ndim - 1; d++) {
+        uint32_t q = (__umulhi(idx, pl.div[d].mul) + idx) >> pl.div[d].shift;
+        off += (idx - q * pl.size[d]) * pl.stride[d];
+        idx = q;
+    }
+    return off + idx * pl.stride[pl.ndim - 1];
+}
+
+// MODE 0: dense[i] = strided[at(i)]   (range get, permute with the innermost dim kept)
+// MODE 1: strided[at(i)] = dense[i]   (range set)
+// MODE 2: strided[at(i)] = value      (range fill)
+// `units` counts float4s (VEC) or floats of the dense side.
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(kBlock) void move_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                     uint32_t units, float value, MovePlan pl) {
+    const uint32_t base = blockIdx.x * (kBlock * kMoveUnroll) + threadIdx.x;
+    if (VEC) {
+        v4f v[kMoveUnroll];
+        uint32_t at[kMoveUnroll];
+#pragma unroll
+        for (int k = 0; k < kMoveUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < units) {
+                at[k] = strided_offset(pl, i);
+                if (MODE == 0) v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + at[k]));
+                else if (MODE == 1) v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src) + i);
+                else v[k] = v4f{value, value, value, value};
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kMoveUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < units) {
+                if (MODE == 0) reinterpret_cast<v4f*>(dst)[i] = v[k];
+                else *reinterpret_cast<v4f*>(dst + at[k]) = v[k];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kMoveUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < units) {
+                const uint32_t at = strided_offset(pl, i);
+                if (MODE == 0) dst[i] = src[at];
+                else if (MODE == 1) dst[at] = src[i];
+                else dst[at] = value;
+            }
+        }
+    }
+}
+
+// A permutation that moves the input's contiguous dim X away from the innermost place:
+// the output's innermost dim is Y (input stride y_in_stride), X lands at output stride
+// x_out_stride, and every other dim is a batch dim with its own pair of strides.
+struct TilePlan {
+    uint32_t x_len, y_len;
+    uint32_t x_out_stride, y_in_stride;
+    uint32_t x_tiles, y_tiles;
+    FastDiv  x_tiles_div, y_tiles_div;
+    int      nbatch;
+    uint32_t bsize[KTH_MAX_DIMS];
+    FastDiv  bdiv[KTH_MAX_DIMS];
+    uint32_t b_in[KTH_MAX_DIMS], b_out[KTH_MAX_DIMS];
+};
+
+// One 64x64 tile per workgroup: rows of 64 consecutive x are loaded (256 B per wave
+// instruction), parked in LDS with a padded row so the transposed read is conflict-free,
+// and rows of 64 consecutive y are stored.
+__global__ __launch_bounds__(kBlock) void permute_tile_kernel(const float* __restrict__ in, float* __restrict__ out, TilePlan pl) {
+    __shared__ float tile[kTileDim][kTileDim + 1];
+    uint32_t t = blockIdx.x;
+    uint32_t q = (__umulhi(t, pl.x_tiles_div.mul) + t) >> pl.x_tiles_div.shift;
+    const uint32_t x0 = (t - q * pl.x_tiles) * kTileDim;
+    t = q;
+    q = (__umulhi(t, pl.y_tiles_div.mul) + t) >> pl.y_tiles_div.shift;
+    const uint32_t y0 = (t - q * pl.y_tiles) * kTileDim;
+    t = q;
+    uint32_t in_off = 0, out_off = 0;
+    for (int d = 0; d < pl.nbatch; d++) {
+        q = (__umulhi(t, pl.bdiv[d].mul) + t) >> pl.bdiv[d].shift;
+        const uint32_t r = t - q * pl.bsize[d];
+        in_off += r * pl.b_in[d];
+        out_off += r * pl.b_out[d];
+        t = q;
+    }
+    const uint32_t lx = threadIdx.x % kTileDim, ly = threadIdx.x / kTileDim;
+    float v[kTilePasses];
+#pragma unroll
+    for (int k = 0; k < kTilePasses; k++) {
+        const uint32_t x = x0 + lx, y = y0 + ly + k * kTileRows;
+        if (x < pl.x_len && y < pl.y_len) v[k] = __builtin_nontemporal_load(in + in_off + y * pl.y_in_stride + x);
+    }
+#pragma unroll
+    for (int k = 0; k < kTilePasses; k++) tile[ly + k * kTileRows][lx] = v[k];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTilePasses; k++) {
+        const uint32_t x = x0 + ly + k * kTileRows, y = y0 + lx;
+        if (x < pl.x_len && y < pl.y_len) out[out_off + x * pl.x_out_stride + y] = tile[lx][ly + k * kTileRows];
+    }
+}
+
+int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "%s: %d dims (1..%d)", what, dims, KTH_MAX_DIMS);
+    if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
+    uint64_t n = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0) return fail(KTH_E_ARGUMENT, "%s: negative dim %d", what, shape[i]);
+        n *= static_cast<uint64_t>(shape[i]);
+        if (n > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: more than 2^31-1 elements", what);
+    }
+    *count = n;
+    return KTH_OK;
+}
+
+// A dense logical tensor seen through strides: dims innermost first.
+struct StridedDims {
+    int      n;
+    uint64_t size[KTH_MAX_DIMS];
+    uint64_t stride[KTH_MAX_DIMS];
+};
+
+// Drops size-1 dims and merges a dim into the one inside it when the strided side steps
+// through both as through one longer dim.
+StridedDims coalesce(const StridedDims& in) {
+    StridedDims out{};
+    for (int d = 0; d < in.n; d++) {
+        if (in.size[d] == 1) continue;
+        if (out.n > 0 && in.stride[d] == out.stride[out.n - 1] * out.size[out.n - 1]) out.size[out.n - 1] *= in.size[d];
+        else { out.size[out.n] = in.size[d]; out.stride[out.n] = in.stride[d]; out.n++; }
+    }
+    if (out.n == 0) { out.n = 1; out.size[0] = 1; out.stride[0] = 1; }
+    return out;
+}
+
+// Launches move_kernel<MODE> over `count` dense elements; `dims` must have stride[0] == 1
+// for the float4 form to apply.
+template <int MODE>
+void launch_move(const char* family, const float* src, float* dst, uint64_t count, float value,
+                 const StridedDims& dims, uint64_t base, uint64_t bytes) {
+    MovePlan pl{};
+    pl.ndim = dims.n;
+    pl.base = static_cast<uint32_t>(base);
+    bool vec = dims.stride[0] == 1 && dims.size[0] % 4 == 0 && base % 4 == 0;
+    for (int d = 1; d < dims.n; d++) vec = vec && dims.stride[d] % 4 == 0;
+    for (int d = 0; d < dims.n; d++) {
+        pl.size[d] = static_cast<uint32_t>(dims.size[d]);
+        pl.stride[d] = static_cast<uint32_t>(dims.stride[d]);
+    }
+    uint64_t units = count;
+    if (vec) { pl.size[0] /= 4; pl.stride[0] = 4; units = count / 4; }
+    for (int d = 0; d < dims.n; d++) pl.div[d] = make_div(pl.size[d]);
+    const uint32_t per_block = kBlock * kMoveUnroll;
+    const uint32_t blocks = static_cast<uint32_t>((units + per_block - 1) / per_block);
+    LaunchScope scope(family, vec ? "float4" : "float", bytes);
+    if (vec) hipLaunchKernelGGL((move_kernel<MODE, true>), dim3(blocks), dim3(kBlock), 0, state().stream, src, dst,
+                                static_cast<uint32_t>(units), value, pl);
+    else     hipLaunchKernelGGL((move_kernel<MODE, false>), dim3(blocks), dim3(kBlock), 0, state().stream, src, dst,
+                                static_cast<uint32_t>(units), value, pl);
+}
+
+// Validates normalised inclusive ranges and describes the selected box as the strided side
+// of a move (dense side: the box in row-major order).
+int box_of(const char* what, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
+           StridedDims* box, uint64_t* base, uint64_t* count, uint64_t* total) {
+    if (int rc = shape_count(shape, dims, what, total)) return rc;
+    if (!first || !last) return fail(KTH_E_ARGUMENT, "%s: null range", what);
+    StridedDims raw{};
+    raw.n = dims;
+    uint64_t run = 1, off = 0, n = 1;
+    for (int d = dims - 1, k = 0; d >= 0; d--, k++) {
+        if (first[d] < 0 || last[d] >= shape[d] || first[d] > last[d])
+            return fail(KTH_E_ARGUMENT, "%s: range %d..%d does not index a dim of size %d", what, first[d], last[d], shape[d]);
+        raw.size[k] = static_cast<uint64_t>(last[d] - first[d] + 1);
+        raw.stride[k] = run;
+        off += static_cast<uint64_t>(first[d]) * run;
+        n *= raw.size[k];
+        run *= static_cast<uint64_t>(shape[d]);
+    }
+    *box = coalesce(raw);
+    if (box->n == 1 && box->size[0] == 1) box->stride[0] = 1;
+    *base = off;
+    *count = n;
+    return KTH_OK;
+}
+
+int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims, const int32_t* axes, uint64_t out) {
+    uint64_t n;
+    if (int rc = shape_count(shape, dims, what, &n)) return rc;
+    bool seen[KTH_MAX_DIMS] = {false};
+    for (int d = 0; d < dims; d++) {
+        if (axes[d] < 0 || axes[d] >= dims || seen[axes[d]])
+            return fail(KTH_E_ARGUMENT, "%s: axes must name every dimension once", what);
+        seen[axes[d]] = true;
+    }
+    Store* si = lookup(in, what);
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, what);
+    if (!so) return KTH_E_HANDLE;
+    if (n > si->n_floats || n > so->n_floats) return fail(KTH_E_ARGUMENT, "%s: the shape needs more elements than a store holds", what);
+    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", what);
+    if (n == 0) return KTH_OK;
+
+    uint64_t in_stride[KTH_MAX_DIMS];
+    uint64_t run = 1;
+    for (int d = dims - 1; d >= 0; d--) { in_stride[d] = run; run *= static_cast<uint64_t>(shape[d]); }
+    StridedDims raw{};
+    raw.n = dims;
+    for (int d = dims - 1, k = 0; d >= 0; d--, k++) {      // output dims, innermost first
+        raw.size[k] = static_cast<uint64_t>(shape[axes[d]]);
+        raw.stride[k] = in_stride[axes[d]];
+    }
+    const StridedDims v = coalesce(raw);
+    if (v.stride[0] == 1) {
+        launch_move<0>("move_kernel_permute", si->ptr, so->ptr, n, 0.0f, v, 0, n * 8);
+        KTH_LAUNCH_CHECK("move_kernel");
+        return KTH_OK;
+    }
+    int px = -1;
+    for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
+    if (px < 0) return fail(KTH_E_DEVICE, "%s: no contiguous input dim found", what);
+    TilePlan pl{};
+    pl.x_len = static_cast<uint32_t>(v.size[px]);
+    pl.y_len = static_cast<uint32_t>(v.size[0]);
+    pl.y_in_stride = static_cast<uint32_t>(v.stride[0]);
+    pl.x_tiles = (pl.x_len + kTileDim - 1) / kTileDim;
+    pl.y_tiles = (pl.y_len + kTileDim - 1) / kTileDim;
+    pl.x_tiles_div = make_div(pl.x_tiles);
+    pl.y_tiles_div = make_div(pl.y_tiles);
+    uint64_t out_run = 1, batch = 1;
+    for (int d = 0; d < v.n; d++) {
+        if (d == px) pl.x_out_stride = static_cast<uint32_t>(out_run);
+        else if (d != 0) {
+            pl.bsize[pl.nbatch] = static_cast<uint32_t>(v.size[d]);
+            pl.bdiv[pl.nbatch] = make_div(pl.bsize[pl.nbatch]);
+            pl.b_in[pl.nbatch] = static_cast<uint32_t>(v.stride[d]);
+            pl.b_out[pl.nbatch] = static_cast<uint32_t>(out_run);
+            pl.nbatch++;
+            batch *= v.size[d];
+        }
+        out_run *= v.size[d];
+    }
+    const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
+    if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+    {
+        LaunchScope scope("permute_tile_kernel", "", n * 8);
+        hipLaunchKernelGGL(permute_tile_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, state().stream,
+                           si->ptr, so->ptr, pl);
+    }
+    KTH_LAUNCH_CHECK("permute_tile_kernel");
+    return KTH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int kth_get_range(uint64_t in, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    StridedDims box; uint64_t base, count, total;
+    if (int rc = box_of("kth_get_range", shape, dims, first, last, &box, &base, &count, &total)) return rc;
+    Store* si = lookup(in, "kth_get_range(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_get_range(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (total > si->n_floats || count > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_get_range: a shape needs more elements than its store holds");
+    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "kth_get_range: output aliases the input");
+    launch_move<0>("move_kernel_get", si->ptr, so->ptr, count, 0.0f, box, base, count * 8);
+    KTH_LAUNCH_CHECK("move_kernel");
+    return KTH_OK;
+}
+
+int kth_set_range(uint64_t target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
+                  uint64_t value, uint64_t value_n) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    StridedDims box; uint64_t base, count, total;
+    if (int rc = box_of("kth_set_range", shape, dims, first, last, &box, &base, &count, &total)) return rc;
+    if (count != value_n)
+        return fail(KTH_E_SHAPE, "Cannot set tensor with %llu elements to an index range of %llu elements",
+                    static_cast<unsigned long long>(value_n), static_cast<unsigned long long>(count));
+    Store* st = lookup(target, "kth_set_range(target)");
+    if (!st) return KTH_E_HANDLE;
+    Store* sv = lookup(value, "kth_set_range(value)");
+    if (!sv) return KTH_E_HANDLE;
+    if (total > st->n_floats || value_n > sv->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_set_range: a shape needs more elements than its store holds");
+    if (st->ptr == sv->ptr) return fail(KTH_E_ARGUMENT, "kth_set_range: value aliases the target");
+    launch_move<1>("move_kernel_set", sv->ptr, st->ptr, count, 0.0f, box, base, count * 8);
+    KTH_LAUNCH_CHECK("move_kernel");
+    return KTH_OK;
+}
+
+int kth_fill_range(uint64_t target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, float value) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    StridedDims box; uint64_t base, count, total;
+    if (int rc = box_of("kth_fill_range", shape, dims, first, last, &box, &base, &count, &total)) return rc;
+    Store* st = lookup(target, "kth_fill_range(target)");
+    if (!st) return KTH_E_HANDLE;
+    if (total > st->n_floats) return fail(KTH_E_ARGUMENT, "kth_fill_range: the shape needs more elements than the store holds");
+    launch_move<2>("move_kernel_fill", nullptr, st->ptr, count, value, box, base, count * 4);
+    KTH_LAUNCH_CHECK("move_kernel");
+    return KTH_OK;
+}
+
+int kth_permute(uint64_t in, const int32_t* shape, int dims, const int32_t* axes, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!axes) return fail(KTH_E_ARGUMENT, "kth_permute: null axes");
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "kth_permute: %d dims", dims);
+    return permute_common("kth_permute", in, shape, dims, axes, out);
+}
+
+int kth_transpose(uint64_t in, const int32_t* shape, int dims, int axis1, int axis2, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "kth_transpose: %d dims", dims);
+    if (axis1 < 0 || axis1 >= dims || axis2 < 0 || axis2 >= dims || axis1 == axis2)
+        return fail(KTH_E_ARGUMENT, "Transpose requires different axes as parameters, but got %d and %d", axis1, axis2);
+    int32_t axes[KTH_MAX_DIMS];
+    for (int d = 0; d < dims; d++) axes[d] = d;
+    axes[axis1] = axis2;
+    axes[axis2] = axis1;
+    return permute_common("kth_transpose", in, shape, dims, axes, out);
+}
+
+}  // extern "C"

@@ -17,7 +17,7 @@ import numpy as np
 from . import abi
 from . import shape_functions as sf
 from .abi import Op, check
-from .raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number
+from .raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
 
 _BINARY = {"plus": Op.PLUS, "minus": Op.MINUS, "times": Op.TIMES, "div": Op.DIV, "pow": Op.POW,
            "lt": Op.LT, "lte": Op.LTE, "gt": Op.GT, "gte": Op.GTE, "eq": Op.EQ, "neq": Op.NEQ}
@@ -212,6 +212,69 @@ class HipRawTensor(AbstractRawTensor):
                                        index.storeReference, abi.shape_array(index.shape), src.storeReference,
                                        abi.shape_array(src.shape), self.dimensions, a))
 
+    # --- layout movers -------------------------------------------------------------------
+    def _get_store_range(self, offset, length, resShape):
+        """JVMRawTensor.kt:270-274: one contiguous store range."""
+        self._require_live()
+        res = self._new(resShape)
+        check(self.ops.lib.kth_copy(res.storeReference, 0, self.storeReference, offset, length))
+        return res
+
+    def _set_store_range(self, offset, length, value):
+        """JVMRawTensor.kt:282-289 (tensor) and 306-309 (constant)."""
+        self._require_live()
+        if _is_number(value):
+            check(self.ops.lib.kth_fill(self.storeReference, offset, length, float(value)))
+            return
+        value._require_live()
+        check(self.ops.lib.kth_copy(self.storeReference, offset, value.storeReference, 0, length))
+
+    def _get_ranges(self, first, last, resShape):
+        """JVMRawTensor.kt:276-280."""
+        self._require_live()
+        res = self._new(resShape)
+        check(self.ops.lib.kth_get_range(self.storeReference, abi.shape_array(self.shape), self.dimensions,
+                                         abi.shape_array(first), abi.shape_array(last), res.storeReference))
+        return res
+
+    def _set_ranges(self, first, last, value):
+        """JVMRawTensor.kt:291-304 (tensor) and 311-315 (constant)."""
+        self._require_live()
+        if _is_number(value):
+            check(self.ops.lib.kth_fill_range(self.storeReference, abi.shape_array(self.shape), self.dimensions,
+                                              abi.shape_array(first), abi.shape_array(last), float(value)))
+            return
+        value._require_live()
+        check(self.ops.lib.kth_set_range(self.storeReference, abi.shape_array(self.shape), self.dimensions,
+                                         abi.shape_array(first), abi.shape_array(last), value.storeReference, value.size))
+
+    def _transpose(self, axis1, axis2, resShape):
+        """JVMRawTensor.kt:437-451; the axis swap of Tensor.kt:1028-1058."""
+        self._require_live()
+        res = self._new(resShape)
+        check(self.ops.lib.kth_transpose(self.storeReference, abi.shape_array(self.shape), self.dimensions, axis1, axis2,
+                                         res.storeReference))
+        return res
+
+    def _permute(self, axes, resShape):
+        """JVMRawTensor.kt:453-466."""
+        self._require_live()
+        res = self._new(resShape)
+        check(self.ops.lib.kth_permute(self.storeReference, abi.shape_array(self.shape), self.dimensions,
+                                       abi.shape_array(axes), res.storeReference))
+        return res
+
+    def maskedFill(self, mask, value):
+        """JVMRawTensor.kt:537-540: the mask broadcasts to this tensor's shape."""
+        self._require_live(); mask._require_live()
+        if mask.shape != self.shape:
+            sf.infer_explicit_broadcast_shape(mask.shape, self.shape)
+        res = self._new(self.shape)
+        check(self.ops.lib.kth_masked_fill(self.storeReference, abi.shape_array(self.shape), self.dimensions,
+                                           mask.storeReference, abi.shape_array(mask.shape), mask.dimensions,
+                                           float(value), res.storeReference))
+        return res
+
     def copy(self, shallow: bool = False):
         """JVMRawTensor.kt:257-262; a shallow copy shares the store (OCLRawTensor.kt:252-258)."""
         self._require_live()
@@ -347,6 +410,10 @@ class HipTensorOperations:
         """TensorOperations.pow(constant, raw): constant ^ x elementwise
         (AbstractJVMTensorOperations.kt:94-96)."""
         return rawTensor._scalar("pow", float(constant), reverse=True)
+
+    def concat(self, axis: int, inputs) -> HipRawTensor:
+        """TensorOperations.kt:41."""
+        return raw_concat(self, axis, inputs)
 
     # --- Tensor-level factories (BasicTensorOperations.kt:10-12) ----------------------------
     def create(self, shape, requiresGrad: bool = False, init=None):

@@ -8,8 +8,8 @@ common-shape calculation) restated once here so that every backend shares them, 
 the reference. Kotlin's overloads on (tensor | Float) become one Python method that
 dispatches on the argument type; Kotlin operators are also exposed as Python operators.
 
-Members of the contract that lie outside the accelerated path (indexed get/set,
-transpose/permute, indexSelect/indexAdd, BLAS, nn) are not part of this mirror.
+Members of the contract that lie outside the accelerated path (indexSelect/indexAdd, dot,
+BLAS, nn) are not part of this mirror.
 """
 from enum import Enum
 from typing import List, Sequence
@@ -231,6 +231,71 @@ class AbstractRawTensor:
         res.inplaceScatter(axis, index, src)
         return res
 
+    # --- get / set by index (AbstractRawTensor.kt:27-37) --------------------------------
+    # An index is a sequence of ints (Kotlin IntArray: leading dims, negative values wrap)
+    # or a sequence of shape_functions.IntRange / (first, last) pairs / ALL (Kotlin
+    # Array<IntRange>, both ends inclusive). Backends supply moves of one contiguous store
+    # range and of a box of ranges.
+    def _get_store_range(self, offset: int, length: int, resShape): raise NotImplementedError
+    def _set_store_range(self, offset: int, length: int, value): raise NotImplementedError     # value: tensor or float
+    def _get_ranges(self, first, last, resShape): raise NotImplementedError
+    def _set_ranges(self, first, last, value): raise NotImplementedError                       # value: tensor or float
+    def _permute(self, axes, resShape): raise NotImplementedError
+    def _transpose(self, axis1: int, axis2: int, resShape): raise NotImplementedError
+    def maskedFill(self, mask, value: float): raise NotImplementedError
+
+    def get(self, index):
+        index = list(index)
+        if sf.is_range_index(index):                                   # JVMRawTensor.kt:276-280
+            norm, res_shape = sf.normalized_range_indexed_shape(self.shape, index)
+            first, last = sf.full_ranges(self.shape, norm)
+            return self._get_ranges(first, last, res_shape)
+        norm, res_shape = sf.normalized_indexed_shape(self.shape, index)   # JVMRawTensor.kt:270-274
+        offset, length = sf.store_range(self.shape, norm)
+        return self._get_store_range(offset, length, res_shape)
+
+    def set(self, index, value):
+        index = list(index)
+        if sf.is_range_index(index):                                   # JVMRawTensor.kt:291-304,311-315
+            norm = sf.normalize_range_index(self.shape, index)
+            first, last = sf.full_ranges(self.shape, norm)
+            if not _is_number(value):
+                size = sf.to_store_size([l - f + 1 for f, l in zip(first, last)])
+                if size != sf.to_store_size(value.shape):
+                    raise ValueError(f"Cannot set tensor with shape {value.shape} to tensor with shape: {self.shape} "
+                                     f"at index: {[tuple(sf.as_range(r)) for r in index]}")
+            self._set_ranges(first, last, value)
+            return
+        norm = sf.normalize_index(self.shape, index)                   # JVMRawTensor.kt:282-289,306-309
+        offset, length = sf.store_range(self.shape, norm)
+        if not _is_number(value) and sf.to_store_size(value.shape) != length:
+            raise ValueError(f"Cannot set tensor with shape: {value.shape} to tensor with shape: {self.shape} "
+                             f"at index: {index}")
+        self._set_store_range(offset, length, value)
+
+    def __getitem__(self, index):
+        return self.get(index if isinstance(index, (tuple, list)) and not isinstance(index, sf.IntRange) else [index])
+
+    def __setitem__(self, index, value):
+        self.set(index if isinstance(index, (tuple, list)) and not isinstance(index, sf.IntRange) else [index], value)
+
+    # --- transpose / permute / narrow (AbstractRawTensor.kt:228-232) --------------------
+    def transpose(self, axis1: int, axis2: int):
+        new_shape, a1, a2 = sf.transpose_normalize_axes(self.shape, axis1, axis2)
+        return self._transpose(a1, a2, new_shape)
+
+    def permute(self, axes):
+        axes = list(axes)
+        return self._permute(axes, sf.permute(self.shape, axes))
+
+    def narrow(self, axis: int, start: int, length: int):
+        """JVMRawTensor.kt:468-473: the range start until start + length at the axis, every
+        other dim in full, through the range get (which also validates the range)."""
+        a = sf.normalize_axis(self.shape, axis)
+        ranges = sf.to_index_ranges(self.shape)
+        ranges[a] = sf.IntRange(start, start + length - 1)
+        return self.get(ranges)
+
     # --- broadcasting (AbstractRawTensor.kt:170-192) -----------------------------------
     def calculateCommonShapeWith(self, other) -> List[int]:
         """Right-align, keep the longer operand's extra leading dims, per-dim max.
@@ -246,3 +311,21 @@ class AbstractRawTensor:
             res.extend(b[:-diff]); b = b[-diff:]
         res.extend(max(x, y) for x, y in zip(a, b))
         return res
+
+
+def concat(ops, axis: int, inputs):
+    """TensorOperations.concat (TensorOperations.kt:41) as the JVM backend builds it
+    (AbstractJVMTensorOperations.kt:106-120): a new tensor of the concatenated shape, then one
+    range set per input at its offset along the axis."""
+    inputs = list(inputs)
+    shapes = [t.shape for t in inputs]
+    res_shape = sf.concat_shapes(shapes, axis)
+    a = sf.normalize_axis(shapes[0], axis)
+    target = sf.to_index_ranges(res_shape)
+    res = ops.createRaw(res_shape)
+    last = 0
+    for t in inputs:
+        target[a] = sf.IntRange(last, last + t.shape[a] - 1)
+        res.set(target, t)
+        last += t.shape[a]
+    return res

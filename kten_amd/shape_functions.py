@@ -6,7 +6,7 @@ broadcast / reduction path uses. Shapes are Python lists of ints; every function
 ValueError where the reference throws IllegalArgumentException, before anything is
 launched on the device.
 """
-from typing import List, Sequence
+from typing import NamedTuple, List, Sequence
 
 
 def to_store_size(shape: Sequence[int]) -> int:
@@ -157,3 +157,115 @@ def normalized_axis_scatter(shape: Sequence[int], axis: int, index_shape: Sequen
             raise ValueError("Scatter requires that index.shape[a] <= target.shape[a] for all axis 'a', except the specified "
                              f"'axis' of the operation, but got tensors with shapes: index: {list(index_shape)}, target: {list(shape)}")
     return a
+
+
+# ---------------------------------------------------------------- range indexing
+
+class IntRange(NamedTuple):
+    """A Kotlin `first..last` range: both ends inclusive."""
+    first: int
+    last: int
+
+
+#: The reference's `all` range (kten-api/.../tensor/Constants.kt): every index of the dim.
+ALL = IntRange(-2 ** 31, 2 ** 31 - 1)
+
+
+def as_range(item) -> IntRange:
+    """Accepts IntRange, ALL, or a (first, last) pair."""
+    if isinstance(item, IntRange):
+        return item
+    if isinstance(item, (tuple, list)) and len(item) == 2:
+        return IntRange(int(item[0]), int(item[1]))
+    raise TypeError(f"Not an index range: {item!r}")
+
+
+def normalized_indexed_shape(shape: Sequence[int], index: Sequence[int]):
+    """ShapeFunctions.kt:232-238 — an Int index selects the sub-tensor under its leading
+    dims; a full index selects one element, with shape [1]."""
+    norm = normalize_index(shape, index)
+    return norm, ([1] if len(norm) == len(shape) else list(shape[len(norm):]))
+
+
+def normalize_range_index(shape: Sequence[int], index: Sequence) -> List[IntRange]:
+    """ShapeFunctions.kt:240-259 — `all` becomes 0 until size; a range with a negative end has
+    its negative ends wrapped; afterwards both ends must lie inside the dim, in order."""
+    ranges = [as_range(r) for r in index]
+    out = []
+    invalid = len(ranges) > len(shape)
+    for size, r in zip(shape, ranges):
+        if r == ALL:
+            r = IntRange(0, size - 1)
+        elif r.first < 0 or r.last < 0:
+            r = IntRange(size + r.first if r.first < 0 else r.first, size + r.last if r.last < 0 else r.last)
+        if r.first < 0 or r.last < 0 or r.first >= size or r.last >= size or r.first > r.last:
+            invalid = True
+        out.append(r)
+    if invalid:
+        raise ValueError(f"Cannot index tensor with shape: {list(shape)} with index: {[tuple(r) for r in ranges]}")
+    return out
+
+
+def normalized_range_indexed_shape(shape: Sequence[int], index: Sequence):
+    """ShapeFunctions.kt:261-268 — range lengths, then the unindexed trailing dims."""
+    norm = normalize_range_index(shape, index)
+    return norm, [r.last - r.first + 1 for r in norm] + list(shape[len(norm):])
+
+
+def is_range_index(index) -> bool:
+    """Kotlin picks the overload by type: IntArray or Array<IntRange>."""
+    return len(index) > 0 and not all(isinstance(i, int) and not isinstance(i, bool) for i in index)
+
+
+def store_range(shape: Sequence[int], norm_index: Sequence[int]):
+    """AbstractIndexing.kt:43-54 SimpleTensorIndexing.storeRange as (offset, length)."""
+    start = 0
+    for size, i in zip(shape, norm_index):
+        start = start * size + i
+    sub = to_store_size(shape[len(norm_index):])
+    return start * sub, sub
+
+
+def full_ranges(shape: Sequence[int], norm_ranges: Sequence[IntRange]):
+    """One (first, last) per dim: the given ranges, then every unindexed dim in full."""
+    first = [r.first for r in norm_ranges] + [0] * (len(shape) - len(norm_ranges))
+    last = [r.last for r in norm_ranges] + [s - 1 for s in shape[len(norm_ranges):]]
+    return first, last
+
+
+def to_index_ranges(shape: Sequence[int]) -> List[IntRange]:
+    """ShapeFunctions.kt:310-312."""
+    return [IntRange(0, s - 1) for s in shape]
+
+
+def transpose_normalize_axes(shape: Sequence[int], axis1: int, axis2: int):
+    """ShapeFunctions.kt:115-129."""
+    a1, a2 = normalize_axis(shape, axis1), normalize_axis(shape, axis2)
+    if a1 == a2:
+        raise ValueError(f"Transpose requires different axes as parameters, but got {axis1} (normalized: {a1}) "
+                         f"and {axis2} (normalized: {a2})")
+    res = list(shape)
+    res[a1], res[a2] = shape[a2], shape[a1]
+    return res, a1, a2
+
+
+def permute(shape: Sequence[int], axes: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:106-113 — every dim must be named; negative axes are not accepted."""
+    if len(shape) != len(axes) or not all(d in axes for d in range(len(shape))):
+        raise ValueError(f"Tensor with shape: {list(shape)} cannot be permuted by axes: {list(axes)}. "
+                         "All dimensions must be indexed.")
+    return [shape[a] for a in axes]
+
+
+def concat_shapes(shapes: Sequence[Sequence[int]], axis: int) -> List[int]:
+    """ShapeFunctions.kt:85-104 — equal dim counts and equal sizes off the axis."""
+    if len({len(s) for s in shapes}) == 1:
+        a = normalize_axis(shapes[0], axis)
+        rest = {tuple(s[:a]) + tuple(s[a + 1:]) for s in shapes}
+        if len(rest) == 1:
+            res = list(shapes[0])
+            res[a] = sum(s[a] for s in shapes)
+            return res
+    raise ValueError(f"Cannot concatenate tensors with shapes: {[list(s) for s in shapes]} at axis: {axis} "
+                     "(All tensors must have the same number of dimenisons, and have the same size at all dimenions "
+                     "except at the dimension indexed by the axis)")

@@ -15,7 +15,7 @@ from ctypes import POINTER, c_double, c_float, c_int, c_int32, c_int64, c_void_p
 import numpy as np
 
 from kten_amd import shape_functions as sf
-from kten_amd.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number
+from kten_amd.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libkten_jvm_oracle.so")
@@ -74,6 +74,15 @@ def lib():
     L.kjo_scatter.restype = c_int
     L.kjo_scatter_fill.argtypes = [fp, ip, fp, ip, c_int, c_int, c_float]
     L.kjo_scatter_fill.restype = c_int
+    L.kjo_range_size.argtypes = [ip, c_int, ip, ip]
+    L.kjo_range_size.restype = c_int64
+    L.kjo_get_range.argtypes = [fp, ip, c_int, ip, ip, fp]
+    L.kjo_set_range.argtypes = [fp, ip, c_int, ip, ip, fp, c_int64]
+    L.kjo_set_range.restype = c_int
+    L.kjo_fill_range.argtypes = [fp, ip, c_int, ip, ip, c_float]
+    L.kjo_transpose_jvm.argtypes = [fp, ip, c_int, c_int, c_int, fp, fp]
+    L.kjo_permute.argtypes = [fp, ip, c_int, ip, fp]
+    L.kjo_masked_fill.argtypes = [fp, fp, c_float, fp, c_int64]
     L.kjo_unary_f64.argtypes = [c_int, c_float]
     L.kjo_unary_f64.restype = c_double
     _lib = L
@@ -171,6 +180,53 @@ def axis_sum_f64(a, axis: int):
     return out, ab
 
 
+def get_range(a, first, last) -> np.ndarray:
+    """get(Array<IntRange>) with one normalised inclusive range per dim; keeps the dims."""
+    a = _f32(a)
+    shape = [l - f + 1 for f, l in zip(first, last)]
+    out = np.empty(shape, dtype=np.float32)
+    lib().kjo_get_range(_p(a), _sh(a.shape), a.ndim, _sh(first), _sh(last), _p(out))
+    return out
+
+
+def set_range(target, first, last, value) -> np.ndarray:
+    """set(Array<IntRange>, tensor | Float) on a copy of `target`."""
+    t = _f32(target).copy()
+    if isinstance(value, (int, float)):
+        lib().kjo_fill_range(_p(t), _sh(t.shape), t.ndim, _sh(first), _sh(last), float(value))
+        return t
+    v = _f32(value)
+    if lib().kjo_set_range(_p(t), _sh(t.shape), t.ndim, _sh(first), _sh(last), _p(v), v.size) != 0:
+        raise ValueError(f"Cannot set tensor with shape {list(v.shape)} to tensor with shape: {list(t.shape)}")
+    return t
+
+
+def transpose_jvm(a, axis1: int, axis2: int) -> np.ndarray:
+    """kten-jvm's slab-copy transpose, literally (equals the axis swap for adjacent axes)."""
+    a = _f32(a)
+    shape = list(a.shape); shape[axis1], shape[axis2] = shape[axis2], shape[axis1]
+    out = np.empty(shape, dtype=np.float32)
+    scratch = np.empty(max(a.size // max(a.shape[axis1], 1), 1), dtype=np.float32)
+    lib().kjo_transpose_jvm(_p(a), _sh(a.shape), a.ndim, axis1, axis2, _p(out), _p(scratch))
+    return out
+
+
+def permute(a, axes) -> np.ndarray:
+    a = _f32(a)
+    out = np.empty([a.shape[x] for x in axes], dtype=np.float32)
+    lib().kjo_permute(_p(a), _sh(a.shape), a.ndim, _sh(axes), _p(out))
+    return out
+
+
+def masked_fill(a, mask, value: float) -> np.ndarray:
+    a, mask = _f32(a), _f32(mask)
+    if mask.shape != a.shape:
+        mask = broadcast_to(mask, a.shape)
+    out = np.empty_like(a)
+    lib().kjo_masked_fill(_p(a), _p(mask), value, _p(out), a.size)
+    return out
+
+
 def unary_f64(op: str, x: float) -> float:
     return lib().kjo_unary_f64(OPS[op], x)
 
@@ -263,6 +319,38 @@ class JvmOracleRawTensor(AbstractRawTensor):
         if rc != 0:
             raise ValueError("Scatter got invalid index, an index value is out of bounds at the axis")
 
+    def _get_store_range(self, offset, length, resShape):                      # JVM:270-274 sliceArray
+        return JvmOracleRawTensor(list(resShape), self.storeReference[offset:offset + length].copy(), self.ops)
+
+    def _set_store_range(self, offset, length, value):                         # JVM:282-289,306-309
+        if _is_number(value):
+            self.storeReference[offset:offset + length] = np.float32(value)
+        else:
+            self.storeReference[offset:offset + length] = value.storeReference[:length]
+
+    def _get_ranges(self, first, last, resShape):
+        out = np.empty(sf.to_store_size(resShape), dtype=np.float32)
+        lib().kjo_get_range(_p(self.storeReference), _sh(self.shape), self.dimensions, _sh(first), _sh(last), _p(out))
+        return JvmOracleRawTensor(list(resShape), out, self.ops)
+
+    def _set_ranges(self, first, last, value):
+        if _is_number(value):
+            lib().kjo_fill_range(_p(self.storeReference), _sh(self.shape), self.dimensions, _sh(first), _sh(last), float(value))
+        elif lib().kjo_set_range(_p(self.storeReference), _sh(self.shape), self.dimensions, _sh(first), _sh(last),
+                                 _p(value.storeReference), value.storeReference.size) != 0:
+            raise ValueError(f"Cannot set tensor with shape {value.shape} to tensor with shape: {self.shape}")
+
+    def _transpose(self, axis1, axis2, resShape):
+        return self._wrap(transpose_jvm(self._nd(), axis1, axis2))
+
+    def _permute(self, axes, resShape):
+        return self._wrap(permute(self._nd(), axes))
+
+    def maskedFill(self, mask, value):
+        if mask.shape != self.shape:
+            sf.infer_explicit_broadcast_shape(mask.shape, self.shape)
+        return self._wrap(masked_fill(self._nd(), mask._nd(), float(value)))
+
     def copy(self, shallow=False):
         if shallow:
             return JvmOracleRawTensor(list(self.shape), self.storeReference, self.ops)
@@ -330,6 +418,9 @@ class JvmOracleOperations:
 
     def pow(self, constant, rawTensor):
         return rawTensor._scalar("pow", float(constant), reverse=True)
+
+    def concat(self, axis, inputs):
+        return raw_concat(self, axis, inputs)
 
     def create(self, shape, requiresGrad=False, init=None):
         from kten_amd.autograd import NoGradVariable, Variable

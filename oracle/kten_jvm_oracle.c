@@ -386,6 +386,131 @@ int kjo_scatter_fill(float* target, const int32_t* target_shape, const float* in
     return 0;
 }
 
+/* ---------------------------------------------------------------- layout movers */
+
+/* IDX:65-88 RangeTensorIndexing.sparseStoreRanges for normalised inclusive ranges
+ * first[d]..last[d], one per dim of `shape`: trailing dims indexed by their full range
+ * are dropped; the remaining k ranges give one store range per combination of the first
+ * k-1 of them (row-major), each from (.., first[k-1]) * sub to (.., last[k-1] + 1) * sub
+ * where sub is the volume of the dropped dims. Calls visit(lo, hi_exclusive) in order. */
+typedef void (*range_visitor)(int64_t lo, int64_t hi, void* ctx);
+
+static void sparse_store_ranges(const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
+                                range_visitor visit, void* ctx) {
+    int k = dims;
+    while (k > 0 && first[k - 1] == 0 && last[k - 1] == shape[k - 1] - 1) k--;
+    if (k == 0) { visit(0, store_size(shape, dims), ctx); return; }
+    int64_t sub = 1;
+    for (int d = k; d < dims; d++) sub *= shape[d];
+    int64_t ranges = 1;
+    int32_t span[KJO_MAX_DIMS];
+    for (int d = 0; d < k - 1; d++) { span[d] = last[d] - first[d] + 1; ranges *= span[d]; }
+    for (int64_t r = 0; r < ranges; r++) {
+        int32_t idx[KJO_MAX_DIMS];
+        int64_t i = r;
+        for (int d = k - 2; d >= 0; d--) { idx[d] = (int32_t)(i % span[d]) + first[d]; i /= span[d]; }
+        idx[k - 1] = first[k - 1];
+        int64_t lo = index_base(idx, shape, k) * sub;
+        idx[k - 1] = last[k - 1] + 1;
+        int64_t hi = index_base(idx, shape, k) * sub;
+        visit(lo, hi, ctx);
+    }
+}
+
+struct range_ctx { const float* src; float* dst; int64_t at; float value; int64_t count; };
+
+static void visit_count(int64_t lo, int64_t hi, void* c) { ((struct range_ctx*)c)->count += hi - lo; }
+static void visit_get(int64_t lo, int64_t hi, void* c) {
+    struct range_ctx* x = (struct range_ctx*)c;
+    memcpy(x->dst + x->at, x->src + lo, (size_t)(hi - lo) * sizeof(float));
+    x->at += hi - lo;
+}
+static void visit_set(int64_t lo, int64_t hi, void* c) {
+    struct range_ctx* x = (struct range_ctx*)c;
+    memcpy(x->dst + lo, x->src + x->at, (size_t)(hi - lo) * sizeof(float));
+    x->at += hi - lo;
+}
+static void visit_fill(int64_t lo, int64_t hi, void* c) {
+    struct range_ctx* x = (struct range_ctx*)c;
+    for (int64_t i = lo; i < hi; i++) x->dst[i] = x->value;
+}
+
+/* Number of elements the ranges select. */
+int64_t kjo_range_size(const int32_t* shape, int dims, const int32_t* first, const int32_t* last) {
+    struct range_ctx c = {0};
+    sparse_store_ranges(shape, dims, first, last, visit_count, &c);
+    return c.count;
+}
+
+/* JVM:276-280 get(Array<IntRange>): the selected store ranges, concatenated in order. */
+void kjo_get_range(const float* in, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, float* out) {
+    struct range_ctx c = {0};
+    c.src = in; c.dst = out;
+    sparse_store_ranges(shape, dims, first, last, visit_get, &c);
+}
+
+/* JVM:291-304 set(Array<IntRange>, tensor): the value's elements, in store order, fill the
+ * selected ranges in order. Only the element COUNT is checked (JVM:295-296): returns -1 when
+ * it differs (the reference throws IllegalArgumentException), else 0. */
+int kjo_set_range(float* target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
+                  const float* value, int64_t value_n) {
+    if (kjo_range_size(shape, dims, first, last) != value_n) return -1;
+    struct range_ctx c = {0};
+    c.src = value; c.dst = target;
+    sparse_store_ranges(shape, dims, first, last, visit_set, &c);
+    return 0;
+}
+
+/* JVM:311-315 set(Array<IntRange>, Float). */
+void kjo_fill_range(float* target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, float value) {
+    struct range_ctx c = {0};
+    c.dst = target; c.value = value;
+    sparse_store_ranges(shape, dims, first, last, visit_fill, &c);
+}
+
+/* JVM:437-451 transpose, literally: res starts as a copy with the swapped shape; then for
+ * every i along axis1, the slab this[.., axis1 = i, ..] is read in store order and written,
+ * in store order, into res[.., axis2 = i, ..]. For adjacent axes (or when every dim between
+ * them has size 1) this is the axis swap the contract documents; for other axis pairs the
+ * two store orders differ and kten-jvm's result is NOT the axis swap (its OpenCL backend,
+ * kernels.cl:263-287, swaps the indices and does give the axis swap). `scratch` holds one slab. */
+void kjo_transpose_jvm(const float* in, const int32_t* shape, int dims, int axis1, int axis2, float* out, float* scratch) {
+    int32_t new_shape[KJO_MAX_DIMS], f_in[KJO_MAX_DIMS], l_in[KJO_MAX_DIMS], f_out[KJO_MAX_DIMS], l_out[KJO_MAX_DIMS];
+    for (int d = 0; d < dims; d++) new_shape[d] = shape[d];
+    new_shape[axis1] = shape[axis2];
+    new_shape[axis2] = shape[axis1];
+    memcpy(out, in, (size_t)store_size(shape, dims) * sizeof(float));
+    for (int d = 0; d < dims; d++) { f_in[d] = 0; l_in[d] = shape[d] - 1; f_out[d] = 0; l_out[d] = new_shape[d] - 1; }
+    for (int32_t i = 0; i < shape[axis1]; i++) {
+        f_in[axis1] = l_in[axis1] = i;
+        f_out[axis2] = l_out[axis2] = i;
+        kjo_get_range(in, shape, dims, f_in, l_in, scratch);
+        kjo_set_range(out, new_shape, dims, f_out, l_out, scratch, kjo_range_size(shape, dims, f_in, l_in));
+    }
+}
+
+/* JVM:453-466 permute: res.shape[d] = shape[axes[d]]; every source element at multi-index t
+ * goes to the multi-index (t[axes[0]], t[axes[1]], ..) of res. */
+void kjo_permute(const float* in, const int32_t* shape, int dims, const int32_t* axes, float* out) {
+    int32_t new_shape[KJO_MAX_DIMS];
+    for (int d = 0; d < dims; d++) new_shape[d] = shape[axes[d]];
+    const int64_t n = store_size(shape, dims);
+    #pragma omp parallel for num_threads(g_threads) schedule(static) if (n > 65536)
+    for (int64_t it = 0; it < n; it++) {
+        int32_t t[KJO_MAX_DIMS], by_axes[KJO_MAX_DIMS];
+        int64_t i = it;
+        for (int d = dims - 1; d >= 0; d--) { t[d] = (int32_t)(i % shape[d]); i /= shape[d]; }   /* IDX:104-115 */
+        for (int d = 0; d < dims; d++) by_axes[d] = t[axes[d]];
+        out[index_base(by_axes, new_shape, dims)] = in[it];
+    }
+}
+
+/* JVM:537-540 maskedFill on a mask already broadcast to the tensor's shape (the caller
+ * broadcasts with kjo_broadcast_to, as JVM:538 does): mask == 1f selects the value. */
+void kjo_masked_fill(const float* a, const float* mask, float value, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = (mask[i] == 1.0f) ? value : a[i];
+}
+
 /* ---------------------------------------------------------------- reductions */
 
 /* JVM:146-148 sum() = kotlin FloatArray.sum(): float accumulator from 0f, index order. */

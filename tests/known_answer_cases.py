@@ -9,7 +9,8 @@ import os
 
 import numpy as np
 
-from kten_amd.autograd import ones, tensorOf
+from kten_amd.autograd import concat, ones, tensorOf
+from kten_amd.shape_functions import ALL
 
 with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
     K = json.load(f)
@@ -331,6 +332,89 @@ def case_readme_sum_of_squares(ops):
     t = T(ops, c["t1"], True)
     (t ** 2).sum().backward()
     assertTensorEquals(c["grad"], t.grad(), c["tol"], c["t1"]["shape"])
+
+
+def _idx(spec):
+    """JSON index -> Python index: ints stay, [first, last] pairs are inclusive ranges, "all" is ALL."""
+    return tuple(ALL if i == "all" else (tuple(i) if isinstance(i, list) else i) for i in spec)
+
+
+def case_set_element_from_tensor_with_grads(ops):
+    c = K["set_element_from_tensor_with_grads"]
+    t1 = T(ops, c["t1"], True)
+    t2 = filled(ops, c["t2_fill"], c["t2_shape"])
+    t2[_idx(c["index"])] = t1[_idx(c["value_index"])] ** float(c["power"])
+    t2.sum().backward()
+    t1.sum().backward()
+    assertTensorEquals(c["t2_expected"], t2, c["tol"], c["t2_expected"]["shape"])
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_grad"]["shape"])
+
+
+def case_set_element_range_from_tensor_with_grads(ops):
+    c = K["set_element_range_from_tensor_with_grads"]
+    t1 = filled(ops, c["t1_fill"], c["t1_shape"])
+    t2 = filled(ops, c["t2_fill"], c["t2_shape"])
+    t2[_idx(c["set_index"])] = (t1[_idx(c["get_index"])] ** float(c["power"])).unsqueeze(c["unsqueeze"])
+    t2.sum().backward()
+    t1.sum().backward()
+    assertTensorEquals(c["t2_expected"], t2, c["tol"], c["t2_expected"]["shape"])
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_grad"]["shape"])
+
+
+def _set_constant(ops, name):
+    c = K[name]
+    t1 = filled(ops, c["t1_fill"], c["t1_shape"])
+    t1[_idx(c["index"])] = c["value"]
+    assertTensorEquals(c["t1_expected"], t1, c["tol"], c["t1_expected"]["shape"])
+    t1.sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_grad"]["shape"])
+
+
+def case_set_constant_at_single_index_with_grads(ops): _set_constant(ops, "set_constant_at_single_index_with_grads")
+def case_set_constant_by_range_with_grads(ops): _set_constant(ops, "set_constant_by_range_with_grads")
+
+
+def case_transpose_with_grads(ops):
+    c = K["transpose_with_grads"]
+    t1 = T(ops, c["t1"], True)
+    res = t1.transpose(*c["axes"])
+    assertTensorEquals(c["expected"], res, c["tol"], c["expected"]["shape"])
+    res.backward(T(ops, c["backward_with"]))
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_grad"]["shape"])
+
+
+def case_permute_with_grads(ops):
+    c = K["permute_with_grads"]
+    t1 = T(ops, c["t1"], True)
+    res = t1.permute(*c["axes"])
+    assertTensorEquals(c["expected"], res, c["tol"], c["expected"]["shape"])
+    (res ** 2.0).sum().backward()
+    assertTensorEquals(c["t1_grad"], t1.grad(), c["tol"], c["t1_grad"]["shape"])
+
+
+def case_concat_with_grads(ops):
+    c = K["concat_with_grads"]
+    ts = [tensorOf(ops, *c[k]["values"]).expand(c[k]["expand"]).asVariable(requiresGrad=True) for k in ("t1", "t2", "t3")]
+    res = concat(*ts)
+    assertTensorEquals(c["expected"], res, c["tol"], c["expected"]["shape"])
+    (res ** 2.0).sum().backward()
+    for t, k in zip(ts, ("t1_grad", "t2_grad", "t3_grad")):
+        assertTensorEquals(c[k], t.grad(), c["tol"], c[k]["shape"])
+
+
+def case_fill_partially(ops):
+    c = K["fill_partially"]
+    t1 = ones(ops, *c["shape"])
+    t1 = t1 * c["times"]
+    t1[_idx(c["index"])] = c["value"]
+    assertTensorEquals(c["expected"], t1, c["tol"], c["expected"]["shape"])
+
+
+def case_doc_transpose_and_permute(ops):
+    for name, method in (("doc_transpose_3d", "transpose"), ("doc_permute_3d", "permute")):
+        c = K[name]
+        t = tensorOf(ops, *range(c["arrange"])).reshape(c["shape"])
+        assertTensorEquals(c["expected"], getattr(t, method)(*c["axes"]), c["tol"], c["expected"]["shape"])
 
 
 CASES = [v for k, v in sorted(globals().items()) if k.startswith("case_")]

@@ -1,0 +1,180 @@
+"""Layout movers on the device against the CPU checker, bit-exact: get / set / fill by
+index and by ranges, narrow, concat, transpose, permute, maskedFill; float4 and scalar
+forms, tile edges, error behaviour, and size-independent properties at large sizes."""
+import itertools
+
+import numpy as np
+import pytest
+
+from kten_amd.shape_functions import ALL
+from oracle import jvm_oracle as jo
+from parity import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def both(gc, array):
+    shape = list(array.shape)
+    return gc.createRaw(shape, array), jo.JvmOracleOperations().createRaw(shape, array.reshape(-1))
+
+
+def boxes(rng, shape, count):
+    out = []
+    for _ in range(count):
+        k = int(rng.integers(1, len(shape) + 1))
+        out.append([(f, int(rng.integers(f, shape[d]))) for d in range(k) for f in [int(rng.integers(0, shape[d]))]])
+    return out
+
+
+SHAPES = [[7], [4096], [5, 9], [64, 256], [33, 1024], [3, 4, 5], [6, 16, 64], [2, 3, 4, 5], [4, 8, 12, 16],
+          [2, 3, 2, 3, 2, 3], [1, 1, 8], [300, 700]]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_range_get_set_fill_parity(shape, gc):
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    aligned = [[(0, shape[0] - 1)] + [(0, s - 1) if s % 4 else (4 * (s // 8), s - 1) for s in shape[1:]]]
+    for box in boxes(rng, shape, 12) + aligned + [[ALL] * len(shape)]:
+        g, c = both(gc, x)
+        got, want = g.get(box), c.get(box)
+        assert got.shape == want.shape
+        assert_bits_equal(got.toArray(), want.toArray(), f"get {box}")
+        v = rng.standard_normal(want.shape).astype(np.float32)
+        gv, cv = both(gc, v)
+        g.set(box, gv); c.set(box, cv)
+        assert_bits_equal(g.toArray(), c.toArray(), f"set {box}")
+        g.set(box, -3.5); c.set(box, -3.5)
+        assert_bits_equal(g.toArray(), c.toArray(), f"fill {box}")
+
+
+def test_int_index_get_set_parity(gc):
+    x = np.arange(2 * 3 * 40, dtype=np.float32).reshape(2, 3, 40)
+    for index in ([1], [-1, 2], [0, -1, 39], [1, 0]):
+        g, c = both(gc, x)
+        assert g.get(index).shape == c.get(index).shape
+        assert_bits_equal(g.get(index).toArray(), c.get(index).toArray(), f"get {index}")
+        v = np.full(c.get(index).shape, 0.5, dtype=np.float32)
+        gv, cv = both(gc, v)
+        g.set(index, gv); c.set(index, cv)
+        assert_bits_equal(g.toArray(), c.toArray(), f"set {index}")
+        g.set(index, 9.0); c.set(index, 9.0)
+        assert_bits_equal(g.toArray(), c.toArray(), f"fill {index}")
+
+
+def test_indexing_errors_match_the_reference(gc):
+    x = gc.createRaw([3, 4], np.zeros(12, dtype=np.float32))
+    for bad in ([(0, 4)], [(2, 1)], [(0, 0), (0, 0), (0, 0)], [(-5, 0)]):
+        with pytest.raises(ValueError):
+            x.get(bad)
+        with pytest.raises(ValueError):
+            x.set(bad, 1.0)
+    with pytest.raises(ValueError):
+        x.get([3])
+    with pytest.raises(ValueError):
+        x.set([(0, 1), (0, 1)], gc.createRaw([3], [1.0, 2.0, 3.0]))          # JVM:295-296 element count
+    with pytest.raises(ValueError):
+        x.set([1], gc.createRaw([3], [1.0, 2.0, 3.0]))                       # JVM:284-285
+    x.set([(0, 1), (0, 1)], gc.createRaw([4], [1.0, 2.0, 3.0, 4.0]))         # only the count matters
+    assert x.toArray()[:2, :2].reshape(-1).tolist() == [1.0, 2.0, 3.0, 4.0]
+    with pytest.raises(ValueError):
+        x.narrow(1, 3, 2)
+    with pytest.raises(ValueError):
+        x.transpose(1, -1)
+    with pytest.raises(ValueError):
+        x.permute([0, 0])
+    with pytest.raises(ValueError):
+        x.permute([0, 1, 2])
+    with pytest.raises(ValueError):
+        x.maskedFill(gc.createRaw([3], [1.0, 0.0, 1.0]), 0.0)
+    with pytest.raises(ValueError):
+        gc.concat(0, [x, gc.createRaw([3, 5], np.zeros(15, dtype=np.float32))])
+
+
+TRANSPOSE_SHAPES = [[2, 3], [64, 64], [65, 63], [1, 7], [130, 257], [3, 5, 7], [2, 64, 128], [4, 3, 66, 70], [2, 3, 4, 5, 6],
+                    [3, 1, 129], [1000, 3], [3, 1000]]
+
+
+@pytest.mark.parametrize("shape", TRANSPOSE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_transpose_every_axis_pair(shape, gc):
+    x = np.random.default_rng(len(shape) + shape[-1]).standard_normal(shape).astype(np.float32)
+    g, c = both(gc, x)
+    for a1, a2 in itertools.permutations(range(len(shape)), 2):
+        got = g.transpose(a1, a2)
+        assert got.shape == list(np.swapaxes(x, a1, a2).shape)
+        assert_bits_equal(got.toArray(), np.swapaxes(x, a1, a2), f"transpose({a1},{a2}) vs the axis swap")
+        lo, hi = min(a1, a2), max(a1, a2)
+        if all(s == 1 for s in shape[lo + 1:hi]):
+            # where kten-jvm's slab copy is the axis swap, the device equals the restatement of kten-jvm
+            assert_bits_equal(got.toArray(), c.transpose(a1, a2).toArray(), f"transpose({a1},{a2}) vs kten-jvm")
+    assert_bits_equal(g.transpose(-1, 0).toArray(), np.swapaxes(x, -1, 0), "negative axis")
+
+
+PERMUTE_SHAPES = [[2, 3, 2], [5, 6, 7], [8, 64, 68], [2, 3, 4, 5], [3, 4, 64, 65], [4, 16, 20, 24], [2, 2, 3, 3, 4, 4],
+                  [128, 3], [6, 1, 5, 1]]
+
+
+@pytest.mark.parametrize("shape", PERMUTE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_permute_parity(shape, gc):
+    x = np.random.default_rng(shape[0] * 31 + len(shape)).standard_normal(shape).astype(np.float32)
+    g, c = both(gc, x)
+    perms = list(itertools.permutations(range(len(shape))))
+    if len(perms) > 40:
+        perms = [perms[i] for i in np.random.default_rng(1).choice(len(perms), 40, replace=False)]
+    for axes in perms:
+        got, want = g.permute(list(axes)), c.permute(list(axes))
+        assert got.shape == want.shape
+        assert_bits_equal(got.toArray(), want.toArray(), f"permute{axes}")
+
+
+def test_masked_fill_parity(gc):
+    rng = np.random.default_rng(3)
+    for shape, mshape in (([4, 5, 6], [5, 1]), ([4, 5, 6], [1]), ([4, 5, 8], [4, 5, 8]), ([32, 16, 8, 8], [16, 1, 1]),
+                          ([1000, 7], [1000, 1]), ([128, 256], [256]), ([9], [9])):
+        x = rng.standard_normal(shape).astype(np.float32)
+        x.reshape(-1)[::7] = np.nan
+        m = rng.choice(np.array([0.0, 1.0, 0.99999994, 2.0, np.nan, -1.0], dtype=np.float32), size=mshape)
+        g, c = both(gc, x); gm, cm = both(gc, m)
+        for value in (0.0, -2.5, float("inf")):
+            assert_bits_equal(g.maskedFill(gm, value).toArray(), c.maskedFill(cm, value).toArray(), f"maskedFill {shape} {mshape}")
+        assert_bits_equal(g.toArray(), x, "maskedFill must not touch its receiver")
+
+
+def test_concat_and_narrow_parity(gc):
+    rng = np.random.default_rng(4)
+    cpu = jo.JvmOracleOperations()
+    for shape, axis, sizes in (([3, 4], 0, [1, 2, 3]), ([3, 4], 1, [4, 1]), ([2, 3, 8], -2, [2, 5]), ([5], 0, [1, 1, 7]),
+                               ([16, 8, 32], 1, [8, 24, 4]), ([4, 6, 10], 2, [3, 9])):
+        parts = []
+        for s in sizes:
+            sh = list(shape); sh[axis] = s
+            parts.append(rng.standard_normal(sh).astype(np.float32))
+        got = gc.concat(axis, [gc.createRaw(list(p.shape), p) for p in parts])
+        want = cpu.concat(axis, [cpu.createRaw(list(p.shape), p.reshape(-1)) for p in parts])
+        assert got.shape == want.shape
+        assert_bits_equal(got.toArray(), want.toArray(), f"concat {shape} axis {axis}")
+        end = 0
+        for p, s in zip(parts, sizes):
+            assert_bits_equal(got.narrow(axis, end, s).toArray(), p, f"narrow {end}+{s}")
+            end += s
+
+
+def test_large_properties(gc):
+    """At sizes the CPU checker would take long for: a transpose applied twice, a permute
+    followed by its inverse and a narrow / concat round trip return the input bits, and a row
+    of a transpose is a column of the input."""
+    from kten_amd import inputs
+    n = 4096
+    x = inputs.SplitMix64(5).uniform([n, n], -1.0, 1.0)
+    g = gc.createRaw([n, n], x)
+    t = g.transpose(0, 1)
+    assert_bits_equal(t.transpose(0, 1).toArray(), x, "transpose twice")
+    assert_bits_equal(t.get([(17, 17), ALL]).toArray().reshape(-1), x[:, 17], "row of the transpose = column of the input")
+    y = inputs.SplitMix64(6).uniform([16, 64, 56, 56], -1.0, 1.0)
+    gy = gc.createRaw([16, 64, 56, 56], y)
+    nhwc = gy.permute([0, 2, 3, 1])
+    assert nhwc.shape == [16, 56, 56, 64]
+    assert_bits_equal(nhwc.get([(3, 3), (5, 5), (7, 7), ALL]).toArray().reshape(-1), y[3, :, 5, 7], "NHWC pixel = NCHW channel column")
+    assert_bits_equal(nhwc.permute([0, 3, 1, 2]).toArray(), y, "permute then its inverse")
+    halves = [gy.narrow(1, 0, 24), gy.narrow(1, 24, 40)]
+    assert_bits_equal(gc.concat(1, halves).toArray(), y, "narrow then concat")
