@@ -94,7 +94,7 @@ def cpu_baseline(name, threads):
     wl = WORKLOADS[name]
     sample = {"cfg1": dict(wl.full_dims), "cfg2": dict(wl.full_dims), "cfg3": dict(wl.full_dims),
               "cfg4": dict(wl.full_dims), "cfg5": {"rows": 8192, "cols": 4096},
-              "max_backward": dict(wl.full_dims), "softmax_ce": {"batch": 8192, "classes": 2048}}[name]
+              "max_backward": dict(wl.full_dims), "softmax_ce": {"batch": 8192, "classes": 2048}}.get(name, dict(wl.full_dims))
     inputs = wl.make_inputs(sample)
     jo.set_threads(threads)
     try:
@@ -117,7 +117,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="cfg5",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce"])
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce", "transpose", "permute",
+                             "concat_mask"])
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,

@@ -184,7 +184,68 @@ def _bytes_sce(d):
     return 4 * (24 * n + 16 * b + 2)
 
 
+# ---- layout movers -------------------------------------------------------------------------
+
+def _in_tr(d):
+    return {"x": SplitMix64(7).uniform([d["rows"], d["cols"]], -1.0, 1.0)}
+
+
+def _run_tr(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    return {"xt": x.transpose(0, 1)}
+
+
+def _bytes_tr(d):
+    return 4 * 2 * d["rows"] * d["cols"]
+
+
+def _in_perm(d):
+    return {"x": SplitMix64(8).uniform([d["n"], d["c"], d["h"], d["w"]], -1.0, 1.0)}
+
+
+def _run_perm(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    nhwc = x.permute(0, 2, 3, 1)
+    return {"nhwc": nhwc, "back": nhwc.permute(0, 3, 1, 2)}
+
+
+def _bytes_perm(d):
+    return 4 * 4 * d["n"] * d["c"] * d["h"] * d["w"]
+
+
+def _in_cat(d):
+    g = SplitMix64(9)
+    return {"a": g.uniform([d["rows"], d["left"]], -1.0, 1.0), "b": g.uniform([d["rows"], d["right"]], -1.0, 1.0),
+            "mask": (g.uniform([d["left"] + d["right"]], 0.0, 1.0) < 0.25).astype(np.float32)}
+
+
+def _run_cat(ops, inp):
+    from .autograd import concat
+    from .shape_functions import ALL
+    a = ops.create(list(inp["a"].shape), False, inp["a"])
+    b = ops.create(list(inp["b"].shape), False, inp["b"])
+    mask = ops.create(list(inp["mask"].shape), False, inp["mask"])
+    cat = concat(a, b, axis=1)
+    masked = cat.maskedFill(mask, 0.0)
+    right = masked[ALL, (inp["a"].shape[1], -1)]
+    masked[(0, -1), (0, inp["a"].shape[1] - 1)] = 1.0
+    return {"cat": cat, "masked": masked, "right": right}
+
+
+def _bytes_cat(d):
+    n, la, lb = d["rows"] * (d["left"] + d["right"]), d["rows"] * d["left"], d["rows"] * d["right"]
+    # concat: two range sets (2 la + 2 lb); maskedFill (2 n + mask); range get (2 lb); range fill (la)
+    return 4 * (2 * n + 2 * n + (d["left"] + d["right"]) + 2 * lb + la)
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "transpose": Workload("transpose", "x.transpose(0, 1): x[8192,8192], U(-1,1), seed 7", {"rows": 8192, "cols": 8192},
+                          _in_tr, _run_tr, _bytes_tr),
+    "permute": Workload("permute", "x.permute(0,2,3,1) then .permute(0,3,1,2): NCHW [64,128,56,56] to NHWC and back, seed 8",
+                        {"n": 64, "c": 128, "h": 56, "w": 56}, _in_perm, _run_perm, _bytes_perm),
+    "concat_mask": Workload("concat_mask", "concat([8192,4096],[8192,4096], axis=1); maskedFill(mask[8192], 0); range get "
+                                           "of the right half; range fill of the left half; seed 9",
+                            {"rows": 8192, "left": 4096, "right": 4096}, _in_cat, _run_cat, _bytes_cat),
     "max_backward": Workload("max_backward", "x.max(-1).sum().backward(): x[8192,8192], N(0,1), seed 5 "
                                              "(max, argMax, zerosLike, inplaceScatter, gradient +=)",
                              {"rows": 8192, "cols": 8192}, _in_max, _run_max, _bytes_max),

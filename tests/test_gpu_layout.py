@@ -178,3 +178,39 @@ def test_large_properties(gc):
     assert_bits_equal(nhwc.permute([0, 3, 1, 2]).toArray(), y, "permute then its inverse")
     halves = [gy.narrow(1, 0, 24), gy.narrow(1, 24, 40)]
     assert_bits_equal(gc.concat(1, halves).toArray(), y, "narrow then concat")
+
+
+@pytest.mark.parametrize("name,dims", [("transpose", {"rows": 300, "cols": 520}), ("permute", {"n": 6, "c": 16, "h": 12, "w": 20}),
+                                       ("concat_mask", {"rows": 96, "left": 200, "right": 120})])
+def test_layout_workloads_small_against_the_checker(name, dims, gc):
+    from kten_amd.workloads import WORKLOADS
+    wl = WORKLOADS[name]
+    inputs = wl.make_inputs(dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inputs).items()}
+    want = {k: v.toArray() for k, v in wl.run(jo.JvmOracleOperations(), inputs).items()}
+    for k in want:
+        assert_bits_equal(got[k], want[k], f"{name}.{k}")
+
+
+def test_layout_workloads_full_size(gc):
+    """The benchmark shapes, against numpy's own movers (independent of both the device code
+    and the checker)."""
+    from kten_amd.workloads import WORKLOADS
+    wl = WORKLOADS["transpose"]
+    inp = wl.make_inputs(wl.full_dims)
+    assert_bits_equal(wl.run(gc, inp)["xt"].toArray(), inp["x"].T, "transpose")
+    wl = WORKLOADS["permute"]
+    inp = wl.make_inputs(wl.full_dims)
+    out = wl.run(gc, inp)
+    assert_bits_equal(out["nhwc"].toArray(), np.transpose(inp["x"], (0, 2, 3, 1)), "NCHW -> NHWC")
+    assert_bits_equal(out["back"].toArray(), inp["x"], "and back")
+    wl = WORKLOADS["concat_mask"]
+    inp = wl.make_inputs(wl.full_dims)
+    out = wl.run(gc, inp)
+    cat = np.concatenate([inp["a"], inp["b"]], axis=1)
+    masked = np.where(inp["mask"] == 1.0, np.float32(0.0), cat)
+    left = inp["a"].shape[1]
+    assert_bits_equal(out["cat"].toArray(), cat, "concat")
+    assert_bits_equal(out["right"].toArray(), masked[:, left:], "range get")
+    masked[:, :left] = 1.0
+    assert_bits_equal(out["masked"].toArray(), masked, "maskedFill then range fill")

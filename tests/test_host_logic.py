@@ -206,6 +206,12 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
     wrap("_scatter", lambda s, a, r: size(a[1]) * (2 if isinstance(a[2], float) else 4 if a[3] else 3))
     wrap("inplaceFill", lambda s, a, r: size(s))
     wrap("copy", lambda s, a, r: 0 if (a and a[0]) else 2 * size(s))        # deep copies only
+    box = lambda first, last: int(np.prod([l - f + 1 for f, l in zip(first, last)]))
+    wrap("_get_ranges", lambda s, a, r: 2 * size(r))
+    wrap("_set_ranges", lambda s, a, r: box(a[0], a[1]) * (1 if isinstance(a[2], float) else 2))
+    wrap("_transpose", lambda s, a, r: 2 * size(s))
+    wrap("_permute", lambda s, a, r: 2 * size(s))
+    wrap("maskedFill", lambda s, a, r: 2 * size(s) + size(a[0]))
     orig_create = type(oracle_ops).createRaw
     def counting_create(self, shape, init=None):
         if callable(init):                      # the [1] seed gradient of backward(): one store
@@ -230,7 +236,9 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
     try:
         small = {"cfg1": {"rows": 8, "cols": 12}, "cfg2": {"n": 100}, "cfg3": {"rows": 6, "cols": 10},
                  "cfg4": {"n": 2, "c": 3, "h": 4, "w": 5}, "cfg5": {"rows": 8, "cols": 12},
-                 "max_backward": {"rows": 6, "cols": 10}, "softmax_ce": {"batch": 6, "classes": 10}}
+                 "max_backward": {"rows": 6, "cols": 10}, "softmax_ce": {"batch": 6, "classes": 10},
+                 "transpose": {"rows": 6, "cols": 10}, "permute": {"n": 2, "c": 3, "h": 4, "w": 5},
+                 "concat_mask": {"rows": 6, "left": 4, "right": 8}}
         for name, dims in small.items():
             wl = WORKLOADS[name]
             counted[0] = 0
