@@ -241,6 +241,30 @@ int kth_permute(uint64_t in, const int32_t* shape, int dims, const int32_t* axes
 int kth_masked_fill(uint64_t a, const int32_t* ashape, int adims, uint64_t mask, const int32_t* mshape, int mdims,
                     float value, uint64_t out);
 
+/* ------------------------------------------------------------------ fused batch normalisation */
+
+/* BatchNormOperation.calculateOutput (kten-api/.../tensor/operations/nn/BatchNormOperation.kt:7-13,
+ * obtained from TensorOperations.batchNorm(axis, momentum, epsilon, training),
+ * kten-api/.../tensor/operations/TensorOperations.kt:129; arithmetic of
+ * backend/kten-jvm/.../operations/nn/JVMBatchNorm.kt:33-99). `in` has `shape`; every
+ * per-channel tensor holds shape[axis] floats. running_mean and running_var are both given
+ * or both 0 (a handle is never 0); they are required when training == 0 and are updated in
+ * place when training != 0. gamma and beta may be 0 (1 and 0). Outputs: out (same shape),
+ * current_mean and current_std = 1 / sqrt(var + epsilon) per channel (zeros in inference
+ * mode, as the reference leaves them). */
+int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis, int training, float momentum, float epsilon,
+                           uint64_t running_mean, uint64_t running_var, uint64_t gamma, uint64_t beta,
+                           uint64_t out, uint64_t current_mean, uint64_t current_std);
+
+/* BatchNormOperation.calculateGrads (BatchNormOperation.kt:15-26; JVMBatchNorm.kt:101-183).
+ * grad_in, grad_gamma, grad_beta are outputs; 0 means "not required" (the reference's
+ * inRequiresGrad / gammaRequiresGrad / betaRequiresGrad flags). Training mode reads
+ * current_mean / current_std as returned by the forward call, inference mode reads
+ * running_mean / running_var. */
+int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axis, int training, float epsilon,
+                            uint64_t running_mean, uint64_t running_var, uint64_t current_mean, uint64_t current_std,
+                            uint64_t gamma, uint64_t grad_out, uint64_t grad_in, uint64_t grad_gamma, uint64_t grad_beta);
+
 /* ------------------------------------------------------------------ control and metrics */
 
 /* Wait for everything launched so far. */

@@ -18,6 +18,7 @@
 #pragma once
 
 #include <algorithm>
+#include <climits>
 #include <cstdint>
 #include <functional>
 #include <memory>
@@ -120,6 +121,64 @@ inline Shape unsqueezeShape(const Shape& s, int axis) {            // ShapeFunct
     return res;
 }
 
+/// A Kotlin `first..last` range, both ends inclusive; `All` stands for the reference's `all`
+/// (kten-api/.../tensor/Constants.kt:7).
+struct IntRange {
+    int first, last;
+    bool operator==(const IntRange& o) const { return first == o.first && last == o.last; }
+};
+inline constexpr IntRange All{INT32_MIN, INT32_MAX};
+
+inline std::vector<int> normalizeIndex(const Shape& s, const std::vector<int>& index) {   // ShapeFunctions.kt:217-230
+    if (index.size() > s.size()) throw std::invalid_argument("Cannot index tensor with shape: " + to_string(s));
+    std::vector<int> out;
+    for (size_t d = 0; d < index.size(); d++) {
+        const int i = index[d] < 0 ? s[d] + index[d] : index[d];
+        if (i < 0 || i >= s[d]) throw std::invalid_argument("Cannot index tensor with shape: " + to_string(s));
+        out.push_back(i);
+    }
+    return out;
+}
+
+inline std::vector<IntRange> normalizeIndex(const Shape& s, const std::vector<IntRange>& index) {   // ShapeFunctions.kt:240-259
+    bool invalid = index.size() > s.size();
+    std::vector<IntRange> out;
+    for (size_t d = 0; d < index.size() && d < s.size(); d++) {
+        IntRange r = index[d];
+        if (r == All) r = IntRange{0, s[d] - 1};
+        else if (r.first < 0 || r.last < 0) r = IntRange{r.first < 0 ? s[d] + r.first : r.first, r.last < 0 ? s[d] + r.last : r.last};
+        if (r.first < 0 || r.last < 0 || r.first >= s[d] || r.last >= s[d] || r.first > r.last) invalid = true;
+        out.push_back(r);
+    }
+    if (invalid) throw std::invalid_argument("Cannot index tensor with shape: " + to_string(s) + " with the given ranges");
+    return out;
+}
+
+inline Shape permuteShape(const Shape& s, const std::vector<int>& axes) {                 // ShapeFunctions.kt:106-113
+    bool ok = s.size() == axes.size();
+    for (size_t d = 0; ok && d < s.size(); d++) ok = std::find(axes.begin(), axes.end(), static_cast<int>(d)) != axes.end();
+    if (!ok) throw std::invalid_argument("Tensor with shape: " + to_string(s) + " cannot be permuted by the given axes. All dimensions must be indexed.");
+    Shape out;
+    for (int a : axes) out.push_back(s[a]);
+    return out;
+}
+
+inline Shape concatShapes(const std::vector<Shape>& shapes, int axis) {                   // ShapeFunctions.kt:85-104
+    bool ok = !shapes.empty();
+    for (const Shape& sh : shapes) ok = ok && sh.size() == shapes[0].size();
+    if (ok) {
+        const int a = normalizeAxis(shapes[0], axis);
+        int total = 0;
+        for (const Shape& sh : shapes) {
+            for (size_t d = 0; d < sh.size(); d++) ok = ok && (static_cast<int>(d) == a || sh[d] == shapes[0][d]);
+            total += sh[a];
+        }
+        if (ok) { Shape res = shapes[0]; res[a] = total; return res; }
+    }
+    throw std::invalid_argument("Cannot concatenate tensors at axis: " + std::to_string(axis) + " (All tensors must have the same number of "
+                                "dimenisons, and have the same size at all dimenions except at the dimension indexed by the axis)");
+}
+
 enum class AggregatingOperation { SUM = KTH_SUM, MEAN = KTH_MEAN, MAX = KTH_MAX, MIN = KTH_MIN,
                                   ARG_MAX = KTH_ARG_MAX, ARG_MIN = KTH_ARG_MIN };   // AggregatingOperation.kt:3-5
 
@@ -152,6 +211,7 @@ public:
     Raw zerosLike(const Raw& t);                                    // :24
     void zeroOut(const Raw& t);                                     // :26
     Raw pow(float constant, const Raw& t);                          // :39
+    Raw concat(int axis, const std::vector<Raw>& inputs);           // :41
     void release(const Raw& t);                                     // :22
     void incrementRef(const Raw& t);                                // :28
     void markSurviveGC(const Raw& t);                               // :30-33 / OCLTensorOperations.kt:96-98
@@ -305,6 +365,85 @@ public:
     }
     Raw scatter(int axis, const Raw& index, const Raw& src) { Raw res = copy(); res->inplaceScatter(axis, index, src); return res; }
 
+    // --- get / set by index and by ranges (AbstractRawTensor.kt:27-37; JVMRawTensor.kt:270-315)
+    Raw get(const std::vector<int>& index) {
+        live();
+        const std::vector<int> norm = normalizeIndex(shape, index);
+        int64_t offset, length;
+        storeRange(norm, offset, length);
+        Raw res = ops->createRaw(norm.size() == shape.size() ? Shape{1} : Shape(shape.begin() + norm.size(), shape.end()));
+        check(kth_copy(res->storeReference, 0, storeReference, static_cast<uint64_t>(offset), static_cast<uint64_t>(length)));
+        return res;
+    }
+    Raw get(const std::vector<IntRange>& index) {
+        live();
+        Shape first, last, resShape;
+        fullRanges(normalizeIndex(shape, index), first, last, resShape);
+        Raw res = ops->createRaw(resShape);
+        check(kth_get_range(storeReference, shape.data(), dimensions(), first.data(), last.data(), res->storeReference));
+        return res;
+    }
+    void set(const std::vector<int>& index, const Raw& value) {
+        live(); value->live();
+        int64_t offset, length;
+        storeRange(normalizeIndex(shape, index), offset, length);
+        if (value->size() != length)
+            throw std::invalid_argument("Cannot set tensor with shape: " + to_string(value->shape) + " to tensor with shape: " + to_string(shape));
+        check(kth_copy(storeReference, static_cast<uint64_t>(offset), value->storeReference, 0, static_cast<uint64_t>(length)));
+    }
+    void set(const std::vector<int>& index, float value) {
+        live();
+        int64_t offset, length;
+        storeRange(normalizeIndex(shape, index), offset, length);
+        check(kth_fill(storeReference, static_cast<uint64_t>(offset), static_cast<uint64_t>(length), value));
+    }
+    void set(const std::vector<IntRange>& index, const Raw& value) {
+        live(); value->live();
+        Shape first, last, resShape;
+        fullRanges(normalizeIndex(shape, index), first, last, resShape);
+        check(kth_set_range(storeReference, shape.data(), dimensions(), first.data(), last.data(), value->storeReference,
+                            static_cast<uint64_t>(value->size())));
+    }
+    void set(const std::vector<IntRange>& index, float value) {
+        live();
+        Shape first, last, resShape;
+        fullRanges(normalizeIndex(shape, index), first, last, resShape);
+        check(kth_fill_range(storeReference, shape.data(), dimensions(), first.data(), last.data(), value));
+    }
+
+    // --- transpose / permute / narrow / maskedFill (AbstractRawTensor.kt:228-232,246)
+    Raw transpose(int axis1, int axis2) {
+        live();
+        const int a1 = normalizeAxis(shape, axis1), a2 = normalizeAxis(shape, axis2);
+        if (a1 == a2) throw std::invalid_argument("Transpose requires different axes as parameters");
+        Shape res = shape;
+        std::swap(res[a1], res[a2]);
+        Raw out = ops->createRaw(res);
+        check(kth_transpose(storeReference, shape.data(), dimensions(), a1, a2, out->storeReference));
+        return out;
+    }
+    Raw permute(const std::vector<int>& axes) {
+        live();
+        Raw out = ops->createRaw(permuteShape(shape, axes));
+        check(kth_permute(storeReference, shape.data(), dimensions(), axes.data(), out->storeReference));
+        return out;
+    }
+    Raw narrow(int axis, int start, int length) {                    // JVMRawTensor.kt:468-473
+        const int a = normalizeAxis(shape, axis);
+        std::vector<IntRange> ranges;
+        for (int d : shape) ranges.push_back(IntRange{0, d - 1});
+        ranges[a] = IntRange{start, start + length - 1};
+        return get(ranges);
+    }
+    Raw maskedFill(const Raw& mask, float value) {                   // JVMRawTensor.kt:537-540
+        live(); mask->live();
+        if (mask->shape != shape) inferExplicitBroadcastShape(mask->shape, shape);
+        Raw out = ops->createRaw(shape);
+        check(kth_masked_fill(storeReference, shape.data(), dimensions(), mask->storeReference, mask->shape.data(),
+                              mask->dimensions(), value, out->storeReference));
+        return out;
+    }
+
     // --- shape-only members and copies (AbstractRawTensor.kt:77-90,124-144,168)
     Raw copy(bool shallow = false) {
         live();
@@ -352,6 +491,21 @@ public:
 private:
     HipRawTensor(const Shape& s, uint64_t handle, HipTensorOperations* o) : shape(s), storeReference(handle), ops(o) {}
     int refCount_ = 1;
+
+    void storeRange(const std::vector<int>& norm, int64_t& offset, int64_t& length) const {   // AbstractIndexing.kt:43-54
+        int64_t start = 0;
+        for (size_t d = 0; d < norm.size(); d++) start = start * shape[d] + norm[d];
+        length = 1;
+        for (size_t d = norm.size(); d < shape.size(); d++) length *= shape[d];
+        offset = start * length;
+    }
+    void fullRanges(const std::vector<IntRange>& norm, Shape& first, Shape& last, Shape& resShape) const {
+        for (size_t d = 0; d < shape.size(); d++) {
+            const IntRange r = d < norm.size() ? norm[d] : IntRange{0, shape[d] - 1};
+            first.push_back(r.first); last.push_back(r.last);
+            resShape.push_back(r.last - r.first + 1);
+        }
+    }
 
     void live() const { if (refCount_ <= 0) throw std::runtime_error("Raw tensor with shape " + to_string(shape) + " was released"); }
 
@@ -452,6 +606,22 @@ inline Raw HipTensorOperations::createRawFill(const Shape& shape, float constant
 inline Raw HipTensorOperations::zerosLike(const Raw& t) { return createRawFill(t->shape, 0.0f); }
 inline void HipTensorOperations::zeroOut(const Raw& t) { t->inplaceFill(0.0f); }
 inline Raw HipTensorOperations::pow(float constant, const Raw& t) { return t->scalar(KTH_POW, constant, true); }
+inline Raw HipTensorOperations::concat(int axis, const std::vector<Raw>& inputs) {   // AbstractJVMTensorOperations.kt:106-120
+    std::vector<Shape> shapes;
+    for (const Raw& t : inputs) shapes.push_back(t->shape);
+    const Shape resShape = concatShapes(shapes, axis);
+    const int a = normalizeAxis(shapes[0], axis);
+    std::vector<IntRange> target;
+    for (int d : resShape) target.push_back(IntRange{0, d - 1});
+    Raw res = createRaw(resShape);
+    int last = 0;
+    for (const Raw& t : inputs) {
+        target[a] = IntRange{last, last + t->shape[a] - 1};
+        res->set(target, t);
+        last += t->shape[a];
+    }
+    return res;
+}
 inline void HipTensorOperations::release(const Raw& t) { t->release(); }
 inline void HipTensorOperations::incrementRef(const Raw& t) { t->incrementRef(); }
 inline void HipTensorOperations::markSurviveGC(const Raw& t) { t->mustSurviveGC = true; }

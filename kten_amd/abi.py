@@ -64,6 +64,10 @@ SIGNATURES = {
     "kth_transpose": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_int, c_uint64]),
     "kth_permute": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), c_uint64]),
     "kth_masked_fill": (c_int, [c_uint64, POINTER(c_int32), c_int, c_uint64, POINTER(c_int32), c_int, c_float, c_uint64]),
+    "kth_batch_norm_forward": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_int, c_float, c_float,
+                                       c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
+    "kth_batch_norm_backward": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_int, c_float,
+                                        c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
     "kth_sync": (c_int, []),
     "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
     "kth_timer_begin": (c_int, []),

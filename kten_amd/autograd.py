@@ -184,6 +184,19 @@ class AGTensor(Tensor):
     def gather(self, axis, index): return Gather(self.ops)(self, axis, index)
     def scatter(self, axis, index, source): return Scatter(self.ops)(self, axis, index, source)
 
+    def batchNorm(self, axis, runningMean, runningVar, training, momentum=0.1, epsilon=1e-5, gamma=None, beta=None):
+        """functions/nn/TensorExtensions.kt: Tensor.batchNorm."""
+        return BatchNormalizationFunction(axis, momentum, epsilon, training, self.ops)(self, runningMean, runningVar, gamma, beta)
+
+    def meanVariance(self, axis, keepDimensions=False, unbiased=True):
+        """AGTensor.kt:454-461."""
+        tensor = _safe(self)
+        mean = tensor.mean(axis, True)
+        elements = tensor.shape[sf.normalize_axis(tensor.shape, axis)] - (1 if unbiased else 0)
+        zeroCentered = tensor - mean
+        variance = (zeroCentered ** 2.0).sum(axis, keepDimensions) / float(elements)
+        return mean, variance
+
     def softmaxCrossEntropy(self, targets):
         """functions/nn/TensorExtensions.kt: logits.softmaxCrossEntropy(targets)."""
         return SoftmaxCrossEntropy(self.ops)(self, targets)
@@ -218,6 +231,7 @@ class AGTensor(Tensor):
     def rsqrt(self): return Rsqrt(self.ops)(self)
     def _reshape(self, newShape): return Reshape(self.ops)(self, newShape)
     def _expand(self, newShape): return Expand(self.ops)(self, newShape)
+    def view(self, *newShape): return Reshape(self.ops, viewMode=True)(self, _as_list(newShape))   # AGTensor.kt:473-475
 
     def noGrad(self):
         """AGTensor.kt:531-535."""
@@ -949,6 +963,10 @@ class Min(SelectionFunction):                                                   
 class Reshape(UnaryTensorFunction):                                                   # :200-231
     modifiesShape = True
 
+    def __init__(self, ops, viewMode=False):
+        super().__init__(ops)
+        self.viewMode = viewMode
+
     def __call__(self, tensor, newShape):
         self.cachedShape = sf.reshape(tensor.shape, newShape)
         super().__call__(tensor)
@@ -957,10 +975,10 @@ class Reshape(UnaryTensorFunction):                                             
 
     def doForward(self, input):
         self.oldShape = list(input.shape)
-        self.output = input.reshape(self.newShape)
+        self.output = input.view(self.newShape) if self.viewMode else input.reshape(self.newShape)
 
     def doBackward(self, gradient):
-        return [gradient.reshape(self.oldShape)]
+        return [gradient.view(self.oldShape) if self.viewMode else gradient.reshape(self.oldShape)]
 
 
 class Expand(UnaryTensorFunction):                                                    # :233-284
@@ -1243,6 +1261,78 @@ class MaskedFill(UnaryTensorFunction):                                          
 
     def doBackward(self, gradient):
         return [gradient.maskedFill(self.mask, 0.0)]
+
+
+class BatchNormalizationFunction(Function):
+    """functions/nn/BatchNormalizationFunction.kt:12-150 — one raw call forward
+    (calculateOutput) and one backward (calculateGrads); running statistics are updated in
+    place by the forward call in training mode."""
+
+    def __init__(self, axis, momentum, epsilon, training, ops):
+        super().__init__(ops)
+        self.axis, self.momentum, self.epsilon, self.training = axis, float(momentum), float(epsilon), bool(training)
+        self.runningMean = self.runningVar = self.gamma = self.beta = None
+
+    def __call__(self, input, runningMean, runningVar, gamma, beta):
+        self.input = _safe(input)
+        if runningMean is not None and runningVar is None:
+            raise ValueError("Running mean and running var must be both set to non-null or both has to be null")
+        if runningMean is None and runningVar is None and not self.training:
+            raise ValueError("Running mean and running var must be non-null for inference mode")
+        if runningMean is not None:
+            if not isinstance(runningMean, NoGradVariable) or not isinstance(runningVar, NoGradVariable):
+                raise ValueError("Running mean and running var parameters for batch normalization must be variables "
+                                 "requiring no gradients")
+            self.runningMean, self.runningVar = runningMean, runningVar
+            runningMean.incrementRef(); runningVar.incrementRef()
+        self.gamma = _safe(gamma) if gamma is not None else None
+        self.beta = _safe(beta) if beta is not None else None
+        normAxis = sf.normalize_axis(input.shape, self.axis)
+        self.keepOutput = True
+        size = self.input.shape[normAxis]
+        if runningMean is not None and runningVar is not None:
+            if (runningMean.dimensions != 1 or runningVar.dimensions != 1
+                    or (self.gamma.dimensions if self.gamma is not None else 1) != 1
+                    or (self.beta.dimensions if self.beta is not None else 1) != 1
+                    or runningMean.shape[0] != size or runningVar.shape[0] != size):
+                raise ValueError("Running mean and running var parameters for batch normalization all must have "
+                                 f"shape: [{size}], but got tensors with shapes: running mean: {runningMean.shape} "
+                                 f"running var: {runningVar.shape} ")
+        if ((self.gamma.shape[0] if self.gamma is not None else size) != size
+                or (self.beta.shape[0] if self.beta is not None else size) != size):
+            raise ValueError(f"Gamma and beta parameters for batch normalization all must have shape: [{size}]")
+        self.batchNormOp = self.ops.batchNorm(normAxis, self.momentum, self.epsilon, self.training)
+        self.cachedShape = list(input.shape)
+        return self
+
+    def getInputsAsList(self):
+        return [t for t in (self.input, self.gamma, self.beta) if t is not None]
+
+    def internalForward(self):
+        super().internalForward()
+        if self.hasValue():
+            return
+        fns = [t for t in (self.input, self.runningMean, self.runningVar, self.gamma, self.beta) if isinstance(t, Function)]
+        for f in fns:
+            f.internalForward()
+        if not self.hasValue():
+            raw = lambda t: None if t is None else t.getRawValue()
+            output, currentMean, currentStd = self.batchNormOp.calculateOutput(
+                raw(self.input), raw(self.runningMean), raw(self.runningVar), raw(self.gamma), raw(self.beta))
+            self._saved = (raw(self.input), currentMean, currentStd, raw(self.runningMean), raw(self.runningVar), raw(self.gamma))
+            self.saveForBackward(*[v for v in self._saved if v is not None])
+            self.output = output
+        for f in fns:
+            f.mayFreeOutput()
+
+    def doBackward(self, gradient):
+        input, currentMean, currentStd, runningMean, runningVar, gamma = self._saved
+        if gradient.shape != input.shape:
+            raise RuntimeError(f"Gradient shape mismatch, output grad shape: {gradient.shape} input shape: {input.shape}")
+        return list(self.batchNormOp.calculateGrads(
+            input, runningMean, runningVar, currentMean, currentStd, gamma, gradient,
+            self.input.requiresGrad, self.gamma.requiresGrad if self.gamma is not None else False,
+            self.beta.requiresGrad if self.beta is not None else False))
 
 
 class SoftmaxCrossEntropy(UnaryTensorFunction):

@@ -1,0 +1,577 @@
+// Fused batch normalisation over one axis (reference:
+// kten-api/.../tensor/operations/nn/BatchNormOperation.kt:5-41 and
+// backend/kten-jvm/.../operations/nn/JVMBatchNorm.kt:33-183).
+//
+// The tensor is seen as [outer, channels, inner] around the axis. Per channel the reference
+// makes serial float passes: sum -> mean, sum of squared deviations -> 1/sqrt(var + eps),
+// then the affine map; backward: sum of gradOut, dot of (x - mean) with gradOut, then the
+// input gradient. Here every pass over the data is one launch over all channels:
+//
+//   stats    one read of x (forward) or of x and gradOut (backward); two f64 sums per channel.
+//            Forward sums d = x - k and d*d for k = the channel's first element, exactly in
+//            f64; the sum of squared deviations from the rounded mean follows from them
+//            (S2 - 2 (mean - k) S1 + n (mean - k)^2). Because k is one of the channel's own
+//            elements the cancellation costs at most n * 2^-53 relative.
+//   finalize one thread per channel folds the partials in a fixed order and does the scalar
+//            float arithmetic of the reference (JVMBatchNorm.kt:57-82,128-137,150-152,
+//            171-177) in its order, writing the per-channel parameters.
+//   apply    one read (+ gradOut) and one write; the float expression of JVMBatchNorm.kt:88-90
+//            / :153-164, evaluated left to right without contraction, so given equal
+//            statistics the output bits equal the reference's.
+//
+// Sums accumulate in f64 in a fixed order: deterministic, and closer to the exact sums than
+// the reference's serial float accumulation.
+#include "kth_internal.h"
+
+using namespace kth;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kBatch = 4;          // loads in flight per thread in the stats kernels
+constexpr int kApplyUnroll = 2;
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct Geometry {
+    uint32_t outer, channels, inner;
+    uint32_t per_channel;           // outer * inner
+};
+
+// ---------------------------------------------------------------- block fold of two doubles
+
+__device__ __forceinline__ void block_fold2(double& a, double& b, double* lds) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_xor(a, off);
+        b += __shfl_xor(b, off);
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { lds[wave * 2] = a; lds[wave * 2 + 1] = b; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        a = lds[0]; b = lds[1];
+        for (int w = 1; w < kBlock / 64; w++) { a += lds[w * 2]; b += lds[w * 2 + 1]; }
+    }
+}
+
+// ---------------------------------------------------------------- stats, long runs (inner >= 64)
+
+// Work of one channel: outer runs of `inner` contiguous floats, cut into chunks of
+// kBlock * W floats (W = 4 with float4 loads); a workgroup takes the chunks
+// [seg * chunks_per_seg, (seg + 1) * chunks_per_seg) of channel blockIdx.x / segments.
+struct RunPlan {
+    Geometry g;
+    uint32_t segments, chunks_per_seg, total_chunks, chunks_per_run;
+    FastDiv  run_div, seg_div;
+};
+
+// BACKWARD false: (sum of d, sum of d*d), d = x - k. BACKWARD true: (sum of g, sum of (x - mean) g).
+template <bool BACKWARD, bool VEC>
+__global__ __launch_bounds__(kBlock) void bn_stats_runs_kernel(const float* __restrict__ x, const float* __restrict__ go,
+                                                              const float* __restrict__ mean, double* __restrict__ partial, RunPlan pl) {
+    __shared__ double lds[2 * kBlock / 64];
+    constexpr uint32_t W = VEC ? 4 : 1;
+    const uint32_t b = blockIdx.x;
+    const uint32_t c = (__umulhi(b, pl.seg_div.mul) + b) >> pl.seg_div.shift;
+    const uint32_t seg = b - c * pl.segments;
+    const uint32_t first = seg * pl.chunks_per_seg;
+    uint32_t last = first + pl.chunks_per_seg;
+    if (last > pl.total_chunks) last = pl.total_chunks;
+    const double shift = BACKWARD ? static_cast<double>(mean[c]) : static_cast<double>(x[static_cast<uint64_t>(c) * pl.g.inner]);
+    double s1 = 0.0, s2 = 0.0;
+    for (uint32_t q0 = first; q0 < last; q0 += kBatch) {
+        v4f vx[kBatch], vg[kBatch];
+        bool ok[kBatch];
+        uint32_t valid[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const uint32_t q = q0 + k;
+            ok[k] = q < last;
+            valid[k] = 0;
+            if (ok[k]) {
+                const uint32_t o = (__umulhi(q, pl.run_div.mul) + q) >> pl.run_div.shift;
+                const uint32_t off = (q - o * pl.chunks_per_run) * (kBlock * W) + threadIdx.x * W;
+                if (off < pl.g.inner) {
+                    const uint64_t at = (static_cast<uint64_t>(o) * pl.g.channels + c) * pl.g.inner + off;
+                    if (VEC) {
+                        valid[k] = 4;
+                        vx[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + at));
+                        if (BACKWARD) vg[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(go + at));
+                    } else {
+                        valid[k] = 1;
+                        vx[k].x = x[at];
+                        if (BACKWARD) vg[k].x = go[at];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            if (valid[k] == 0) continue;
+#pragma unroll
+            for (int e = 0; e < static_cast<int>(W); e++) {
+                const double d = static_cast<double>(vx[k][e]) - shift;
+                if (BACKWARD) { const double g = static_cast<double>(vg[k][e]); s1 += g; s2 += d * g; }
+                else { s1 += d; s2 += d * d; }
+            }
+        }
+    }
+    block_fold2(s1, s2, lds);
+    if (threadIdx.x == 0) {
+        partial[(static_cast<uint64_t>(c) * pl.segments + seg) * 2] = s1;
+        partial[(static_cast<uint64_t>(c) * pl.segments + seg) * 2 + 1] = s2;
+    }
+}
+
+// ---------------------------------------------------------------- stats, short runs (inner < 64)
+
+// The tensor as a matrix [outer, width = channels * inner]: a thread owns a column, the 4
+// waves of a workgroup take rows r = first + wave, first + wave + 4, ...; a wave's loads are
+// 256 contiguous bytes. Partials are per (segment, column).
+struct ColPlan {
+    Geometry g;
+    uint32_t width, col_blocks, segments, rows_per_seg;
+    FastDiv  col_div, inner_div;
+};
+
+template <bool BACKWARD>
+__global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __restrict__ x, const float* __restrict__ go,
+                                                              const float* __restrict__ mean, double* __restrict__ partial, ColPlan pl) {
+    __shared__ double lds[kBlock * 2];
+    const uint32_t b = blockIdx.x;
+    const uint32_t seg = (__umulhi(b, pl.col_div.mul) + b) >> pl.col_div.shift;
+    const uint32_t col = (b - seg * pl.col_blocks) * 64 + (threadIdx.x & 63);
+    const uint32_t lane_row = threadIdx.x >> 6;
+    double s1 = 0.0, s2 = 0.0;
+    if (col < pl.width) {
+        const uint32_t ch = (__umulhi(col, pl.inner_div.mul) + col) >> pl.inner_div.shift;
+        const double shift = BACKWARD ? static_cast<double>(mean[ch]) : static_cast<double>(x[static_cast<uint64_t>(ch) * pl.g.inner]);
+        const uint32_t first = seg * pl.rows_per_seg;
+        uint32_t last = first + pl.rows_per_seg;
+        if (last > pl.g.outer) last = pl.g.outer;
+        for (uint32_t r0 = first + lane_row; r0 < last; r0 += 4 * kBatch) {
+            float vx[kBatch], vg[kBatch];
+#pragma unroll
+            for (int k = 0; k < kBatch; k++) {
+                const uint32_t r = r0 + 4 * k;
+                if (r < last) {
+                    const uint64_t at = static_cast<uint64_t>(r) * pl.width + col;
+                    vx[k] = x[at];
+                    if (BACKWARD) vg[k] = go[at];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kBatch; k++) {
+                if (r0 + 4 * k < last) {
+                    const double d = static_cast<double>(vx[k]) - shift;
+                    if (BACKWARD) { const double g = static_cast<double>(vg[k]); s1 += g; s2 += d * g; }
+                    else { s1 += d; s2 += d * d; }
+                }
+            }
+        }
+    }
+    lds[threadIdx.x * 2] = s1;
+    lds[threadIdx.x * 2 + 1] = s2;
+    __syncthreads();
+    if (lane_row == 0 && col < pl.width) {
+        for (int w = 1; w < 4; w++) { s1 += lds[(threadIdx.x + 64 * w) * 2]; s2 += lds[(threadIdx.x + 64 * w) * 2 + 1]; }
+        partial[(static_cast<uint64_t>(seg) * pl.width + col) * 2] = s1;
+        partial[(static_cast<uint64_t>(seg) * pl.width + col) * 2 + 1] = s2;
+    }
+}
+
+// ---------------------------------------------------------------- finalize
+
+// Per-channel parameters for the apply kernels.
+struct ForwardParams { float mean, stdev, gamma, beta; };
+struct BackwardParams { float mean, stdev, gamma, dot_std_sq, grad_mean, pad0, pad1, pad2; };
+
+// Folds the partials of channel c in a fixed order. by_cols: partials are [segment][column].
+__device__ __forceinline__ void fold_partials(const double* partial, uint32_t c, uint32_t segments, bool by_cols,
+                                              uint32_t width, uint32_t inner, double& s1, double& s2) {
+    s1 = 0.0; s2 = 0.0;
+    if (by_cols) {
+        for (uint32_t s = 0; s < segments; s++)
+            for (uint32_t i = 0; i < inner; i++) {
+                const uint64_t at = (static_cast<uint64_t>(s) * width + static_cast<uint64_t>(c) * inner + i) * 2;
+                s1 += partial[at]; s2 += partial[at + 1];
+            }
+    } else {
+        for (uint32_t s = 0; s < segments; s++) {
+            const uint64_t at = (static_cast<uint64_t>(c) * segments + s) * 2;
+            s1 += partial[at]; s2 += partial[at + 1];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float* __restrict__ x, const double* __restrict__ partial,
+                                                                    Geometry g, uint32_t segments, int by_cols, int training,
+                                                                    float momentum, float epsilon, float* running_mean, float* running_var,
+                                                                    const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                                    float* __restrict__ current_mean, float* __restrict__ current_std,
+                                                                    ForwardParams* __restrict__ params) {
+    const uint32_t c = blockIdx.x * kBlock + threadIdx.x;
+    if (c >= g.channels) return;
+    float mean, stdev = 0.0f;
+    if (training) {
+        double s1, s2;
+        fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
+        const double n = static_cast<double>(g.per_channel);
+        const double k = static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]);
+        mean = static_cast<float>(k + s1 / n);                                  // JVMBatchNorm.kt:57-58
+        const double dm = static_cast<double>(mean) - k;
+        double ssd = s2 - 2.0 * dm * s1 + n * dm * dm;
+        if (ssd < 0.0) ssd = 0.0;
+        const float sum = static_cast<float>(ssd);                              // :60-64
+        const float count = static_cast<float>(g.per_channel);
+        if (sum != 0.0f || epsilon != 0.0f) stdev = 1.0f / sqrtf(sum / count + epsilon);   // :66-68
+        current_mean[c] = mean;
+        current_std[c] = stdev;
+        if (running_mean != nullptr && running_var != nullptr) {                // :72-76
+            running_mean[c] = (momentum * mean) + ((1.0f - momentum) * running_mean[c]);
+            const float unbiased = sum / static_cast<float>(g.per_channel - 1);
+            running_var[c] = (momentum * unbiased) + ((1.0f - momentum) * running_var[c]);
+        }
+    } else {                                                                    // :78-81
+        mean = running_mean[c];
+        stdev = 1.0f / sqrtf(running_var[c] + epsilon);
+        current_mean[c] = 0.0f;
+        current_std[c] = 0.0f;
+    }
+    ForwardParams p;
+    p.mean = mean; p.stdev = stdev;
+    p.gamma = gamma != nullptr ? gamma[c] : 1.0f;                               // :84-85
+    p.beta = beta != nullptr ? beta[c] : 0.0f;
+    params[c] = p;
+}
+
+__global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const double* __restrict__ partial, Geometry g, uint32_t segments,
+                                                                     int by_cols, int have_sums, int training, float epsilon,
+                                                                     const float* __restrict__ running_mean, const float* __restrict__ running_var,
+                                                                     const float* __restrict__ current_mean, const float* __restrict__ current_std,
+                                                                     const float* __restrict__ gamma, float* __restrict__ grad_gamma,
+                                                                     float* __restrict__ grad_beta, BackwardParams* __restrict__ params) {
+    const uint32_t c = blockIdx.x * kBlock + threadIdx.x;
+    if (c >= g.channels) return;
+    float mean, stdev;
+    if (training) { mean = current_mean[c]; stdev = current_std[c]; }           // JVMBatchNorm.kt:131-133
+    else {                                                                      // :134-137
+        mean = running_mean[c];
+        stdev = static_cast<float>(1.0 / sqrt(static_cast<double>(running_var[c] + epsilon)));
+    }
+    float sum = 0.0f, dot = 0.0f;
+    if (have_sums) {
+        double s1, s2;
+        fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
+        sum = static_cast<float>(s1);                                           // :139-147
+        dot = static_cast<float>(s2);
+    }
+    const float count = static_cast<float>(g.per_channel);
+    BackwardParams p;
+    p.mean = mean; p.stdev = stdev;
+    p.gamma = gamma != nullptr ? gamma[c] : 1.0f;
+    p.dot_std_sq = dot * stdev * stdev / count;                                 // :151
+    p.grad_mean = sum / count;                                                  // :152
+    p.pad0 = p.pad1 = p.pad2 = 0.0f;
+    params[c] = p;
+    if (grad_gamma != nullptr) grad_gamma[c] = dot * stdev;                     // :171-173
+    if (grad_beta != nullptr) grad_beta[c] = sum;                               // :175-177
+}
+
+// ---------------------------------------------------------------- apply
+
+struct ApplyPlan {
+    uint32_t units;                 // float4s (VEC) or floats
+    uint32_t channels;
+    FastDiv  inner_div, channel_div;   // inner counted in the kernel's units
+};
+
+__device__ __forceinline__ uint32_t channel_of(const ApplyPlan& pl, uint32_t i) {
+    const uint32_t q = (__umulhi(i, pl.inner_div.mul) + i) >> pl.inner_div.shift;
+    const uint32_t r = (__umulhi(q, pl.channel_div.mul) + q) >> pl.channel_div.shift;
+    return q - r * pl.channels;
+}
+
+__device__ __forceinline__ float bn_forward(float x, const ForwardParams& p) {
+    return (x - p.mean) * p.stdev * p.gamma + p.beta;                           // JVMBatchNorm.kt:88-90
+}
+__device__ __forceinline__ float bn_backward_training(float x, float go, const BackwardParams& p) {
+    const float base = (x - p.mean) * p.dot_std_sq;                             // :154-156
+    return (go - p.grad_mean - base) * p.stdev * p.gamma;
+}
+__device__ __forceinline__ float bn_backward_inference(float go, const BackwardParams& p) {
+    return go * p.stdev * p.gamma;                                              // :160-162
+}
+
+// MODE 0: forward. MODE 1: input gradient, training. MODE 2: input gradient, inference.
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float* __restrict__ x, const float* __restrict__ go, float* __restrict__ out,
+                                                         const ForwardParams* __restrict__ fparams,
+                                                         const BackwardParams* __restrict__ bparams, ApplyPlan pl) {
+    const uint32_t base = blockIdx.x * (kBlock * kApplyUnroll) + threadIdx.x;
+    if (VEC) {
+        v4f vx[kApplyUnroll], vg[kApplyUnroll];
+#pragma unroll
+        for (int k = 0; k < kApplyUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < pl.units) {
+                if (MODE != 2) vx[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x) + i);
+                if (MODE != 0) vg[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(go) + i);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kApplyUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < pl.units) {
+                const uint32_t c = channel_of(pl, i);
+                v4f r;
+                if (MODE == 0) {
+                    const ForwardParams p = fparams[c];
+                    r.x = bn_forward(vx[k].x, p); r.y = bn_forward(vx[k].y, p); r.z = bn_forward(vx[k].z, p); r.w = bn_forward(vx[k].w, p);
+                } else if (MODE == 1) {
+                    const BackwardParams p = bparams[c];
+                    r.x = bn_backward_training(vx[k].x, vg[k].x, p); r.y = bn_backward_training(vx[k].y, vg[k].y, p);
+                    r.z = bn_backward_training(vx[k].z, vg[k].z, p); r.w = bn_backward_training(vx[k].w, vg[k].w, p);
+                } else {
+                    const BackwardParams p = bparams[c];
+                    r.x = bn_backward_inference(vg[k].x, p); r.y = bn_backward_inference(vg[k].y, p);
+                    r.z = bn_backward_inference(vg[k].z, p); r.w = bn_backward_inference(vg[k].w, p);
+                }
+                reinterpret_cast<v4f*>(out)[i] = r;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kApplyUnroll; k++) {
+            const uint32_t i = base + k * kBlock;
+            if (i < pl.units) {
+                const uint32_t c = channel_of(pl, i);
+                if (MODE == 0) out[i] = bn_forward(x[i], fparams[c]);
+                else if (MODE == 1) out[i] = bn_backward_training(x[i], go[i], bparams[c]);
+                else out[i] = bn_backward_inference(go[i], bparams[c]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- host side
+
+int geometry_of(const char* what, const int32_t* shape, int dims, int axis, Geometry* g, uint64_t* n) {
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "%s: %d dims", what, dims);
+    if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
+    if (axis < 0 || axis >= dims) return fail(KTH_E_ARGUMENT, "%s: axis %d of %d dims", what, axis, dims);
+    uint64_t outer = 1, inner = 1;
+    for (int d = 0; d < dims; d++) {
+        if (shape[d] < 1) return fail(KTH_E_ARGUMENT, "%s: dim %d is %d", what, d, shape[d]);
+        if (d < axis) outer *= static_cast<uint64_t>(shape[d]);
+        if (d > axis) inner *= static_cast<uint64_t>(shape[d]);
+        if (outer * inner * static_cast<uint64_t>(shape[axis]) > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: more than 2^31-1 elements", what);
+    }
+    g->outer = static_cast<uint32_t>(outer);
+    g->channels = static_cast<uint32_t>(shape[axis]);
+    g->inner = static_cast<uint32_t>(inner);
+    g->per_channel = static_cast<uint32_t>(outer * inner);
+    *n = outer * inner * g->channels;
+    return KTH_OK;
+}
+
+// A per-channel operand: 0 means "not given"; otherwise it must hold `channels` floats.
+int channel_store(const char* what, uint64_t handle, uint32_t channels, float** ptr) {
+    *ptr = nullptr;
+    if (handle == 0) return KTH_OK;
+    Store* s = lookup(handle, what);
+    if (!s) return KTH_E_HANDLE;
+    if (s->n_floats < channels) return fail(KTH_E_SHAPE, "%s holds %llu values, the axis has %u", what,
+                                             static_cast<unsigned long long>(s->n_floats), channels);
+    *ptr = s->ptr;
+    return KTH_OK;
+}
+
+struct StatsLaunch {
+    bool     by_cols;
+    uint32_t segments;
+    uint64_t partial_doubles;
+    RunPlan  run;
+    ColPlan  col;
+    bool     vec;
+};
+
+StatsLaunch plan_stats(const Geometry& g) {
+    StatsLaunch st{};
+    const uint32_t target = static_cast<uint32_t>(state().compute_units > 0 ? state().compute_units : 256) * 8;
+    if (g.inner >= 64) {
+        st.by_cols = false;
+        st.vec = g.inner % 4 == 0;
+        const uint32_t chunk = kBlock * (st.vec ? 4 : 1);
+        RunPlan& p = st.run;
+        p.g = g;
+        p.chunks_per_run = (g.inner + chunk - 1) / chunk;
+        p.total_chunks = g.outer * p.chunks_per_run;
+        uint32_t segments = (target + g.channels - 1) / g.channels;
+        const uint32_t max_segments = (p.total_chunks + kBatch - 1) / kBatch;      // at least one batch of chunks each
+        if (segments > max_segments) segments = max_segments;
+        if (segments < 1) segments = 1;
+        p.chunks_per_seg = (p.total_chunks + segments - 1) / segments;
+        p.segments = (p.total_chunks + p.chunks_per_seg - 1) / p.chunks_per_seg;
+        p.run_div = make_div(p.chunks_per_run);
+        p.seg_div = make_div(p.segments);
+        st.segments = p.segments;
+        st.partial_doubles = static_cast<uint64_t>(g.channels) * p.segments * 2;
+    } else {
+        st.by_cols = true;
+        ColPlan& p = st.col;
+        p.g = g;
+        p.width = g.channels * g.inner;
+        p.col_blocks = (p.width + 63) / 64;
+        uint32_t segments = (target + p.col_blocks - 1) / p.col_blocks;
+        const uint32_t max_segments = (g.outer + 4 * kBatch - 1) / (4 * kBatch);
+        if (segments > max_segments) segments = max_segments;
+        if (segments < 1) segments = 1;
+        p.rows_per_seg = (g.outer + segments - 1) / segments;
+        p.segments = (g.outer + p.rows_per_seg - 1) / p.rows_per_seg;
+        p.col_div = make_div(p.col_blocks);
+        p.inner_div = make_div(g.inner);
+        st.segments = p.segments;
+        st.partial_doubles = static_cast<uint64_t>(p.segments) * p.width * 2;
+    }
+    return st;
+}
+
+template <bool BACKWARD>
+void launch_stats(const StatsLaunch& st, const float* x, const float* go, const float* mean, double* partial, uint64_t n) {
+    hipStream_t stream = state().stream;
+    const uint64_t bytes = (BACKWARD ? 2 : 1) * n * 4;
+    if (st.by_cols) {
+        LaunchScope scope("bn_stats_cols_kernel", BACKWARD ? "backward" : "forward", bytes);
+        hipLaunchKernelGGL((bn_stats_cols_kernel<BACKWARD>), dim3(st.col.col_blocks * st.col.segments), dim3(kBlock), 0, stream,
+                           x, go, mean, partial, st.col);
+    } else {
+        LaunchScope scope("bn_stats_runs_kernel", BACKWARD ? "backward" : "forward", bytes);
+        const dim3 grid(st.run.g.channels * st.run.segments);
+        if (st.vec) hipLaunchKernelGGL((bn_stats_runs_kernel<BACKWARD, true>), grid, dim3(kBlock), 0, stream, x, go, mean, partial, st.run);
+        else        hipLaunchKernelGGL((bn_stats_runs_kernel<BACKWARD, false>), grid, dim3(kBlock), 0, stream, x, go, mean, partial, st.run);
+    }
+}
+
+template <int MODE>
+void launch_apply(const Geometry& g, uint64_t n, const float* x, const float* go, float* out, const ForwardParams* fp, const BackwardParams* bp) {
+    ApplyPlan pl{};
+    const bool vec = g.inner % 4 == 0;
+    pl.units = static_cast<uint32_t>(vec ? n / 4 : n);
+    pl.channels = g.channels;
+    pl.inner_div = make_div(vec ? g.inner / 4 : g.inner);
+    pl.channel_div = make_div(g.channels);
+    const uint32_t per_block = kBlock * kApplyUnroll;
+    const dim3 grid((pl.units + per_block - 1) / per_block);
+    const uint64_t bytes = (MODE == 0 ? 2 : MODE == 1 ? 3 : 2) * n * 4;
+    LaunchScope scope("bn_apply_kernel", MODE == 0 ? "forward" : MODE == 1 ? "backward_training" : "backward_inference", bytes);
+    if (vec) hipLaunchKernelGGL((bn_apply_kernel<MODE, true>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
+    else     hipLaunchKernelGGL((bn_apply_kernel<MODE, false>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
+}
+
+uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
+
+}  // namespace
+
+extern "C" {
+
+int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis, int training, float momentum, float epsilon,
+                           uint64_t running_mean, uint64_t running_var, uint64_t gamma, uint64_t beta,
+                           uint64_t out, uint64_t current_mean, uint64_t current_std) {
+    std::lock_guard<std::mutex> guard(lock());
+    KTH_REQUIRE_INIT();
+    Geometry g; uint64_t n;
+    if (int rc = geometry_of("kth_batch_norm_forward", shape, dims, axis, &g, &n)) return rc;
+    if ((running_mean == 0) != (running_var == 0))
+        return fail(KTH_E_ARGUMENT, "Running mean and running var must be both set or both absent");
+    if (!training && running_mean == 0)
+        return fail(KTH_E_ARGUMENT, "Running mean and running var must be given for inference mode");
+    Store* si = lookup(in, "kth_batch_norm_forward(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_batch_norm_forward(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (n > si->n_floats || n > so->n_floats) return fail(KTH_E_ARGUMENT, "kth_batch_norm_forward: the shape needs more elements than a store holds");
+    float *rm, *rv, *ga, *be, *cm, *cs;
+    if (int rc = channel_store("kth_batch_norm_forward(running_mean)", running_mean, g.channels, &rm)) return rc;
+    if (int rc = channel_store("kth_batch_norm_forward(running_var)", running_var, g.channels, &rv)) return rc;
+    if (int rc = channel_store("kth_batch_norm_forward(gamma)", gamma, g.channels, &ga)) return rc;
+    if (int rc = channel_store("kth_batch_norm_forward(beta)", beta, g.channels, &be)) return rc;
+    if (int rc = channel_store("kth_batch_norm_forward(current_mean)", current_mean, g.channels, &cm)) return rc;
+    if (int rc = channel_store("kth_batch_norm_forward(current_std)", current_std, g.channels, &cs)) return rc;
+    if (!cm || !cs) return fail(KTH_E_ARGUMENT, "kth_batch_norm_forward: current_mean and current_std are outputs and must be given");
+
+    const StatsLaunch st = training ? plan_stats(g) : StatsLaunch{};
+    const uint64_t params_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(ForwardParams));
+    const uint64_t ws_bytes = params_bytes + st.partial_doubles * sizeof(double);
+    uint64_t cap;
+    char* ws = reinterpret_cast<char*>(workspace_acquire(ws_bytes, &cap));
+    if (!ws) return fail(KTH_E_MEMORY, "kth_batch_norm_forward: no workspace of %llu bytes", static_cast<unsigned long long>(ws_bytes));
+    ForwardParams* params = reinterpret_cast<ForwardParams*>(ws);
+    double* partial = reinterpret_cast<double*>(ws + params_bytes);
+    if (training) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
+    {
+        LaunchScope scope("bn_finalize_forward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
+        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + kBlock - 1) / kBlock), dim3(kBlock), 0, state().stream,
+                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params);
+    }
+    launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr);
+    workspace_release(reinterpret_cast<float*>(ws), cap);
+    KTH_LAUNCH_CHECK("batch_norm_forward");
+    return KTH_OK;
+}
+
+int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axis, int training, float epsilon,
+                            uint64_t running_mean, uint64_t running_var, uint64_t current_mean, uint64_t current_std,
+                            uint64_t gamma, uint64_t grad_out, uint64_t grad_in, uint64_t grad_gamma, uint64_t grad_beta) {
+    std::lock_guard<std::mutex> guard(lock());
+    KTH_REQUIRE_INIT();
+    Geometry g; uint64_t n;
+    if (int rc = geometry_of("kth_batch_norm_backward", shape, dims, axis, &g, &n)) return rc;
+    if (grad_in == 0 && grad_gamma == 0 && grad_beta == 0) return KTH_OK;         // JVMBatchNorm.kt:113-115
+    Store* si = lookup(in, "kth_batch_norm_backward(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* sg = lookup(grad_out, "kth_batch_norm_backward(grad_out)");
+    if (!sg) return KTH_E_HANDLE;
+    Store* sgi = nullptr;
+    if (grad_in != 0) { sgi = lookup(grad_in, "kth_batch_norm_backward(grad_in)"); if (!sgi) return KTH_E_HANDLE; }
+    if (n > si->n_floats || n > sg->n_floats || (sgi && n > sgi->n_floats))
+        return fail(KTH_E_ARGUMENT, "kth_batch_norm_backward: the shape needs more elements than a store holds");
+    float *rm, *rv, *cm, *cs, *ga, *gg, *gb;
+    if (int rc = channel_store("kth_batch_norm_backward(running_mean)", running_mean, g.channels, &rm)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(running_var)", running_var, g.channels, &rv)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(current_mean)", current_mean, g.channels, &cm)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(current_std)", current_std, g.channels, &cs)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(gamma)", gamma, g.channels, &ga)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(grad_gamma)", grad_gamma, g.channels, &gg)) return rc;
+    if (int rc = channel_store("kth_batch_norm_backward(grad_beta)", grad_beta, g.channels, &gb)) return rc;
+    if (training ? (!cm || !cs) : (!rm || !rv))
+        return fail(KTH_E_ARGUMENT, "kth_batch_norm_backward: %s", training ? "current_mean and current_std are needed in training mode"
+                                                                            : "running_mean and running_var are needed in inference mode");
+    // The two sums feed gradGamma, gradBeta and the training-mode input gradient; the
+    // inference-mode input gradient does not use them.
+    const bool need_sums = training || gg != nullptr || gb != nullptr;
+    const StatsLaunch st = need_sums ? plan_stats(g) : StatsLaunch{};
+    const uint64_t params_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(BackwardParams));
+    const uint64_t ws_bytes = params_bytes + st.partial_doubles * sizeof(double);
+    uint64_t cap;
+    char* ws = reinterpret_cast<char*>(workspace_acquire(ws_bytes, &cap));
+    if (!ws) return fail(KTH_E_MEMORY, "kth_batch_norm_backward: no workspace of %llu bytes", static_cast<unsigned long long>(ws_bytes));
+    BackwardParams* params = reinterpret_cast<BackwardParams*>(ws);
+    double* partial = reinterpret_cast<double*>(ws + params_bytes);
+    if (need_sums) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
+    {
+        LaunchScope scope("bn_finalize_backward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
+        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + kBlock - 1) / kBlock), dim3(kBlock), 0, state().stream,
+                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params);
+    }
+    if (sgi) {
+        if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params);
+        else launch_apply<2>(g, n, nullptr, sg->ptr, sgi->ptr, nullptr, params);
+    }
+    workspace_release(reinterpret_cast<float*>(ws), cap);
+    KTH_LAUNCH_CHECK("batch_norm_backward");
+    return KTH_OK;
+}
+
+}  // extern "C"

@@ -321,6 +321,48 @@ class HipRawTensor(AbstractRawTensor):
         return self.toArray().reshape(-1).tolist()
 
 
+class HipBatchNorm:
+    """BatchNormOperation (kten-api/.../tensor/operations/nn/BatchNormOperation.kt:5-41) on the
+    device: calculateOutput / calculateGrads return the reference's data classes as tuples."""
+
+    def __init__(self, axis, momentum, epsilon, training, ops):
+        self.axis, self.momentum, self.epsilon, self.training, self.ops = axis, float(momentum), float(epsilon), bool(training), ops
+
+    @staticmethod
+    def _h(t):
+        if t is None:
+            return 0
+        t._require_live()
+        return t.storeReference
+
+    def calculateOutput(self, input, runningMean, runningVar, gamma, beta):
+        input._require_live()
+        channels = input.shape[sf.normalize_axis(input.shape, self.axis)]
+        output = self.ops.createRaw(input.shape)
+        currentMean = self.ops.createRaw([channels])
+        currentStd = self.ops.createRaw([channels])
+        check(self.ops.lib.kth_batch_norm_forward(
+            input.storeReference, abi.shape_array(input.shape), input.dimensions, self.axis, 1 if self.training else 0,
+            self.momentum, self.epsilon, self._h(runningMean), self._h(runningVar), self._h(gamma), self._h(beta),
+            output.storeReference, currentMean.storeReference, currentStd.storeReference))
+        return output, currentMean, currentStd
+
+    def calculateGrads(self, input, runningMean, runningVar, currentMean, currentStd, gamma, gradOut,
+                       inRequiresGrad, gammaRequiresGrad, betaRequiresGrad):
+        if not (inRequiresGrad or gammaRequiresGrad or betaRequiresGrad):
+            return None, None, None
+        input._require_live(); gradOut._require_live()
+        channels = input.shape[self.axis]
+        gradIn = self.ops.createRaw(input.shape) if inRequiresGrad else None
+        gradGamma = self.ops.createRaw([channels]) if gammaRequiresGrad else None
+        gradBeta = self.ops.createRaw([channels]) if betaRequiresGrad else None
+        check(self.ops.lib.kth_batch_norm_backward(
+            input.storeReference, abi.shape_array(input.shape), input.dimensions, self.axis, 1 if self.training else 0,
+            self.epsilon, self._h(runningMean), self._h(runningVar), self._h(currentMean), self._h(currentStd), self._h(gamma),
+            gradOut.storeReference, self._h(gradIn), self._h(gradGamma), self._h(gradBeta)))
+        return gradIn, gradGamma, gradBeta
+
+
 class HipTensorOperations:
     """TensorOperations for the HIP platform (kten-api/.../operations/TensorOperations.kt:9-135),
     restricted to the members the broadcast / reduction path uses. Lifetime management
@@ -414,6 +456,10 @@ class HipTensorOperations:
     def concat(self, axis: int, inputs) -> HipRawTensor:
         """TensorOperations.kt:41."""
         return raw_concat(self, axis, inputs)
+
+    def batchNorm(self, axis: int, momentum: float, epsilon: float, training: bool) -> "HipBatchNorm":
+        """TensorOperations.kt:129."""
+        return HipBatchNorm(axis, momentum, epsilon, training, self)
 
     # --- Tensor-level factories (BasicTensorOperations.kt:10-12) ----------------------------
     def create(self, shape, requiresGrad: bool = False, init=None):

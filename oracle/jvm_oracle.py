@@ -83,6 +83,10 @@ def lib():
     L.kjo_transpose_jvm.argtypes = [fp, ip, c_int, c_int, c_int, fp, fp]
     L.kjo_permute.argtypes = [fp, ip, c_int, ip, fp]
     L.kjo_masked_fill.argtypes = [fp, fp, c_float, fp, c_int64]
+    L.kjo_batch_norm_apply.argtypes = [fp, ip, c_int, c_int, fp, fp, fp, fp, fp]
+    L.kjo_batch_norm_output.argtypes = [fp, ip, c_int, c_int, c_int, c_float, c_float, fp, fp, fp, fp, fp, fp, fp]
+    L.kjo_batch_norm_grad_in.argtypes = [fp, ip, c_int, c_int, c_int, fp, fp, fp, fp, fp, fp, fp]
+    L.kjo_batch_norm_grads.argtypes = [fp, ip, c_int, c_int, c_int, c_float, fp, fp, fp, fp, fp, fp, fp, fp, fp]
     L.kjo_unary_f64.argtypes = [c_int, c_float]
     L.kjo_unary_f64.restype = c_double
     _lib = L
@@ -224,6 +228,29 @@ def masked_fill(a, mask, value: float) -> np.ndarray:
         mask = broadcast_to(mask, a.shape)
     out = np.empty_like(a)
     lib().kjo_masked_fill(_p(a), _p(mask), value, _p(out), a.size)
+    return out
+
+
+def _po(a):
+    return None if a is None else _p(a)
+
+
+def batch_norm_apply(x, axis, mean, stdev, gamma=None, beta=None) -> np.ndarray:
+    """The elementwise half of calculateOutput from given per-channel statistics."""
+    x = _f32(x); out = np.empty_like(x)
+    mean, stdev = _f32(mean), _f32(stdev)
+    gamma = None if gamma is None else _f32(gamma); beta = None if beta is None else _f32(beta)
+    lib().kjo_batch_norm_apply(_p(x), _sh(x.shape), x.ndim, axis, _p(mean), _p(stdev), _po(gamma), _po(beta), _p(out))
+    return out
+
+
+def batch_norm_grad_in(x, axis, training, mean, stdev, gamma, grad_out, sums, dots) -> np.ndarray:
+    """The elementwise half of calculateGrads from given per-channel scalars."""
+    x, grad_out = _f32(x), _f32(grad_out); out = np.empty_like(x)
+    mean, stdev, sums, dots = _f32(mean), _f32(stdev), _f32(sums), _f32(dots)
+    gamma = None if gamma is None else _f32(gamma)
+    lib().kjo_batch_norm_grad_in(_p(x), _sh(x.shape), x.ndim, axis, 1 if training else 0, _p(mean), _p(stdev), _po(gamma),
+                                 _p(grad_out), _p(sums), _p(dots), _p(out))
     return out
 
 
@@ -375,6 +402,41 @@ class JvmOracleRawTensor(AbstractRawTensor):
         return self.storeReference.tolist()
 
 
+class JvmOracleBatchNorm:
+    """JVMBatchNorm (backend/kten-jvm/.../operations/nn/JVMBatchNorm.kt) through the C restatement."""
+
+    def __init__(self, axis, momentum, epsilon, training, ops):
+        self.axis, self.momentum, self.epsilon, self.training, self.ops = axis, float(momentum), float(epsilon), bool(training), ops
+
+    @staticmethod
+    def _s(t):
+        return None if t is None else _p(t.storeReference)
+
+    def calculateOutput(self, input, runningMean, runningVar, gamma, beta):
+        channels = input.shape[self.axis]
+        output = self.ops.createRaw(input.shape)
+        currentMean, currentStd = self.ops.createRaw([channels]), self.ops.createRaw([channels])
+        lib().kjo_batch_norm_output(_p(input.storeReference), _sh(input.shape), input.dimensions, self.axis,
+                                    1 if self.training else 0, self.momentum, self.epsilon, self._s(runningMean),
+                                    self._s(runningVar), self._s(gamma), self._s(beta), _p(output.storeReference),
+                                    _p(currentMean.storeReference), _p(currentStd.storeReference))
+        return output, currentMean, currentStd
+
+    def calculateGrads(self, input, runningMean, runningVar, currentMean, currentStd, gamma, gradOut,
+                       inRequiresGrad, gammaRequiresGrad, betaRequiresGrad):
+        if not (inRequiresGrad or gammaRequiresGrad or betaRequiresGrad):
+            return None, None, None
+        channels = input.shape[self.axis]
+        gradIn = self.ops.createRaw(input.shape) if inRequiresGrad else None
+        gradGamma = self.ops.createRaw([channels]) if gammaRequiresGrad else None
+        gradBeta = self.ops.createRaw([channels]) if betaRequiresGrad else None
+        lib().kjo_batch_norm_grads(_p(input.storeReference), _sh(input.shape), input.dimensions, self.axis,
+                                   1 if self.training else 0, self.epsilon, self._s(runningMean), self._s(runningVar),
+                                   self._s(currentMean), self._s(currentStd), self._s(gamma), _p(gradOut.storeReference),
+                                   self._s(gradIn), self._s(gradGamma), self._s(gradBeta))
+        return gradIn, gradGamma, gradBeta
+
+
 class JvmOracleOperations:
     """The operations object of the CPU checker. Lifetime calls are no-ops, as on the
     JVM backend (AbstractJVMTensorOperations.kt:73-79,90-92)."""
@@ -421,6 +483,9 @@ class JvmOracleOperations:
 
     def concat(self, axis, inputs):
         return raw_concat(self, axis, inputs)
+
+    def batchNorm(self, axis, momentum, epsilon, training):
+        return JvmOracleBatchNorm(axis, momentum, epsilon, training, self)
 
     def create(self, shape, requiresGrad=False, init=None):
         from kten_amd.autograd import NoGradVariable, Variable

@@ -511,6 +511,126 @@ void kjo_masked_fill(const float* a, const float* mask, float value, float* out,
     for (int64_t i = 0; i < n; i++) out[i] = (mask[i] == 1.0f) ? value : a[i];
 }
 
+/* ---------------------------------------------------------------- fused batch normalisation */
+
+/* BN = backend/kten-jvm/src/main/kotlin/eu/redbean/kten/jvm/tensor/operations/nn/JVMBatchNorm.kt
+ * The tensor is seen as [outer, channels, inner] around the axis; BN:19-31 applyForAxis walks
+ * one channel's elements in store order: (o, i) with i fastest. */
+#define BN_FOR_CHANNEL(o_, i_, at_) \
+    for (int64_t o_ = 0; o_ < outer; o_++) \
+        for (int64_t i_ = 0, at_ = (o_ * channels + c) * inner; i_ < inner; i_++, at_++)
+
+static void bn_geometry(const int32_t* shape, int dims, int axis, int64_t* outer, int64_t* channels, int64_t* inner) {
+    *outer = 1; *inner = 1;
+    for (int d = 0; d < axis; d++) *outer *= shape[d];
+    for (int d = axis + 1; d < dims; d++) *inner *= shape[d];
+    *channels = shape[axis];
+}
+
+/* BN:87-92: out = (x - mean) * stdev * g + b, left to right in float, for one channel. */
+static void bn_apply_channel(const float* in, float* out, int64_t outer, int64_t channels, int64_t inner, int64_t c,
+                             float mean, float stdev, float g, float b) {
+    BN_FOR_CHANNEL(o, i, at) out[at] = (in[at] - mean) * stdev * g + b;
+}
+
+/* The elementwise half of calculateOutput for given per-channel statistics (gamma / beta may
+ * be NULL: 1 and 0, BN:84-85). Used to check a backend's output bit for bit from ITS OWN
+ * statistics, whose low bits depend on the summation order. */
+void kjo_batch_norm_apply(const float* in, const int32_t* shape, int dims, int axis, const float* mean, const float* stdev,
+                          const float* gamma, const float* beta, float* out) {
+    int64_t outer, channels, inner;
+    bn_geometry(shape, dims, axis, &outer, &channels, &inner);
+    for (int64_t c = 0; c < channels; c++)
+        bn_apply_channel(in, out, outer, channels, inner, c, mean[c], stdev[c], gamma ? gamma[c] : 1.0f, beta ? beta[c] : 0.0f);
+}
+
+/* BN:33-99 calculateOutput. running_mean / running_var (both or neither), gamma, beta may be
+ * NULL. current_mean / current_std are written in training mode only (they stay as
+ * allocated, zero, in inference mode: BN:41-42,79-82). */
+void kjo_batch_norm_output(const float* in, const int32_t* shape, int dims, int axis, int training, float momentum, float epsilon,
+                           float* running_mean, float* running_var, const float* gamma, const float* beta,
+                           float* out, float* current_mean, float* current_std) {
+    int64_t outer, channels, inner;
+    bn_geometry(shape, dims, axis, &outer, &channels, &inner);
+    const int64_t n = outer * inner;
+    #pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t c = 0; c < channels; c++) {
+        float mean, stdev = 0.0f;
+        if (training) {
+            float sum = 0.0f;
+            BN_FOR_CHANNEL(o, i, at) sum += in[at];
+            mean = sum / (float)n;
+            current_mean[c] = mean;
+            sum = 0.0f;
+            BN_FOR_CHANNEL(o2, i2, at2) { float d = in[at2] - mean; sum += d * d; }
+            if (sum != 0.0f || epsilon != 0.0f) stdev = 1.0f / sqrtf(sum / (float)n + epsilon);
+            current_std[c] = stdev;
+            if (running_mean && running_var) {
+                running_mean[c] = (momentum * mean) + ((1.0f - momentum) * running_mean[c]);
+                float unbiased = sum / (float)(n - 1);
+                running_var[c] = (momentum * unbiased) + ((1.0f - momentum) * running_var[c]);
+            }
+        } else {
+            mean = running_mean[c];
+            stdev = 1.0f / sqrtf(running_var[c] + epsilon);
+        }
+        bn_apply_channel(in, out, outer, channels, inner, c, mean, stdev, gamma ? gamma[c] : 1.0f, beta ? beta[c] : 0.0f);
+    }
+}
+
+/* BN:148-168: gradIn for one channel from the channel's scalars. */
+static void bn_grad_in_channel(const float* in, const float* grad_out, float* grad_in, int64_t outer, int64_t channels, int64_t inner,
+                               int64_t c, int training, float mean, float stdev, float g, float sum, float dot) {
+    const int64_t n = outer * inner;
+    if (training) {
+        const float dot_std_sq = dot * stdev * stdev / (float)n;
+        const float grad_mean = sum / (float)n;
+        BN_FOR_CHANNEL(o, i, at) {
+            float base = (in[at] - mean) * dot_std_sq;
+            grad_in[at] = (grad_out[at] - grad_mean - base) * stdev * g;
+        }
+    } else {
+        BN_FOR_CHANNEL(o, i, at) grad_in[at] = grad_out[at] * stdev * g;
+    }
+}
+
+/* The elementwise half of calculateGrads for given per-channel scalars (sum of gradOut and
+ * dot product of (x - mean) with gradOut), for the same purpose as kjo_batch_norm_apply. */
+void kjo_batch_norm_grad_in(const float* in, const int32_t* shape, int dims, int axis, int training, const float* mean,
+                            const float* stdev, const float* gamma, const float* grad_out, const float* sum, const float* dot,
+                            float* grad_in) {
+    int64_t outer, channels, inner;
+    bn_geometry(shape, dims, axis, &outer, &channels, &inner);
+    for (int64_t c = 0; c < channels; c++)
+        bn_grad_in_channel(in, grad_out, grad_in, outer, channels, inner, c, training, mean[c], stdev[c], gamma ? gamma[c] : 1.0f,
+                           sum ? sum[c] : 0.0f, dot ? dot[c] : 0.0f);
+}
+
+/* BN:101-183 calculateGrads. grad_in / grad_gamma / grad_beta may be NULL (not required). In
+ * inference mode the statistics come from the running tensors, with the standard deviation
+ * through double arithmetic (BN:136). */
+void kjo_batch_norm_grads(const float* in, const int32_t* shape, int dims, int axis, int training, float epsilon,
+                          const float* running_mean, const float* running_var, const float* current_mean, const float* current_std,
+                          const float* gamma, const float* grad_out, float* grad_in, float* grad_gamma, float* grad_beta) {
+    if (!grad_in && !grad_gamma && !grad_beta) return;
+    int64_t outer, channels, inner;
+    bn_geometry(shape, dims, axis, &outer, &channels, &inner);
+    #pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t c = 0; c < channels; c++) {
+        const float g = gamma ? gamma[c] : 1.0f;
+        float mean, stdev;
+        if (training) { mean = current_mean[c]; stdev = current_std[c]; }
+        else { mean = running_mean[c]; stdev = (float)(1.0 / sqrt((double)(running_var[c] + epsilon))); }
+        float sum = 0.0f;
+        BN_FOR_CHANNEL(o, i, at) sum += grad_out[at];
+        float dot = 0.0f;
+        BN_FOR_CHANNEL(o2, i2, at2) dot += (in[at2] - mean) * grad_out[at2];
+        if (grad_in) bn_grad_in_channel(in, grad_out, grad_in, outer, channels, inner, c, training, mean, stdev, g, sum, dot);
+        if (grad_gamma) grad_gamma[c] = dot * stdev;
+        if (grad_beta) grad_beta[c] = sum;
+    }
+}
+
 /* ---------------------------------------------------------------- reductions */
 
 /* JVM:146-148 sum() = kotlin FloatArray.sum(): float accumulator from 0f, index order. */

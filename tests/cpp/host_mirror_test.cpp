@@ -109,6 +109,28 @@ int main() {
         expect_illegal_argument([&] { t1->view({3, -1, -1}); }, "view with two inferred dimensions");
         expect_illegal_argument([&] { g->gather(1, tensor(ops, {2, 2}, {0, 2, 0, 0})); }, "gather index out of range (JVMRawTensor.kt:345-346)");
 
+        // TensorTestsBase.kt:1190-1221 transpose, :1232-1270 permute, :1272-1315 concat, :1876-1888 partial fill
+        Raw tr = tensor(ops, {2, 3}, {1, 2, 3, 4, 5, 6});
+        expect_values(tr->transpose(0, 1), {3, 2}, {1, 4, 2, 5, 3, 6}, 0.0f, "transpose(0, 1)");
+        Raw pm = tensor(ops, {2, 3, 2}, {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12});
+        expect_values(pm->permute({2, 0, 1}), {2, 2, 3}, {1, 3, 5, 7, 9, 11, 2, 4, 6, 8, 10, 12}, 0.0f, "permute(2, 0, 1)");
+        Raw cat = ops.concat(0, {tensor(ops, {1, 3}, {1, 2, 3})->broadcastTo({2, 3}), tensor(ops, {1, 3}, {4, 5, 6}), tensor(ops, {1, 3}, {7, 8, 9})});
+        expect_values(cat, {4, 3}, {1, 2, 3, 1, 2, 3, 4, 5, 6, 7, 8, 9}, 0.0f, "concat along axis 0");
+        expect_values(cat->narrow(0, 2, 2), {2, 3}, {4, 5, 6, 7, 8, 9}, 0.0f, "narrow");
+        Raw pf = ops.createRawFill({2, 3}, 2.0f);
+        pf->set(std::vector<IntRange>{{0, 0}, {1, 2}}, 0.0f);
+        expect_values(pf, {2, 3}, {2, 0, 0, 2, 2, 2}, 0.0f, "set(ranges, Float)");
+        // TensorTestsBase.kt:152-188: t2[1..1, all, 1..-1] = value of shape [1, 3, 2]
+        Raw big = ops.createRawFill({3, 3, 3}, 1.0f);
+        big->set(std::vector<IntRange>{{1, 1}, All, {1, -1}}, ops.createRawFill({1, 3, 2}, 0.01f));
+        expect_values(big->get(std::vector<int>{1}), {3, 3}, {1, 0.01f, 0.01f, 1, 0.01f, 0.01f, 1, 0.01f, 0.01f}, 0.0f, "set(ranges, tensor) and get(IntArray)");
+        expect_values(big->get(std::vector<IntRange>{All, {0, 0}, {2, 2}}), {3, 1, 1}, {1, 0.01f, 1}, 0.0f, "get(ranges)");
+        expect_values(tr->maskedFill(tensor(ops, {3}, {1, 0, 1}), -1.0f), {2, 3}, {-1, 2, -1, -1, 5, -1}, 0.0f, "maskedFill with a broadcast mask");
+        expect_illegal_argument([&] { big->get(std::vector<IntRange>{{2, 1}}); }, "range with first > last");
+        expect_illegal_argument([&] { big->set(std::vector<IntRange>{{0, 0}}, ops.createRawFill({2}, 1.0f)); }, "set(ranges) with a different element count");
+        expect_illegal_argument([&] { pm->permute({0, 0, 1}); }, "permute must name every axis");
+        expect_illegal_argument([&] { tr->transpose(1, -1); }, "transpose needs two different axes");
+
         // in-place arithmetic and NaN detection
         Raw acc = ops.zerosLike(t1);
         acc->plusAssign(t1);

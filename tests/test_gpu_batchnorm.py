@@ -1,0 +1,155 @@
+"""Fused batch normalisation on the device: the reference's own tests, parity with the CPU
+checker (statistics to the reduction bar against float64; the elementwise halves bit-exact
+from the device's own statistics), every data layout the kernels distinguish, determinism
+and error behaviour."""
+import numpy as np
+import pytest
+
+import batchnorm_cases as bnc
+from kten_amd.inputs import SplitMix64
+from oracle import jvm_oracle as jo
+from parity import assert_bits_equal, assert_reduction_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name,case", bnc.CASES, ids=[n for n, _ in bnc.CASES])
+def test_reference_batch_norm_tests(name, case, gc):
+    case(gc)
+
+
+def make(ops, arrays):
+    return {k: (None if v is None else ops.createRaw(list(v.shape), v.reshape(-1) if ops.platformKey.startswith("JVM") else v))
+            for k, v in arrays.items()}
+
+
+def inputs_for(shape, axis, seed, affine, running):
+    gen = SplitMix64(seed)
+    c = shape[axis]
+    return {"x": gen.normal(shape) * np.float32(1.7) + np.float32(0.3), "go": gen.normal(shape),
+            "gamma": gen.normal([c]) if affine else None, "beta": gen.normal([c]) if affine else None,
+            "rm": gen.normal([c]) if running else None, "rv": np.abs(gen.normal([c])) if running else None}
+
+
+def channel_sums64(a, axis):
+    red = tuple(d for d in range(a.ndim) if d != axis)
+    return a.astype(np.float64).sum(red)
+
+
+# (shape, axis): long runs with float4 loads, long runs with scalar loads, short runs, channel-last, one channel,
+# more channels than workgroup columns, a single row
+LAYOUTS = [([10, 3, 4, 5], 1), ([8, 16, 32, 32], 1), ([4, 6, 67], 1), ([4, 5, 257], 1), ([64, 33, 7], 1), ([512, 40], 1),
+           ([300, 129], 1), ([40, 512], 0), ([3, 2000], 0), ([2, 3, 4, 5], 3), ([6, 1, 300], 1), ([1, 8, 4096], 1),
+           ([9, 4, 1024], 1), ([10, 3, 4, 5], 2)]
+
+
+@pytest.mark.parametrize("affine,running", [(True, True), (False, False)])
+@pytest.mark.parametrize("shape,axis", LAYOUTS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else f"axis{v}")
+def test_training_mode_parity(shape, axis, affine, running, gc):
+    eps, momentum = 1e-3, 0.1
+    arrays = inputs_for(shape, axis, sum(shape) * 7 + axis, affine, running)
+    cpu = jo.JvmOracleOperations()
+    g, c = make(gc, arrays), make(cpu, arrays)
+    gop, cop = gc.batchNorm(axis, momentum, eps, True), cpu.batchNorm(axis, momentum, eps, True)
+    gout, gmean, gstd = gop.calculateOutput(g["x"], g["rm"], g["rv"], g["gamma"], g["beta"])
+    cout, cmean, cstd = cop.calculateOutput(c["x"], c["rm"], c["rv"], c["gamma"], c["beta"])
+    x64 = arrays["x"].astype(np.float64)
+    n = arrays["x"].size // shape[axis]
+    bshape = [1] * len(shape); bshape[axis] = shape[axis]
+    mean64 = channel_sums64(arrays["x"], axis) / n
+    assert_reduction_close(gmean.toArray(), mean64, cmean.toArray(), "currentMean")
+    # the reciprocal standard deviation, against float64 from the device's own rounded mean
+    dev_mean = gmean.toArray().astype(np.float64).reshape(bshape)
+    ssd64 = channel_sums64((x64 - dev_mean) ** 2, axis)
+    std64 = 1.0 / np.sqrt(ssd64 / n + eps)
+    jvm_mean = cmean.toArray().astype(np.float64).reshape(bshape)
+    jvm_std64 = 1.0 / np.sqrt(channel_sums64((x64 - jvm_mean) ** 2, axis) / n + eps)
+    err = np.abs(gstd.toArray() - std64)
+    assert np.all((err <= 1e-5 * std64) | (err <= np.abs(cstd.toArray() - jvm_std64))), "currentStd"
+    # the elementwise half, bit for bit from the device's own statistics
+    assert_bits_equal(gout.toArray(), jo.batch_norm_apply(arrays["x"], axis, gmean.toArray(), gstd.toArray(),
+                                                          arrays["gamma"], arrays["beta"]), "output")
+    if running:
+        assert np.allclose(g["rm"].toArray(), c["rm"].toArray(), rtol=1e-5, atol=1e-6)
+        assert np.allclose(g["rv"].toArray(), c["rv"].toArray(), rtol=1e-5, atol=1e-6)
+        f = np.float32
+        want_rm = (f(momentum) * gmean.toArray() + (f(1) - f(momentum)) * arrays["rm"]).astype(f)
+        assert_bits_equal(g["rm"].toArray(), want_rm, "running mean from the device's mean, in the reference's float order")
+
+    ggin, ggg, ggb = gop.calculateGrads(g["x"], g["rm"], g["rv"], gmean, gstd, g["gamma"], g["go"], True, affine, affine)
+    cgin, cgg, cgb = cop.calculateGrads(c["x"], c["rm"], c["rv"], cmean, cstd, c["gamma"], c["go"], True, affine, affine)
+    go64 = arrays["go"].astype(np.float64)
+    sum64 = channel_sums64(arrays["go"], axis)
+    dot64 = channel_sums64((x64 - dev_mean) * go64, axis)
+    if affine:
+        assert_reduction_close(ggb.toArray(), sum64, cgb.toArray(), "gradBeta")
+        jvm_dot64 = channel_sums64((x64 - jvm_mean) * go64, axis)
+        err = np.abs(ggg.toArray() - dot64 * gstd.toArray())
+        jerr = np.abs(cgg.toArray() - jvm_dot64 * cstd.toArray())
+        assert np.all((err <= 1e-5 * np.abs(dot64 * gstd.toArray())) | (err <= jerr) | (err <= 1e-6)), "gradGamma"
+    want_gin = jo.batch_norm_grad_in(arrays["x"], axis, True, gmean.toArray(), gstd.toArray(), arrays["gamma"], arrays["go"],
+                                     sum64.astype(np.float32), dot64.astype(np.float32))
+    assert_bits_equal(ggin.toArray(), want_gin, "gradIn from the device's statistics and the correctly rounded sums")
+    scale = np.abs(cgin.toArray()).max()
+    assert np.abs(ggin.toArray() - cgin.toArray()).max() <= 2e-5 * scale, "gradIn against the checker end to end"
+
+
+@pytest.mark.parametrize("shape,axis", [([10, 3, 4, 5], 2), ([8, 16, 32, 32], 1), ([512, 40], 1), ([4, 6, 67], 1)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else f"axis{v}")
+def test_inference_mode_is_bit_exact(shape, axis, gc):
+    """No reduction feeds the inference output or input gradient, so they match the checker
+    bit for bit; gradGamma / gradBeta are sums and go through the reduction bar."""
+    eps = 1e-3
+    arrays = inputs_for(shape, axis, sum(shape) + 100 * axis, True, True)
+    cpu = jo.JvmOracleOperations()
+    g, c = make(gc, arrays), make(cpu, arrays)
+    gop, cop = gc.batchNorm(axis, 0.1, eps, False), cpu.batchNorm(axis, 0.1, eps, False)
+    gout, gmean, gstd = gop.calculateOutput(g["x"], g["rm"], g["rv"], g["gamma"], g["beta"])
+    cout, cmean, cstd = cop.calculateOutput(c["x"], c["rm"], c["rv"], c["gamma"], c["beta"])
+    assert_bits_equal(gout.toArray(), cout.toArray(), "output")
+    assert_bits_equal(gmean.toArray(), cmean.toArray(), "currentMean stays zero")
+    assert_bits_equal(gstd.toArray(), cstd.toArray(), "currentStd stays zero")
+    assert_bits_equal(g["rm"].toArray(), arrays["rm"], "running mean untouched")
+    assert_bits_equal(g["rv"].toArray(), arrays["rv"], "running var untouched")
+    ggin, ggg, ggb = gop.calculateGrads(g["x"], g["rm"], g["rv"], gmean, gstd, g["gamma"], g["go"], True, True, True)
+    cgin, cgg, cgb = cop.calculateGrads(c["x"], c["rm"], c["rv"], cmean, cstd, c["gamma"], c["go"], True, True, True)
+    assert_bits_equal(ggin.toArray(), cgin.toArray(), "gradIn")
+    assert_reduction_close(ggb.toArray(), channel_sums64(arrays["go"], axis), cgb.toArray(), "gradBeta")
+    bshape = [1] * len(shape); bshape[axis] = shape[axis]
+    std = (1.0 / np.sqrt((arrays["rv"] + np.float32(eps)).astype(np.float64))).astype(np.float32)
+    dot64 = channel_sums64((arrays["x"].astype(np.float64) - arrays["rm"].reshape(bshape)) * arrays["go"], axis)
+    assert_reduction_close(ggg.toArray(), dot64 * std, cgg.toArray(), "gradGamma")
+    only_in, none_g, none_b = gop.calculateGrads(g["x"], g["rm"], g["rv"], gmean, gstd, g["gamma"], g["go"], True, False, False)
+    assert none_g is None and none_b is None
+    assert_bits_equal(only_in.toArray(), cgin.toArray(), "gradIn alone (no statistics pass)")
+
+
+def test_batch_norm_is_deterministic_and_handles_degenerate_channels(gc):
+    arrays = inputs_for([32, 24, 28, 28], 1, 5, True, False)
+    arrays["x"][:, 3] = 2.5                                   # a constant channel
+    g = make(gc, arrays)
+    op = gc.batchNorm(1, 0.1, 0.0, True)                      # epsilon 0: the constant channel's 1/std stays 0
+    first = [t.toArray() for t in op.calculateOutput(g["x"], None, None, g["gamma"], g["beta"])]
+    again = [t.toArray() for t in op.calculateOutput(g["x"], None, None, g["gamma"], g["beta"])]
+    for a, b, name in zip(first, again, ("output", "currentMean", "currentStd")):
+        assert_bits_equal(a, b, f"{name} on a second run")
+    assert first[1][3] == np.float32(2.5) and first[2][3] == 0.0
+    assert_bits_equal(first[0][:, 3], np.full([32, 28, 28], arrays["beta"][3], dtype=np.float32), "constant channel -> beta")
+
+
+def test_batch_norm_argument_errors(gc):
+    x = gc.createRaw([4, 3, 8], np.zeros(96, dtype=np.float32))
+    three, two = gc.createRaw([3], [1.0, 1.0, 1.0]), gc.createRaw([2], [1.0, 1.0])
+    with pytest.raises(ValueError):
+        gc.batchNorm(1, 0.1, 1e-3, False).calculateOutput(x, None, None, None, None)          # inference needs running statistics
+    with pytest.raises(ValueError):
+        gc.batchNorm(1, 0.1, 1e-3, True).calculateOutput(x, three, None, None, None)          # both or neither
+    with pytest.raises(ValueError):
+        gc.batchNorm(1, 0.1, 1e-3, True).calculateOutput(x, None, None, two, None)            # gamma too short
+    with pytest.raises(ValueError):
+        gc.batchNorm(3, 0.1, 1e-3, True).calculateOutput(x, None, None, None, None)           # axis out of range
+    t = gc.create([4, 3, 8], True, np.zeros([4, 3, 8], dtype=np.float32))
+    with pytest.raises(ValueError):
+        t.batchNorm(1, None, None, False)
+    with pytest.raises(ValueError):
+        t.batchNorm(1, gc.create([3], True, np.zeros(3, dtype=np.float32)), gc.create([3], False, np.ones(3, dtype=np.float32)), True)
