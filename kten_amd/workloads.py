@@ -238,7 +238,38 @@ def _bytes_cat(d):
     return 4 * (2 * n + 2 * n + (d["left"] + d["right"]) + 2 * lb + la)
 
 
+# ---- fused batch normalisation ------------------------------------------------------------------
+
+def _in_bn(d):
+    g = SplitMix64(10)
+    n, c, h, w = d["n"], d["c"], d["h"], d["w"]
+    return {"x": g.normal([n, c, h, w]) * np.float32(1.5) + np.float32(0.25), "grad_out": g.normal([n, c, h, w]),
+            "gamma": g.uniform([c], 0.5, 1.5), "beta": g.uniform([c], -0.1, 0.1),
+            "running_mean": np.zeros([c], dtype=np.float32), "running_var": np.ones([c], dtype=np.float32)}
+
+
+def _run_bn(ops, inp):
+    from .autograd import NoGradVariable
+    raw = {k: ops.create(list(v.shape), False, v).getRawValue() for k, v in inp.items()}
+    op = ops.batchNorm(1, 0.1, 1e-5, True)
+    out, mean, std = op.calculateOutput(raw["x"], raw["running_mean"], raw["running_var"], raw["gamma"], raw["beta"])
+    grad_in, grad_gamma, grad_beta = op.calculateGrads(raw["x"], raw["running_mean"], raw["running_var"], mean, std,
+                                                       raw["gamma"], raw["grad_out"], True, True, True)
+    res = {"out": out, "mean": mean, "std": std, "grad_in": grad_in, "grad_gamma": grad_gamma, "grad_beta": grad_beta}
+    return {k: NoGradVariable(ops, v) for k, v in res.items()}
+
+
+def _bytes_bn(d):
+    full, c = d["n"] * d["c"] * d["h"] * d["w"], d["c"]
+    # forward: statistics (read x), normalise (read x, write out); backward: sums (read x and gradOut),
+    # input gradient (read x and gradOut, write); per-channel operands and results: 8 C forward, 6 C backward
+    return 4 * (8 * full + 14 * c)
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "batch_norm": Workload("batch_norm", "BatchNormOperation over axis 1 of NCHW [64,128,56,56], training mode: calculateOutput "
+                                         "then calculateGrads (input, gamma and beta gradients); seed 10",
+                           {"n": 64, "c": 128, "h": 56, "w": 56}, _in_bn, _run_bn, _bytes_bn),
     "transpose": Workload("transpose", "x.transpose(0, 1): x[8192,8192], U(-1,1), seed 7", {"rows": 8192, "cols": 8192},
                           _in_tr, _run_tr, _bytes_tr),
     "permute": Workload("permute", "x.permute(0,2,3,1) then .permute(0,3,1,2): NCHW [64,128,56,56] to NHWC and back, seed 8",

@@ -27,6 +27,12 @@
  *   - index map, + - * / sqrt, compare, max/min/argmax/argmin, round/sign/trunc/floor/ceil:
  *     pinned by the reference's own known-answer tests (tests/golden/known_answers.json)
  *     and by brute-force / IEEE closed forms.
+ *   - range get / set / fill, permute, maskedFill, the literal kten-jvm transpose: pinned by the
+ *     reference's indexing / transpose / permute / concat tests and documented examples and
+ *     by numpy's slicing, transpose, where and concatenate (tests/test_oracle_layout.py).
+ *   - fused batch normalisation: pinned by the reference's four batch-norm tests (fused op
+ *     against the composed computation), float64 closed forms with an independently derived
+ *     gradient, and one channel worked by hand in float32 (tests/test_oracle_batchnorm.py).
  *   - exp log pow tanh sinh cosh sin cos tan asin acos atan at ULP granularity:
  *     "parity unpinned" by the reference (its tests check six points at 1e-4 absolute);
  *     pinned here only to the closed form (float)libm_f64((double)x) and those six points.

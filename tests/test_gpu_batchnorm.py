@@ -153,3 +153,37 @@ def test_batch_norm_argument_errors(gc):
         t.batchNorm(1, None, None, False)
     with pytest.raises(ValueError):
         t.batchNorm(1, gc.create([3], True, np.zeros(3, dtype=np.float32)), gc.create([3], False, np.ones(3, dtype=np.float32)), True)
+
+
+def test_batch_norm_workload_at_benchmark_size(gc):
+    """NCHW [64,128,56,56], training forward + backward: statistics against float64, the two
+    elementwise halves bit for bit from the device's statistics, and what batch normalisation
+    guarantees of its own output (per-channel mean beta, variance gamma^2 var / (var + eps))."""
+    from kten_amd.workloads import WORKLOADS
+    wl = WORKLOADS["batch_norm"]
+    inp = wl.make_inputs(wl.full_dims)
+    out = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    x64 = inp["x"].astype(np.float64)
+    n = inp["x"].size // 128
+    mean64 = x64.sum((0, 2, 3)) / n
+    assert np.abs(out["mean"] - mean64).max() <= 1e-5 * np.abs(mean64).max()
+    dev_mean = out["mean"].astype(np.float64).reshape(1, 128, 1, 1)
+    var64 = ((x64 - dev_mean) ** 2).sum((0, 2, 3)) / n
+    std64 = 1.0 / np.sqrt(var64 + 1e-5)
+    assert np.abs(out["std"] - std64).max() <= 1e-5 * std64.max()
+    assert_bits_equal(out["out"], jo.batch_norm_apply(inp["x"], 1, out["mean"], out["std"], inp["gamma"], inp["beta"]), "output")
+    o64 = out["out"].astype(np.float64)
+    assert np.abs(o64.mean((0, 2, 3)) - inp["beta"]).max() <= 1e-5
+    assert np.allclose(o64.var((0, 2, 3)), inp["gamma"].astype(np.float64) ** 2 * var64 / (var64 + 1e-5), rtol=1e-5)
+    go64 = inp["grad_out"].astype(np.float64)
+    sum64, dot64 = go64.sum((0, 2, 3)), ((x64 - dev_mean) * go64).sum((0, 2, 3))
+    assert np.abs(out["grad_beta"] - sum64).max() <= 1e-5 * np.abs(sum64).max()
+    assert np.abs(out["grad_gamma"] - dot64 * out["std"]).max() <= 1e-5 * np.abs(dot64 * out["std"]).max()
+    want = jo.batch_norm_grad_in(inp["x"], 1, True, out["mean"], out["std"], inp["gamma"], inp["grad_out"],
+                                 sum64.astype(np.float32), dot64.astype(np.float32))
+    assert_bits_equal(out["grad_in"], want, "gradIn")
+    # the input gradient of batch normalisation sums to zero per channel and is orthogonal to x - mean
+    gi64 = out["grad_in"].astype(np.float64)
+    # (to float rounding of the 200 704 terms of a channel: a few 1e-7 of their absolute sum)
+    assert np.all(np.abs(gi64.sum((0, 2, 3))) <= 1e-6 * np.abs(gi64).sum((0, 2, 3)))
+    assert np.all(np.abs((gi64 * (x64 - dev_mean)).sum((0, 2, 3))) <= 1e-6 * np.abs(gi64 * (x64 - dev_mean)).sum((0, 2, 3)))

@@ -239,6 +239,7 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
                  "max_backward": {"rows": 6, "cols": 10}, "softmax_ce": {"batch": 6, "classes": 10},
                  "transpose": {"rows": 6, "cols": 10}, "permute": {"n": 2, "c": 3, "h": 4, "w": 5},
                  "concat_mask": {"rows": 6, "left": 4, "right": 8}}
+        assert WORKLOADS["batch_norm"].algorithmic_bytes({"n": 2, "c": 3, "h": 4, "w": 5}) == 4 * (8 * 120 + 14 * 3)
         for name, dims in small.items():
             wl = WORKLOADS[name]
             counted[0] = 0
