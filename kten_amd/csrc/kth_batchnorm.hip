@@ -187,21 +187,30 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
 struct ForwardParams { float mean, stdev, gamma, beta; };
 struct BackwardParams { float mean, stdev, gamma, dot_std_sq, grad_mean, pad0, pad1, pad2; };
 
-// Folds the partials of channel c in a fixed order. by_cols: partials are [segment][column].
+// One wave folds the partials of channel c, always in the same order: lane l takes the items
+// l, l + 64, ... (item t of a by-columns layout is segment t / inner, column c * inner + t % inner),
+// then the lanes are folded by xor-shuffles. Every lane returns the totals.
 __device__ __forceinline__ void fold_partials(const double* partial, uint32_t c, uint32_t segments, bool by_cols,
                                               uint32_t width, uint32_t inner, double& s1, double& s2) {
     s1 = 0.0; s2 = 0.0;
+    const uint32_t lane = threadIdx.x & 63;
     if (by_cols) {
-        for (uint32_t s = 0; s < segments; s++)
-            for (uint32_t i = 0; i < inner; i++) {
-                const uint64_t at = (static_cast<uint64_t>(s) * width + static_cast<uint64_t>(c) * inner + i) * 2;
-                s1 += partial[at]; s2 += partial[at + 1];
-            }
-    } else {
-        for (uint32_t s = 0; s < segments; s++) {
-            const uint64_t at = (static_cast<uint64_t>(c) * segments + s) * 2;
+        const uint32_t items = segments * inner;
+        for (uint32_t t = lane; t < items; t += 64) {
+            const uint32_t seg = t / inner, i = t - seg * inner;
+            const uint64_t at = (static_cast<uint64_t>(seg) * width + static_cast<uint64_t>(c) * inner + i) * 2;
             s1 += partial[at]; s2 += partial[at + 1];
         }
+    } else {
+        for (uint32_t t = lane; t < segments; t += 64) {
+            const uint64_t at = (static_cast<uint64_t>(c) * segments + t) * 2;
+            s1 += partial[at]; s2 += partial[at + 1];
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        s1 += __shfl_xor(s1, off);
+        s2 += __shfl_xor(s2, off);
     }
 }
 
@@ -211,12 +220,13 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
                                                                     const float* __restrict__ gamma, const float* __restrict__ beta,
                                                                     float* __restrict__ current_mean, float* __restrict__ current_std,
                                                                     ForwardParams* __restrict__ params) {
-    const uint32_t c = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
     if (c >= g.channels) return;
     float mean, stdev = 0.0f;
+    double s1 = 0.0, s2 = 0.0;
+    if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
+    if ((threadIdx.x & 63) != 0) return;
     if (training) {
-        double s1, s2;
-        fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
         const double n = static_cast<double>(g.per_channel);
         const double k = static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]);
         mean = static_cast<float>(k + s1 / n);                                  // JVMBatchNorm.kt:57-58
@@ -252,8 +262,11 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
                                                                      const float* __restrict__ current_mean, const float* __restrict__ current_std,
                                                                      const float* __restrict__ gamma, float* __restrict__ grad_gamma,
                                                                      float* __restrict__ grad_beta, BackwardParams* __restrict__ params) {
-    const uint32_t c = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
     if (c >= g.channels) return;
+    double s1 = 0.0, s2 = 0.0;
+    if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
+    if ((threadIdx.x & 63) != 0) return;
     float mean, stdev;
     if (training) { mean = current_mean[c]; stdev = current_std[c]; }           // JVMBatchNorm.kt:131-133
     else {                                                                      // :134-137
@@ -262,8 +275,6 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
     }
     float sum = 0.0f, dot = 0.0f;
     if (have_sums) {
-        double s1, s2;
-        fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
         sum = static_cast<float>(s1);                                           // :139-147
         dot = static_cast<float>(s2);
     }
@@ -305,7 +316,10 @@ __device__ __forceinline__ float bn_backward_inference(float go, const BackwardP
 }
 
 // MODE 0: forward. MODE 1: input gradient, training. MODE 2: input gradient, inference.
-template <int MODE, bool VEC>
+// VEC: one float4 per unit. UNIFORM: inner % 4 == 0, so the four lanes of a float4 share a
+// channel (pl.inner_div counts float4s); otherwise each lane finds its own channel
+// (pl.inner_div counts floats).
+template <int MODE, bool VEC, bool UNIFORM>
 __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float* __restrict__ x, const float* __restrict__ go, float* __restrict__ out,
                                                          const ForwardParams* __restrict__ fparams,
                                                          const BackwardParams* __restrict__ bparams, ApplyPlan pl) {
@@ -324,19 +338,13 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float* __restric
         for (int k = 0; k < kApplyUnroll; k++) {
             const uint32_t i = base + k * kBlock;
             if (i < pl.units) {
-                const uint32_t c = channel_of(pl, i);
                 v4f r;
-                if (MODE == 0) {
-                    const ForwardParams p = fparams[c];
-                    r.x = bn_forward(vx[k].x, p); r.y = bn_forward(vx[k].y, p); r.z = bn_forward(vx[k].z, p); r.w = bn_forward(vx[k].w, p);
-                } else if (MODE == 1) {
-                    const BackwardParams p = bparams[c];
-                    r.x = bn_backward_training(vx[k].x, vg[k].x, p); r.y = bn_backward_training(vx[k].y, vg[k].y, p);
-                    r.z = bn_backward_training(vx[k].z, vg[k].z, p); r.w = bn_backward_training(vx[k].w, vg[k].w, p);
-                } else {
-                    const BackwardParams p = bparams[c];
-                    r.x = bn_backward_inference(vg[k].x, p); r.y = bn_backward_inference(vg[k].y, p);
-                    r.z = bn_backward_inference(vg[k].z, p); r.w = bn_backward_inference(vg[k].w, p);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t c = UNIFORM ? channel_of(pl, i) : channel_of(pl, i * 4 + e);
+                    if (MODE == 0) r[e] = bn_forward(vx[k][e], fparams[c]);
+                    else if (MODE == 1) r[e] = bn_backward_training(vx[k][e], vg[k][e], bparams[c]);
+                    else r[e] = bn_backward_inference(vg[k][e], bparams[c]);
                 }
                 reinterpret_cast<v4f*>(out)[i] = r;
             }
@@ -457,17 +465,18 @@ void launch_stats(const StatsLaunch& st, const float* x, const float* go, const 
 template <int MODE>
 void launch_apply(const Geometry& g, uint64_t n, const float* x, const float* go, float* out, const ForwardParams* fp, const BackwardParams* bp) {
     ApplyPlan pl{};
-    const bool vec = g.inner % 4 == 0;
+    const bool vec = n % 4 == 0, uniform = g.inner % 4 == 0;
     pl.units = static_cast<uint32_t>(vec ? n / 4 : n);
     pl.channels = g.channels;
-    pl.inner_div = make_div(vec ? g.inner / 4 : g.inner);
+    pl.inner_div = make_div(uniform ? g.inner / 4 : g.inner);
     pl.channel_div = make_div(g.channels);
     const uint32_t per_block = kBlock * kApplyUnroll;
     const dim3 grid((pl.units + per_block - 1) / per_block);
     const uint64_t bytes = (MODE == 0 ? 2 : MODE == 1 ? 3 : 2) * n * 4;
     LaunchScope scope("bn_apply_kernel", MODE == 0 ? "forward" : MODE == 1 ? "backward_training" : "backward_inference", bytes);
-    if (vec) hipLaunchKernelGGL((bn_apply_kernel<MODE, true>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
-    else     hipLaunchKernelGGL((bn_apply_kernel<MODE, false>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
+    if (uniform)  hipLaunchKernelGGL((bn_apply_kernel<MODE, true, true>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
+    else if (vec) hipLaunchKernelGGL((bn_apply_kernel<MODE, true, false>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
+    else          hipLaunchKernelGGL((bn_apply_kernel<MODE, false, false>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
 }
 
 uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
@@ -512,7 +521,7 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     if (training) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
     {
         LaunchScope scope("bn_finalize_forward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + kBlock - 1) / kBlock), dim3(kBlock), 0, state().stream,
+        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
                            si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params);
     }
     launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr);
@@ -562,7 +571,7 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     if (need_sums) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
     {
         LaunchScope scope("bn_finalize_backward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + kBlock - 1) / kBlock), dim3(kBlock), 0, state().stream,
+        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
                            partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params);
     }
     if (sgi) {

@@ -280,18 +280,39 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* _
     }
 }
 
-// Any shapes: one output element per (thread, k); strides in floats, dim 0 in elements.
-template <class Op>
-__global__ __launch_bounds__(kBlock) void binary_bcast_scalar_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                                     float* __restrict__ out, uint32_t n, float eps, BcastPlan pl) {
+// Any shapes, four consecutive outputs per (thread, k): the output and every operand that
+// has the output's element count (AL / BL: it is then laid out exactly like the output) move
+// as float4; a broadcast operand is gathered element by element through the plan (dim 0 in
+// elements), which the caches serve. The last, partial group of four is done by elements.
+template <class Op, bool AL, bool BL>
+__global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                   float* __restrict__ out, uint32_t n, float eps, BcastPlan pl) {
     const uint32_t base = blockIdx.x * kBcastTile + threadIdx.x;
 #pragma unroll
     for (int k = 0; k < kBcastUnroll; k++) {
-        uint32_t i = base + k * kBlock;
-        if (i < n) {
-            uint32_t ao, bo;
-            decompose(pl, i, ao, bo);
-            out[i] = Op::apply(a[ao], b[bo], eps);
+        const uint32_t e0 = (base + k * kBlock) * 4;
+        if (e0 >= n) continue;
+        if (e0 + 4 <= n) {
+            float va[4], vb[4];
+            if (AL) { const float4 v = ld4(a, e0 >> 2); va[0] = v.x; va[1] = v.y; va[2] = v.z; va[3] = v.w; }
+            if (BL) { const float4 v = ld4(b, e0 >> 2); vb[0] = v.x; vb[1] = v.y; vb[2] = v.z; vb[3] = v.w; }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                uint32_t ao, bo;
+                decompose(pl, e0 + j, ao, bo);
+                if (!AL) va[j] = a[ao];
+                if (!BL) vb[j] = b[bo];
+            }
+            float4 r;
+            r.x = Op::apply(va[0], vb[0], eps); r.y = Op::apply(va[1], vb[1], eps);
+            r.z = Op::apply(va[2], vb[2], eps); r.w = Op::apply(va[3], vb[3], eps);
+            st4(out, e0 >> 2, r);
+        } else {
+            for (uint32_t e = e0; e < n; e++) {
+                uint32_t ao, bo;
+                decompose(pl, e, ao, bo);
+                out[e] = Op::apply(a[ao], b[bo], eps);
+            }
         }
     }
 }
@@ -421,7 +442,7 @@ template <class Op>
 void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n, float eps,
                          BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec, uint64_t bytes) {
     hipStream_t st = state().stream;
-    LaunchScope scope(!vec_ok ? "binary_bcast_scalar_kernel" : (a_vec && b_vec) ? "binary_bcast_vec_kernel_vv"
+    LaunchScope scope(!vec_ok ? "binary_bcast_mixed_kernel" : (a_vec && b_vec) ? "binary_bcast_vec_kernel_vv"
                       : a_vec ? "binary_bcast_vec_kernel_vs" : b_vec ? "binary_bcast_vec_kernel_sv"
                       : "binary_bcast_vec_kernel_ss", Op::name, bytes);
     if (vec_ok) {
@@ -433,8 +454,13 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
         else if (b_vec)      hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n4, eps, plan);
         else                 hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n4, eps, plan);
     } else {
-        hipLaunchKernelGGL((binary_bcast_scalar_kernel<Op>), dim3(static_cast<uint32_t>((static_cast<uint64_t>(n) + kBcastTile - 1) / kBcastTile)),
-                           dim3(kBlock), 0, st, a, b, out, n, eps, plan);
+        const uint64_t groups = (static_cast<uint64_t>(n) + 3) / 4;
+        dim3 grid(static_cast<uint32_t>((groups + kBcastTile - 1) / kBcastTile)), block(kBlock);
+        const bool al = plan.a_stream, bl = plan.b_stream;
+        if (al && bl)  hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, true>), grid, block, 0, st, a, b, out, n, eps, plan);
+        else if (al)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, false>), grid, block, 0, st, a, b, out, n, eps, plan);
+        else if (bl)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n, eps, plan);
+        else           hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n, eps, plan);
     }
 }
 
