@@ -126,58 +126,81 @@ __global__ __launch_bounds__(kBlock) void bn_stats_runs_kernel(const float* __re
 
 // ---------------------------------------------------------------- stats, short runs (inner < 64)
 
-// The tensor as a matrix [outer, width = channels * inner]: a thread owns a column, the 4
-// waves of a workgroup take rows r = first + wave, first + wave + 4, ...; a wave's loads are
-// 256 contiguous bytes. Partials are per (segment, column).
+// The tensor as a matrix [outer, width = channels * inner]: a thread owns W adjacent columns
+// (4 with float4 loads when width % 4 == 0, else 1), the 4 waves of a workgroup take rows
+// r = first + wave, first + wave + 4, ...; a wave's loads are 1 KiB (256 B) of one row.
+// Partials are per (segment, column).
 struct ColPlan {
     Geometry g;
     uint32_t width, col_blocks, segments, rows_per_seg;
     FastDiv  col_div, inner_div;
 };
 
-template <bool BACKWARD>
+template <bool BACKWARD, int W>
 __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __restrict__ x, const float* __restrict__ go,
                                                               const float* __restrict__ mean, double* __restrict__ partial, ColPlan pl) {
-    __shared__ double lds[kBlock * 2];
+    __shared__ double lds[kBlock * 2 * W];
     const uint32_t b = blockIdx.x;
     const uint32_t seg = (__umulhi(b, pl.col_div.mul) + b) >> pl.col_div.shift;
-    const uint32_t col = (b - seg * pl.col_blocks) * 64 + (threadIdx.x & 63);
+    const uint32_t col = ((b - seg * pl.col_blocks) * 64 + (threadIdx.x & 63)) * W;   // first of this thread's W columns
     const uint32_t lane_row = threadIdx.x >> 6;
-    double s1 = 0.0, s2 = 0.0;
+    double s1[W], s2[W];
+#pragma unroll
+    for (int e = 0; e < W; e++) { s1[e] = 0.0; s2[e] = 0.0; }
     if (col < pl.width) {
-        const uint32_t ch = (__umulhi(col, pl.inner_div.mul) + col) >> pl.inner_div.shift;
-        const double shift = BACKWARD ? static_cast<double>(mean[ch]) : static_cast<double>(x[static_cast<uint64_t>(ch) * pl.g.inner]);
+        double shift[W];
+#pragma unroll
+        for (int e = 0; e < W; e++) {
+            const uint32_t ce = col + e;
+            const uint32_t ch = (__umulhi(ce, pl.inner_div.mul) + ce) >> pl.inner_div.shift;
+            shift[e] = BACKWARD ? static_cast<double>(mean[ch]) : static_cast<double>(x[static_cast<uint64_t>(ch) * pl.g.inner]);
+        }
         const uint32_t first = seg * pl.rows_per_seg;
         uint32_t last = first + pl.rows_per_seg;
         if (last > pl.g.outer) last = pl.g.outer;
         for (uint32_t r0 = first + lane_row; r0 < last; r0 += 4 * kBatch) {
-            float vx[kBatch], vg[kBatch];
+            v4f vx[kBatch], vg[kBatch];
 #pragma unroll
             for (int k = 0; k < kBatch; k++) {
                 const uint32_t r = r0 + 4 * k;
                 if (r < last) {
                     const uint64_t at = static_cast<uint64_t>(r) * pl.width + col;
-                    vx[k] = x[at];
-                    if (BACKWARD) vg[k] = go[at];
+                    if (W == 4) {
+                        vx[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + at));
+                        if (BACKWARD) vg[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(go + at));
+                    } else {
+                        vx[k].x = x[at];
+                        if (BACKWARD) vg[k].x = go[at];
+                    }
                 }
             }
 #pragma unroll
             for (int k = 0; k < kBatch; k++) {
                 if (r0 + 4 * k < last) {
-                    const double d = static_cast<double>(vx[k]) - shift;
-                    if (BACKWARD) { const double g = static_cast<double>(vg[k]); s1 += g; s2 += d * g; }
-                    else { s1 += d; s2 += d * d; }
+#pragma unroll
+                    for (int e = 0; e < W; e++) {
+                        const double d = static_cast<double>(vx[k][e]) - shift[e];
+                        if (BACKWARD) { const double g = static_cast<double>(vg[k][e]); s1[e] += g; s2[e] += d * g; }
+                        else { s1[e] += d; s2[e] += d * d; }
+                    }
                 }
             }
         }
     }
-    lds[threadIdx.x * 2] = s1;
-    lds[threadIdx.x * 2 + 1] = s2;
+#pragma unroll
+    for (int e = 0; e < W; e++) {
+        lds[(threadIdx.x * W + e) * 2] = s1[e];
+        lds[(threadIdx.x * W + e) * 2 + 1] = s2[e];
+    }
     __syncthreads();
     if (lane_row == 0 && col < pl.width) {
-        for (int w = 1; w < 4; w++) { s1 += lds[(threadIdx.x + 64 * w) * 2]; s2 += lds[(threadIdx.x + 64 * w) * 2 + 1]; }
-        partial[(static_cast<uint64_t>(seg) * pl.width + col) * 2] = s1;
-        partial[(static_cast<uint64_t>(seg) * pl.width + col) * 2 + 1] = s2;
+#pragma unroll
+        for (int e = 0; e < W; e++) {
+            double a = s1[e], c = s2[e];
+            for (int w = 1; w < 4; w++) { a += lds[((threadIdx.x + 64 * w) * W + e) * 2]; c += lds[((threadIdx.x + 64 * w) * W + e) * 2 + 1]; }
+            partial[(static_cast<uint64_t>(seg) * pl.width + col + e) * 2] = a;
+            partial[(static_cast<uint64_t>(seg) * pl.width + col + e) * 2 + 1] = c;
+        }
     }
 }
 
@@ -431,7 +454,9 @@ StatsLaunch plan_stats(const Geometry& g) {
         ColPlan& p = st.col;
         p.g = g;
         p.width = g.channels * g.inner;
-        p.col_blocks = (p.width + 63) / 64;
+        st.vec = p.width % 4 == 0;                     // every row then starts 16-byte aligned
+        const uint32_t cols_per_block = st.vec ? 256 : 64;
+        p.col_blocks = (p.width + cols_per_block - 1) / cols_per_block;
         uint32_t segments = (target + p.col_blocks - 1) / p.col_blocks;
         const uint32_t max_segments = (g.outer + 4 * kBatch - 1) / (4 * kBatch);
         if (segments > max_segments) segments = max_segments;
@@ -452,8 +477,9 @@ void launch_stats(const StatsLaunch& st, const float* x, const float* go, const 
     const uint64_t bytes = (BACKWARD ? 2 : 1) * n * 4;
     if (st.by_cols) {
         LaunchScope scope("bn_stats_cols_kernel", BACKWARD ? "backward" : "forward", bytes);
-        hipLaunchKernelGGL((bn_stats_cols_kernel<BACKWARD>), dim3(st.col.col_blocks * st.col.segments), dim3(kBlock), 0, stream,
-                           x, go, mean, partial, st.col);
+        const dim3 grid(st.col.col_blocks * st.col.segments);
+        if (st.vec) hipLaunchKernelGGL((bn_stats_cols_kernel<BACKWARD, 4>), grid, dim3(kBlock), 0, stream, x, go, mean, partial, st.col);
+        else        hipLaunchKernelGGL((bn_stats_cols_kernel<BACKWARD, 1>), grid, dim3(kBlock), 0, stream, x, go, mean, partial, st.col);
     } else {
         LaunchScope scope("bn_stats_runs_kernel", BACKWARD ? "backward" : "forward", bytes);
         const dim3 grid(st.run.g.channels * st.run.segments);

@@ -98,6 +98,37 @@ struct OpSigmoidT {
     }
 };
 
+struct OpTanhT {
+    static constexpr const char* name = "OpTanh";
+    static constexpr int kTableDoubles = kExpTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_tanh(x, lds); }
+};
+struct OpSinhT {
+    static constexpr const char* name = "OpSinh";
+    static constexpr int kTableDoubles = kExpTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_sinh(x, lds); }
+};
+struct OpCoshT {
+    static constexpr const char* name = "OpCosh";
+    static constexpr int kTableDoubles = kExpTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_cosh(x, lds); }
+};
+
+// pow(tensor | Float): the common operands (finite non-zero base, finite exponent) go through
+// the exp / log tables, read from global memory (3 KiB, cache resident); zeros, infinities
+// and NaNs take jpow's spelled-out Java rules over the library routine.
+struct OpPowT {
+    static constexpr const char* name = "OpPow";
+    static __device__ __forceinline__ float apply(float a, float b, float) {
+        const bool common = (a != 0.0f) && (fabsf(a) < INFINITY) && (fabsf(b) < INFINITY) && (b != 0.0f);
+        if (common) return table_pow_finite(a, b, g_log_table, g_exp_table);
+        return jpow(a, b);
+    }
+};
+
 // Unary map whose op reads a small f64 table through LDS. The data loads of the tile are
 // issued first, the table copy overlaps them. Four float4 per thread, so the 1-2 KiB
 // table is amortised over a 16 KiB tile.
@@ -470,7 +501,7 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
     case KTH_MINUS: CALL(OpMinus); break;                      \
     case KTH_TIMES: CALL(OpTimes); break;                      \
     case KTH_DIV:   CALL(OpDiv);   break;                      \
-    case KTH_POW:   CALL(OpPow);   break;                      \
+    case KTH_POW:   CALL(OpPowT);  break;                      \
     case KTH_LT:    CALL(OpLt);    break;                      \
     case KTH_LTE:   CALL(OpLte);   break;                      \
     case KTH_GT:    CALL(OpGt);    break;                      \
@@ -522,9 +553,10 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
     case KTH_NEG: U(OpNeg); break;           case KTH_RECIPROCAL: U(OpReciprocal); break;
     case KTH_LOG: if (n32) launch_unary_lds<OpLogT>(pa, po, n32); break;
     case KTH_EXP: if (n32) launch_unary_lds<OpExpT>(pa, po, n32); break;
-    case KTH_TANH: U(OpTanh); break;
+    case KTH_TANH: if (n32) launch_unary_lds<OpTanhT>(pa, po, n32); break;
     case KTH_SIGMOID: if (n32) launch_unary_lds<OpSigmoidT>(pa, po, n32); break;
-    case KTH_SINH: U(OpSinh); break;         case KTH_COSH: U(OpCosh); break;
+    case KTH_SINH: if (n32) launch_unary_lds<OpSinhT>(pa, po, n32); break;
+    case KTH_COSH: if (n32) launch_unary_lds<OpCoshT>(pa, po, n32); break;
     case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
     case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSin); break;
     case KTH_COS: U(OpCos); break;           case KTH_TAN: U(OpTan); break;

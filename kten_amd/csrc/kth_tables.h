@@ -28,8 +28,8 @@ struct LogEntry { double invc, logc; };
 
 constexpr uint64_t kLogOff = 0x3fe6000000000000ull;   // 0.6875
 
-__device__ __forceinline__ float table_log(float x, const LogEntry* tab) {
-    const double d = static_cast<double>(x);                 // exact; fp32 denormals become normal doubles
+// log of a positive finite double (normal), to about 1e-16 relative.
+__device__ __forceinline__ double table_log_d(double d, const LogEntry* tab) {
     const uint64_t ix = static_cast<uint64_t>(__double_as_longlong(d));
     const uint64_t tmp = ix - kLogOff;
     const int i = static_cast<int>(tmp >> 45) & (kLogTableEntries - 1);
@@ -43,8 +43,12 @@ __device__ __forceinline__ float table_log(float x, const LogEntry* tab) {
     p = fma(r, p, 1.0 / 3.0);
     p = fma(r, p, -1.0 / 2.0);
     const double l1p = fma(r * r, p, r);
-    const double y = fma(static_cast<double>(k), 0.693147180559945309417232121458, e.logc) + l1p;
-    float res = static_cast<float>(y);
+    return fma(static_cast<double>(k), 0.693147180559945309417232121458, e.logc) + l1p;
+}
+
+__device__ __forceinline__ float table_log(float x, const LogEntry* tab) {
+    // The conversion is exact; fp32 denormals become normal doubles.
+    float res = static_cast<float>(table_log_d(static_cast<double>(x), tab));
     // Math.log: NaN or negative -> NaN, +-0 -> -inf, +inf -> +inf.
     if (x == 0.0f) res = -INFINITY;
     if (x < 0.0f) res = __uint_as_float(0x7fc00000u);
@@ -52,9 +56,8 @@ __device__ __forceinline__ float table_log(float x, const LogEntry* tab) {
     return res;
 }
 
-__device__ __forceinline__ float table_exp(float x, const double* tab) {
-    // Outside [-120, 100] the fp32 result is already 0 or inf; clamping keeps k in int range.
-    const double d = fmin(fmax(static_cast<double>(x), -120.0), 100.0);
+// e^d for d in [-120, 100], to about 1e-16 relative.
+__device__ __forceinline__ double table_exp_d(double d, const double* tab) {
     const double kd = rint(d * 184.664965233787316142070359168242182);   // 128 / ln2
     const int k = static_cast<int>(kd);
     // ln2 / 128 split so that kd * hi is exact for |kd| < 2^16.
@@ -66,9 +69,87 @@ __device__ __forceinline__ float table_exp(float x, const double* tab) {
     p = fma(r, p, 1.0 / 6.0);
     p = fma(r, p, 0.5);
     p = fma(r * r, p, r);                                    // e^r - 1
-    const double y = ldexp(fma(s, p, s), k >> 7);
-    float res = static_cast<float>(y);
+    return ldexp(fma(s, p, s), k >> 7);
+}
+
+__device__ __forceinline__ float table_exp(float x, const double* tab) {
+    // Outside [-120, 100] the fp32 result is already 0 or inf; clamping keeps k in int range.
+    float res = static_cast<float>(table_exp_d(fmin(fmax(static_cast<double>(x), -120.0), 100.0), tab));
     if (x != x) res = x;
+    return res;
+}
+
+// 1 / d for d in [1, 1e45]: the hardware estimate and two Newton steps (error about 1e-16
+// relative), without the scaling and fix-up code of an IEEE division.
+__device__ __forceinline__ double newton_rcp(double d) {
+    double r = __builtin_amdgcn_rcp(d);
+    r = fma(fma(-d, r, 1.0), r, r);
+    r = fma(fma(-d, r, 1.0), r, r);
+    return r;
+}
+
+// tanh, sinh, cosh from t = e^|x| (Math.tanh / sinh / cosh of the double, rounded once).
+// Below 2^-5 the odd functions use their Taylor series, so nothing cancels; above it the
+// differences t - 1/t and t^2 - 1 lose at most five bits of the 53.
+__device__ __forceinline__ float table_tanh(float x, const double* tab) {
+    const double a = fabs(static_cast<double>(x));
+    double y;
+    if (a < 0.03125) {
+        const double z = a * a;
+        double p = fma(z, -1382.0 / 155925.0, 62.0 / 2835.0);
+        p = fma(z, p, -17.0 / 315.0);
+        p = fma(z, p, 2.0 / 15.0);
+        p = fma(z, p, -1.0 / 3.0);
+        y = fma(a * z, p, a);
+    } else {
+        const double t = table_exp_d(2.0 * fmin(a, 20.0), tab);     // tanh(20) rounds to 1 in f64 already
+        y = (t - 1.0) * newton_rcp(t + 1.0);
+    }
+    float res = copysignf(static_cast<float>(y), x);
+    if (x != x) res = x;
+    return res;
+}
+
+__device__ __forceinline__ float table_sinh(float x, const double* tab) {
+    const double a = fabs(static_cast<double>(x));
+    double y;
+    if (a < 0.03125) {
+        const double z = a * a;
+        double p = fma(z, 1.0 / 362880.0, 1.0 / 5040.0);
+        p = fma(z, p, 1.0 / 120.0);
+        p = fma(z, p, 1.0 / 6.0);
+        y = fma(a * z, p, a);
+    } else {
+        const double t = table_exp_d(fmin(a, 100.0), tab);          // e^100 / 2 is beyond fp32: rounds to inf
+        y = 0.5 * (t - newton_rcp(t));
+    }
+    float res = copysignf(static_cast<float>(y), x);
+    if (x != x) res = x;
+    return res;
+}
+
+__device__ __forceinline__ float table_cosh(float x, const double* tab) {
+    const double t = table_exp_d(fmin(fabs(static_cast<double>(x)), 100.0), tab);
+    float res = static_cast<float>(0.5 * (t + newton_rcp(t)));
+    if (x != x) res = x;
+    return res;
+}
+
+// Math.pow(double, double) rounded to float, for the operands the tables cover: a finite
+// base other than 0 and a finite exponent. |a|^b = e^(b ln|a|); the error of b ln|a| is at
+// most about 2e-14 absolute, i.e. the result is within 2e-14 relative of the exact power
+// before the rounding to fp32. A negative base takes the sign of an odd integer exponent and
+// gives NaN for a non-integer one (Java and C agree on these).
+__device__ __forceinline__ float table_pow_finite(float a, float b, const LogEntry* log_tab, const double* exp_tab) {
+    const double l = table_log_d(fabs(static_cast<double>(a)), log_tab);
+    const double y = table_exp_d(fmin(fmax(static_cast<double>(b) * l, -120.0), 100.0), exp_tab);
+    float res = static_cast<float>(y);
+    if (a < 0.0f) {
+        const float t = truncf(b);
+        if (t != b) return __uint_as_float(0x7fc00000u);
+        // odd integer: |b| < 2^24 and its lowest bit set (larger floats are all even)
+        if (fabsf(b) < 16777216.0f && (static_cast<int>(fabsf(b)) & 1)) res = -res;
+    }
     return res;
 }
 
