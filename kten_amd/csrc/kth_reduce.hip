@@ -114,7 +114,7 @@ __device__ __forceinline__ void emit(const Geom& g, uint32_t o, uint32_t s, uint
 
 // ---------------------------------------------------------------- rows: inner == 1
 
-// G lanes per row (G in 1..64 a power of two, or 256 = the whole workgroup).
+// G lanes per row (G in {1, 2, 4, 16, 64}, or 256 = the whole workgroup).
 // VEC = 4 requires axis % 4 == 0 and seg_len % 4 == 0 so every row segment is 16-byte aligned.
 template <class R, int G, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
@@ -176,6 +176,98 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
         }
     } else {
         if (lane == 0 && row < g.outer) emit<R>(g, row, s, 0, acc, out, partial);
+    }
+}
+
+// ---------------------------------------------------------------- short rows: inner == 1, 8 <= axis < 256
+
+// Rows this short are contiguous in memory one after the other, so a workgroup takes a tile of
+// `rows` whole rows (a power of two in 32..1024, rows * axis <= kShortTile floats) as ONE contiguous
+// span: it is loaded with coalesced float4s whatever the row length, parked in LDS at an odd
+// row stride (conflict-free), and then `256 / rows` lanes fold each row from LDS, in index
+// order within a lane.
+constexpr uint32_t kShortTile = 8192;        // floats per tile: 32 KiB of LDS (+ padding)
+constexpr uint32_t kShortLoads = kShortTile / 4 / kBlock;
+
+struct ShortPlan {
+    uint32_t outer, axis, rows, stride;      // row length (axis, or axis * inner for slabs); stride = length | 1
+    uint32_t inner;                          // slabs only
+    FastDiv  axis_div, inner_div;
+};
+
+// Loads `floats` contiguous floats from `base` (16-byte aligned) and parks element e at
+// tile[(e / axis) * stride + e % axis].
+__device__ __forceinline__ void stage_short_tile(const float* __restrict__ base, uint32_t floats, const ShortPlan& pl, float* tile) {
+    float4 v[kShortLoads];
+#pragma unroll
+    for (uint32_t k = 0; k < kShortLoads; k++) {
+        const uint32_t e = (k * kBlock + threadIdx.x) * 4;
+        if (e + 4 <= floats) v[k] = ld4_stream(base + e);
+        else {
+            v[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (e < floats) v[k].x = base[e];
+            if (e + 1 < floats) v[k].y = base[e + 1];
+            if (e + 2 < floats) v[k].z = base[e + 2];
+        }
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kShortLoads; k++) {
+        const uint32_t e = (k * kBlock + threadIdx.x) * 4;
+        const float vals[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+            const uint32_t ee = e + j;
+            if (ee < floats) {
+                const uint32_t r = (__umulhi(ee, pl.axis_div.mul) + ee) >> pl.axis_div.shift;
+                tile[r * pl.stride + (ee - r * pl.axis)] = vals[j];
+            }
+        }
+    }
+}
+
+template <class R, int G>
+__global__ __launch_bounds__(kBlock) void reduce_short_rows_kernel(const float* __restrict__ in, float* __restrict__ out, ShortPlan pl) {
+    using Acc = typename R::Acc;
+    __shared__ float tile[kShortTile + kShortTile / 8 + 8];
+    const uint32_t first_row = blockIdx.x * pl.rows;
+    const uint32_t rows_here = min(pl.rows, pl.outer - first_row);
+    const uint32_t floats = rows_here * pl.axis;
+    stage_short_tile(in + static_cast<size_t>(first_row) * pl.axis, floats, pl, tile);      // rows * axis % 4 == 0: 16-byte aligned
+    __syncthreads();
+    // G > 1: G lanes per row, kBlock / G rows. G == 1: a thread takes rows r, r + kBlock, ...
+    const uint32_t lane = threadIdx.x % G;
+    for (uint32_t r = threadIdx.x / G; r < pl.rows; r += kBlock / G) {
+        Acc acc = R::init();
+        if (r < rows_here) {
+            const float* row = tile + r * pl.stride;
+            for (uint32_t j = lane; j < pl.axis; j += G) R::step(acc, row[j], j);
+        }
+#pragma unroll
+        for (int m = G / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
+        if (lane == 0 && r < rows_here) out[first_row + r] = R::finish(acc, pl.axis);
+    }
+}
+
+// The same staging for a reduction over a middle axis with a small inner size: a "row" is
+// the contiguous slab [axis, inner] of one outer index (pl.axis holds axis * inner), and the
+// outputs of the tile, rows * inner of them, are dealt to the threads in output order:
+// output (r, i) folds tile[r][j * inner + i] over j.
+template <class R>
+__global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float* __restrict__ in, float* __restrict__ out, ShortPlan pl) {
+    using Acc = typename R::Acc;
+    __shared__ float tile[kShortTile + kShortTile / 8 + 8];
+    const uint32_t first_row = blockIdx.x * pl.rows;
+    const uint32_t rows_here = min(pl.rows, pl.outer - first_row);
+    stage_short_tile(in + static_cast<size_t>(first_row) * pl.axis, rows_here * pl.axis, pl, tile);
+    __syncthreads();
+    const uint32_t outputs = rows_here * pl.inner, steps = pl.axis / pl.inner;
+    float* dst = out + static_cast<size_t>(first_row) * pl.inner;
+    for (uint32_t item = threadIdx.x; item < outputs; item += kBlock) {
+        const uint32_t r = (__umulhi(item, pl.inner_div.mul) + item) >> pl.inner_div.shift;
+        const float* p = tile + r * pl.stride + (item - r * pl.inner);
+        Acc acc = R::init();
+        for (uint32_t j = 0; j < steps; j++) R::step(acc, p[j * pl.inner], j);
+        dst[item] = R::finish(acc, steps);
     }
 }
 
@@ -356,6 +448,46 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     Geom g{outer, axis, inner, 1, axis};
     const uint64_t n_out = static_cast<uint64_t>(outer) * inner;
 
+    if (inner == 1 && axis >= 8 && axis < 256) {
+        // rows per tile: the largest power of two with rows * axis <= kShortTile, at most kBlock
+        ShortPlan pl{};
+        uint32_t rows = 4 * kBlock;
+        while (rows * axis > kShortTile) rows >>= 1;
+        pl.outer = outer; pl.axis = axis; pl.rows = rows; pl.stride = axis | 1u;
+        pl.axis_div = make_div(axis);
+        const dim3 grid(static_cast<uint32_t>(ceil_div(outer, rows)));
+        hipError_t e;
+        {
+            LaunchScope scope("reduce_short_rows_kernel", R::name, (static_cast<uint64_t>(outer) * axis + n_out) * 4);
+            switch (rows >= kBlock ? 1 : kBlock / rows) {
+            case 1: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 1>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
+            case 2: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 2>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
+            case 4: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 4>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
+            default: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 8>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
+            }
+            e = hipGetLastError();
+        }
+        if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+        return KTH_OK;
+    }
+
+    if (inner > 1 && inner < 64 && static_cast<uint64_t>(axis) * inner <= 256 && axis >= 2) {
+        ShortPlan pl{};
+        const uint32_t length = axis * inner;
+        uint32_t rows = 4 * kBlock;
+        while (rows * length > kShortTile) rows >>= 1;
+        pl.outer = outer; pl.axis = length; pl.rows = rows; pl.stride = length | 1u; pl.inner = inner;
+        pl.axis_div = make_div(length); pl.inner_div = make_div(inner);
+        hipError_t e;
+        {
+            LaunchScope scope("reduce_short_slabs_kernel", R::name, (static_cast<uint64_t>(outer) * length + n_out) * 4);
+            hipLaunchKernelGGL((reduce_short_slabs_kernel<R>), dim3(static_cast<uint32_t>(ceil_div(outer, rows))), dim3(kBlock), 0, stream, in, out, pl);
+            e = hipGetLastError();
+        }
+        if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+        return KTH_OK;
+    }
+
     enum { ROWS, COLS, STRIDED } kind;
     int G = 1, VEC = 1, WY = 4;
     uint32_t tiles = 0;
@@ -364,7 +496,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         kind = ROWS;
         VEC = (axis % 4 == 0) ? 4 : 1;
         const uint32_t per_lane = axis / VEC;          // loads per row
-        G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : 1;
+        G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : per_lane >= 2 ? 2 : 1;
         const uint64_t base_blocks = ceil_div(outer, kBlock / G);
         plan_segments(&g, base_blocks, target / 2, G * VEC, G * VEC * 16);
         blocks = base_blocks * g.segments;
@@ -403,10 +535,12 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
 #define ROWS_LAUNCH(GG, VV) hipLaunchKernelGGL((reduce_rows_kernel<R, GG, VV>), grid, dim3(kBlock), 0, stream, in, out, partial, g)
             if (VEC == 4) {
                 switch (G) { case 256: ROWS_LAUNCH(256, 4); break; case 64: ROWS_LAUNCH(64, 4); break;
-                             case 16: ROWS_LAUNCH(16, 4); break; case 4: ROWS_LAUNCH(4, 4); break; default: ROWS_LAUNCH(1, 4); }
+                             case 16: ROWS_LAUNCH(16, 4); break; case 4: ROWS_LAUNCH(4, 4); break; case 2: ROWS_LAUNCH(2, 4); break;
+                             default: ROWS_LAUNCH(1, 4); }
             } else {
                 switch (G) { case 256: ROWS_LAUNCH(256, 1); break; case 64: ROWS_LAUNCH(64, 1); break;
-                             case 16: ROWS_LAUNCH(16, 1); break; case 4: ROWS_LAUNCH(4, 1); break; default: ROWS_LAUNCH(1, 1); }
+                             case 16: ROWS_LAUNCH(16, 1); break; case 4: ROWS_LAUNCH(4, 1); break; case 2: ROWS_LAUNCH(2, 1); break;
+                             default: ROWS_LAUNCH(1, 1); }
             }
 #undef ROWS_LAUNCH
         } else if (kind == COLS) {

@@ -20,6 +20,11 @@ GEOMETRIES = [
     ([8, 64], 0), ([100, 256], 0), ([5000, 128], 0), ([70000, 64], 0), ([333, 1000], 0), ([40000, 65], 0),
     ([4, 50, 64], 1), ([3, 2000, 68], 1), ([2, 3, 4], 0), ([2, 3, 4], 1), ([6, 30000, 5], 1), ([10, 56, 56], 1),
     ([128, 56, 56], 1), ([64, 16, 49], 0), ([3, 17, 1, 9], 1), ([2, 2, 2, 2, 2, 2, 2, 2, 2, 5], 4),
+    # short rows staged through LDS (8 <= length < 256), every lanes-per-row variant, ragged last tile
+    ([5000, 8], 1), ([1030, 9], 1), ([777, 31], 1), ([3001, 32], 1), ([515, 50], 1), ([130, 100], 1), ([67, 129], 1),
+    ([33, 255], 1), ([1, 200], 1), ([300, 10], 1),
+    # short slabs (axis * inner <= 256, inner < 64)
+    ([5000, 8, 8], 1), ([1000, 2, 2], 1), ([999, 3, 40], 1), ([257, 16, 16], 1), ([100, 4, 63], 1), ([70, 2, 3, 5], 2),
 ]
 OPS = ["sum", "mean", "max", "min", "argMax", "argMin"]
 CODE = {"sum": "sum", "mean": "mean", "max": "max", "min": "min", "argMax": "arg_max", "argMin": "arg_min"}
@@ -56,7 +61,7 @@ def test_axis_reductions(shape, axis, gc):
 
 
 @pytest.mark.parametrize("shape,axis", [([64, 40], 1), ([9, 1000], 1), ([3, 5000], 1), ([333, 1000], 0), ([4, 50, 64], 1),
-                                        ([6, 3000, 5], 1), ([2, 70000], 1), ([70000, 64], 0)],
+                                        ([6, 3000, 5], 1), ([2, 70000], 1), ([70000, 64], 0), ([600, 100], 1), ([300, 12, 9], 1)],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
 def test_special_values_in_reductions(shape, axis, gc):
     """NaN propagation in max/min, NaN skipping in arg ops, signed zeros, lanes of -inf / +inf, ties."""
