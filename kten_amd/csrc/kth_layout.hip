@@ -9,8 +9,8 @@
 //   - permute reads the input through permuted strides.
 // When the innermost dim of the dense side is also contiguous on the strided side the copy
 // is a plain coalesced move (move_kernel, float4 when offsets allow). When the permutation
-// changes the innermost dim, 64x64 tiles go through LDS so that both the loads and the
-// stores are coalesced (permute_tile_kernel).
+// changes the innermost dim, tiles of 4096 elements go through LDS so that both the loads and
+// the stores are coalesced (permute_tile_kernel; 64 x 64, or narrow along a short dim).
 #include "kth_internal.h"
 
 using namespace kth;
@@ -19,11 +19,10 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kMoveUnroll = 2;
-constexpr int kTileDim = 64;
-constexpr int kTileRows = kBlock / kTileDim;          // rows of a tile one pass of the block covers
-constexpr int kTilePasses = kTileDim / kTileRows;
+constexpr int kTileElems = 4096;
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 
 // The strided side of a move. Dim 0 is the innermost dim of the dense side; for the float4
 // kernel size[0] is counted in float4s and stride[0] is 4. Strides and base are in floats.
@@ -102,17 +101,25 @@ struct TilePlan {
     uint32_t b_in[KTH_MAX_DIMS], b_out[KTH_MAX_DIMS];
 };
 
-// One 64x64 tile per workgroup: rows of 64 consecutive x are loaded (256 B per wave
-// instruction), parked in LDS with a padded row so the transposed read is conflict-free,
-// and rows of 64 consecutive y are stored.
-__global__ __launch_bounds__(kBlock) void permute_tile_kernel(const float* __restrict__ in, float* __restrict__ out, TilePlan pl) {
-    __shared__ float tile[kTileDim][kTileDim + 1];
+// One TX x TY tile of 4096 elements per workgroup (TX along the input's contiguous dim, TY
+// along the output's). Element k * 256 + t of the tile is loaded by thread t in x-fastest
+// order and stored in y-fastest order, so a wave instruction reads min(TX, 64) consecutive x
+// and writes min(TY, 64) consecutive y; 64 x 64 is the square case, the narrow shapes serve a
+// short x or y dim (channels-last images, small trailing dims), where consecutive rows of the
+// short dim are usually adjacent in memory and the accesses stay contiguous across rows.
+// The LDS row pitch TX + 1 is odd: both phases are free of bank conflicts.
+// V is the element: a float, or a float2 / float4 when the permutation keeps an innermost
+// dim of 2 or 4 floats in place (lengths, strides and offsets of the plan then count elements).
+template <int TX, int TY, class V>
+__global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restrict__ in, V* __restrict__ out, TilePlan pl) {
+    static_assert(TX * TY * sizeof(V) == kTileElems * sizeof(float), "a tile holds 16 KiB");
+    __shared__ V tile[TY * (TX + 1)];
     uint32_t t = blockIdx.x;
     uint32_t q = (__umulhi(t, pl.x_tiles_div.mul) + t) >> pl.x_tiles_div.shift;
-    const uint32_t x0 = (t - q * pl.x_tiles) * kTileDim;
+    const uint32_t x0 = (t - q * pl.x_tiles) * TX;
     t = q;
     q = (__umulhi(t, pl.y_tiles_div.mul) + t) >> pl.y_tiles_div.shift;
-    const uint32_t y0 = (t - q * pl.y_tiles) * kTileDim;
+    const uint32_t y0 = (t - q * pl.y_tiles) * TY;
     t = q;
     uint32_t in_off = 0, out_off = 0;
     for (int d = 0; d < pl.nbatch; d++) {
@@ -122,20 +129,88 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const float* __res
         out_off += r * pl.b_out[d];
         t = q;
     }
-    const uint32_t lx = threadIdx.x % kTileDim, ly = threadIdx.x / kTileDim;
-    float v[kTilePasses];
+    constexpr int kPasses = TX * TY / kBlock;
+    V v[kPasses];
 #pragma unroll
-    for (int k = 0; k < kTilePasses; k++) {
-        const uint32_t x = x0 + lx, y = y0 + ly + k * kTileRows;
+    for (int k = 0; k < kPasses; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        const uint32_t x = x0 + e % TX, y = y0 + e / TX;
         if (x < pl.x_len && y < pl.y_len) v[k] = __builtin_nontemporal_load(in + in_off + y * pl.y_in_stride + x);
     }
 #pragma unroll
-    for (int k = 0; k < kTilePasses; k++) tile[ly + k * kTileRows][lx] = v[k];
+    for (int k = 0; k < kPasses; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        tile[(e / TX) * (TX + 1) + e % TX] = v[k];
+    }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < kTilePasses; k++) {
-        const uint32_t x = x0 + ly + k * kTileRows, y = y0 + lx;
-        if (x < pl.x_len && y < pl.y_len) out[out_off + x * pl.x_out_stride + y] = tile[lx][ly + k * kTileRows];
+    for (int k = 0; k < kPasses; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        const uint32_t lx = e / TY, ly = e % TY;
+        const uint32_t x = x0 + lx, y = y0 + ly;
+        if (x < pl.x_len && y < pl.y_len) out[out_off + x * pl.x_out_stride + y] = tile[ly * (TX + 1) + lx];
+    }
+}
+
+// Many small transposes: the (x, y) slab of x_len * y_len floats is contiguous on both sides
+// and so is the batch dim right outside it, so a workgroup moves a run of whole slabs: one
+// contiguous span in, the same span out, the transposition done by the LDS addressing (rows
+// parked at an odd pitch).
+struct SlabPlan {
+    uint32_t x_len, y_len, slab, pitch;      // pitch = x_len | 1: LDS position of (y, x) is y * pitch + x
+    uint32_t group, groups, batch0;          // slabs per workgroup, workgroups per outer batch entry, slabs per outer entry
+    FastDiv  slab_div, x_div, y_div, groups_div;
+    int      nbatch;                         // batch dims outside the innermost one
+    uint32_t bsize[KTH_MAX_DIMS];
+    FastDiv  bdiv[KTH_MAX_DIMS];
+    uint32_t b_in[KTH_MAX_DIMS], b_out[KTH_MAX_DIMS];
+};
+
+constexpr uint32_t kSlabTile = 4096;
+
+__global__ __launch_bounds__(kBlock) void permute_slabs_kernel(const float* __restrict__ in, float* __restrict__ out, SlabPlan pl) {
+    __shared__ float tile[kSlabTile + kSlabTile / 2 + 8];
+    uint32_t t = blockIdx.x;
+    uint32_t q = (__umulhi(t, pl.groups_div.mul) + t) >> pl.groups_div.shift;
+    const uint32_t first = (t - q * pl.groups) * pl.group;
+    t = q;
+    uint32_t in_off = first * pl.slab, out_off = first * pl.slab;
+    for (int d = 0; d < pl.nbatch; d++) {
+        q = (__umulhi(t, pl.bdiv[d].mul) + t) >> pl.bdiv[d].shift;
+        const uint32_t r = t - q * pl.bsize[d];
+        in_off += r * pl.b_in[d];
+        out_off += r * pl.b_out[d];
+        t = q;
+    }
+    const uint32_t slabs = min(pl.group, pl.batch0 - first);
+    const uint32_t floats = slabs * pl.slab, lds_slab = pl.y_len * pl.pitch;
+    constexpr uint32_t kLoads = kSlabTile / kBlock;
+    float v[kLoads];
+#pragma unroll
+    for (uint32_t k = 0; k < kLoads; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        if (e < floats) v[k] = __builtin_nontemporal_load(in + in_off + e);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kLoads; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        if (e < floats) {                                     // input order inside a slab: (y, x), x fastest
+            const uint32_t g = (__umulhi(e, pl.slab_div.mul) + e) >> pl.slab_div.shift;
+            const uint32_t r = e - g * pl.slab;
+            const uint32_t y = (__umulhi(r, pl.x_div.mul) + r) >> pl.x_div.shift;
+            tile[g * lds_slab + y * pl.pitch + (r - y * pl.x_len)] = v[k];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < kLoads; k++) {
+        const uint32_t e = k * kBlock + threadIdx.x;
+        if (e < floats) {                                     // output order inside a slab: (x, y), y fastest
+            const uint32_t g = (__umulhi(e, pl.slab_div.mul) + e) >> pl.slab_div.shift;
+            const uint32_t r = e - g * pl.slab;
+            const uint32_t x = (__umulhi(r, pl.y_div.mul) + r) >> pl.y_div.shift;
+            out[out_off + e] = tile[g * lds_slab + (r - x * pl.y_len) * pl.pitch + x];
+        }
     }
 }
 
@@ -223,6 +298,96 @@ int box_of(const char* what, const int32_t* shape, int dims, const int32_t* firs
     return KTH_OK;
 }
 
+// Permutes through LDS tiles. `v`: the output's dims innermost first with the input's strides,
+// in units of `elem` floats (1, 2 or 4), stride[0] != 1. Returns KTH_OK after launching.
+int launch_tiles(const char* what, const StridedDims& v, int elem, const float* in, float* out, uint64_t n) {
+    int px = -1;
+    for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
+    if (px < 0) return fail(KTH_E_DEVICE, "%s: no contiguous input dim found", what);
+    const uint32_t x_len = static_cast<uint32_t>(v.size[px]), y_len = static_cast<uint32_t>(v.size[0]);
+    const uint32_t y_in_stride = static_cast<uint32_t>(v.stride[0]);
+    uint64_t x_out_stride = 1;
+    for (int d = 0; d < px; d++) x_out_stride *= v.size[d];
+    hipStream_t stream = state().stream;
+
+    // Batch dims: every dim but X and Y, innermost first, with input and output strides.
+    int nb = 0;
+    uint32_t bsize[KTH_MAX_DIMS], b_in[KTH_MAX_DIMS], b_out[KTH_MAX_DIMS];
+    uint64_t out_run = 1, batch = 1;
+    for (int d = 0; d < v.n; d++) {
+        if (d != px && d != 0) {
+            bsize[nb] = static_cast<uint32_t>(v.size[d]);
+            b_in[nb] = static_cast<uint32_t>(v.stride[d]);
+            b_out[nb] = static_cast<uint32_t>(out_run);
+            nb++;
+            batch *= v.size[d];
+        }
+        out_run *= v.size[d];
+    }
+
+    const uint32_t slab = x_len * y_len;
+    if (elem == 1 && slab <= kSlabTile / 2 && y_in_stride == x_len && x_out_stride == y_len && nb >= 1 &&
+        b_in[0] == slab && b_out[0] == slab) {
+        SlabPlan pl{};
+        pl.x_len = x_len; pl.y_len = y_len; pl.slab = slab; pl.pitch = x_len | 1u;
+        pl.batch0 = bsize[0];
+        pl.group = kSlabTile / slab;
+        if (pl.group > pl.batch0) pl.group = pl.batch0;
+        pl.groups = (pl.batch0 + pl.group - 1) / pl.group;
+        pl.slab_div = make_div(slab); pl.x_div = make_div(x_len); pl.y_div = make_div(y_len); pl.groups_div = make_div(pl.groups);
+        uint64_t outer = 1;
+        for (int d = 1; d < nb; d++) {
+            pl.bsize[pl.nbatch] = bsize[d]; pl.bdiv[pl.nbatch] = make_div(bsize[d]);
+            pl.b_in[pl.nbatch] = b_in[d]; pl.b_out[pl.nbatch] = b_out[d];
+            pl.nbatch++;
+            outer *= bsize[d];
+        }
+        const uint64_t blocks = static_cast<uint64_t>(pl.groups) * outer;
+        if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+        LaunchScope scope("permute_slabs_kernel", "", n * 8);
+        hipLaunchKernelGGL(permute_slabs_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, in, out, pl);
+        return KTH_OK;
+    }
+
+    TilePlan pl{};
+    pl.x_len = x_len; pl.y_len = y_len; pl.y_in_stride = y_in_stride;
+    pl.x_out_stride = static_cast<uint32_t>(x_out_stride);
+    // Tile shape: narrow along a dim shorter than 64 (the smallest power of two that holds it), square
+    // otherwise; vector elements use one shape of 16 KiB.
+    uint32_t tx = 64, ty = 64;
+    if (elem == 4) { tx = 32; ty = 32; }
+    else if (elem == 2) { tx = 64; ty = 32; }
+    else if (pl.x_len < 64 && pl.x_len <= pl.y_len) { tx = 2; while (tx < pl.x_len) tx <<= 1; ty = kTileElems / tx; }
+    else if (pl.y_len < 64) { ty = 2; while (ty < pl.y_len) ty <<= 1; tx = kTileElems / ty; }
+    pl.x_tiles = (pl.x_len + tx - 1) / tx;
+    pl.y_tiles = (pl.y_len + ty - 1) / ty;
+    pl.x_tiles_div = make_div(pl.x_tiles);
+    pl.y_tiles_div = make_div(pl.y_tiles);
+    pl.nbatch = nb;
+    for (int d = 0; d < nb; d++) { pl.bsize[d] = bsize[d]; pl.bdiv[d] = make_div(bsize[d]); pl.b_in[d] = b_in[d]; pl.b_out[d] = b_out[d]; }
+    const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
+    if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+    const dim3 grid(static_cast<uint32_t>(blocks));
+    LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
+    if (elem == 4) {
+        hipLaunchKernelGGL((permute_tile_kernel<32, 32, v4f>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const v4f*>(in),
+                           reinterpret_cast<v4f*>(out), pl);
+    } else if (elem == 2) {
+        hipLaunchKernelGGL((permute_tile_kernel<64, 32, v2f>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const v2f*>(in),
+                           reinterpret_cast<v2f*>(out), pl);
+    } else {
+#define KTH_TILE(TX, TY) hipLaunchKernelGGL((permute_tile_kernel<TX, TY, float>), grid, dim3(kBlock), 0, stream, in, out, pl)
+        switch (tx) {
+        case 2: KTH_TILE(2, 2048); break;    case 4: KTH_TILE(4, 1024); break;    case 8: KTH_TILE(8, 512); break;
+        case 16: KTH_TILE(16, 256); break;   case 32: KTH_TILE(32, 128); break;   case 64: KTH_TILE(64, 64); break;
+        case 128: KTH_TILE(128, 32); break;  case 256: KTH_TILE(256, 16); break;  case 512: KTH_TILE(512, 8); break;
+        case 1024: KTH_TILE(1024, 4); break; default: KTH_TILE(2048, 2); break;
+        }
+#undef KTH_TILE
+    }
+    return KTH_OK;
+}
+
 int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims, const int32_t* axes, uint64_t out) {
     uint64_t n;
     if (int rc = shape_count(shape, dims, what, &n)) return rc;
@@ -250,42 +415,26 @@ int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims
         raw.stride[k] = in_stride[axes[d]];
     }
     const StridedDims v = coalesce(raw);
+    if (v.stride[0] == 1 && (v.size[0] == 2 || v.size[0] == 4) && v.n >= 3) {
+        // An innermost dim of 2 or 4 floats that stays in place: permute float2 / float4 elements
+        // through tiles when the dims that do move are long enough to fill them.
+        const uint64_t elem = v.size[0];
+        StridedDims w{};
+        for (int d = 1; d < v.n; d++) { w.size[w.n] = v.size[d]; w.stride[w.n] = v.stride[d] / elem; w.n++; }
+        int wx = -1;
+        for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
+        if (w.stride[0] != 1 && wx > 0 && w.size[0] >= 16 && w.size[wx] >= 16) {
+            if (int rc = launch_tiles(what, w, static_cast<int>(elem), si->ptr, so->ptr, n)) return rc;
+            KTH_LAUNCH_CHECK("permute_tile_kernel");
+            return KTH_OK;
+        }
+    }
     if (v.stride[0] == 1) {
         launch_move<0>("move_kernel_permute", si->ptr, so->ptr, n, 0.0f, v, 0, n * 8);
         KTH_LAUNCH_CHECK("move_kernel");
         return KTH_OK;
     }
-    int px = -1;
-    for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
-    if (px < 0) return fail(KTH_E_DEVICE, "%s: no contiguous input dim found", what);
-    TilePlan pl{};
-    pl.x_len = static_cast<uint32_t>(v.size[px]);
-    pl.y_len = static_cast<uint32_t>(v.size[0]);
-    pl.y_in_stride = static_cast<uint32_t>(v.stride[0]);
-    pl.x_tiles = (pl.x_len + kTileDim - 1) / kTileDim;
-    pl.y_tiles = (pl.y_len + kTileDim - 1) / kTileDim;
-    pl.x_tiles_div = make_div(pl.x_tiles);
-    pl.y_tiles_div = make_div(pl.y_tiles);
-    uint64_t out_run = 1, batch = 1;
-    for (int d = 0; d < v.n; d++) {
-        if (d == px) pl.x_out_stride = static_cast<uint32_t>(out_run);
-        else if (d != 0) {
-            pl.bsize[pl.nbatch] = static_cast<uint32_t>(v.size[d]);
-            pl.bdiv[pl.nbatch] = make_div(pl.bsize[pl.nbatch]);
-            pl.b_in[pl.nbatch] = static_cast<uint32_t>(v.stride[d]);
-            pl.b_out[pl.nbatch] = static_cast<uint32_t>(out_run);
-            pl.nbatch++;
-            batch *= v.size[d];
-        }
-        out_run *= v.size[d];
-    }
-    const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
-    if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
-    {
-        LaunchScope scope("permute_tile_kernel", "", n * 8);
-        hipLaunchKernelGGL(permute_tile_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, state().stream,
-                           si->ptr, so->ptr, pl);
-    }
+    if (int rc = launch_tiles(what, v, 1, si->ptr, so->ptr, n)) return rc;
     KTH_LAUNCH_CHECK("permute_tile_kernel");
     return KTH_OK;
 }

@@ -111,7 +111,9 @@ def test_transpose_every_axis_pair(shape, gc):
 
 
 PERMUTE_SHAPES = [[2, 3, 2], [5, 6, 7], [8, 64, 68], [2, 3, 4, 5], [3, 4, 64, 65], [4, 16, 20, 24], [2, 2, 3, 3, 4, 4],
-                  [128, 3], [6, 1, 5, 1]]
+                  [128, 3], [6, 1, 5, 1],
+                  # float4 / float2 elements kept innermost; batched small slabs; narrow tiles with ragged edges
+                  [20, 33, 4], [17, 40, 2], [3, 18, 21, 4], [50, 6, 7], [1000, 16, 4], [70, 3, 100], [5, 9, 130, 3]]
 
 
 @pytest.mark.parametrize("shape", PERMUTE_SHAPES, ids=lambda s: "x".join(map(str, s)))
