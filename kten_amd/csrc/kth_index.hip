@@ -61,14 +61,28 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
     if (pos >= positions) return;
     uint32_t io, ao, bo;
     locate(pl, pos, io, ao, bo);
-    for (uint32_t i = 0; i < pl.i_axis_len; i++) {
-        const int sel = static_cast<int>(index[io + i * pl.i_axis_stride]);
-        if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
-        float* to = target + ao + static_cast<uint32_t>(sel) * pl.a_axis_stride;
-        if (MODE == 2) *to = value;
-        else {
-            const float v = src[bo + i * pl.b_axis_stride];
-            if (MODE == 1) *to = *to + v; else *to = v;
+    // The index and source values of kScatterBatch steps are loaded before the first of their
+    // stores, so the loads overlap; the stores stay in ascending order of i.
+    constexpr uint32_t kScatterBatch = 8;
+    for (uint32_t i0 = 0; i0 < pl.i_axis_len; i0 += kScatterBatch) {
+        float fi[kScatterBatch], fv[kScatterBatch];
+#pragma unroll
+        for (uint32_t k = 0; k < kScatterBatch; k++) {
+            if (i0 + k < pl.i_axis_len) {
+                fi[k] = index[io + (i0 + k) * pl.i_axis_stride];
+                if (MODE != 2) fv[k] = src[bo + (i0 + k) * pl.b_axis_stride];
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < kScatterBatch; k++) {
+            if (i0 + k < pl.i_axis_len) {
+                const int sel = static_cast<int>(fi[k]);
+                if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
+                float* to = target + ao + static_cast<uint32_t>(sel) * pl.a_axis_stride;
+                if (MODE == 2) *to = value;
+                else if (MODE == 1) *to = *to + fv[k];
+                else *to = fv[k];
+            }
         }
     }
 }

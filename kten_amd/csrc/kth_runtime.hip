@@ -337,6 +337,22 @@ int kth_read_scalar(uint64_t handle, uint64_t index, float* out) {
     return kth_download(out, handle, index, 1);
 }
 
+namespace {
+
+typedef float copy_v4f __attribute__((ext_vector_type(4)));
+
+// Store-to-store copy of n floats between 16-byte aligned addresses: one float4 per thread,
+// non-temporal load, ordinary store (the copy stays in the memory-side cache for the kernel
+// that reads it next); the last n % 4 floats are moved by workgroup 0.
+__global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ src, float* __restrict__ dst, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t n4 = n >> 2;
+    if (i < n4) reinterpret_cast<copy_v4f*>(dst)[i] = __builtin_nontemporal_load(reinterpret_cast<const copy_v4f*>(src) + i);
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) dst[(n4 << 2) + threadIdx.x] = src[(n4 << 2) + threadIdx.x];
+}
+
+}  // namespace
+
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
@@ -353,6 +369,14 @@ int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offse
         if (hi - lo < n) return fail(KTH_E_ARGUMENT, "kth_copy: overlapping ranges in one store");
     }
     State& s = state();
+    if (dst_offset % 4 == 0 && src_offset % 4 == 0 && n <= kMaxElements) {
+        LaunchScope scope("copy_kernel", "", n * 8);
+        const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + 255) / 256);
+        hipLaunchKernelGGL(copy_kernel, dim3(blocks == 0 ? 1 : blocks), dim3(256), 0, s.stream, sst->ptr + src_offset,
+                           d->ptr + dst_offset, static_cast<uint32_t>(n));
+        KTH_LAUNCH_CHECK("copy_kernel");
+        return KTH_OK;
+    }
     LaunchScope scope("memcpy_d2d", "", n * 8);
     KTH_HIP(hipMemcpyAsync(d->ptr + dst_offset, sst->ptr + src_offset, n * 4, hipMemcpyDeviceToDevice, s.stream));
     return KTH_OK;
