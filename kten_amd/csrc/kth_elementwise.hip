@@ -70,6 +70,7 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const float* a, float* ou
 
 __device__ LogEntry g_log_table[kLogTableEntries];
 __device__ double   g_exp_table[kExpTableEntries];
+__device__ double   g_atan_table[kAtanTableEntries];
 
 struct OpLogT {
     static constexpr const char* name = "OpLog";
@@ -116,6 +117,29 @@ struct OpCoshT {
     static __device__ __forceinline__ const double* table() { return g_exp_table; }
     static __device__ __forceinline__ float apply(float x, const double* lds) { return table_cosh(x, lds); }
 };
+
+struct OpAtanT {
+    static constexpr const char* name = "OpAtan";
+    static constexpr int kTableDoubles = kAtanTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_atan_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_atan(x, lds); }
+};
+struct OpAsinT {
+    static constexpr const char* name = "OpAsin";
+    static constexpr int kTableDoubles = kAtanTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_atan_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_asin(x, lds); }
+};
+struct OpAcosT {
+    static constexpr const char* name = "OpAcos";
+    static constexpr int kTableDoubles = kAtanTableEntries;
+    static __device__ __forceinline__ const double* table() { return g_atan_table; }
+    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_acos(x, lds); }
+};
+// sin, cos, tan need no table: reduction constants and Taylor coefficients are immediates.
+struct OpSinT { static constexpr const char* name = "OpSin"; static __device__ __forceinline__ float apply(float x, float, float) { return table_sin(x); } };
+struct OpCosT { static constexpr const char* name = "OpCos"; static __device__ __forceinline__ float apply(float x, float, float) { return table_cos(x); } };
+struct OpTanT { static constexpr const char* name = "OpTan"; static __device__ __forceinline__ float apply(float x, float, float) { return table_tan(x); } };
 
 // pow(tensor | Float): the common operands (finite non-zero base, finite exponent) go through
 // the exp / log tables, read from global memory (3 KiB, cache resident); zeros, infinities
@@ -558,10 +582,11 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
     case KTH_SINH: if (n32) launch_unary_lds<OpSinhT>(pa, po, n32); break;
     case KTH_COSH: if (n32) launch_unary_lds<OpCoshT>(pa, po, n32); break;
     case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
-    case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSin); break;
-    case KTH_COS: U(OpCos); break;           case KTH_TAN: U(OpTan); break;
-    case KTH_ASIN: U(OpAsin); break;         case KTH_ACOS: U(OpAcos); break;
-    case KTH_ATAN: U(OpAtan); break;         case KTH_FLOOR: U(OpFloor); break;
+    case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSinT); break;
+    case KTH_COS: U(OpCosT); break;          case KTH_TAN: U(OpTanT); break;
+    case KTH_ASIN: if (n32) launch_unary_lds<OpAsinT>(pa, po, n32); break;
+    case KTH_ACOS: if (n32) launch_unary_lds<OpAcosT>(pa, po, n32); break;
+    case KTH_ATAN: if (n32) launch_unary_lds<OpAtanT>(pa, po, n32); break;         case KTH_FLOOR: U(OpFloor); break;
     case KTH_CEIL: U(OpCeil); break;         case KTH_ROUND: U(OpRound); break;
     case KTH_TRUNC: U(OpTrunc); break;       case KTH_RSQRT: U(OpRsqrt); break;
     default: return fail(KTH_E_ARGUMENT, "kth_unary: op %d is not a unary map", op);
@@ -796,9 +821,13 @@ hipError_t init_math_tables() {
     }
     for (int i = 0; i < kExpTableEntries; i++)
         exp_tab[i] = static_cast<double>(exp2l(static_cast<long double>(i) / kExpTableEntries));
+    double atan_tab[kAtanTableEntries];
+    for (int i = 0; i < kAtanTableEntries; i++) atan_tab[i] = static_cast<double>(atanl(static_cast<long double>(i) / 64.0L));
     hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_log_table), log_tab, sizeof(log_tab));
     if (e != hipSuccess) return e;
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_exp_table), exp_tab, sizeof(exp_tab));
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_exp_table), exp_tab, sizeof(exp_tab));
+    if (e != hipSuccess) return e;
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_atan_table), atan_tab, sizeof(atan_tab));
 }
 
 }  // namespace kth

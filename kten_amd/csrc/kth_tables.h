@@ -23,6 +23,7 @@ namespace kth {
 
 constexpr int kLogTableEntries = 128;     // {invc, logc} pairs
 constexpr int kExpTableEntries = 128;
+constexpr int kAtanTableEntries = 65;     // atan(i / 64), i = 0..64
 
 struct LogEntry { double invc, logc; };
 
@@ -151,6 +152,124 @@ __device__ __forceinline__ float table_pow_finite(float a, float b, const LogEnt
         if (fabsf(b) < 16777216.0f && (static_cast<int>(fabsf(b)) & 1)) res = -res;
     }
     return res;
+}
+
+// ---------------------------------------------------------------- sin / cos / tan
+
+// Arguments up to 1e6 in magnitude are reduced in f64 by k = round(x * 2/pi) and
+// r = x - k * pi/2 with pi/2 split into 33 + 33 + 53 bits (k p1 and k p2 are exact products, the
+// subtractions of nearly equal values are exact), so r is good to about 1e-16 relative even
+// when x is the float closest to a multiple of pi/2. sin r and cos r on [-pi/4, pi/4] come from
+// their Taylor series (to r^17 and r^16: truncation below 1e-18). Larger arguments need a
+// multi-word reduction and take the library routine.
+constexpr double kTrigFastLimit = 1.0e6;
+
+__device__ __forceinline__ void sincos_reduced(double x, double& s, double& c, int& k) {
+    const double kd = rint(x * 0x1.45f306dc9c883p-1);
+    k = static_cast<int>(kd);
+    double r = fma(kd, -0x1.921fb54400000p+0, x);
+    r = fma(kd, -0x1.0b4611a600000p-34, r);
+    r = fma(kd, -0x1.3198a2e037073p-69, r);
+    if (kd == 0.0) r = x;                                    // keeps the sign of -0
+    const double z = r * r;
+    double p = fma(z, 1.0 / 355687428096000.0, -1.0 / 1307674368000.0);
+    p = fma(z, p, 1.0 / 6227020800.0);
+    p = fma(z, p, -1.0 / 39916800.0);
+    p = fma(z, p, 1.0 / 362880.0);
+    p = fma(z, p, -1.0 / 5040.0);
+    p = fma(z, p, 1.0 / 120.0);
+    p = fma(z, p, -1.0 / 6.0);
+    s = fma(r * z, p, r);
+    double q = fma(z, 1.0 / 20922789888000.0, -1.0 / 87178291200.0);
+    q = fma(z, q, 1.0 / 479001600.0);
+    q = fma(z, q, -1.0 / 3628800.0);
+    q = fma(z, q, 1.0 / 40320.0);
+    q = fma(z, q, -1.0 / 720.0);
+    q = fma(z, q, 1.0 / 24.0);
+    c = fma(z * z, q, fma(z, -0.5, 1.0));
+}
+
+// 1 / d for any normal d whose reciprocal is normal: hardware estimate and two Newton steps.
+__device__ __forceinline__ double newton_rcp_any(double d) {
+    double r = __builtin_amdgcn_rcp(d);
+    r = fma(fma(-d, r, 1.0), r, r);
+    r = fma(fma(-d, r, 1.0), r, r);
+    return r;
+}
+
+__device__ __forceinline__ float table_sin(float x) {
+    const double d = static_cast<double>(x);
+    if (!(fabs(d) <= kTrigFastLimit)) return static_cast<float>(sin(d));      // large, inf (-> NaN), NaN
+    double s, c; int k;
+    sincos_reduced(d, s, c, k);
+    const double y = (k & 1) ? c : s;
+    return static_cast<float>((k & 2) ? -y : y);
+}
+
+__device__ __forceinline__ float table_cos(float x) {
+    const double d = static_cast<double>(x);
+    if (!(fabs(d) <= kTrigFastLimit)) return static_cast<float>(cos(d));
+    double s, c; int k;
+    sincos_reduced(d, s, c, k);
+    const double y = (k & 1) ? s : c;
+    return static_cast<float>(((k + 1) & 2) ? -y : y);
+}
+
+__device__ __forceinline__ float table_tan(float x) {
+    const double d = static_cast<double>(x);
+    if (!(fabs(d) <= kTrigFastLimit)) return static_cast<float>(tan(d));
+    double s, c; int k;
+    sincos_reduced(d, s, c, k);
+    // cos r >= 0.7 on the reduced range; sin r of an odd quadrant is at least 1e-9 for a float argument
+    return static_cast<float>((k & 1) ? -c * newton_rcp_any(s) : s * newton_rcp_any(c));
+}
+
+// ---------------------------------------------------------------- atan / asin / acos
+
+// atan of a in [0, 1]: c = round(64 a) / 64, t = (a - c) / (1 + a c), atan a = atan c + atan t
+// with |t| <= 1/128, atan t by its Taylor series to t^9 (next term below 2^-77).
+__device__ __forceinline__ double atan_unit(double a, const double* tab) {
+    const double id = rint(a * 64.0);
+    const double c = id * 0.015625;
+    const double t = (a - c) * newton_rcp_any(fma(a, c, 1.0));
+    const double z = t * t;
+    double p = fma(z, 1.0 / 9.0, -1.0 / 7.0);
+    p = fma(z, p, 1.0 / 5.0);
+    p = fma(z, p, -1.0 / 3.0);
+    return tab[static_cast<int>(id)] + fma(t * z, p, t);
+}
+
+constexpr double kPio2Hi = 0x1.921fb54442d18p+0, kPio2Lo = 0x1.1a62633145c07p-54;
+
+// atan of a >= 0 (finite or inf).
+__device__ __forceinline__ double atan_positive(double a, const double* tab) {
+    if (a <= 1.0) return atan_unit(a, tab);
+    const double inv = a > 1.0e300 ? 0.0 : newton_rcp_any(a);
+    return (kPio2Hi - atan_unit(inv, tab)) + kPio2Lo;
+}
+
+__device__ __forceinline__ float table_atan(float x, const double* tab) {
+    float res = copysignf(static_cast<float>(atan_positive(fabs(static_cast<double>(x)), tab)), x);
+    if (x != x) res = x;
+    return res;
+}
+
+// asin a = 2 atan(a / (1 + sqrt((1 - a)(1 + a)))) on [0, 1]; NaN outside [-1, 1] (Math.asin).
+__device__ __forceinline__ float table_asin(float x, const double* tab) {
+    const double a = fabs(static_cast<double>(x));
+    if (!(a <= 1.0)) return __uint_as_float(0x7fc00000u);
+    const double w = sqrt((1.0 - a) * (1.0 + a));
+    const double u = a * newton_rcp_any(1.0 + w);
+    return copysignf(static_cast<float>(2.0 * atan_unit(u, tab)), x);
+}
+
+// acos x = 2 atan(sqrt((1 - x) / (1 + x))) on (-1, 1], pi at -1; NaN outside [-1, 1] (Math.acos).
+__device__ __forceinline__ float table_acos(float x, const double* tab) {
+    const double d = static_cast<double>(x);
+    if (!(fabs(d) <= 1.0)) return __uint_as_float(0x7fc00000u);
+    if (d == -1.0) return static_cast<float>(2.0 * kPio2Hi);
+    const double ratio = (1.0 - d) * newton_rcp_any(1.0 + d);
+    return static_cast<float>(2.0 * atan_positive(sqrt(ratio), tab));
 }
 
 }  // namespace kth
