@@ -212,6 +212,23 @@ public:
     void zeroOut(const Raw& t);                                     // :26
     Raw pow(float constant, const Raw& t);                          // :39
     Raw concat(int axis, const std::vector<Raw>& inputs);           // :41
+
+    // TensorOperations.kt:129 batchNorm(axis, momentum, epsilon, training): BatchNormOperation
+    // (kten-api/.../tensor/operations/nn/BatchNormOperation.kt:5-41). Absent tensors are null.
+    struct BatchNormOutputs { Raw output, currentMean, currentStd; };
+    struct BatchNormGrads { Raw gradIn, gradGamma, gradBeta; };
+    class BatchNorm {
+    public:
+        BatchNorm(int axis, float momentum, float epsilon, bool training, HipTensorOperations* ops)
+            : axis_(axis), momentum_(momentum), epsilon_(epsilon), training_(training), ops_(ops) {}
+        BatchNormOutputs calculateOutput(const Raw& input, const Raw& runningMean, const Raw& runningVar, const Raw& gamma, const Raw& beta);
+        BatchNormGrads calculateGrads(const Raw& input, const Raw& runningMean, const Raw& runningVar, const Raw& currentMean,
+                                      const Raw& currentStd, const Raw& gamma, const Raw& gradOut,
+                                      bool inRequiresGrad, bool gammaRequiresGrad, bool betaRequiresGrad);
+    private:
+        int axis_; float momentum_, epsilon_; bool training_; HipTensorOperations* ops_;
+    };
+    BatchNorm batchNorm(int axis, float momentum, float epsilon, bool training) { return BatchNorm(axis, momentum, epsilon, training, this); }
     void release(const Raw& t);                                     // :22
     void incrementRef(const Raw& t);                                // :28
     void markSurviveGC(const Raw& t);                               // :30-33 / OCLTensorOperations.kt:96-98
@@ -621,6 +638,31 @@ inline Raw HipTensorOperations::concat(int axis, const std::vector<Raw>& inputs)
         last += t->shape[a];
     }
     return res;
+}
+inline HipTensorOperations::BatchNormOutputs HipTensorOperations::BatchNorm::calculateOutput(
+        const Raw& input, const Raw& runningMean, const Raw& runningVar, const Raw& gamma, const Raw& beta) {
+    const int axis = normalizeAxis(input->shape, axis_);
+    const auto h = [](const Raw& t) -> uint64_t { return t ? t->storeReference : 0; };
+    BatchNormOutputs r{ops_->createRaw(input->shape), ops_->createRaw({input->shape[axis]}), ops_->createRaw({input->shape[axis]})};
+    check(kth_batch_norm_forward(input->storeReference, input->shape.data(), input->dimensions(), axis, training_ ? 1 : 0, momentum_,
+                                 epsilon_, h(runningMean), h(runningVar), h(gamma), h(beta), r.output->storeReference,
+                                 r.currentMean->storeReference, r.currentStd->storeReference));
+    return r;
+}
+inline HipTensorOperations::BatchNormGrads HipTensorOperations::BatchNorm::calculateGrads(
+        const Raw& input, const Raw& runningMean, const Raw& runningVar, const Raw& currentMean, const Raw& currentStd,
+        const Raw& gamma, const Raw& gradOut, bool inRequiresGrad, bool gammaRequiresGrad, bool betaRequiresGrad) {
+    BatchNormGrads r{};
+    if (!inRequiresGrad && !gammaRequiresGrad && !betaRequiresGrad) return r;          // JVMBatchNorm.kt:113-115
+    const int axis = normalizeAxis(input->shape, axis_);
+    const auto h = [](const Raw& t) -> uint64_t { return t ? t->storeReference : 0; };
+    if (inRequiresGrad) r.gradIn = ops_->createRaw(input->shape);
+    if (gammaRequiresGrad) r.gradGamma = ops_->createRaw({input->shape[axis]});
+    if (betaRequiresGrad) r.gradBeta = ops_->createRaw({input->shape[axis]});
+    check(kth_batch_norm_backward(input->storeReference, input->shape.data(), input->dimensions(), axis, training_ ? 1 : 0, epsilon_,
+                                  h(runningMean), h(runningVar), h(currentMean), h(currentStd), h(gamma), gradOut->storeReference,
+                                  h(r.gradIn), h(r.gradGamma), h(r.gradBeta)));
+    return r;
 }
 inline void HipTensorOperations::release(const Raw& t) { t->release(); }
 inline void HipTensorOperations::incrementRef(const Raw& t) { t->incrementRef(); }

@@ -131,6 +131,23 @@ int main() {
         expect_illegal_argument([&] { pm->permute({0, 0, 1}); }, "permute must name every axis");
         expect_illegal_argument([&] { tr->transpose(1, -1); }, "transpose needs two different axes");
 
+        // BatchNormOperation, inference mode (TensorTestsBase.kt:2064-2084): (x - mean) / sqrt(var + eps) * gamma + beta
+        Raw bx = tensor(ops, {2, 2, 2}, {1, 2, 3, 4, 5, 6, 7, 8});
+        Raw bmean = tensor(ops, {2}, {1, 3}), bvar = tensor(ops, {2}, {3, 15}), bgamma = tensor(ops, {2}, {2, 4}), bbeta = tensor(ops, {2}, {1, -1});
+        auto bn = ops.batchNorm(1, 0.1f, 1.0f, false).calculateOutput(bx, bmean, bvar, bgamma, bbeta);
+        expect_values(bn.output, {2, 2, 2}, {1, 2, -1, 0, 5, 6, 3, 4}, 0.0f, "batchNorm inference: exact for var + eps = 4 and 16");
+        // training mode: channel mean and the reciprocal standard deviation (biased variance 4.25, eps 0)
+        auto bt = ops.batchNorm(1, 0.1f, 0.0f, true).calculateOutput(bx, nullptr, nullptr, nullptr, nullptr);
+        expect_values(bt.currentMean, {2}, {3.5f, 5.5f}, 0.0f, "batchNorm training: channel means");
+        expect_values(bt.currentStd, {2}, {0.48507125f, 0.48507125f}, 1e-7f, "batchNorm training: 1 / sqrt(var)");
+        auto bg = ops.batchNorm(1, 0.1f, 0.0f, true).calculateGrads(bx, nullptr, nullptr, bt.currentMean, bt.currentStd, nullptr,
+                                                                    ops.createRawFill({2, 2, 2}, 1.0f), true, false, true);
+        expect_values(bg.gradBeta, {2}, {4, 4}, 0.0f, "batchNorm gradBeta = sum of gradOut");
+        expect_values(bg.gradIn, {2, 2, 2}, {0, 0, 0, 0, 0, 0, 0, 0}, 1e-6f, "batchNorm gradIn of a constant gradient is zero");
+        expect(bg.gradGamma == nullptr, "a gradient that is not required is not produced");
+        expect_illegal_argument([&] { ops.batchNorm(1, 0.1f, 1e-3f, false).calculateOutput(bx, nullptr, nullptr, nullptr, nullptr); },
+                                "inference mode needs running statistics");
+
         // in-place arithmetic and NaN detection
         Raw acc = ops.zerosLike(t1);
         acc->plusAssign(t1);
