@@ -93,7 +93,7 @@ def cpu_baseline(name, threads):
     from oracle import jvm_oracle as jo
     wl = WORKLOADS[name]
     sample = {"cfg1": dict(wl.full_dims), "cfg2": dict(wl.full_dims), "cfg3": dict(wl.full_dims),
-              "cfg4": dict(wl.full_dims), "cfg5": {"rows": 8192, "cols": 4096},
+              "cfg4": dict(wl.full_dims), "cfg5": dict(wl.full_dims),
               "max_backward": dict(wl.full_dims), "softmax_ce": {"batch": 8192, "classes": 2048}}.get(name, dict(wl.full_dims))
     inputs = wl.make_inputs(sample)
     jo.set_threads(threads)
