@@ -196,6 +196,16 @@ int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t 
 int kth_scatter_fill(uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
                      int dims, int axis, float value);
 
+/* indexSelect (RAW:236; JVM:484-501): index holds k floats; out has `shape` with the axis
+ * resized to k: out[p, i] = in[p, (int) index[i]]. Blocking: an index outside
+ * [0, shape[axis]) returns KTH_E_ARGUMENT (JVM:494-496). */
+int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint64_t index, uint64_t k, uint64_t out);
+
+/* indexAdd (RAW:238; JVM:503-516): target[p, (int) index[i]] += src[p, i] * alpha, i
+ * ascending, so repeated indices accumulate in index order. src has `shape` with the axis
+ * resized to k (checked on the host by ShapeFunctions.kt:280-293). Blocking, as above. */
+int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uint64_t index, uint64_t k, uint64_t src, float alpha);
+
 /* ------------------------------------------------------------------ layout movers */
 
 /* get(Array<IntRange>) (RAW:29; JVM:276-280) and narrow (RAW:232; JVM:468-473): copies the

@@ -58,6 +58,8 @@ SIGNATURES = {
     "kth_scatter": (c_int, [c_int, c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32),
                             c_int, c_int]),
     "kth_scatter_fill": (c_int, [c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_int, c_int, c_float]),
+    "kth_index_select": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_uint64, c_uint64, c_uint64]),
+    "kth_index_add": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_uint64, c_uint64, c_uint64, c_float]),
     "kth_get_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_uint64]),
     "kth_set_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_uint64, c_uint64]),
     "kth_fill_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_float]),

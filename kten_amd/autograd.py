@@ -182,6 +182,7 @@ class AGTensor(Tensor):
     def max(self, axis, keepDimensions=False): return Max(self.ops)(self, axis, keepDimensions)
     def min(self, axis, keepDimensions=False): return Min(self.ops)(self, axis, keepDimensions)
     def gather(self, axis, index): return Gather(self.ops)(self, axis, index)
+    def indexSelect(self, axis, index): return IndexSelect(self.ops)(self, index, axis)           # AGTensor.kt:305-307
     def scatter(self, axis, index, source): return Scatter(self.ops)(self, axis, index, source)
 
     def batchNorm(self, axis, runningMean, runningVar, training, momentum=0.1, epsilon=1e-5, gamma=None, beta=None):
@@ -298,6 +299,7 @@ class NoGradVariable(AGTensor):
     def max(self, axis, keepDimensions=False): return self._new(self.rawValue.max(axis, keepDimensions))
     def min(self, axis, keepDimensions=False): return self._new(self.rawValue.min(axis, keepDimensions))
     def gather(self, axis, index): return self._new(self.rawValue.gather(axis, index.getRawValue()))          # :196
+    def indexSelect(self, axis, index): return self._new(self.rawValue.indexSelect(axis, index.getRawValue()))   # :202
 
     def scatter(self, axis, index, source):                                                                   # :198-202
         if source.requiresGrad:
@@ -1191,6 +1193,29 @@ class Permute(UnaryTensorFunction):                                             
 
     def doBackward(self, gradient):
         return [gradient.permute(self.reverseShapeIndices)]
+
+
+class IndexSelect(UnaryTensorFunction):                                               # :314-347
+    modifiesShape = True
+
+    def __call__(self, tensor, index, axis):
+        if index.requiresGrad:
+            raise ValueError("Index select cannot differentiate the index. The index tensor passed to index select should "
+                             "never require gradients.")
+        normAxis, outputShape = sf.index_select_norm_axis_shape(tensor.shape, axis, index.shape)
+        super().__call__(tensor)
+        self.cachedShape = outputShape
+        self.originalTensorShape = list(tensor.shape)
+        self.axis, self.index = normAxis, index
+        return self
+
+    def doForward(self, input):
+        self.output = input.indexSelect(self.axis, self.index.getRawValue())
+
+    def doBackward(self, gradient):
+        gradInput = self.ops.createRawFill(self.originalTensorShape, 0.0)
+        gradInput.indexAdd(self.axis, self.index.getRawValue(), gradient)
+        return [gradInput]
 
 
 class Concat(AnyTensorFunction):                                                      # :349-378

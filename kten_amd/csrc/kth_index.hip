@@ -87,6 +87,58 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
     }
 }
 
+// indexSelect / indexAdd (JVMRawTensor.kt:484-516): the index is one list of k rows along the
+// axis, shared by every position. The tensor is seen as [outer, axis, inner].
+struct RowsPlan {
+    uint32_t axis_len, k, inner;       // inner in the kernel's units (float4s for the vector form)
+    FastDiv  inner_div, k_div;
+};
+
+// One thread per unit of the result [outer, k, inner]: out[o, i, :] = in[o, index[i], :].
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void index_select_kernel(const float* __restrict__ in, const float* __restrict__ index,
+                                                             float* __restrict__ out, uint32_t units, RowsPlan pl, int* bad) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= units) return;
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t col = e - row * pl.inner;
+    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
+    const int sel = static_cast<int>(index[row - o * pl.k]);
+    if (sel < 0 || static_cast<uint32_t>(sel) >= pl.axis_len) { *bad = 1; return; }
+    const uint32_t from = (o * pl.axis_len + static_cast<uint32_t>(sel)) * pl.inner + col;
+    if (VEC) reinterpret_cast<float4*>(out)[e] = reinterpret_cast<const float4*>(in)[from];
+    else out[e] = in[from];
+}
+
+// One thread per position (o, column): target[o, index[i], column] += src[o, i, column] * alpha
+// for i ascending, so repeated indices accumulate in index order as on the JVM.
+__global__ __launch_bounds__(kBlock) void index_add_kernel(float* __restrict__ target, const float* __restrict__ index,
+                                                          const float* __restrict__ src, float alpha, uint32_t positions,
+                                                          RowsPlan pl, int* bad) {
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= positions) return;
+    const uint32_t o = (__umulhi(p, pl.inner_div.mul) + p) >> pl.inner_div.shift;
+    const uint32_t col = p - o * pl.inner;
+    float* t = target + static_cast<size_t>(o) * pl.axis_len * pl.inner + col;
+    const float* s = src + static_cast<size_t>(o) * pl.k * pl.inner + col;
+    constexpr uint32_t kBatch = 8;
+    for (uint32_t i0 = 0; i0 < pl.k; i0 += kBatch) {
+        float fi[kBatch], fv[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; j++)
+            if (i0 + j < pl.k) { fi[j] = index[i0 + j]; fv[j] = s[static_cast<size_t>(i0 + j) * pl.inner]; }
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; j++) {
+            if (i0 + j < pl.k) {
+                const int sel = static_cast<int>(fi[j]);
+                if (sel < 0 || static_cast<uint32_t>(sel) >= pl.axis_len) { *bad = 1; continue; }
+                float* to = t + static_cast<size_t>(sel) * pl.inner;
+                *to = *to + fv[j] * alpha;
+            }
+        }
+    }
+}
+
 __global__ void clear_int_kernel(int* p) { *p = 0; }
 
 int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
@@ -242,6 +294,76 @@ int kth_scatter_fill(uint64_t target, const int32_t* target_shape, uint64_t inde
                      int dims, int axis, float value) {
     std::lock_guard<std::mutex> g(lock());
     return scatter_common(2, target, target_shape, index, index_shape, 0, nullptr, dims, axis, value);
+}
+
+static int rows_geometry(const char* what, const int32_t* shape, int dims, int axis, uint64_t* outer, uint64_t* inner, uint64_t* total) {
+    if (dims < 1 || dims > KTH_MAX_DIMS) return fail(KTH_E_ARGUMENT, "%s: %d dims", what, dims);
+    if (axis < 0 || axis >= dims) return fail(KTH_E_ARGUMENT, "%s: axis %d of %d dims", what, axis, dims);
+    if (int rc = shape_count(shape, dims, what, total)) return rc;
+    *outer = 1; *inner = 1;
+    for (int d = 0; d < axis; d++) *outer *= static_cast<uint64_t>(shape[d]);
+    for (int d = axis + 1; d < dims; d++) *inner *= static_cast<uint64_t>(shape[d]);
+    return KTH_OK;
+}
+
+int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint64_t index, uint64_t k, uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    uint64_t outer, inner, total;
+    if (int rc = rows_geometry("kth_index_select", shape, dims, axis, &outer, &inner, &total)) return rc;
+    const uint64_t n_out = outer * k * inner;
+    if (n_out > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_select: more than 2^31-1 result elements");
+    Store* si = lookup(in, "kth_index_select(in)");
+    if (!si) return KTH_E_HANDLE;
+    Store* sx = lookup(index, "kth_index_select(index)");
+    if (!sx) return KTH_E_HANDLE;
+    Store* so = lookup(out, "kth_index_select(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (total > si->n_floats || k > sx->n_floats || n_out > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_index_select: a shape needs more elements than its store holds");
+    if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_index_select: output aliases an input");
+    if (n_out == 0) return KTH_OK;
+    const bool vec = inner % 4 == 0;
+    RowsPlan pl{};
+    pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k);
+    pl.inner = static_cast<uint32_t>(vec ? inner / 4 : inner);
+    pl.inner_div = make_div(pl.inner); pl.k_div = make_div(pl.k);
+    const uint32_t units = static_cast<uint32_t>(vec ? n_out / 4 : n_out);
+    const uint32_t blocks = (units + kBlock - 1) / kBlock;
+    return with_index_check("Index select", [&](int* flag) {
+        LaunchScope scope("index_select_kernel", vec ? "float4" : "float", 2 * n_out * 4 + k * 4);
+        if (vec) hipLaunchKernelGGL((index_select_kernel<true>), dim3(blocks), dim3(kBlock), 0, state().stream, si->ptr, sx->ptr, so->ptr, units, pl, flag);
+        else     hipLaunchKernelGGL((index_select_kernel<false>), dim3(blocks), dim3(kBlock), 0, state().stream, si->ptr, sx->ptr, so->ptr, units, pl, flag);
+    });
+}
+
+int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uint64_t index, uint64_t k, uint64_t src, float alpha) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    uint64_t outer, inner, total;
+    if (int rc = rows_geometry("kth_index_add", shape, dims, axis, &outer, &inner, &total)) return rc;
+    const uint64_t n_src = outer * k * inner;
+    if (n_src > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_add: more than 2^31-1 source elements");
+    Store* st = lookup(target, "kth_index_add(target)");
+    if (!st) return KTH_E_HANDLE;
+    Store* sx = lookup(index, "kth_index_add(index)");
+    if (!sx) return KTH_E_HANDLE;
+    Store* ss = lookup(src, "kth_index_add(src)");
+    if (!ss) return KTH_E_HANDLE;
+    if (total > st->n_floats || k > sx->n_floats || n_src > ss->n_floats)
+        return fail(KTH_E_ARGUMENT, "kth_index_add: a shape needs more elements than its store holds");
+    if (st->ptr == sx->ptr || st->ptr == ss->ptr) return fail(KTH_E_ARGUMENT, "kth_index_add: target aliases an input");
+    const uint64_t positions = outer * inner;
+    if (positions == 0 || k == 0) return KTH_OK;
+    RowsPlan pl{};
+    pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k); pl.inner = static_cast<uint32_t>(inner);
+    pl.inner_div = make_div(pl.inner); pl.k_div = make_div(pl.k);
+    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+    return with_index_check("Index Add", [&](int* flag) {
+        LaunchScope scope("index_add_kernel", "", 3 * n_src * 4 + k * 4);
+        hipLaunchKernelGGL(index_add_kernel, dim3(blocks), dim3(kBlock), 0, state().stream, st->ptr, sx->ptr, ss->ptr, alpha,
+                           static_cast<uint32_t>(positions), pl, flag);
+    });
 }
 
 }  // extern "C"

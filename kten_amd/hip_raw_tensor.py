@@ -212,6 +212,20 @@ class HipRawTensor(AbstractRawTensor):
                                        index.storeReference, abi.shape_array(index.shape), src.storeReference,
                                        abi.shape_array(src.shape), self.dimensions, a))
 
+    def _index_select(self, axis, index, resShape):
+        """JVMRawTensor.kt:484-501."""
+        self._require_live(); index._require_live()
+        res = self._new(resShape)
+        check(self.ops.lib.kth_index_select(self.storeReference, abi.shape_array(self.shape), self.dimensions, axis,
+                                            index.storeReference, index.shape[0], res.storeReference))
+        return res
+
+    def _index_add(self, axis, index, src, alpha):
+        """JVMRawTensor.kt:503-516."""
+        self._require_live(); index._require_live(); src._require_live()
+        check(self.ops.lib.kth_index_add(self.storeReference, abi.shape_array(self.shape), self.dimensions, axis,
+                                         index.storeReference, index.shape[0], src.storeReference, alpha))
+
     # --- layout movers -------------------------------------------------------------------
     def _get_store_range(self, offset, length, resShape):
         """JVMRawTensor.kt:270-274: one contiguous store range."""

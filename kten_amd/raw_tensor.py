@@ -8,8 +8,8 @@ common-shape calculation) restated once here so that every backend shares them, 
 the reference. Kotlin's overloads on (tensor | Float) become one Python method that
 dispatches on the argument type; Kotlin operators are also exposed as Python operators.
 
-Members of the contract that lie outside the accelerated path (indexSelect/indexAdd, dot,
-BLAS, nn) are not part of this mirror.
+Members of the contract that lie outside the accelerated path (dot, BLAS, nn other than
+batch normalisation) are not part of this mirror.
 """
 from enum import Enum
 from typing import List, Sequence
@@ -295,6 +295,18 @@ class AbstractRawTensor:
         ranges = sf.to_index_ranges(self.shape)
         ranges[a] = sf.IntRange(start, start + length - 1)
         return self.get(ranges)
+
+    # --- indexSelect / indexAdd (AbstractRawTensor.kt:236-238) ---------------------------
+    def _index_select(self, axis: int, index, resShape): raise NotImplementedError
+    def _index_add(self, axis: int, index, src, alpha: float): raise NotImplementedError
+
+    def indexSelect(self, axis: int, index):
+        a, res_shape = sf.index_select_norm_axis_shape(self.shape, axis, index.shape)
+        return self._index_select(a, index, res_shape)
+
+    def indexAdd(self, axis: int, index, src, alpha: float = 1.0):
+        a = sf.index_add_check_shapes_norm_axis(self.shape, axis, index.shape, src.shape)
+        self._index_add(a, index, src, float(alpha))
 
     # --- broadcasting (AbstractRawTensor.kt:170-192) -----------------------------------
     def calculateCommonShapeWith(self, other) -> List[int]:

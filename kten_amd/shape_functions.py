@@ -233,6 +233,30 @@ def full_ranges(shape: Sequence[int], norm_ranges: Sequence[IntRange]):
     return first, last
 
 
+def index_select_norm_axis_shape(shape: Sequence[int], axis: int, index_shape: Sequence[int]):
+    """ShapeFunctions.kt:270-278."""
+    a = normalize_axis(shape, axis)
+    if len(index_shape) != 1:
+        raise ValueError(f"Index select requires singleton tensor as index, but got index tensor with shape: {list(index_shape)}")
+    res = list(shape)
+    res[a] = index_shape[0]
+    return a, res
+
+
+def index_add_check_shapes_norm_axis(shape: Sequence[int], axis: int, index_shape: Sequence[int], src_shape: Sequence[int]) -> int:
+    """ShapeFunctions.kt:280-293."""
+    if len(index_shape) != 1:
+        raise ValueError(f"Index add requires index tensor to have 1 dimension, but got tensor with shape: {list(index_shape)}")
+    a = normalize_axis(shape, axis)
+    expected = list(shape)
+    expected[a] = index_shape[0]
+    if list(src_shape) != expected:
+        raise ValueError("Index add expects source tensor to have same size as index size at the specified axis, and same size "
+                         f"as this tensor for every other axis, but got source tensor with shape: {list(src_shape)} axis: {axis} "
+                         f"and this tensor have shape: {list(shape)}")
+    return a
+
+
 def to_index_ranges(shape: Sequence[int]) -> List[IntRange]:
     """ShapeFunctions.kt:310-312."""
     return [IntRange(0, s - 1) for s in shape]

@@ -74,6 +74,10 @@ def lib():
     L.kjo_scatter.restype = c_int
     L.kjo_scatter_fill.argtypes = [fp, ip, fp, ip, c_int, c_int, c_float]
     L.kjo_scatter_fill.restype = c_int
+    L.kjo_index_select.argtypes = [fp, ip, c_int, c_int, fp, c_int64, fp]
+    L.kjo_index_select.restype = c_int
+    L.kjo_index_add.argtypes = [fp, ip, c_int, c_int, fp, c_int64, fp, c_float]
+    L.kjo_index_add.restype = c_int
     L.kjo_range_size.argtypes = [ip, c_int, ip, ip]
     L.kjo_range_size.restype = c_int64
     L.kjo_get_range.argtypes = [fp, ip, c_int, ip, ip, fp]
@@ -345,6 +349,18 @@ class JvmOracleRawTensor(AbstractRawTensor):
                                    _sh(index.shape), _p(src.storeReference), _sh(src.shape), self.dimensions, a)
         if rc != 0:
             raise ValueError("Scatter got invalid index, an index value is out of bounds at the axis")
+
+    def _index_select(self, axis, index, resShape):
+        out = np.zeros(sf.to_store_size(resShape), dtype=np.float32)
+        if lib().kjo_index_select(_p(self.storeReference), _sh(self.shape), self.dimensions, axis, _p(index.storeReference),
+                                  index.storeReference.size, _p(out)) != 0:
+            raise ValueError("Index select got invalid index, an index value is out of bounds at the axis")
+        return JvmOracleRawTensor(list(resShape), out, self.ops)
+
+    def _index_add(self, axis, index, src, alpha):
+        if lib().kjo_index_add(_p(self.storeReference), _sh(self.shape), self.dimensions, axis, _p(index.storeReference),
+                               index.storeReference.size, _p(src.storeReference), alpha) != 0:
+            raise ValueError("Index Add got invalid index, an index value is out of bounds at the axis")
 
     def _get_store_range(self, offset, length, resShape):                      # JVM:270-274 sliceArray
         return JvmOracleRawTensor(list(resShape), self.storeReference[offset:offset + length].copy(), self.ops)

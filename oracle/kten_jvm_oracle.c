@@ -392,6 +392,43 @@ int kjo_scatter_fill(float* target, const int32_t* target_shape, const float* in
     return 0;
 }
 
+/* JVM:484-501 indexSelect: index is 1-D with k entries; res has this tensor's shape with the
+ * axis resized to k; res[p, i] = this[p, (int) index[i]] for every position p without the
+ * axis. Returns -1 at an index outside [0, shape[axis]) (IllegalArgumentException). */
+int kjo_index_select(const float* in, const int32_t* shape, int dims, int axis, const float* index, int64_t k, float* out) {
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < axis; d++) outer *= shape[d];
+    for (int d = axis + 1; d < dims; d++) inner *= shape[d];
+    const int64_t len = shape[axis];
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t j = 0; j < inner; j++)
+            for (int64_t i = 0; i < k; i++) {
+                const int32_t sel = f2i(index[i]);
+                if (sel < 0 || sel >= len) return -1;
+                out[(o * k + i) * inner + j] = in[(o * len + sel) * inner + j];
+            }
+    return 0;
+}
+
+/* JVM:503-516 indexAdd: this[p, (int) index[i]] += src[p, i] * alpha, i ascending within a
+ * position, so repeated indices accumulate in index order. */
+int kjo_index_add(float* target, const int32_t* shape, int dims, int axis, const float* index, int64_t k,
+                  const float* src, float alpha) {
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < axis; d++) outer *= shape[d];
+    for (int d = axis + 1; d < dims; d++) inner *= shape[d];
+    const int64_t len = shape[axis];
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t j = 0; j < inner; j++)
+            for (int64_t i = 0; i < k; i++) {
+                const int32_t sel = f2i(index[i]);
+                if (sel < 0 || sel >= len) return -1;
+                float* to = target + (o * len + sel) * inner + j;
+                *to = *to + src[(o * k + i) * inner + j] * alpha;
+            }
+    return 0;
+}
+
 /* ---------------------------------------------------------------- layout movers */
 
 /* IDX:65-88 RangeTensorIndexing.sparseStoreRanges for normalised inclusive ranges

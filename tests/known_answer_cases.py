@@ -402,6 +402,15 @@ def case_concat_with_grads(ops):
         assertTensorEquals(c[k], t.grad(), c["tol"], c[k]["shape"])
 
 
+def case_index_select_with_grads(ops):
+    c = K["index_select_with_grads"]
+    tensor = tensorOf(ops, *range(c["arrange"])).reshape(c["shape"]).asVariable(requiresGrad=True)
+    res = tensor.indexSelect(c["axis"], tensorOf(ops, *c["index"]))
+    assertTensorEquals(c["expected"], res, c["tol"], c["expected"]["shape"])
+    res.sum().backward()
+    assertTensorEquals(c["grad"], tensor.grad(), c["tol"], c["grad"]["shape"])
+
+
 def case_fill_partially(ops):
     c = K["fill_partially"]
     t1 = ones(ops, *c["shape"])

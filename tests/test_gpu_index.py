@@ -76,3 +76,41 @@ def test_max_backward_at_scale_matches_checker(gc):
     assert_bits_equal(out[0][0], out[1][0], "grad of max")
     assert abs(float(out[0][1][0]) - float(out[1][1][0])) <= 1e-6 * abs(float(out[1][1][0]))
     np.testing.assert_allclose(out[0][2], out[1][2], rtol=0, atol=1e-9)
+
+
+ROW_CASES = [([3, 3, 3], 1, 3), ([5, 7], 0, 9), ([5, 7], -1, 4), ([2, 3, 4, 5], 2, 6), ([6], 0, 10), ([1000, 64], 0, 5000),
+             ([50, 300, 8], 1, 700), ([4096, 33], 0, 100), ([7, 9, 130], 0, 20), ([64, 1000], 1, 256)]
+
+
+@pytest.mark.parametrize("shape,axis,k", ROW_CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_index_select_and_index_add_parity(shape, axis, k, gc):
+    rng = np.random.default_rng(sum(shape) + k)
+    ax = axis % len(shape)
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = rng.integers(0, shape[ax], [k]).astype(np.float32)
+    gx, cx = both(gc, shape, x); gi, ci = both(gc, [k], idx)
+    got, want = gx.indexSelect(axis, gi), cx.indexSelect(axis, ci)
+    assert got.shape == want.shape
+    assert_bits_equal(got.toArray(), want.toArray(), "indexSelect")
+    src = rng.standard_normal(want.shape).astype(np.float32)
+    gs, cs = both(gc, want.shape, src)
+    for alpha in (1.0, -0.3):
+        gt, ct = both(gc, shape, x)
+        gt.indexAdd(axis, gi, gs, alpha); ct.indexAdd(axis, ci, cs, alpha)
+        assert_bits_equal(gt.toArray(), ct.toArray(), f"indexAdd alpha {alpha} (repeated indices accumulate in index order)")
+
+
+def test_index_select_errors(gc):
+    x = gc.createRaw([2, 3], np.arange(6, dtype=np.float32))
+    for bad in (3.0, -1.0):
+        with pytest.raises(ValueError):
+            x.indexSelect(1, gc.createRaw([2], [0.0, bad]))
+        with pytest.raises(ValueError):
+            x.indexAdd(1, gc.createRaw([2], [0.0, bad]), gc.createRaw([2, 2], np.ones(4, dtype=np.float32)))
+    with pytest.raises(ValueError):
+        x.indexSelect(1, gc.createRaw([1, 2], [0.0, 1.0]))
+    with pytest.raises(ValueError):
+        x.indexAdd(1, gc.createRaw([2], [0.0, 1.0]), gc.createRaw([2, 3], np.ones(6, dtype=np.float32)))
+    t = gc.createRaw([1], [0.0])
+    t.indexAdd(0, gc.createRaw([3], [0.0, 0.0, 0.0]), gc.createRaw([3], [1e8, 1.0, -1e8]))
+    assert t.toArray()[0] == 0.0

@@ -141,3 +141,44 @@ def test_concat_and_narrow_equal_numpy(oracle_ops):
         oracle_ops.concat(0, [oracle_ops.createRaw([2, 3]), oracle_ops.createRaw([3])])
     with pytest.raises(ValueError):
         oracle_ops.createRaw([2, 3]).narrow(1, 2, 2)
+
+
+def test_index_select_and_index_add_equal_numpy(oracle_ops):
+    rng = np.random.default_rng(12)
+    for shape, axis, k in (([3, 3, 3], 1, 3), ([5, 7], 0, 9), ([5, 7], -1, 4), ([2, 3, 4, 5], 2, 6), ([6], 0, 10)):
+        a = rng.standard_normal(shape).astype(np.float32)
+        ax = axis % len(shape)
+        idx = rng.integers(0, shape[ax], k)
+        t, it = oracle_ops.createRaw(shape, a.reshape(-1)), oracle_ops.createRaw([k], idx.astype(np.float32))
+        got = t.indexSelect(axis, it)
+        want = np.take(a, idx, axis=ax)
+        assert got.shape == list(want.shape) and np.array_equal(got.toArray(), want)
+        # indexAdd with alpha 1 against np.add.at; repeated indices accumulate (small integers: exact in any order)
+        src = rng.integers(-8, 8, want.shape).astype(np.float32)
+        base = rng.integers(-8, 8, shape).astype(np.float32)
+        t2 = oracle_ops.createRaw(shape, base.reshape(-1))
+        t2.indexAdd(axis, it, oracle_ops.createRaw(list(src.shape), src.reshape(-1)), 2.0)
+        want2 = base.copy()
+        sl = [slice(None)] * len(shape)
+        for i, sel in enumerate(idx):
+            sl_t = list(sl); sl_t[ax] = sel
+            sl_s = list(sl); sl_s[ax] = i
+            want2[tuple(sl_t)] += src[tuple(sl_s)] * np.float32(2.0)
+        assert np.array_equal(t2.toArray(), want2)
+    t = oracle_ops.createRaw([2, 3], np.zeros(6, dtype=np.float32))
+    with pytest.raises(ValueError):
+        t.indexSelect(1, oracle_ops.createRaw([2], [0.0, 3.0]))                    # JVM:494-496
+    with pytest.raises(ValueError):
+        t.indexSelect(1, oracle_ops.createRaw([1, 2], [0.0, 1.0]))                 # the index must be 1-D
+    with pytest.raises(ValueError):
+        t.indexAdd(1, oracle_ops.createRaw([2], [0.0, 1.0]), oracle_ops.createRaw([2, 3], np.zeros(6, dtype=np.float32)))
+
+
+def test_index_add_accumulates_in_index_order(oracle_ops):
+    # 1e8 + 1 - 1e8 in float: the order of the three additions decides between 0 and 1 (JVM:511-513)
+    t = oracle_ops.createRaw([1], [0.0])
+    t.indexAdd(0, oracle_ops.createRaw([3], [0.0, 0.0, 0.0]), oracle_ops.createRaw([3], [1e8, 1.0, -1e8]))
+    assert t.toArray()[0] == 0.0
+    t = oracle_ops.createRaw([1], [0.0])
+    t.indexAdd(0, oracle_ops.createRaw([3], [0.0, 0.0, 0.0]), oracle_ops.createRaw([3], [1e8, -1e8, 1.0]))
+    assert t.toArray()[0] == 1.0
