@@ -183,6 +183,7 @@ class AGTensor(Tensor):
     def min(self, axis, keepDimensions=False): return Min(self.ops)(self, axis, keepDimensions)
     def gather(self, axis, index): return Gather(self.ops)(self, axis, index)
     def indexSelect(self, axis, index): return IndexSelect(self.ops)(self, index, axis)           # AGTensor.kt:305-307
+    def dot(self, vector): return Dot(self.ops)(self, vector)
     def scatter(self, axis, index, source): return Scatter(self.ops)(self, axis, index, source)
 
     def batchNorm(self, axis, runningMean, runningVar, training, momentum=0.1, epsilon=1e-5, gamma=None, beta=None):
@@ -300,6 +301,11 @@ class NoGradVariable(AGTensor):
     def min(self, axis, keepDimensions=False): return self._new(self.rawValue.min(axis, keepDimensions))
     def gather(self, axis, index): return self._new(self.rawValue.gather(axis, index.getRawValue()))          # :196
     def indexSelect(self, axis, index): return self._new(self.rawValue.indexSelect(axis, index.getRawValue()))   # :202
+
+    def dot(self, vector):
+        if vector.requiresGrad:
+            return super().dot(vector)
+        return self._new(self.rawValue.dot(vector.getRawValue()))
 
     def scatter(self, axis, index, source):                                                                   # :198-202
         if source.requiresGrad:
@@ -1193,6 +1199,24 @@ class Permute(UnaryTensorFunction):                                             
 
     def doBackward(self, gradient):
         return [gradient.permute(self.reverseShapeIndices)]
+
+
+class Dot(BiTensorFunction):                                                          # functions/BlasFunctions.kt:102-127
+    broadcastingOperation = False
+
+    def __call__(self, a, b):
+        self.cachedShape = sf.dot_shape(a.shape, b.shape)
+        return super().__call__(a, b)
+
+    def doForward(self, a, b):
+        self.saveForBackward(a, b)
+        self.output = a.dot(b)
+
+    def doBackward(self, gradient):
+        vector1, vector2 = self.valuesSaved
+        first, second = self.inputs
+        return [vector2 * gradient.broadcastTo(self.bShape) if first.requiresGrad else None,
+                vector1 * gradient.broadcastTo(self.aShape) if second.requiresGrad else None]
 
 
 class IndexSelect(UnaryTensorFunction):                                               # :314-347

@@ -8,8 +8,8 @@ common-shape calculation) restated once here so that every backend shares them, 
 the reference. Kotlin's overloads on (tensor | Float) become one Python method that
 dispatches on the argument type; Kotlin operators are also exposed as Python operators.
 
-Members of the contract that lie outside the accelerated path (dot, BLAS, nn other than
-batch normalisation) are not part of this mirror.
+Members of the contract that lie outside the accelerated path (BLAS level 2 and 3, nn other
+than batch normalisation) are not part of this mirror.
 """
 from enum import Enum
 from typing import List, Sequence
@@ -307,6 +307,16 @@ class AbstractRawTensor:
     def indexAdd(self, axis: int, index, src, alpha: float = 1.0):
         a = sf.index_add_check_shapes_norm_axis(self.shape, axis, index.shape, src.shape)
         self._index_add(a, index, src, float(alpha))
+
+    # --- dot (AbstractRawTensor.kt:234) ---------------------------------------------------
+    def dot(self, vector):
+        """JVMRawTensor.kt:475-482: elementwise products rounded to float, then their sum. A
+        backend may override it; this composition is two operations of the path (times, sum)."""
+        sf.dot_shape(self.shape, vector.shape)
+        products = self.times(vector)
+        res = products._sum_all()
+        self.ops.release(products)
+        return res
 
     # --- broadcasting (AbstractRawTensor.kt:170-192) -----------------------------------
     def calculateCommonShapeWith(self, other) -> List[int]:

@@ -257,6 +257,14 @@ def index_add_check_shapes_norm_axis(shape: Sequence[int], axis: int, index_shap
     return a
 
 
+def dot_shape(shape: Sequence[int], other: Sequence[int]) -> List[int]:
+    """ShapeFunctions.kt:373-380."""
+    if len(shape) != 1 or list(shape) != list(other):
+        raise ValueError("Dot product can only applied to vectors (1D tensors) with same shape, but got tensors with shapes: "
+                         f"{list(shape)} and {list(other)}")
+    return [1]
+
+
 def to_index_ranges(shape: Sequence[int]) -> List[IntRange]:
     """ShapeFunctions.kt:310-312."""
     return [IntRange(0, s - 1) for s in shape]

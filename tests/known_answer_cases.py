@@ -411,6 +411,15 @@ def case_index_select_with_grads(ops):
     assertTensorEquals(c["grad"], tensor.grad(), c["tol"], c["grad"]["shape"])
 
 
+def case_dot_with_grad(ops):
+    c = K["dot_with_grad"]
+    t1 = tensorOf(ops, *range(c["arrange"])).reshape(c["shape"]).asVariable(requiresGrad=True)
+    res = t1[0].dot(t1[1])
+    assertTensorEquals([c["expected"]], res, c["tol"], [1])
+    res.backward()
+    assertTensorEquals(c["grad"], t1.grad(), c["tol"], c["grad"]["shape"])
+
+
 def case_fill_partially(ops):
     c = K["fill_partially"]
     t1 = ones(ops, *c["shape"])
