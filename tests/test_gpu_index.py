@@ -11,7 +11,10 @@ pytestmark = pytest.mark.gpu
 
 CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([3, 4, 5], [2, 4, 2], 2), ([6], [9], 0),
          ([2, 3, 4, 5], [2, 3, 7, 5], 2), ([1000, 300], [1000, 1], 1), ([1000, 300], [1, 300], 0), ([64, 2048], [64, 1], 1),
-         ([70000, 7], [70000, 3], 1), ([5, 3, 2, 2, 3, 2, 2, 2, 3, 4], [5, 3, 2, 2, 6, 2, 2, 2, 3, 4], 4)]
+         ([70000, 7], [70000, 3], 1), ([5, 3, 2, 2, 3, 2, 2, 2, 3, 4], [5, 3, 2, 2, 6, 2, 2, 2, 3, 4], 4),
+         # long axes with many repeated indices (the last entry of a position wins)
+         ([300, 400], [300, 400], 1), ([300, 400], [300, 400], 0), ([64, 2048], [64, 2048], 1), ([2048, 64], [2048, 40], 0),
+         ([8, 100, 128], [8, 90, 128], 1), ([50, 33, 70], [50, 33, 64], 2), ([40, 10], [40, 2000], 1)]
 
 
 def both(gc, shape, array):
