@@ -192,12 +192,30 @@ constexpr uint32_t kShortLoads = kShortTile / 4 / kBlock;
 struct ShortPlan {
     uint32_t outer, axis, rows, stride;      // row length (axis, or axis * inner for slabs); stride = length | 1
     uint32_t inner;                          // slabs only
+    uint32_t aligned;                        // every tile starts 16-byte aligned: float4 loads
+    uint32_t lanes;                          // slabs only: lanes that share one output (power of two, <= 64)
     FastDiv  axis_div, inner_div;
 };
 
 // Loads `floats` contiguous floats from `base` (16-byte aligned) and parks element e at
 // tile[(e / axis) * stride + e % axis].
 __device__ __forceinline__ void stage_short_tile(const float* __restrict__ base, uint32_t floats, const ShortPlan& pl, float* tile) {
+    if (!pl.aligned) {                       // tiles that start off a 16-byte boundary: coalesced scalar loads
+        for (uint32_t e0 = 0; e0 < floats; e0 += kBlock * 8) {
+            float w[8];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) { const uint32_t e = e0 + k * kBlock + threadIdx.x; if (e < floats) w[k] = ld1_stream(base + e); }
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) {
+                const uint32_t e = e0 + k * kBlock + threadIdx.x;
+                if (e < floats) {
+                    const uint32_t r = (__umulhi(e, pl.axis_div.mul) + e) >> pl.axis_div.shift;
+                    tile[r * pl.stride + (e - r * pl.axis)] = w[k];
+                }
+            }
+        }
+        return;
+    }
     float4 v[kShortLoads];
 #pragma unroll
     for (uint32_t k = 0; k < kShortLoads; k++) {
@@ -250,7 +268,8 @@ __global__ __launch_bounds__(kBlock) void reduce_short_rows_kernel(const float* 
 
 // The same staging for a reduction over a middle axis with a small inner size: a "row" is
 // the contiguous slab [axis, inner] of one outer index (pl.axis holds axis * inner), and the
-// outputs of the tile, rows * inner of them, are dealt to the threads in output order:
+// (1 to 1024 slabs per tile), and the outputs of the tile, rows * inner of them, are dealt to
+// the threads in output order:
 // output (r, i) folds tile[r][j * inner + i] over j.
 template <class R>
 __global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float* __restrict__ in, float* __restrict__ out, ShortPlan pl) {
@@ -262,12 +281,16 @@ __global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float*
     __syncthreads();
     const uint32_t outputs = rows_here * pl.inner, steps = pl.axis / pl.inner;
     float* dst = out + static_cast<size_t>(first_row) * pl.inner;
-    for (uint32_t item = threadIdx.x; item < outputs; item += kBlock) {
+    // pl.lanes adjacent lanes share an output when the tile has fewer outputs than threads: lane l
+    // takes the axis positions l, l + lanes, ... in ascending order, then the lanes are merged.
+    const uint32_t lane = threadIdx.x & (pl.lanes - 1), group = threadIdx.x / pl.lanes;
+    for (uint32_t item = group; item < outputs; item += kBlock / pl.lanes) {
         const uint32_t r = (__umulhi(item, pl.inner_div.mul) + item) >> pl.inner_div.shift;
         const float* p = tile + r * pl.stride + (item - r * pl.inner);
         Acc acc = R::init();
-        for (uint32_t j = 0; j < steps; j++) R::step(acc, p[j * pl.inner], j);
-        dst[item] = R::finish(acc, steps);
+        for (uint32_t j = lane; j < steps; j += pl.lanes) R::step(acc, p[j * pl.inner], j);
+        for (uint32_t m = pl.lanes >> 1; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, static_cast<int>(m)));
+        if (lane == 0) dst[item] = R::finish(acc, steps);
     }
 }
 
@@ -453,7 +476,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         ShortPlan pl{};
         uint32_t rows = 4 * kBlock;
         while (rows * axis > kShortTile) rows >>= 1;
-        pl.outer = outer; pl.axis = axis; pl.rows = rows; pl.stride = axis | 1u;
+        pl.outer = outer; pl.axis = axis; pl.rows = rows; pl.stride = axis | 1u; pl.aligned = 1;
         pl.axis_div = make_div(axis);
         const dim3 grid(static_cast<uint32_t>(ceil_div(outer, rows)));
         hipError_t e;
@@ -471,12 +494,24 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         return KTH_OK;
     }
 
-    if (inner > 1 && inner < 64 && static_cast<uint64_t>(axis) * inner <= 256 && axis >= 2) {
+    // Slabs [axis, inner] of at most a tile, and enough of them to give every CU a workgroup.
+    uint32_t slab_rows = 0;
+    // Measured: better than the column and strided kernels for slabs of at most 256 floats with a
+    // small inner size, and for any slab that fits a tile when the axis is short (<= 16).
+    const uint64_t slab = static_cast<uint64_t>(axis) * inner;
+    if (inner > 1 && axis >= 2 && ((inner < 64 && slab <= 256) || (axis <= 16 && slab <= kShortTile))) {
+        slab_rows = static_cast<uint32_t>(kShortTile / slab);
+        if (slab_rows > 4 * kBlock) slab_rows = 4 * kBlock;
+        if (ceil_div(outer, slab_rows) < static_cast<uint64_t>(st.compute_units)) slab_rows = 0;
+    }
+    if (slab_rows > 0) {
         ShortPlan pl{};
         const uint32_t length = axis * inner;
-        uint32_t rows = 4 * kBlock;
-        while (rows * length > kShortTile) rows >>= 1;
+        const uint32_t rows = slab_rows;
         pl.outer = outer; pl.axis = length; pl.rows = rows; pl.stride = length | 1u; pl.inner = inner;
+        pl.aligned = (static_cast<uint64_t>(rows) * length) % 4 == 0 ? 1 : 0;
+        pl.lanes = 1;
+        while (pl.lanes < 64 && static_cast<uint64_t>(rows) * inner * pl.lanes * 2 <= kBlock && pl.lanes * 2 <= axis) pl.lanes <<= 1;
         pl.axis_div = make_div(length); pl.inner_div = make_div(inner);
         hipError_t e;
         {
