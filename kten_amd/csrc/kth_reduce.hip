@@ -1,12 +1,14 @@
 // Axis and full reductions over a row-major tensor seen as [outer, axis, inner].
 //
-// Three first-pass kernels cover the layouts:
+// These first-pass kernels cover the layouts (short rows and slabs have LDS-staged variants below):
 //   rows    (inner == 1): G lanes of a wave64 (or a whole 256-thread workgroup) walk one
 //           contiguous row with float4 loads, combine by xor shuffles (+ LDS across waves);
 //   columns (inner >= 64): a wave owns 64 float4-wide (or scalar) columns so every load
 //           instruction is a contiguous 1 KiB (256 B) span; the waves of a workgroup
 //           take different rows and combine through LDS;
-//   strided (small inner): one thread per output element, serial walk down the axis.
+//   stream  (small inner, slab of 2048 floats or more): a workgroup per slab, threads stay on
+//           their column while the workgroup walks the slab as one contiguous span;
+//   strided (other small inner): one thread per output element, serial walk down the axis.
 // When the output alone gives too few workgroups to fill 256 CUs, the axis is cut into
 // S segments; each (output, segment) writes a partial and a second kernel combines the
 // S partials in a fixed order. No atomics anywhere: the same input always gives the
@@ -392,6 +394,72 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __r
     emit<R>(g, o, s, i, acc, out, partial);
 }
 
+// ---------------------------------------------------------------- stream: small inner, long axis
+
+// One workgroup per (outer index, segment): its slab is one contiguous span. `lanes` groups of
+// inner / VEC threads walk the rows `lanes` apart, so a load instruction of the workgroup covers
+// lanes * inner consecutive floats and every thread stays on its own column(s). The lanes'
+// partials meet in LDS and one thread per column merges them in lane order.
+// VEC = 4 requires inner % 4 == 0 (every row then starts 16-byte aligned).
+template <class R, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                              typename R::Acc* __restrict__ partial, Geom g,
+                                                              uint32_t lanes, FastDiv cols_div) {
+    using Acc = typename R::Acc;
+    __shared__ Acc fold[kBlock * VEC];
+    const uint32_t s = blockIdx.x % g.segments;
+    const uint32_t o = blockIdx.x / g.segments;
+    const uint32_t cols = g.inner / VEC;
+    const uint32_t t = threadIdx.x;
+    const uint32_t lane = (__umulhi(t, cols_div.mul) + t) >> cols_div.shift;
+    const uint32_t c = t - lane * cols;
+    const uint32_t begin = s * g.seg_len;
+    const uint32_t end = min(begin + g.seg_len, g.axis);
+    Acc acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = R::init();
+    if (lane < lanes) {
+        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + c * VEC;
+        constexpr uint32_t kBatch = VEC == 4 ? 4 : 8;
+        uint32_t r = begin + lane;
+        if (VEC == 4) {
+            for (; r + (kBatch - 1) * lanes < end; r += kBatch * lanes) {
+                float4 w[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) w[k] = ld4_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) {
+                    R::step(acc[0], w[k].x, r + k * lanes); R::step(acc[VEC > 1 ? 1 : 0], w[k].y, r + k * lanes);
+                    R::step(acc[VEC > 2 ? 2 : 0], w[k].z, r + k * lanes); R::step(acc[VEC > 3 ? 3 : 0], w[k].w, r + k * lanes);
+                }
+            }
+            for (; r < end; r += lanes) {
+                const float4 w = ld4_stream(base + static_cast<size_t>(r) * g.inner);
+                R::step(acc[0], w.x, r); R::step(acc[VEC > 1 ? 1 : 0], w.y, r);
+                R::step(acc[VEC > 2 ? 2 : 0], w.z, r); R::step(acc[VEC > 3 ? 3 : 0], w.w, r);
+            }
+        } else {
+            for (; r + (kBatch - 1) * lanes < end; r += kBatch * lanes) {
+                float w[kBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) w[k] = ld1_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
+#pragma unroll
+                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], w[k], r + k * lanes);
+            }
+            for (; r < end; r += lanes) R::step(acc[0], ld1_stream(base + static_cast<size_t>(r) * g.inner), r);
+        }
+    }
+    // fold[lane][column]: thread t owns columns c * VEC .. c * VEC + VEC - 1 of lane t / cols
+#pragma unroll
+    for (int v = 0; v < VEC; v++) fold[t * VEC + v] = acc[v];
+    __syncthreads();
+    if (t < g.inner) {
+        Acc a = fold[t];
+        for (uint32_t l = 1; l < lanes; l++) a = R::merge(a, fold[l * g.inner + t]);
+        emit<R>(g, o, s, t, a, out, partial);
+    }
+}
+
 // ---------------------------------------------------------------- second pass
 
 // Combines the `segments` partials of each output, always in the same order.
@@ -462,6 +530,10 @@ void plan_segments(Geom* g, uint64_t base_blocks, uint64_t target, uint32_t quan
     g->segments = ceil_div(g->axis, len);
 }
 
+// Measured: from slabs of about 2048 floats on, streaming a slab per workgroup beats one thread
+// per output (6 TB/s against 1-4.5); below that the per-workgroup fold dominates.
+constexpr uint64_t kStreamMinSlab = 2048;
+
 template <class R>
 int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
     using Acc = typename R::Acc;
@@ -523,8 +595,9 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         return KTH_OK;
     }
 
-    enum { ROWS, COLS, STRIDED } kind;
+    enum { ROWS, COLS, STRIDED, STREAM } kind;
     int G = 1, VEC = 1, WY = 4;
+    uint32_t stream_lanes = 0;
     uint32_t tiles = 0;
     uint64_t blocks = 0;
     if (inner == 1) {
@@ -545,6 +618,13 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         WY = (base_blocks * 4 < target && axis >= 2048) ? 16 : 4;
         plan_segments(&g, base_blocks, WY == 16 ? target / 4 : target, WY, WY * 8);
         blocks = base_blocks * g.segments;
+    } else if (slab >= kStreamMinSlab && outer <= 0x7fffffffu / 64) {
+        // A long axis over a small inner size: one workgroup streams a whole slab (or a segment of it).
+        kind = STREAM;
+        VEC = (inner % 4 == 0) ? 4 : 1;
+        stream_lanes = kBlock / (inner / VEC);
+        plan_segments(&g, outer, target / 2, stream_lanes, stream_lanes * 8);
+        blocks = static_cast<uint64_t>(outer) * g.segments;
     } else {
         kind = STRIDED;
         const uint64_t base_blocks = ceil_div(n_out, kBlock);
@@ -564,7 +644,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     const uint64_t bytes = (static_cast<uint64_t>(outer) * axis * inner + n_out) * 4;
     hipError_t e;
     {
-        LaunchScope scope(kind == ROWS ? "reduce_rows_kernel" : kind == COLS ? "reduce_cols_kernel" : "reduce_strided_kernel",
+        LaunchScope scope(kind == ROWS ? "reduce_rows_kernel" : kind == COLS ? "reduce_cols_kernel" : kind == STREAM ? "reduce_stream_kernel" : "reduce_strided_kernel",
                           R::name, bytes);
         if (kind == ROWS) {
 #define ROWS_LAUNCH(GG, VV) hipLaunchKernelGGL((reduce_rows_kernel<R, GG, VV>), grid, dim3(kBlock), 0, stream, in, out, partial, g)
@@ -583,6 +663,10 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
             else if (VEC == 4)        hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
             else if (WY == 16)        hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 16>), grid, dim3(kWave, 16), 0, stream, in, out, partial, g, tiles);
             else                      hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+        } else if (kind == STREAM) {
+            const FastDiv cols_div = make_div(inner / VEC);
+            if (VEC == 4) hipLaunchKernelGGL((reduce_stream_kernel<R, 4>), grid, dim3(kBlock), 0, stream, in, out, partial, g, stream_lanes, cols_div);
+            else          hipLaunchKernelGGL((reduce_stream_kernel<R, 1>), grid, dim3(kBlock), 0, stream, in, out, partial, g, stream_lanes, cols_div);
         } else {
             hipLaunchKernelGGL((reduce_strided_kernel<R>), grid, dim3(kBlock), 0, stream, in, out, partial, g);
         }
