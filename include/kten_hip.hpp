@@ -498,6 +498,20 @@ public:
     }
     bool containsNan() { live(); int flag = 0; check(kth_contains_nan(storeReference, static_cast<uint64_t>(size()), &flag)); return flag != 0; }
     void inplaceFill(float value) { live(); check(kth_fill(storeReference, 0, static_cast<uint64_t>(size()), value)); }
+    // inplaceResize (AbstractRawTensor.kt:242; JVMRawTensor.kt:524-531): a new store that keeps the
+    // leading values and holds zeros beyond them; this wrapper's reference on the old store is returned.
+    void inplaceResize(const Shape& to) {
+        live();
+        const uint64_t nNew = static_cast<uint64_t>(toStoreSize(to)), nOld = static_cast<uint64_t>(size());
+        uint64_t fresh = 0;
+        check(kth_alloc(nNew, &fresh));
+        const uint64_t kept = nNew < nOld ? nNew : nOld;
+        check(kth_copy(fresh, 0, storeReference, 0, kept));
+        if (nNew > kept) check(kth_fill(fresh, kept, nNew - kept, 0.0f));
+        check(kth_release(storeReference));
+        storeReference = fresh;
+        shape = to;
+    }
     std::vector<float> toVector() {
         live();
         std::vector<float> host(static_cast<size_t>(size()));

@@ -324,6 +324,24 @@ class HipRawTensor(AbstractRawTensor):
         self._require_live()
         check(self.ops.lib.kth_fill(self.storeReference, 0, self.size, float(value)))
 
+    def inplaceResize(self, *shape):
+        """inplaceResize (AbstractRawTensor.kt:242): a new store of the new size that keeps the
+        leading values and holds zeros beyond them (FloatArray.copyOf, JVMRawTensor.kt:524-531);
+        this wrapper's reference on the old store is given back (OCLRawTensor.kt:383-390)."""
+        self._require_live()
+        new_shape = list(shape[0]) if len(shape) == 1 and not isinstance(shape[0], int) else list(shape)
+        n_new, n_old = sf.to_store_size(new_shape), self.size
+        handle = ctypes.c_uint64()
+        lib = self.ops.lib
+        check(lib.kth_alloc(n_new, ctypes.byref(handle)))
+        kept = min(n_new, n_old)
+        check(lib.kth_copy(handle, 0, self.storeReference, 0, kept))
+        if n_new > kept:
+            check(lib.kth_fill(handle, kept, n_new - kept, 0.0))
+        check(lib.kth_release(self.storeReference))
+        self.storeReference = handle.value
+        self.shape = new_shape
+
     def toArray(self) -> np.ndarray:
         """Device -> host copy shaped like the tensor (the backend's toSerializableData)."""
         self._require_live()

@@ -67,6 +67,7 @@ class AbstractRawTensor:
     def getSingleValue(self, indexes) -> float: raise NotImplementedError
     def containsNan(self) -> bool: raise NotImplementedError
     def inplaceFill(self, value: float): raise NotImplementedError
+    def inplaceResize(self, *shape): raise NotImplementedError               # new store: leading values kept, zeros beyond
     def toList(self): raise NotImplementedError                              # flat host copy (serializable data)
 
     # --- arithmetic (AbstractRawTensor.kt:39-73) ---------------------------------------

@@ -411,6 +411,17 @@ class JvmOracleRawTensor(AbstractRawTensor):
     def inplaceFill(self, value):
         lib().kjo_fill(_p(self.storeReference), self.storeReference.size, value)
 
+    def inplaceResize(self, *shape):
+        """JVMRawTensor.kt:524-531: storeReference.copyOf(new size) keeps the leading values and
+        pads with zeros."""
+        new_shape = list(shape[0]) if len(shape) == 1 and not isinstance(shape[0], int) else list(shape)
+        n = sf.to_store_size(new_shape)
+        store = np.zeros(n, dtype=np.float32)
+        kept = min(n, self.storeReference.size)
+        store[:kept] = self.storeReference[:kept]
+        self.storeReference = store
+        self.shape = new_shape
+
     def toArray(self):
         return self.storeReference.reshape(self.shape).copy()
 

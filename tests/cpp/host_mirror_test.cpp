@@ -157,6 +157,15 @@ int main() {
         expect(!acc->containsNan(), "containsNan on finite values");
         expect(tensor(ops, {2}, {1.0f, NAN})->containsNan(), "containsNan finds a NaN");
 
+        // inplaceResize keeps the leading values and pads with zeros; a shallow copy keeps the old store
+        Raw grown = tensor(ops, {3}, {1, 2, 3});
+        Raw alias = grown->copy(true);
+        grown->inplaceResize({2, 3});
+        expect_values(grown, {2, 3}, {1, 2, 3, 0, 0, 0}, 0.0f, "inplaceResize grows with zeros");
+        grown->inplaceResize({2});
+        expect_values(grown, {2}, {1, 2}, 0.0f, "inplaceResize truncates");
+        expect_values(alias, {3}, {1, 2, 3}, 0.0f, "a shallow copy still sees the store it shares");
+
         // survive the scope
         ops.markSurviveGC(t1);
         gc.close();

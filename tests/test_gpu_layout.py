@@ -216,3 +216,16 @@ def test_layout_workloads_full_size(gc):
     assert_bits_equal(out["right"].toArray(), masked[:, left:], "range get")
     masked[:, :left] = 1.0
     assert_bits_equal(out["masked"].toArray(), masked, "maskedFill then range fill")
+
+
+@pytest.mark.parametrize("old,new", [([6], [2, 5]), ([2, 5], [3]), ([1000, 33], [1000, 40]), ([64, 64], [63, 65]), ([4099], [4099])])
+def test_inplace_resize_parity(old, new, gc):
+    x = np.random.default_rng(sum(old) + sum(new)).standard_normal(old).astype(np.float32)
+    g, c = both(gc, x)
+    shared = g.copy(shallow=True)
+    g.inplaceResize(*new); c.inplaceResize(*new)
+    assert g.shape == c.shape == new
+    assert_bits_equal(g.toArray().reshape(-1), c.toArray().reshape(-1), f"inplaceResize {old} -> {new}")
+    assert_bits_equal(shared.toArray().reshape(-1), x.reshape(-1), "the shallow copy keeps the old store")
+    g.plusAssign(1.0); c.plusAssign(1.0)                      # the new store is an ordinary store
+    assert_bits_equal(g.toArray().reshape(-1), c.toArray().reshape(-1), "arithmetic on the resized tensor")

@@ -182,3 +182,13 @@ def test_index_add_accumulates_in_index_order(oracle_ops):
     t = oracle_ops.createRaw([1], [0.0])
     t.indexAdd(0, oracle_ops.createRaw([3], [0.0, 0.0, 0.0]), oracle_ops.createRaw([3], [1e8, -1e8, 1.0]))
     assert t.toArray()[0] == 1.0
+
+
+def test_inplace_resize_keeps_the_leading_values_and_pads_with_zeros(oracle_ops):
+    """FloatArray.copyOf (JVMRawTensor.kt:528-531): the ones-buffer of the convolution code is
+    resized this way (JVMSpatialConvolutionBase.kt:66)."""
+    t = oracle_ops.createRaw([2, 3], np.arange(1, 7, dtype=np.float32))
+    t.inplaceResize(3, 3)
+    assert t.shape == [3, 3] and t.toList() == [1, 2, 3, 4, 5, 6, 0, 0, 0]
+    t.inplaceResize([2, 2])
+    assert t.shape == [2, 2] and t.toList() == [1, 2, 3, 4]
