@@ -298,19 +298,22 @@ __global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float*
 
 // ---------------------------------------------------------------- columns: inner >= 64
 
-// Workgroup = 64 x WY threads: lane x owns VEC adjacent columns of a 64*VEC-column tile,
-// wave y takes rows y, y + WY, ... of the segment.
-template <class R, int VEC, int WY>
+// Workgroup = 64 x WY threads over a tile of TW * 64 * VEC columns: lane x of wave y owns VEC
+// adjacent columns of sub-tile y % TW (so TW waves side by side read one contiguous span of a
+// row), and takes rows y / TW, y / TW + WY / TW, ... of the segment.
+template <class R, int VEC, int WY, int TW>
 __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                                  typename R::Acc* __restrict__ partial, Geom g, uint32_t tiles) {
     using Acc = typename R::Acc;
+    constexpr uint32_t WR = WY / TW;            // row lanes
     const uint32_t bid = blockIdx.x;
     const uint32_t tile = bid % tiles;
     const uint32_t rest = bid / tiles;
     const uint32_t s = rest % g.segments;
     const uint32_t o = rest / g.segments;
     const uint32_t tx = threadIdx.x, ty = threadIdx.y;
-    const uint32_t col = (tile * kWave + tx) * VEC;
+    const uint32_t sub = ty % TW, lane = ty / TW;
+    const uint32_t col = ((tile * TW + sub) * kWave + tx) * VEC;
     const bool active = col < g.inner;          // inner % VEC == 0, so a float4 is all in or all out
     Acc acc[VEC];
 #pragma unroll
@@ -320,27 +323,27 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
         const uint32_t begin = s * g.seg_len;
         const uint32_t end = min(begin + g.seg_len, g.axis);
         constexpr uint32_t kBatch = 8;          // loads in flight per thread
-        uint32_t r = begin + ty;
-        for (; r + (kBatch - 1) * WY < end; r += kBatch * WY) {
+        uint32_t r = begin + lane;
+        for (; r + (kBatch - 1) * WR < end; r += kBatch * WR) {
             if (VEC == 4) {
                 float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WY) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
-                    const uint32_t rr = r + k * WY;
+                    const uint32_t rr = r + k * WR;
                     R::step(acc[0], v[k].x, rr); R::step(acc[1 % VEC], v[k].y, rr);
                     R::step(acc[2 % VEC], v[k].z, rr); R::step(acc[3 % VEC], v[k].w, rr);
                 }
             } else {
                 float v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + static_cast<size_t>(r + k * WY) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], v[k], r + k * WY);
+                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], v[k], r + k * WR);
             }
         }
-        for (; r < end; r += WY) {
+        for (; r < end; r += WR) {
             const float* p = base + static_cast<size_t>(r) * g.inner;
             if (VEC == 4) {
                 float4 v = ld4_stream(p);
@@ -355,11 +358,11 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
 #pragma unroll
     for (int v = 0; v < VEC; v++) lds[ty][tx * VEC + v] = acc[v];
     __syncthreads();
-    if (ty == 0 && active) {
+    if (lane == 0 && active) {
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
-            Acc t = lds[0][tx * VEC + v];
-            for (int w = 1; w < WY; w++) t = R::merge(t, lds[w][tx * VEC + v]);
+            Acc t = lds[sub][tx * VEC + v];
+            for (uint32_t w = 1; w < WR; w++) t = R::merge(t, lds[w * TW + sub][tx * VEC + v]);
             emit<R>(g, o, s, col + v, t, out, partial);
         }
     }
@@ -600,7 +603,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     const bool stream_fits = slab >= kStreamMinSlab && (inner < 256 || (inner < 512 && inner % 4 == 0)) &&
                              outer <= 0x7fffffffu / 64;
     enum { ROWS, COLS, STRIDED, STREAM } kind;
-    int G = 1, VEC = 1, WY = 4;
+    int G = 1, VEC = 1, WY = 4, TW = 1;
     uint32_t stream_lanes = 0;
     uint32_t tiles = 0;
     uint64_t blocks = 0;
@@ -615,12 +618,15 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     } else if (inner >= 64 && !stream_fits) {
         kind = COLS;
         VEC = (inner % 4 == 0) ? 4 : 1;
-        tiles = ceil_div(inner, kWave * VEC);
+        // Scalar columns: four waves side by side make a row's span 1 KiB instead of 256 B
+        // (measured 51 us against 60 on [4,16384,1001]); with float4 columns the narrow tile is faster.
+        TW = (VEC == 1 && inner >= 256) ? 4 : 1;
+        tiles = ceil_div(inner, kWave * VEC * TW);
         const uint64_t base_blocks = static_cast<uint64_t>(tiles) * outer;
         // Few column tiles and a long axis: 16 waves per workgroup fold 16 rows at a time
         // through LDS, which cuts the number of partials per output by four.
-        WY = (base_blocks * 4 < target && axis >= 2048) ? 16 : 4;
-        plan_segments(&g, base_blocks, WY == 16 ? target / 4 : target, WY, WY * 8);
+        WY = (base_blocks * 4 * TW < target && axis >= 2048) ? 16 : 4;
+        plan_segments(&g, base_blocks, WY == 16 ? target / 4 : target, WY / TW, WY / TW * 8);
         blocks = base_blocks * g.segments;
     } else if (stream_fits) {
         // A long axis over a small inner size: one workgroup streams a whole slab (or a segment of it).
@@ -663,10 +669,15 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
             }
 #undef ROWS_LAUNCH
         } else if (kind == COLS) {
-            if (VEC == 4 && WY == 16) hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 16>), grid, dim3(kWave, 16), 0, stream, in, out, partial, g, tiles);
-            else if (VEC == 4)        hipLaunchKernelGGL((reduce_cols_kernel<R, 4, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
-            else if (WY == 16)        hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 16>), grid, dim3(kWave, 16), 0, stream, in, out, partial, g, tiles);
-            else                      hipLaunchKernelGGL((reduce_cols_kernel<R, 1, 4>), grid, dim3(kWave, 4), 0, stream, in, out, partial, g, tiles);
+#define COLS_LAUNCH(VV, YY, TT) hipLaunchKernelGGL((reduce_cols_kernel<R, VV, YY, TT>), grid, dim3(kWave, YY), 0, stream, in, out, partial, g, tiles)
+            if (TW == 4) {
+                if (VEC == 4 && WY == 16) COLS_LAUNCH(4, 16, 4); else if (VEC == 4) COLS_LAUNCH(4, 4, 4);
+                else if (WY == 16) COLS_LAUNCH(1, 16, 4); else COLS_LAUNCH(1, 4, 4);
+            } else {
+                if (VEC == 4 && WY == 16) COLS_LAUNCH(4, 16, 1); else if (VEC == 4) COLS_LAUNCH(4, 4, 1);
+                else if (WY == 16) COLS_LAUNCH(1, 16, 1); else COLS_LAUNCH(1, 4, 1);
+            }
+#undef COLS_LAUNCH
         } else if (kind == STREAM) {
             const FastDiv cols_div = make_div(inner / VEC);
             if (VEC == 4) hipLaunchKernelGGL((reduce_stream_kernel<R, 4>), grid, dim3(kBlock), 0, stream, in, out, partial, g, stream_lanes, cols_div);

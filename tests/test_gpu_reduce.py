@@ -29,6 +29,8 @@ GEOMETRIES = [
     # a slab (or a segment of it) streamed by one workgroup: scalar and float4 columns, with and without segments
     ([300, 700, 3], 1), ([2, 50000, 12], 1), ([2000, 64, 33], 1), ([1500, 100, 40], 1), ([5, 2049, 1, 63], 1),
     ([3, 40000, 2], 1), ([1, 100000, 7], 1),
+    # scalar columns in tiles four waves wide, with and without segments
+    ([300, 1001], 0), ([3, 500, 257], 1), ([2, 5000, 259], 1), ([7, 300], 0),
     # streamed slabs with wide columns: one group of threads per row, float4 columns up to 511
     ([40, 300, 129], 1), ([30, 64, 200], 1), ([3, 5000, 68], 1), ([20, 50, 300], 1), ([5, 2000, 255], 1), ([9, 40, 508], 1),
 ]
