@@ -23,9 +23,12 @@ GEOMETRIES = [
     # short rows staged through LDS (8 <= length < 256), every lanes-per-row variant, ragged last tile
     ([5000, 8], 1), ([1030, 9], 1), ([777, 31], 1), ([3001, 32], 1), ([515, 50], 1), ([130, 100], 1), ([67, 129], 1),
     ([33, 255], 1), ([1, 200], 1), ([300, 10], 1),
-    # short slabs (axis * inner <= 256, inner < 64)
+    # short slabs, too few of them for the tiled kernel
     ([5000, 8, 8], 1), ([1000, 2, 2], 1), ([999, 3, 40], 1), ([257, 16, 16], 1), ([100, 4, 63], 1), ([70, 2, 3, 5], 2),    # slabs up to a whole tile for short axes: unaligned tiles, several lanes per output
     ([600, 8, 128], 1), ([300, 16, 64], 1), ([257, 3, 1024], 1), ([1100, 2, 300], 1), ([400, 4, 201], 1),
+    # slabs of up to 2047 floats with any axis length, enough of them to take the tiled kernel
+    ([8000, 17, 17], 1), ([7000, 40, 8], 1), ([8000, 100, 3], 1), ([3000, 500, 2], 1), ([1500, 24, 80], 1),
+    ([1500, 19, 100], 1), ([1500, 128, 13], 1),
     # a slab (or a segment of it) streamed by one workgroup: scalar and float4 columns, with and without segments
     ([300, 700, 3], 1), ([2, 50000, 12], 1), ([2000, 64, 33], 1), ([1500, 100, 40], 1), ([5, 2049, 1, 63], 1),
     ([3, 40000, 2], 1), ([1, 100000, 7], 1),
@@ -70,7 +73,8 @@ def test_axis_reductions(shape, axis, gc):
 
 @pytest.mark.parametrize("shape,axis", [([64, 40], 1), ([9, 1000], 1), ([3, 5000], 1), ([333, 1000], 0), ([4, 50, 64], 1),
                                         ([6, 3000, 5], 1), ([2, 70000], 1), ([70000, 64], 0), ([600, 100], 1), ([300, 12, 9], 1),
-                                        ([2, 50000, 12], 1), ([700, 300, 7], 1), ([300, 16, 64], 1)],
+                                        ([2, 50000, 12], 1), ([700, 300, 7], 1), ([300, 16, 64], 1),
+                                        ([8000, 100, 3], 1), ([1500, 24, 80], 1)],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
 def test_special_values_in_reductions(shape, axis, gc):
     """NaN propagation in max/min, NaN skipping in arg ops, signed zeros, lanes of -inf / +inf, ties."""
