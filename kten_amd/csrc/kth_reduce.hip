@@ -260,7 +260,12 @@ __global__ __launch_bounds__(kBlock) void reduce_short_rows_kernel(const float* 
         Acc acc = R::init();
         if (r < rows_here) {
             const float* row = tile + r * pl.stride;
-            for (uint32_t j = lane; j < pl.axis; j += G) R::step(acc, row[j], j);
+            uint32_t j = lane;
+            for (; j + 3 * G < pl.axis; j += 4 * G) {               // four LDS reads in flight
+                const float a0 = row[j], a1 = row[j + G], a2 = row[j + 2 * G], a3 = row[j + 3 * G];
+                R::step(acc, a0, j); R::step(acc, a1, j + G); R::step(acc, a2, j + 2 * G); R::step(acc, a3, j + 3 * G);
+            }
+            for (; j < pl.axis; j += G) R::step(acc, row[j], j);
         }
 #pragma unroll
         for (int m = G / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
@@ -290,7 +295,13 @@ __global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float*
         const uint32_t r = (__umulhi(item, pl.inner_div.mul) + item) >> pl.inner_div.shift;
         const float* p = tile + r * pl.stride + (item - r * pl.inner);
         Acc acc = R::init();
-        for (uint32_t j = lane; j < steps; j += pl.lanes) R::step(acc, p[j * pl.inner], j);
+        uint32_t j = lane;
+        for (; j + 3 * pl.lanes < steps; j += 4 * pl.lanes) {       // four LDS reads in flight
+            const float a0 = p[j * pl.inner], a1 = p[(j + pl.lanes) * pl.inner];
+            const float a2 = p[(j + 2 * pl.lanes) * pl.inner], a3 = p[(j + 3 * pl.lanes) * pl.inner];
+            R::step(acc, a0, j); R::step(acc, a1, j + pl.lanes); R::step(acc, a2, j + 2 * pl.lanes); R::step(acc, a3, j + 3 * pl.lanes);
+        }
+        for (; j < steps; j += pl.lanes) R::step(acc, p[j * pl.inner], j);
         for (uint32_t m = pl.lanes >> 1; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, static_cast<int>(m)));
         if (lane == 0) dst[item] = R::finish(acc, steps);
     }
