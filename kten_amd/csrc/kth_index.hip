@@ -139,6 +139,73 @@ __global__ __launch_bounds__(kBlock) void index_add_kernel(float* __restrict__ t
     }
 }
 
+// ---- indexAdd through a sorted index list ------------------------------------------------
+// keys[i] = the target row of source row i (axis_len for a value out of range, which is also
+// reported); vals[i] = i. After a stable sort by key, the source rows that add into one target
+// row stand next to each other in their original order.
+__global__ __launch_bounds__(kBlock) void index_keys_kernel(const float* __restrict__ index, uint32_t k, uint32_t axis_len,
+                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, int* bad) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= k) return;
+    const int sel = static_cast<int>(index[i]);
+    const bool ok = sel >= 0 && static_cast<uint32_t>(sel) < axis_len;
+    if (!ok) *bad = 1;
+    keys[i] = ok ? static_cast<uint32_t>(sel) : axis_len;
+    vals[i] = i;
+}
+
+// One thread per unit (float or float4) of [outer, k, inner] in sorted order. The thread at the
+// head of a run of equal keys owns that target row's unit: it adds the run's source rows in
+// order, target = target + src * alpha each time (two roundings, as JVMRawTensor.kt:515);
+// the other threads of the run have nothing to do. No two threads write the same element.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                 const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                                                                 float alpha, uint32_t units, RowsPlan pl) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= units) return;
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t col = e - row * pl.inner;
+    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
+    const uint32_t i = row - o * pl.k;
+    const uint32_t key = keys[i];
+    if (key >= pl.axis_len) return;
+    if (i > 0 && keys[i - 1] == key) return;
+    const size_t t_at = (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
+    const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
+    if (VEC) {
+        float4* t = reinterpret_cast<float4*>(target) + t_at;
+        const float4* s = reinterpret_cast<const float4*>(src) + s_base;
+        float4 acc = *t;
+        uint32_t r = i;
+        float4 v = s[static_cast<size_t>(vals[r]) * pl.inner];
+        while (true) {
+            const bool more = r + 1 < pl.k && keys[r + 1] == key;
+            float4 next = v;
+            if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];     // in flight during the adds
+            acc.x = acc.x + v.x * alpha; acc.y = acc.y + v.y * alpha; acc.z = acc.z + v.z * alpha; acc.w = acc.w + v.w * alpha;
+            if (!more) break;
+            v = next; r++;
+        }
+        *t = acc;
+    } else {
+        float* t = target + t_at;
+        const float* s = src + s_base;
+        float acc = *t;
+        uint32_t r = i;
+        float v = s[static_cast<size_t>(vals[r]) * pl.inner];
+        while (true) {
+            const bool more = r + 1 < pl.k && keys[r + 1] == key;
+            float next = v;
+            if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];
+            acc = acc + v * alpha;
+            if (!more) break;
+            v = next; r++;
+        }
+        *t = acc;
+    }
+}
+
 __global__ void clear_int_kernel(int* p) { *p = 0; }
 
 int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
@@ -358,12 +425,54 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     RowsPlan pl{};
     pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k); pl.inner = static_cast<uint32_t>(inner);
     pl.inner_div = make_div(pl.inner); pl.k_div = make_div(pl.k);
-    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
-    return with_index_check("Index Add", [&](int* flag) {
-        LaunchScope scope("index_add_kernel", "", 3 * n_src * 4 + k * 4);
-        hipLaunchKernelGGL(index_add_kernel, dim3(blocks), dim3(kBlock), 0, state().stream, st->ptr, sx->ptr, ss->ptr, alpha,
-                           static_cast<uint32_t>(positions), pl, flag);
+    hipStream_t stream = state().stream;
+
+    // A short list: one thread per (outer, column) position walks it in order. The walk is serial,
+    // about half a microsecond per entry, so from kSortedFrom entries on the list is sorted instead
+    // and every touched target row is updated by its own threads.
+    constexpr uint64_t kSortedFrom = 64;
+    uint32_t* keys = nullptr;
+    uint64_t cap = 0;
+    size_t temp_bytes = 0;
+    int end_bit = 1;
+    while (end_bit < 32 && (1ull << end_bit) <= pl.axis_len) end_bit++;      // keys run up to axis_len inclusive
+    const uint64_t k_pad = (k + 63) & ~63ull;                                // keeps the four arrays 256-byte aligned
+    if (k >= kSortedFrom &&
+        sort_pairs_u32(nullptr, &temp_bytes, nullptr, nullptr, nullptr, nullptr, pl.k, end_bit, stream) == hipSuccess)
+        keys = reinterpret_cast<uint32_t*>(workspace_acquire(4 * k_pad * 4 + temp_bytes, &cap));
+    if (!keys) {
+        (void)hipGetLastError();
+        const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+        return with_index_check("Index Add", [&](int* flag) {
+            LaunchScope scope("index_add_kernel", "", 3 * n_src * 4 + k * 4);
+            hipLaunchKernelGGL(index_add_kernel, dim3(blocks), dim3(kBlock), 0, stream, st->ptr, sx->ptr, ss->ptr, alpha,
+                               static_cast<uint32_t>(positions), pl, flag);
+        });
+    }
+    uint32_t* vals = keys + k_pad;
+    uint32_t* keys_sorted = vals + k_pad;
+    uint32_t* vals_sorted = keys_sorted + k_pad;
+    void* temp = vals_sorted + k_pad;
+    const bool vec = inner % 4 == 0;
+    if (vec) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }
+    const uint32_t units = static_cast<uint32_t>(vec ? n_src / 4 : n_src);
+    hipError_t sort_status = hipSuccess;
+    int rc = with_index_check("Index Add", [&](int* flag) {
+        {
+            LaunchScope scope("index_sort", "", k * 4 * 5);
+            hipLaunchKernelGGL(index_keys_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, sx->ptr, pl.k,
+                               pl.axis_len, keys, vals, flag);
+            sort_status = sort_pairs_u32(temp, &temp_bytes, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
+        }
+        if (sort_status != hipSuccess) return;
+        LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : "float", 3 * n_src * 4 + k * 4);
+        const dim3 grid((units + kBlock - 1) / kBlock);
+        if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, alpha, units, pl);
+        else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, alpha, units, pl);
     });
+    workspace_release(reinterpret_cast<float*>(keys), cap);
+    if (sort_status != hipSuccess) return fail(KTH_E_DEVICE, "kth_index_add: sorting the index list failed: %s", hipGetErrorString(sort_status));
+    return rc;
 }
 
 }  // extern "C"

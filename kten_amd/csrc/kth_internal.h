@@ -81,6 +81,11 @@ Store* lookup(uint64_t handle, const char* what);
 float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
 void   workspace_release(float* p, uint64_t cap_bytes);
 
+// Stable sort of n (key, value) pairs by the low `end_bit` bits of the key, on `stream`
+// (kth_sort.hip). With temp == nullptr only *temp_bytes is set, to the scratch size needed.
+hipError_t sort_pairs_u32(void* temp, size_t* temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
+                          const uint32_t* vals_in, uint32_t* vals_out, uint32_t n, int end_bit, hipStream_t stream);
+
 // Computes the exp / log tables on the host (extended precision) and copies them into the
 // device symbols of the elementwise kernels. Called once from kth_init.
 hipError_t init_math_tables();

@@ -82,7 +82,11 @@ def test_max_backward_at_scale_matches_checker(gc):
 
 
 ROW_CASES = [([3, 3, 3], 1, 3), ([5, 7], 0, 9), ([5, 7], -1, 4), ([2, 3, 4, 5], 2, 6), ([6], 0, 10), ([1000, 64], 0, 5000),
-             ([50, 300, 8], 1, 700), ([4096, 33], 0, 100), ([7, 9, 130], 0, 20), ([64, 1000], 1, 256)]
+             ([50, 300, 8], 1, 700), ([4096, 33], 0, 100), ([7, 9, 130], 0, 20), ([64, 1000], 1, 256),
+             # lists of 64 entries or more are sorted on the device: the threshold, long runs of one target row,
+             # a flat tensor, a short middle axis, columns that are not a multiple of 4
+             ([9, 7], 0, 63), ([9, 7], 0, 64), ([3, 40], 0, 5000), ([2, 5, 3], 1, 1000), ([100000], 0, 300000),
+             ([20, 4100], 1, 9000), ([1, 2, 1], 1, 4097)]
 
 
 @pytest.mark.parametrize("shape,axis,k", ROW_CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
@@ -117,3 +121,17 @@ def test_index_select_errors(gc):
     t = gc.createRaw([1], [0.0])
     t.indexAdd(0, gc.createRaw([3], [0.0, 0.0, 0.0]), gc.createRaw([3], [1e8, 1.0, -1e8]))
     assert t.toArray()[0] == 0.0
+    # the same on a list long enough to be sorted: the order of the adds still decides the result
+    idx = np.zeros(300, dtype=np.float32)
+    vals = np.tile(np.array([1e8, 1.0, -1e8], dtype=np.float32), 100)
+    t = gc.createRaw([2], [0.0, 5.0])
+    t.indexAdd(0, gc.createRaw([300], idx), gc.createRaw([300], vals))
+    assert t.toList() == [0.0, 5.0]
+    # a bad value in a long list is reported, and the tensor stays usable
+    idx[150] = 2.0
+    with pytest.raises(ValueError):
+        t.indexAdd(0, gc.createRaw([300], idx), gc.createRaw([300], vals))
+    idx[150] = np.nan                                           # toInt() of NaN is 0
+    t2 = gc.createRaw([2], [0.0, 5.0])
+    t2.indexAdd(0, gc.createRaw([300], idx), gc.createRaw([300], vals))
+    assert t2.toList() == [0.0, 5.0]
