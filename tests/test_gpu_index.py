@@ -135,3 +135,36 @@ def test_index_select_errors(gc):
     t2 = gc.createRaw([2], [0.0, 5.0])
     t2.indexAdd(0, gc.createRaw([300], idx), gc.createRaw([300], vals))
     assert t2.toList() == [0.0, 5.0]
+
+
+def test_index_add_full_size_round_trip(gc):
+    """At the benchmark's [16384, 4096]: adding the rows of src into a zero tensor at a permutation
+    of the rows, then selecting by the same permutation, gives src back bit for bit (0 + s * 1 = s
+    for every s that is not -0); with every row sent to one target row the result is the serial
+    float sum of the rows in order."""
+    rows, cols = 16384, 4096
+    rng = np.random.default_rng(5)
+    src = rng.standard_normal((rows, cols)).astype(np.float32)
+    src[src == 0] = 1.0
+    perm = rng.permutation(rows).astype(np.float32)
+    s = gc.createRaw([rows, cols], src)
+    p = gc.createRaw([rows], perm)
+    t = gc.createRawFill([rows, cols], 0.0)
+    t.indexAdd(0, p, s)
+    back = t.indexSelect(0, p)
+    assert_bits_equal(back.toArray(), src, "indexSelect(indexAdd(0, perm, src), perm)")
+    # along the last axis, the same with a permutation of the columns
+    pc = gc.createRaw([cols], rng.permutation(cols).astype(np.float32))
+    t2 = gc.createRawFill([rows, cols], 0.0)
+    t2.indexAdd(1, pc, s)
+    assert_bits_equal(t2.indexSelect(1, pc).toArray(), src, "the same along the last axis")
+    # 4096 rows into one: the adds happen in list order
+    few = 4096
+    one = gc.createRawFill([2, cols], 0.0)
+    one.indexAdd(0, gc.createRawFill([few], 1.0), gc.createRaw([few, cols], src[:few]))
+    want = np.zeros(cols, dtype=np.float32)
+    for r in range(few):
+        want = want + src[r]
+    got = one.toArray()
+    assert_bits_equal(got[1], want, "serial float sum of the rows, in order")
+    assert not got[0].any()
