@@ -87,6 +87,76 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
     }
 }
 
+// Scatter along the innermost axis when the index rows are long: one workgroup per position
+// keeps the target row in LDS, so the scattered accesses never leave the CU and the row goes
+// back to memory as one contiguous span. The index row is taken THREADS entries at a time, in
+// order; inside such a chunk, entries that name the same target element are put in order
+// through an LDS tag per element:
+//   assign: the element is cleared, every contender raises it to its lane number + 1 with an
+//           atomic max, and the highest lane (the last entry) then stores its value there;
+//   add:    contenders lower the element's tag to their lane number with an atomic min; the
+//           lowest lane adds its value and leaves, and the round repeats until nobody is left
+//           (as many rounds as the most frequent index of the chunk occurs).
+// LDS: a_axis_len floats, plus a_axis_len tags for MODE 1. THREADS = 1024 for rows above 32 KiB of
+// LDS, which leave room for few workgroups on a CU: the chunk is then 1024 entries.
+template <int MODE, int THREADS>
+__global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __restrict__ target, const float* __restrict__ index,
+                                                                 const float* __restrict__ src, float value, IndexPlan pl, int* bad) {
+    extern __shared__ float row_lds[];
+    float* tile = row_lds;
+    uint32_t* tile_bits = reinterpret_cast<uint32_t*>(row_lds);
+    uint32_t* tag = reinterpret_cast<uint32_t*>(row_lds) + pl.a_axis_len;     // MODE 1 only
+    const uint32_t tid = threadIdx.x;
+    uint32_t io, ao, bo;
+    locate(pl, blockIdx.x, io, ao, bo);
+    float* trow = target + ao;
+    const float* irow = index + io;
+    const float* srow = src + bo;
+    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) {
+        tile[j] = trow[j];
+        if (MODE == 1) tag[j] = 0xffffffffu;
+    }
+    // the first chunk's entries are fetched while the row arrives
+    float next_i = 0.0f, next_v = value;
+    if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
+    __syncthreads();
+    for (uint32_t r0 = 0; r0 < pl.i_axis_len; r0 += THREADS) {
+        const uint32_t r = r0 + tid;
+        bool have = r < pl.i_axis_len;
+        const int sel_raw = static_cast<int>(next_i);
+        const float v = next_v;
+        if (r + THREADS < pl.i_axis_len) { next_i = irow[r + THREADS]; if (MODE != 2) next_v = srow[r + THREADS]; }
+        if (have && (sel_raw < 0 || static_cast<uint32_t>(sel_raw) >= pl.a_axis_len)) { *bad = 1; have = false; }
+        const uint32_t sel = have ? static_cast<uint32_t>(sel_raw) : 0u;
+        if (MODE == 2) {
+            if (have) tile[sel] = value;                   // equal values: the order of the stores is immaterial
+        } else if (MODE == 0) {
+            if (have) tile_bits[sel] = 0u;
+            __syncthreads();
+            if (have) atomicMax(&tile_bits[sel], tid + 1u);
+            __syncthreads();
+            const bool last = have && tile_bits[sel] == tid + 1u;
+            __syncthreads();
+            if (last) tile[sel] = v;
+            __syncthreads();
+        } else {
+            bool pending = have;
+            while (true) {
+                if (pending) atomicMin(&tag[sel], tid);
+                __syncthreads();
+                if (pending && tag[sel] == tid) {          // one lane per element gets here
+                    tile[sel] = tile[sel] + v;
+                    tag[sel] = 0xffffffffu;
+                    pending = false;
+                }
+                if (!__syncthreads_or(pending ? 1 : 0)) break;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) trow[j] = tile[j];
+}
+
 // indexSelect / indexAdd (JVMRawTensor.kt:484-516): the index is one list of k rows along the
 // axis, shared by every position. The tensor is seen as [outer, axis, inner].
 struct RowsPlan {
@@ -295,6 +365,128 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
     });
 }
 
+// The limits of scatter_rows_lds_kernel: the innermost axis, a target row that fits the LDS a
+// workgroup may have (with its tags in the add form), index rows long enough that moving the
+// whole row pays.
+// A workgroup may use 64 KiB of dynamic LDS unless the kernel is granted more; gfx950 has 160 KiB
+// per CU, so the three row kernels ask for 128 KiB once and fall back to 64 KiB if refused.
+static uint32_t scatter_lds_limit() {
+    static const uint32_t limit = [] {
+        const int want = 131072;
+        bool ok = true;
+        const void* wide[] = {reinterpret_cast<const void*>(&scatter_rows_lds_kernel<0, 1024>),
+                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<1, 1024>),
+                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<2, 1024>)};
+        for (const void* f : wide) ok = ok && hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, want) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        return ok ? 131072u : 65536u;
+    }();
+    return limit;
+}
+
+static bool scatter_rows_fit_lds(int mode, uint32_t a_axis_len, uint32_t i_axis_len) {
+    const uint64_t lds_bytes = static_cast<uint64_t>(a_axis_len) * (mode == 1 ? 8u : 4u);
+    return lds_bytes <= scatter_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
+}
+
+// Plans and launches on device pointers; shapes are validated by the caller.
+static int scatter_launch(int mode, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
+                          const float* psrc, const int32_t* src_shape, int dims, int axis, float value, uint64_t idx_n) {
+    IndexPlan pl{};
+    pl.ndim = dims - 1;
+    uint64_t positions = 1;
+    int n = 0;
+    for (int d = dims - 1; d >= 0; d--) {
+        if (d == axis) continue;
+        pl.size[n] = static_cast<uint32_t>(index_shape[d]);
+        pl.div[n] = make_div(pl.size[n]);
+        positions *= pl.size[n];
+        n++;
+    }
+    strides_without_axis(index_shape, dims, axis, pl.i_stride, &pl.i_axis_stride);
+    strides_without_axis(target_shape, dims, axis, pl.a_stride, &pl.a_axis_stride);
+    if (mode != 2) strides_without_axis(src_shape, dims, axis, pl.b_stride, &pl.b_axis_stride);
+    pl.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
+    pl.a_axis_len = static_cast<uint32_t>(target_shape[axis]);
+    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
+    const uint64_t bytes = (mode == 2 ? 2 : mode == 1 ? 4 : 3) * idx_n * 4;
+    if (axis == dims - 1 && scatter_rows_fit_lds(mode, pl.a_axis_len, pl.i_axis_len) && positions <= 0x7fffffffull) {
+        const uint32_t lds_bytes = pl.a_axis_len * (mode == 1 ? 8u : 4u);
+        const uint64_t row_bytes = (2ull * pl.a_axis_len * positions + (mode == 2 ? 1 : 2) * idx_n) * 4;
+        return with_index_check("Scatter", [&](int* flag) {
+            LaunchScope scope("scatter_rows_lds_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", row_bytes);
+            const dim3 grid(static_cast<uint32_t>(positions));
+            hipStream_t stream = state().stream;
+#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, value, pl, flag)
+            if (lds_bytes > 32768u) { if (mode == 0) ROWS_LAUNCH(0, 1024); else if (mode == 1) ROWS_LAUNCH(1, 1024); else ROWS_LAUNCH(2, 1024); }
+            else                    { if (mode == 0) ROWS_LAUNCH(0, 256);  else if (mode == 1) ROWS_LAUNCH(1, 256);  else ROWS_LAUNCH(2, 256); }
+#undef ROWS_LAUNCH
+        });
+    }
+    return with_index_check("Scatter", [&](int* flag) {
+        LaunchScope scope("scatter_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
+        const dim3 grid(blocks), block(kBlock);
+        const uint32_t p32 = static_cast<uint32_t>(positions);
+        hipStream_t stream = state().stream;
+        if (mode == 0)      hipLaunchKernelGGL((scatter_kernel<0>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag);
+        else if (mode == 1) hipLaunchKernelGGL((scatter_kernel<1>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag);
+        else                hipLaunchKernelGGL((scatter_kernel<2>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag);
+    });
+}
+
+// A scatter along an axis that is not the innermost walks that axis serially per position, about
+// 0.4 us a step once the positions no longer hide the latency. When the axis is long and the row
+// form above applies, it is cheaper to bring the axis to the innermost place with the permute
+// kernels (target, index and source), scatter rows there and permute the target back:
+// (4 target + 4 index + 2 source) elements of streaming traffic at about 5 TB/s.
+static bool scatter_pays_transposing(int mode, const int32_t* target_shape, const int32_t* index_shape, int dims, int axis,
+                                     uint64_t t_n, uint64_t idx_n, uint64_t src_n) {
+    if (axis == dims - 1) return false;
+    const uint32_t a_len = static_cast<uint32_t>(target_shape[axis]), i_len = static_cast<uint32_t>(index_shape[axis]);
+    if (i_len < 256 || !scatter_rows_fit_lds(mode, a_len, i_len)) return false;
+    const double positions = static_cast<double>(idx_n) / i_len;
+    const double serial_us = 0.4 * i_len * (positions > 5e5 ? positions / 5e5 : 1.0);
+    const double moved_us = 40.0 + (4.0 * t_n + 4.0 * idx_n + 2.0 * src_n) * 4.0 / 5e6;
+    return serial_us > 2.0 * moved_us;
+}
+
+static int scatter_transposed(int mode, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
+                              const float* psrc, const int32_t* src_shape, int dims, int axis, float value,
+                              uint64_t t_n, uint64_t idx_n, uint64_t src_n) {
+    int32_t to_last[KTH_MAX_DIMS], from_last[KTH_MAX_DIMS];          // axis -> innermost, and back
+    int32_t t_shape[KTH_MAX_DIMS], i_shape[KTH_MAX_DIMS], s_shape[KTH_MAX_DIMS];
+    for (int d = 0, k = 0; d < dims; d++) if (d != axis) to_last[k++] = d;
+    to_last[dims - 1] = axis;
+    for (int d = 0; d < dims; d++) {
+        from_last[to_last[d]] = d;
+        t_shape[d] = target_shape[to_last[d]];
+        i_shape[d] = index_shape[to_last[d]];
+        if (mode != 2) s_shape[d] = src_shape[to_last[d]];
+    }
+    uint64_t t_cap = 0, i_cap = 0, s_cap = 0;
+    float* t_moved = workspace_acquire(t_n * 4, &t_cap);
+    float* i_moved = t_moved ? workspace_acquire(idx_n * 4, &i_cap) : nullptr;
+    float* s_moved = (i_moved && mode != 2) ? workspace_acquire(src_n * 4, &s_cap) : nullptr;
+    int rc = KTH_E_MEMORY;
+    if (t_moved && i_moved && (mode == 2 || s_moved)) {
+        rc = permute_device("kth_scatter", target, t_moved, target_shape, dims, to_last);
+        if (rc == KTH_OK) rc = permute_device("kth_scatter", index, i_moved, index_shape, dims, to_last);
+        if (rc == KTH_OK && mode != 2) rc = permute_device("kth_scatter", psrc, s_moved, src_shape, dims, to_last);
+        if (rc == KTH_OK) {
+            rc = scatter_launch(mode, t_moved, t_shape, i_moved, i_shape, s_moved, s_shape, dims, dims - 1, value, idx_n);
+            // also after a reported index: the valid entries have been applied, as in the serial form
+            if (rc == KTH_OK || rc == KTH_E_ARGUMENT) {
+                const int back = permute_device("kth_scatter", t_moved, target, t_shape, dims, from_last);
+                if (back != KTH_OK) rc = back;
+            }
+        }
+    }
+    if (s_moved) workspace_release(s_moved, s_cap);
+    if (i_moved) workspace_release(i_moved, i_cap);
+    if (t_moved) workspace_release(t_moved, t_cap);
+    return rc;
+}
+
 static int scatter_common(int mode, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
                           uint64_t src, const int32_t* src_shape, int dims, int axis, float value) {
     KTH_REQUIRE_INIT();
@@ -321,34 +513,12 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
         return fail(KTH_E_ARGUMENT, "kth_scatter: a shape needs more elements than its store holds");
     if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
     if (idx_n == 0) return KTH_OK;
-    IndexPlan pl{};
-    pl.ndim = dims - 1;
-    uint64_t positions = 1;
-    int n = 0;
-    for (int d = dims - 1; d >= 0; d--) {
-        if (d == axis) continue;
-        pl.size[n] = static_cast<uint32_t>(index_shape[d]);
-        pl.div[n] = make_div(pl.size[n]);
-        positions *= pl.size[n];
-        n++;
-    }
-    strides_without_axis(index_shape, dims, axis, pl.i_stride, &pl.i_axis_stride);
-    strides_without_axis(target_shape, dims, axis, pl.a_stride, &pl.a_axis_stride);
-    if (mode != 2) strides_without_axis(src_shape, dims, axis, pl.b_stride, &pl.b_axis_stride);
-    pl.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
-    pl.a_axis_len = static_cast<uint32_t>(target_shape[axis]);
-    const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
     const float* psrc = ss ? ss->ptr : nullptr;
-    const uint64_t bytes = (mode == 2 ? 2 : mode == 1 ? 4 : 3) * idx_n * 4;
-    return with_index_check("Scatter", [&](int* flag) {
-        LaunchScope scope("scatter_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
-        const dim3 grid(blocks), block(kBlock);
-        const uint32_t p32 = static_cast<uint32_t>(positions);
-        hipStream_t stream = state().stream;
-        if (mode == 0)      hipLaunchKernelGGL((scatter_kernel<0>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
-        else if (mode == 1) hipLaunchKernelGGL((scatter_kernel<1>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
-        else                hipLaunchKernelGGL((scatter_kernel<2>), grid, block, 0, stream, st->ptr, sx->ptr, psrc, value, p32, pl, flag);
-    });
+    if (scatter_pays_transposing(mode, target_shape, index_shape, dims, axis, t_n, idx_n, src_n))
+        if (int rc = scatter_transposed(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value,
+                                        t_n, idx_n, src_n); rc != KTH_E_MEMORY)
+            return rc;                                   // no room for the transposed copies: the serial form below
+    return scatter_launch(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value, idx_n);
 }
 
 int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,

@@ -81,6 +81,10 @@ Store* lookup(uint64_t handle, const char* what);
 float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
 void   workspace_release(float* p, uint64_t cap_bytes);
 
+// out = in with its dims reordered: out dim d is in dim axes[d] (kth_layout.hip). Device pointers
+// to dense tensors of the same, non-zero element count; `axes` names every dim once.
+int permute_device(const char* what, const float* in, float* out, const int32_t* shape, int dims, const int32_t* axes);
+
 // Stable sort of n (key, value) pairs by the low `end_bit` bits of the key, on `stream`
 // (kth_sort.hip). With temp == nullptr only *temp_bytes is set, to the scratch size needed.
 hipError_t sort_pairs_u32(void* temp, size_t* temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,

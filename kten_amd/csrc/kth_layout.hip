@@ -404,7 +404,17 @@ int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims
     if (n > si->n_floats || n > so->n_floats) return fail(KTH_E_ARGUMENT, "%s: the shape needs more elements than a store holds", what);
     if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", what);
     if (n == 0) return KTH_OK;
+    return permute_device(what, si->ptr, so->ptr, shape, dims, axes);
+}
 
+}  // namespace
+
+namespace kth {
+
+// out = in with its dims reordered by `axes` (validated by the caller), both dense, n > 0 elements.
+int permute_device(const char* what, const float* in, float* out, const int32_t* shape, int dims, const int32_t* axes) {
+    uint64_t n = 1;
+    for (int d = 0; d < dims; d++) n *= static_cast<uint64_t>(shape[d]);
     uint64_t in_stride[KTH_MAX_DIMS];
     uint64_t run = 1;
     for (int d = dims - 1; d >= 0; d--) { in_stride[d] = run; run *= static_cast<uint64_t>(shape[d]); }
@@ -424,22 +434,22 @@ int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims
         int wx = -1;
         for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
         if (w.stride[0] != 1 && wx > 0 && w.size[0] >= 16 && w.size[wx] >= 16) {
-            if (int rc = launch_tiles(what, w, static_cast<int>(elem), si->ptr, so->ptr, n)) return rc;
+            if (int rc = launch_tiles(what, w, static_cast<int>(elem), in, out, n)) return rc;
             KTH_LAUNCH_CHECK("permute_tile_kernel");
             return KTH_OK;
         }
     }
     if (v.stride[0] == 1) {
-        launch_move<0>("move_kernel_permute", si->ptr, so->ptr, n, 0.0f, v, 0, n * 8);
+        launch_move<0>("move_kernel_permute", in, out, n, 0.0f, v, 0, n * 8);
         KTH_LAUNCH_CHECK("move_kernel");
         return KTH_OK;
     }
-    if (int rc = launch_tiles(what, v, 1, si->ptr, so->ptr, n)) return rc;
+    if (int rc = launch_tiles(what, v, 1, in, out, n)) return rc;
     KTH_LAUNCH_CHECK("permute_tile_kernel");
     return KTH_OK;
 }
 
-}  // namespace
+}  // namespace kth
 
 extern "C" {
 

@@ -14,7 +14,14 @@ CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([
          ([70000, 7], [70000, 3], 1), ([5, 3, 2, 2, 3, 2, 2, 2, 3, 4], [5, 3, 2, 2, 6, 2, 2, 2, 3, 4], 4),
          # long axes with many repeated indices (the last entry of a position wins)
          ([300, 400], [300, 400], 1), ([300, 400], [300, 400], 0), ([64, 2048], [64, 2048], 1), ([2048, 64], [2048, 40], 0),
-         ([8, 100, 128], [8, 90, 128], 1), ([50, 33, 70], [50, 33, 64], 2), ([40, 10], [40, 2000], 1)]
+         ([8, 100, 128], [8, 90, 128], 1), ([50, 33, 70], [50, 33, 64], 2), ([40, 10], [40, 2000], 1),
+         # rows along the innermost axis that are scattered inside LDS: the size limits of the assign and add forms
+         # and one past them, index dims smaller than the target's, one index value for a whole row
+         ([3, 16384], [3, 5000], 1), ([3, 8192], [3, 3000], 1), ([2, 8193], [2, 2000], 1), ([2, 16385], [2, 4000], 1),
+         ([2, 32768], [2, 5000], 1), ([2, 32769], [2, 5000], 1),
+         ([10, 6, 300], [7, 4, 100], 2), ([5, 1], [5, 700], 1), ([1, 4096], [1, 4096], 1),
+         # a long axis that is not the innermost: scattered as rows between two permutes
+         ([4096, 96], [4096, 96], 0), ([2, 3000, 40], [2, 2500, 33], 1), ([8192, 3, 5], [8000, 2, 5], 0), ([5000, 7], [700, 7], 0)]
 
 
 def both(gc, shape, array):
@@ -168,3 +175,33 @@ def test_index_add_full_size_round_trip(gc):
     got = one.toArray()
     assert_bits_equal(got[1], want, "serial float sum of the rows, in order")
     assert not got[0].any()
+
+
+def test_scatter_rows_with_a_larger_source_and_bad_values(gc):
+    """The source may be larger than the index in every dim (only the index's extent is read), and
+    an index value outside the axis is reported from the LDS form as from the serial one, with the
+    valid entries applied."""
+    rng = np.random.default_rng(11)
+    shape, ishape, sshape = [6, 500], [4, 300], [5, 450]
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = rng.integers(0, 500, size=ishape).astype(np.float32)
+    src = rng.standard_normal(sshape).astype(np.float32)
+    for name in ("inplaceScatter", "inplaceScatterAdd"):
+        gt, ct = both(gc, shape, x)
+        gi, ci = both(gc, ishape, idx); gs, cs = both(gc, sshape, src)
+        getattr(gt, name)(1, gi, gs); getattr(ct, name)(1, ci, cs)
+        assert_bits_equal(gt.toArray(), ct.toArray(), name + " with a larger source")
+    bad = idx.copy(); bad[2, 17] = 500.0; bad[0, 299] = -3.0
+    for name in ("inplaceScatter", "inplaceScatterAdd"):
+        gt = gc.createRaw(shape, x)
+        with pytest.raises(ValueError):
+            getattr(gt, name)(1, gc.createRaw(ishape, bad), gc.createRaw(sshape, src))
+    gt = gc.createRaw(shape, x)
+    with pytest.raises(ValueError):
+        gt.inplaceScatter(1, gc.createRaw(ishape, bad), 2.0)
+    ok = gc.createRaw(shape, x)
+    ok.inplaceScatter(1, gc.createRaw(ishape, idx), 2.0)          # the library is still usable
+    want = x.copy()
+    for r in range(4):
+        want[r, idx[r].astype(int)] = 2.0
+    assert_bits_equal(ok.toArray(), want, "fill after a reported error")
