@@ -1,9 +1,12 @@
 // gather / inplaceScatter / inplaceScatterAdd / inplaceScatter(Float) along an axis
 // (reference: JVMRawTensor.kt:227-255,317-353 with StoreIndexing.applyAt,
 // AbstractIndexing.kt:123-146). Positions run over the index tensor's shape without the
-// axis; one thread owns one position and walks the axis in ascending order, so within a
-// position duplicates resolve exactly as on the JVM ("last write wins", "added in order"),
-// and different positions never touch the same target element.
+// axis. Within a position duplicates resolve exactly as on the JVM ("last write wins", "added
+// in order"), and different positions never touch the same target element. Short index rows:
+// one thread owns one position and walks the axis in ascending order. Long index rows: a
+// workgroup owns the position, keeps its target row in LDS and orders the entries of each
+// chunk through LDS tags (axes other than the innermost are permuted there and back).
+// indexAdd sorts its index list so that every target row is updated by threads of its own.
 // Index values are floats: Kotlin's toInt() (truncate, NaN -> 0, saturate) is what
 // v_cvt_i32_f32 does. An index outside [0, axis length) is skipped and reported: the host
 // turns the report into the reference's IllegalArgumentException.
