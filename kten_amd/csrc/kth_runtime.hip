@@ -18,6 +18,11 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+// Counts kth_init calls that brought the library up. A new table slot starts its generation at
+// epoch << 20, so a handle from before a kth_shutdown does not validate against the stores of a
+// later session (unless a slot saw a million releases).
+static uint32_t g_epoch = 0;
+
 static inline uint64_t make_handle(uint32_t index, uint32_t generation) {
     return (static_cast<uint64_t>(generation) << 32) | static_cast<uint64_t>(index + 1);
 }
@@ -170,6 +175,7 @@ int kth_init(int device) {
     KTH_HIP(init_math_tables());
     s.device = device;
     s.ready = true;
+    g_epoch += 1;
     return KTH_OK;
 }
 
@@ -237,7 +243,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
                     (unsigned long long)s.total_mem);
     uint32_t idx;
     if (!s.free_slots.empty()) { idx = s.free_slots.back(); s.free_slots.pop_back(); }
-    else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); }
+    else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); s.table.back().generation = g_epoch << 20; }
     Store& st = s.table[idx];
     st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1;
     s.live_bytes += cap;
