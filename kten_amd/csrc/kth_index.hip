@@ -55,6 +55,38 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict_
     out[e] = in[ao + static_cast<uint32_t>(sel) * pl.a_axis_stride];
 }
 
+// gather along the innermost axis when the index rows are long: one workgroup per position reads
+// the input row into LDS as one contiguous span and serves out[r] = row[index[r]] from there, so
+// both the reads and the writes of global memory are contiguous. The plan is the scatter form:
+// position dims without the axis, i_stride for index and result, a_stride for the input.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void gather_rows_lds_kernel(const float* __restrict__ in, const float* __restrict__ index,
+                                                                 float* __restrict__ out, IndexPlan pl, int* bad) {
+    extern __shared__ float gather_row[];
+    const uint32_t tid = threadIdx.x;
+    uint32_t io, ao, bo;
+    locate(pl, blockIdx.x, io, ao, bo);
+    const float* arow = in + ao;
+    const float* irow = index + io;
+    float* orow = out + io;
+    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) gather_row[j] = arow[j];
+    __syncthreads();
+    constexpr uint32_t kBatch = 4;
+    for (uint32_t r0 = tid; r0 < pl.i_axis_len; r0 += kBatch * THREADS) {
+        float fi[kBatch];
+#pragma unroll
+        for (uint32_t k = 0; k < kBatch; k++) if (r0 + k * THREADS < pl.i_axis_len) fi[k] = irow[r0 + k * THREADS];
+#pragma unroll
+        for (uint32_t k = 0; k < kBatch; k++) {
+            if (r0 + k * THREADS < pl.i_axis_len) {
+                const int sel = static_cast<int>(fi[k]);
+                if (sel < 0 || static_cast<uint32_t>(sel) >= pl.a_axis_len) { *bad = 1; continue; }
+                orow[r0 + k * THREADS] = gather_row[sel];
+            }
+        }
+    }
+}
+
 // MODE 0: assign from src, 1: add from src, 2: assign the constant.
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ target, const float* __restrict__ index,
@@ -323,6 +355,35 @@ int with_index_check(const char* what, F launch) {
     return KTH_OK;
 }
 
+// The limits of scatter_rows_lds_kernel: the innermost axis, a target row that fits the LDS a
+// workgroup may have (with its tags in the add form), index rows long enough that moving the
+// whole row pays.
+// A workgroup may use 64 KiB of dynamic LDS unless the kernel is granted more; gfx950 has 160 KiB
+// per CU, so the row kernels ask for 128 KiB once and fall back to 64 KiB if refused.
+static uint32_t rows_lds_limit() {
+    static const uint32_t limit = [] {
+        const int want = 131072;
+        bool ok = true;
+        const void* wide[] = {reinterpret_cast<const void*>(&scatter_rows_lds_kernel<0, 1024>),
+                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<1, 1024>),
+                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<2, 1024>)};
+        ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&gather_rows_lds_kernel<1024>), hipFuncAttributeMaxDynamicSharedMemorySize, want) == hipSuccess;
+        for (const void* f : wide) ok = ok && hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, want) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        return ok ? 131072u : 65536u;
+    }();
+    return limit;
+}
+
+static bool gather_rows_fit_lds(uint32_t a_axis_len, uint32_t i_axis_len) {
+    return static_cast<uint64_t>(a_axis_len) * 4u <= rows_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
+}
+
+static bool scatter_rows_fit_lds(int mode, uint32_t a_axis_len, uint32_t i_axis_len) {
+    const uint64_t lds_bytes = static_cast<uint64_t>(a_axis_len) * (mode == 1 ? 8u : 4u);
+    return lds_bytes <= rows_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
+}
+
 }  // namespace
 
 extern "C" {
@@ -349,6 +410,29 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
         return fail(KTH_E_ARGUMENT, "kth_gather: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_gather: output aliases an input");
     if (idx_n == 0) return KTH_OK;
+    if (gather_rows_fit_lds(static_cast<uint32_t>(in_shape[axis]), static_cast<uint32_t>(index_shape[axis])) && axis == dims - 1) {
+        IndexPlan rp{};
+        rp.ndim = dims - 1;
+        uint64_t positions = 1;
+        for (int d = dims - 2, n = 0; d >= 0; d--, n++) {
+            rp.size[n] = static_cast<uint32_t>(index_shape[d]);
+            rp.div[n] = make_div(rp.size[n]);
+            positions *= rp.size[n];
+        }
+        strides_without_axis(index_shape, dims, axis, rp.i_stride, &rp.i_axis_stride);
+        strides_without_axis(in_shape, dims, axis, rp.a_stride, &rp.a_axis_stride);
+        rp.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
+        rp.a_axis_len = static_cast<uint32_t>(in_shape[axis]);
+        const uint32_t lds_bytes = rp.a_axis_len * 4u;
+        return with_index_check("Gather", [&](int* flag) {
+            LaunchScope scope("gather_rows_lds_kernel", "", (positions * rp.a_axis_len + 2 * idx_n) * 4);
+            const dim3 grid(static_cast<uint32_t>(positions));
+            if (lds_bytes > 32768u)
+                hipLaunchKernelGGL((gather_rows_lds_kernel<1024>), grid, dim3(1024), lds_bytes, state().stream, si->ptr, sx->ptr, so->ptr, rp, flag);
+            else
+                hipLaunchKernelGGL((gather_rows_lds_kernel<256>), grid, dim3(256), lds_bytes, state().stream, si->ptr, sx->ptr, so->ptr, rp, flag);
+        });
+    }
     IndexPlan pl{};
     pl.ndim = dims;
     uint64_t in_run = 1;
@@ -366,30 +450,6 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
         hipLaunchKernelGGL(gather_kernel, dim3(blocks), dim3(kBlock), 0, state().stream, si->ptr, sx->ptr, so->ptr,
                            static_cast<uint32_t>(idx_n), pl, flag);
     });
-}
-
-// The limits of scatter_rows_lds_kernel: the innermost axis, a target row that fits the LDS a
-// workgroup may have (with its tags in the add form), index rows long enough that moving the
-// whole row pays.
-// A workgroup may use 64 KiB of dynamic LDS unless the kernel is granted more; gfx950 has 160 KiB
-// per CU, so the three row kernels ask for 128 KiB once and fall back to 64 KiB if refused.
-static uint32_t scatter_lds_limit() {
-    static const uint32_t limit = [] {
-        const int want = 131072;
-        bool ok = true;
-        const void* wide[] = {reinterpret_cast<const void*>(&scatter_rows_lds_kernel<0, 1024>),
-                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<1, 1024>),
-                              reinterpret_cast<const void*>(&scatter_rows_lds_kernel<2, 1024>)};
-        for (const void* f : wide) ok = ok && hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, want) == hipSuccess;
-        if (!ok) (void)hipGetLastError();
-        return ok ? 131072u : 65536u;
-    }();
-    return limit;
-}
-
-static bool scatter_rows_fit_lds(int mode, uint32_t a_axis_len, uint32_t i_axis_len) {
-    const uint64_t lds_bytes = static_cast<uint64_t>(a_axis_len) * (mode == 1 ? 8u : 4u);
-    return lds_bytes <= scatter_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
 }
 
 // Plans and launches on device pointers; shapes are validated by the caller.

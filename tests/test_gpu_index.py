@@ -199,6 +199,10 @@ def test_scatter_rows_with_a_larger_source_and_bad_values(gc):
     gt = gc.createRaw(shape, x)
     with pytest.raises(ValueError):
         gt.inplaceScatter(1, gc.createRaw(ishape, bad), 2.0)
+    with pytest.raises(ValueError):
+        gc.createRaw(shape, x).gather(1, gc.createRaw(ishape, bad))
+    assert_bits_equal(gc.createRaw(shape, x).gather(1, gc.createRaw(ishape, idx)).toArray(),
+                      np.take_along_axis(x[:4], idx.astype(np.int64), 1), "gather of long rows after a reported error")
     ok = gc.createRaw(shape, x)
     ok.inplaceScatter(1, gc.createRaw(ishape, idx), 2.0)          # the library is still usable
     want = x.copy()
