@@ -58,7 +58,8 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict_
 // gather along the innermost axis when the index rows are long: one workgroup per position reads
 // the input row into LDS as one contiguous span and serves out[r] = row[index[r]] from there, so
 // both the reads and the writes of global memory are contiguous. The plan is the scatter form:
-// position dims without the axis, i_stride for index and result, a_stride for the input.
+// position dims without the axis, i_stride for the index, a_stride for the input, b_stride for
+// the result (indexSelect along the innermost axis is the same with one index row for all: i_stride 0).
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void gather_rows_lds_kernel(const float* __restrict__ in, const float* __restrict__ index,
                                                                  float* __restrict__ out, IndexPlan pl, int* bad) {
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(THREADS) void gather_rows_lds_kernel(const float* _
     locate(pl, blockIdx.x, io, ao, bo);
     const float* arow = in + ao;
     const float* irow = index + io;
-    float* orow = out + io;
+    float* orow = out + bo;
     for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) gather_row[j] = arow[j];
     __syncthreads();
     constexpr uint32_t kBatch = 4;
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         const uint32_t r = r0 + tid;
         bool have = r < pl.i_axis_len;
         const int sel_raw = static_cast<int>(next_i);
-        const float v = next_v;
+        const float v = MODE == 1 ? next_v * value : next_v;      // add form: value is the factor on the source (1 for scatterAdd)
         if (r + THREADS < pl.i_axis_len) { next_i = irow[r + THREADS]; if (MODE != 2) next_v = srow[r + THREADS]; }
         if (have && (sel_raw < 0 || static_cast<uint32_t>(sel_raw) >= pl.a_axis_len)) { *bad = 1; have = false; }
         const uint32_t sel = have ? static_cast<uint32_t>(sel_raw) : 0u;
@@ -420,6 +421,7 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
             positions *= rp.size[n];
         }
         strides_without_axis(index_shape, dims, axis, rp.i_stride, &rp.i_axis_stride);
+        strides_without_axis(index_shape, dims, axis, rp.b_stride, &rp.b_axis_stride);
         strides_without_axis(in_shape, dims, axis, rp.a_stride, &rp.a_axis_stride);
         rp.i_axis_len = static_cast<uint32_t>(index_shape[axis]);
         rp.a_axis_len = static_cast<uint32_t>(in_shape[axis]);
@@ -480,7 +482,8 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
             LaunchScope scope("scatter_rows_lds_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", row_bytes);
             const dim3 grid(static_cast<uint32_t>(positions));
             hipStream_t stream = state().stream;
-#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, value, pl, flag)
+            const float factor = mode == 1 ? 1.0f : value;
+#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag)
             if (lds_bytes > 32768u) { if (mode == 0) ROWS_LAUNCH(0, 1024); else if (mode == 1) ROWS_LAUNCH(1, 1024); else ROWS_LAUNCH(2, 1024); }
             else                    { if (mode == 0) ROWS_LAUNCH(0, 256);  else if (mode == 1) ROWS_LAUNCH(1, 256);  else ROWS_LAUNCH(2, 256); }
 #undef ROWS_LAUNCH
@@ -623,6 +626,24 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
         return fail(KTH_E_ARGUMENT, "kth_index_select: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_index_select: output aliases an input");
     if (n_out == 0) return KTH_OK;
+    if (inner == 1 && gather_rows_fit_lds(static_cast<uint32_t>(shape[axis]), static_cast<uint32_t>(k))) {
+        // columns picked from contiguous rows: the gather row kernel with one index row for every position
+        IndexPlan rp{};
+        rp.ndim = 1;
+        rp.size[0] = static_cast<uint32_t>(outer); rp.div[0] = make_div(rp.size[0]);
+        rp.i_stride[0] = 0; rp.a_stride[0] = static_cast<uint32_t>(shape[axis]); rp.b_stride[0] = static_cast<uint32_t>(k);
+        rp.i_axis_stride = rp.a_axis_stride = rp.b_axis_stride = 1;
+        rp.i_axis_len = static_cast<uint32_t>(k); rp.a_axis_len = static_cast<uint32_t>(shape[axis]);
+        const uint32_t lds_bytes = rp.a_axis_len * 4u;
+        return with_index_check("Index select", [&](int* flag) {
+            LaunchScope scope("gather_rows_lds_kernel", "indexSelect", (total + n_out + k) * 4);
+            const dim3 grid(static_cast<uint32_t>(outer));
+            if (lds_bytes > 32768u)
+                hipLaunchKernelGGL((gather_rows_lds_kernel<1024>), grid, dim3(1024), lds_bytes, state().stream, si->ptr, sx->ptr, so->ptr, rp, flag);
+            else
+                hipLaunchKernelGGL((gather_rows_lds_kernel<256>), grid, dim3(256), lds_bytes, state().stream, si->ptr, sx->ptr, so->ptr, rp, flag);
+        });
+    }
     const bool vec = inner % 4 == 0;
     RowsPlan pl{};
     pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k);
@@ -659,6 +680,26 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k); pl.inner = static_cast<uint32_t>(inner);
     pl.inner_div = make_div(pl.inner); pl.k_div = make_div(pl.k);
     hipStream_t stream = state().stream;
+
+    if (inner == 1 && scatter_rows_fit_lds(1, pl.axis_len, pl.k)) {
+        // columns added into contiguous rows: the scatter row kernel in its add form, one index row for
+        // every position and alpha as the factor on the source
+        IndexPlan rp{};
+        rp.ndim = 1;
+        rp.size[0] = static_cast<uint32_t>(outer); rp.div[0] = make_div(rp.size[0]);
+        rp.i_stride[0] = 0; rp.a_stride[0] = pl.axis_len; rp.b_stride[0] = pl.k;
+        rp.i_axis_stride = rp.a_axis_stride = rp.b_axis_stride = 1;
+        rp.i_axis_len = pl.k; rp.a_axis_len = pl.axis_len;
+        const uint32_t lds_bytes = rp.a_axis_len * 8u;
+        return with_index_check("Index Add", [&](int* flag) {
+            LaunchScope scope("scatter_rows_lds_kernel", "indexAdd", (2 * total + n_src + k) * 4);
+            const dim3 grid(static_cast<uint32_t>(outer));
+            if (lds_bytes > 32768u)
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag);
+            else
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag);
+        });
+    }
 
     // A short list: one thread per (outer, column) position walks it in order. The walk is serial,
     // about half a microsecond per entry, so from kSortedFrom entries on the list is sorted instead
