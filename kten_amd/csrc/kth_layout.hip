@@ -87,6 +87,54 @@ __global__ __launch_bounds__(kBlock) void move_kernel(const float* __restrict__ 
     }
 }
 
+// The same moves when the strided side cannot take float4s (odd run lengths or offsets): the
+// dense side still moves as float4s, 16-byte aligned from the start of its store, and the four
+// floats of each meet the strided side one by one. Lanes next to each other stay next to each
+// other on both sides, so the scalar accesses coalesce. `n` counts floats; MODE 0 and 1 only.
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                           uint32_t n, MovePlan pl) {
+    const uint32_t base = blockIdx.x * (kBlock * kMoveUnroll) + threadIdx.x;
+    uint32_t at[kMoveUnroll][4];
+    v4f v[kMoveUnroll];
+#pragma unroll
+    for (int k = 0; k < kMoveUnroll; k++) {
+        const uint32_t i = (base + k * kBlock) * 4u;
+        if (i >= n) continue;
+        // position inside the innermost run decides whether the four floats share it
+        const uint32_t q0 = (__umulhi(i, pl.div[0].mul) + i) >> pl.div[0].shift;
+        const uint32_t r0 = i - q0 * pl.size[0];
+        at[k][0] = strided_offset(pl, i);
+#pragma unroll
+        for (int j = 1; j < 4; j++)
+            at[k][j] = (pl.ndim == 1 || r0 + j < pl.size[0]) ? at[k][0] + j * pl.stride[0] : (i + j < n ? strided_offset(pl, i + j) : at[k][0]);
+        if (MODE == 0) {
+            v[k].x = src[at[k][0]];
+            v[k].y = i + 1 < n ? src[at[k][1]] : 0.0f;
+            v[k].z = i + 2 < n ? src[at[k][2]] : 0.0f;
+            v[k].w = i + 3 < n ? src[at[k][3]] : 0.0f;
+        } else if (i + 3 < n) {
+            v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + i));
+        } else {
+            v[k].x = src[i]; v[k].y = i + 1 < n ? src[i + 1] : 0.0f; v[k].z = i + 2 < n ? src[i + 2] : 0.0f; v[k].w = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kMoveUnroll; k++) {
+        const uint32_t i = (base + k * kBlock) * 4u;
+        if (i >= n) continue;
+        if (MODE == 0) {
+            if (i + 3 < n) *reinterpret_cast<v4f*>(dst + i) = v[k];
+            else { dst[i] = v[k].x; if (i + 1 < n) dst[i + 1] = v[k].y; if (i + 2 < n) dst[i + 2] = v[k].z; }
+        } else {
+            dst[at[k][0]] = v[k].x;
+            if (i + 1 < n) dst[at[k][1]] = v[k].y;
+            if (i + 2 < n) dst[at[k][2]] = v[k].z;
+            if (i + 3 < n) dst[at[k][3]] = v[k].w;
+        }
+    }
+}
+
 // A permutation that moves the input's contiguous dim X away from the innermost place:
 // the output's innermost dim is Y (input stride y_in_stride), X lands at output stride
 // x_out_stride, and every other dim is a batch dim with its own pair of strides.
@@ -265,6 +313,13 @@ void launch_move(const char* family, const float* src, float* dst, uint64_t coun
     if (vec) { pl.size[0] /= 4; pl.stride[0] = 4; units = count / 4; }
     for (int d = 0; d < dims.n; d++) pl.div[d] = make_div(pl.size[d]);
     const uint32_t per_block = kBlock * kMoveUnroll;
+    if constexpr (MODE != 2) if (!vec && count >= 1024) {
+        const uint32_t blocks4 = static_cast<uint32_t>(((count + 3) / 4 + per_block - 1) / per_block);
+        LaunchScope scope(family, "float4 dense side", bytes);
+        hipLaunchKernelGGL((move_mixed_kernel<MODE>), dim3(blocks4), dim3(kBlock), 0, state().stream, src, dst,
+                           static_cast<uint32_t>(count), pl);
+        return;
+    }
     const uint32_t blocks = static_cast<uint32_t>((units + per_block - 1) / per_block);
     LaunchScope scope(family, vec ? "float4" : "float", bytes);
     if (vec) hipLaunchKernelGGL((move_kernel<MODE, true>), dim3(blocks), dim3(kBlock), 0, state().stream, src, dst,
