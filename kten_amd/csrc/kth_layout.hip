@@ -200,6 +200,79 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
     }
 }
 
+// A permutation that keeps a short innermost run of `run` floats (5 ... 63 here) in place and
+// transposes the dims outside it: the tile is T x T runs (T = 16 for runs up to 16 floats, 8
+// above), read as T spans of T * run contiguous floats (x fastest) and written as T spans of
+// T * run contiguous floats (y fastest). LDS holds the tile as [x][y][run] at an odd pitch per x,
+// so the store phase reads it linearly. Lengths, strides and offsets of `t` count runs. The
+// element V is a float4 when the run is a multiple of 4 floats (run, pitch then count float4s).
+struct RunsPlan {
+    TilePlan t;
+    uint32_t run, tile, pitch;               // elements per run, runs per tile side, LDS elements per x
+    FastDiv  in_row_div, run_div, out_row_div;
+};
+
+template <class V>
+__global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restrict__ in, V* __restrict__ out, RunsPlan rp) {
+    constexpr uint32_t kElems = kTileElems * sizeof(float) / sizeof(V);      // 16 KiB of elements
+    __shared__ V tile[kElems + 64];
+    const TilePlan& pl = rp.t;
+    uint32_t t = blockIdx.x;
+    uint32_t q = (__umulhi(t, pl.x_tiles_div.mul) + t) >> pl.x_tiles_div.shift;
+    const uint32_t x0 = (t - q * pl.x_tiles) * rp.tile;
+    t = q;
+    q = (__umulhi(t, pl.y_tiles_div.mul) + t) >> pl.y_tiles_div.shift;
+    const uint32_t y0 = (t - q * pl.y_tiles) * rp.tile;
+    t = q;
+    uint32_t in_off = 0, out_off = 0;
+    for (int d = 0; d < pl.nbatch; d++) {
+        q = (__umulhi(t, pl.bdiv[d].mul) + t) >> pl.bdiv[d].shift;
+        const uint32_t r = t - q * pl.bsize[d];
+        in_off += r * pl.b_in[d];
+        out_off += r * pl.b_out[d];
+        t = q;
+    }
+    const uint32_t row = rp.tile * rp.run;                   // elements of one span
+    const uint32_t floats = rp.tile * row;
+    const V* src = in + (static_cast<size_t>(in_off) + x0) * rp.run;
+    V* dst = out + (static_cast<size_t>(out_off) + y0) * rp.run;
+    const uint32_t x_floats = min(rp.tile, pl.x_len - x0) * rp.run;   // valid part of an input span
+    const uint32_t y_floats = min(rp.tile, pl.y_len - y0) * rp.run;   // valid part of an output span
+    constexpr uint32_t kPasses = kElems / kBlock;
+    V v[kPasses];
+#pragma unroll
+    for (uint32_t k = 0; k < kPasses; k++) {
+        const uint32_t f = k * kBlock + threadIdx.x;
+        if (f < floats) {
+            const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
+            const uint32_t p = f - y * row;
+            if (y0 + y < pl.y_len && p < x_floats)
+                v[k] = __builtin_nontemporal_load(src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p);
+        }
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kPasses; k++) {
+        const uint32_t f = k * kBlock + threadIdx.x;
+        if (f < floats) {
+            const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
+            const uint32_t p = f - y * row;
+            const uint32_t x = (__umulhi(p, rp.run_div.mul) + p) >> rp.run_div.shift;
+            tile[x * rp.pitch + y * rp.run + (p - x * rp.run)] = v[k];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t k = 0; k < kPasses; k++) {
+        const uint32_t f = k * kBlock + threadIdx.x;
+        if (f < floats) {
+            const uint32_t x = (__umulhi(f, rp.out_row_div.mul) + f) >> rp.out_row_div.shift;
+            const uint32_t p = f - x * row;
+            if (x0 + x < pl.x_len && p < y_floats)
+                dst[static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p] = tile[x * rp.pitch + p];
+        }
+    }
+}
+
 // Many small transposes: the (x, y) slab of x_len * y_len floats is contiguous on both sides
 // and so is the batch dim right outside it, so a workgroup moves a run of whole slabs: one
 // contiguous span in, the same span out, the transposition done by the LDS addressing (rows
@@ -354,7 +427,7 @@ int box_of(const char* what, const int32_t* shape, int dims, const int32_t* firs
 }
 
 // Permutes through LDS tiles. `v`: the output's dims innermost first with the input's strides,
-// in units of `elem` floats (1, 2 or 4), stride[0] != 1. Returns KTH_OK after launching.
+// in units of `elem` floats (1, 2, 4, or a run of 5 ... 63), stride[0] != 1. Returns KTH_OK after launching.
 int launch_tiles(const char* what, const StridedDims& v, int elem, const float* in, float* out, uint64_t n) {
     int px = -1;
     for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
@@ -407,6 +480,28 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     TilePlan pl{};
     pl.x_len = x_len; pl.y_len = y_len; pl.y_in_stride = y_in_stride;
     pl.x_out_stride = static_cast<uint32_t>(x_out_stride);
+    if (elem > 4) {
+        RunsPlan rp{};
+        const bool vec = elem % 4 == 0;
+        rp.run = static_cast<uint32_t>(vec ? elem / 4 : elem);
+        rp.tile = elem <= 16 ? 16u : 8u;
+        rp.pitch = (rp.tile * rp.run) | 1u;
+        rp.in_row_div = make_div(rp.tile * rp.run); rp.out_row_div = rp.in_row_div; rp.run_div = make_div(rp.run);
+        pl.x_tiles = (pl.x_len + rp.tile - 1) / rp.tile;
+        pl.y_tiles = (pl.y_len + rp.tile - 1) / rp.tile;
+        pl.x_tiles_div = make_div(pl.x_tiles);
+        pl.y_tiles_div = make_div(pl.y_tiles);
+        pl.nbatch = nb;
+        for (int d = 0; d < nb; d++) { pl.bsize[d] = bsize[d]; pl.bdiv[d] = make_div(bsize[d]); pl.b_in[d] = b_in[d]; pl.b_out[d] = b_out[d]; }
+        rp.t = pl;
+        const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
+        if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+        LaunchScope scope("permute_runs_kernel", vec ? "float4" : "float", n * 8);
+        if (vec) hipLaunchKernelGGL((permute_runs_kernel<v4f>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream,
+                                    reinterpret_cast<const v4f*>(in), reinterpret_cast<v4f*>(out), rp);
+        else     hipLaunchKernelGGL((permute_runs_kernel<float>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, in, out, rp);
+        return KTH_OK;
+    }
     // Tile shape: narrow along a dim shorter than 64 (the smallest power of two that holds it), square
     // otherwise; vector elements use one shape of 16 KiB.
     uint32_t tx = 64, ty = 64;
@@ -491,6 +586,21 @@ int permute_device(const char* what, const float* in, float* out, const int32_t*
         if (w.stride[0] != 1 && wx > 0 && w.size[0] >= 16 && w.size[wx] >= 16) {
             if (int rc = launch_tiles(what, w, static_cast<int>(elem), in, out, n)) return rc;
             KTH_LAUNCH_CHECK("permute_tile_kernel");
+            return KTH_OK;
+        }
+    }
+    if (v.stride[0] == 1 && v.size[0] >= 5 && (v.size[0] < 32 || (v.size[0] < 64 && v.size[0] % 4 != 0)) && v.n >= 3) {
+        // A run of 5 ... 31 floats that stays innermost (up to 63 when it cannot move as float4s): tiles of
+        // runs, when both transposed dims can fill one.
+        const uint64_t run = v.size[0];
+        StridedDims w{};
+        for (int d = 1; d < v.n; d++) { w.size[w.n] = v.size[d]; w.stride[w.n] = v.stride[d] / run; w.n++; }
+        int wx = -1;
+        for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
+        const uint64_t side = run <= 16 ? 16 : 8;
+        if (w.stride[0] != 1 && wx > 0 && w.size[0] >= side && w.size[wx] >= side) {
+            if (int rc = launch_tiles(what, w, static_cast<int>(run), in, out, n)) return rc;
+            KTH_LAUNCH_CHECK("permute_runs_kernel");
             return KTH_OK;
         }
     }

@@ -113,7 +113,11 @@ def test_transpose_every_axis_pair(shape, gc):
 PERMUTE_SHAPES = [[2, 3, 2], [5, 6, 7], [8, 64, 68], [2, 3, 4, 5], [3, 4, 64, 65], [4, 16, 20, 24], [2, 2, 3, 3, 4, 4],
                   [128, 3], [6, 1, 5, 1],
                   # float4 / float2 elements kept innermost; batched small slabs; narrow tiles with ragged edges
-                  [20, 33, 4], [17, 40, 2], [3, 18, 21, 4], [50, 6, 7], [1000, 16, 4], [70, 3, 100], [5, 9, 130, 3]]
+                  [20, 33, 4], [17, 40, 2], [3, 18, 21, 4], [50, 6, 7], [1000, 16, 4], [70, 3, 100], [5, 9, 130, 3],
+                  # a run of 5 ... 63 floats kept innermost: tiles of runs (float4 and scalar), ragged tile edges, exact tiles,
+                  # a batch dim outside, a merged run ([.., 3, 4] -> 12), dims too short for a tile (the strided move instead)
+                  [40, 50, 8], [33, 47, 12], [20, 35, 7], [18, 70, 33], [3, 17, 19, 5], [16, 16, 31], [19, 23, 3, 4], [100, 9, 6],
+                  [9, 10, 63], [16, 48, 28]]
 
 
 @pytest.mark.parametrize("shape", PERMUTE_SHAPES, ids=lambda s: "x".join(map(str, s)))
