@@ -200,9 +200,9 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
     }
 }
 
-// A permutation that keeps a short innermost run of `run` floats (5 ... 63 here) in place and
-// transposes the dims outside it: the tile is T x T runs (T = 16 for runs up to 16 floats, 8
-// above), read as T spans of T * run contiguous floats (x fastest) and written as T spans of
+// A permutation that keeps a short innermost run of `run` floats (3 ... 63 here) in place and
+// transposes the dims outside it: the tile is T x T runs (T = 32 for runs up to 4 floats, 16 up
+// to 16 floats, 8 above), read as T spans of T * run contiguous floats (x fastest) and written as T spans of
 // T * run contiguous floats (y fastest). LDS holds the tile as [x][y][run] at an odd pitch per x,
 // so the store phase reads it linearly. Lengths, strides and offsets of `t` count runs. The
 // element V is a float4 when the run is a multiple of 4 floats (run, pitch then count float4s).
@@ -427,7 +427,7 @@ int box_of(const char* what, const int32_t* shape, int dims, const int32_t* firs
 }
 
 // Permutes through LDS tiles. `v`: the output's dims innermost first with the input's strides,
-// in units of `elem` floats (1, 2, 4, or a run of 5 ... 63), stride[0] != 1. Returns KTH_OK after launching.
+// in units of `elem` floats (1, 2, 4, or a run of 3 ... 63), stride[0] != 1. Returns KTH_OK after launching.
 int launch_tiles(const char* what, const StridedDims& v, int elem, const float* in, float* out, uint64_t n) {
     int px = -1;
     for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
@@ -480,11 +480,11 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     TilePlan pl{};
     pl.x_len = x_len; pl.y_len = y_len; pl.y_in_stride = y_in_stride;
     pl.x_out_stride = static_cast<uint32_t>(x_out_stride);
-    if (elem > 4) {
+    if (elem == 3 || elem > 4) {
         RunsPlan rp{};
         const bool vec = elem % 4 == 0;
         rp.run = static_cast<uint32_t>(vec ? elem / 4 : elem);
-        rp.tile = elem <= 16 ? 16u : 8u;
+        rp.tile = elem <= 4 ? 32u : elem <= 16 ? 16u : 8u;
         rp.pitch = (rp.tile * rp.run) | 1u;
         rp.in_row_div = make_div(rp.tile * rp.run); rp.out_row_div = rp.in_row_div; rp.run_div = make_div(rp.run);
         pl.x_tiles = (pl.x_len + rp.tile - 1) / rp.tile;
@@ -589,15 +589,15 @@ int permute_device(const char* what, const float* in, float* out, const int32_t*
             return KTH_OK;
         }
     }
-    if (v.stride[0] == 1 && v.size[0] >= 5 && (v.size[0] < 32 || (v.size[0] < 64 && v.size[0] % 4 != 0)) && v.n >= 3) {
-        // A run of 5 ... 31 floats that stays innermost (up to 63 when it cannot move as float4s): tiles of
+    if (v.stride[0] == 1 && v.size[0] >= 3 && (v.size[0] < 32 || (v.size[0] < 64 && v.size[0] % 4 != 0)) && v.n >= 3) {
+        // A run of 3 ... 31 floats that stays innermost (up to 63 when it cannot move as float4s): tiles of
         // runs, when both transposed dims can fill one.
         const uint64_t run = v.size[0];
         StridedDims w{};
         for (int d = 1; d < v.n; d++) { w.size[w.n] = v.size[d]; w.stride[w.n] = v.stride[d] / run; w.n++; }
         int wx = -1;
         for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
-        const uint64_t side = run <= 16 ? 16 : 8;
+        const uint64_t side = run <= 4 ? 32 : run <= 16 ? 16 : 8;
         if (w.stride[0] != 1 && wx > 0 && w.size[0] >= side && w.size[wx] >= side) {
             if (int rc = launch_tiles(what, w, static_cast<int>(run), in, out, n)) return rc;
             KTH_LAUNCH_CHECK("permute_runs_kernel");
