@@ -276,8 +276,9 @@ def py_lane(op, lane):
     f32 = np.float32
     if op in ("sum", "mean"):
         acc = f32(0.0)
-        for v in lane:
-            acc = f32(acc + f32(v))
+        with np.errstate(invalid="ignore"):             # inf + -inf is part of the cases
+            for v in lane:
+                acc = f32(acc + f32(v))
         return acc if op == "sum" else f32(acc / f32(len(lane)))
     if op in ("max", "min"):
         acc = f32(-np.inf) if op == "max" else f32(np.inf)
