@@ -117,7 +117,8 @@ __device__ __forceinline__ void emit(const Geom& g, uint32_t o, uint32_t s, uint
 // ---------------------------------------------------------------- rows: inner == 1
 
 // G lanes per row (G in {1, 2, 4, 16, 64}, or 256 = the whole workgroup).
-// VEC = 4 requires axis % 4 == 0 and seg_len % 4 == 0 so every row segment is 16-byte aligned.
+// VEC = 4 requires axis % 4 == 0 and seg_len % 4 == 0 so every row segment is 16-byte aligned;
+// VEC = 1 takes any row and peels it to 16-byte boundaries.
 template <class R, int G, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                             typename R::Acc* __restrict__ partial, Geom g) {
@@ -152,15 +153,30 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
                 R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
             }
         } else {
-            uint32_t j = begin + lane;
-            for (; j + (kBatch - 1) * G < end; j += kBatch * G) {
-                float v[kBatch];
+            // Rows that do not start on 16-byte boundaries: up to three single floats reach the next
+            // boundary, float4s cover the middle, up to three single floats finish the segment. A
+            // lane meets its elements in ascending index order, as the arg reducers require.
+            const uint32_t skew = static_cast<uint32_t>((static_cast<size_t>(row) * g.axis + begin) & 3u);
+            const uint32_t head = min((4u - skew) & 3u, end - begin);
+            for (uint32_t e = begin + lane; e < begin + head; e += G) R::step(acc, ld1_stream(base + e), e);
+            const uint32_t body = begin + head;
+            const uint32_t body_end = body + ((end - body) & ~3u);
+            uint32_t j = body + lane * 4;
+            for (; j + (kBatch - 1) * G * 4 < body_end; j += kBatch * G * 4) {
+                float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + j + k * G);
+                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + j + k * G * 4);
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) R::step(acc, v[k], j + k * G);
+                for (uint32_t k = 0; k < kBatch; k++) {
+                    const uint32_t jj = j + k * G * 4;
+                    R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3);
+                }
             }
-            for (; j < end; j += G) R::step(acc, ld1_stream(base + j), j);
+            for (; j < body_end; j += G * 4) {
+                float4 v = ld4_stream(base + j);
+                R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
+            }
+            for (uint32_t e = body_end + lane; e < end; e += G) R::step(acc, ld1_stream(base + e), e);
         }
     }
     constexpr int kLanes = G < kWave ? G : kWave;
@@ -181,10 +197,10 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
     }
 }
 
-// ---------------------------------------------------------------- short rows: inner == 1, 8 <= axis < 256
+// ---------------------------------------------------------------- short rows: inner == 1, 2 <= axis < 256
 
 // Rows this short are contiguous in memory one after the other, so a workgroup takes a tile of
-// `rows` whole rows (a power of two in 32..1024, rows * axis <= kShortTile floats) as ONE contiguous
+// `rows` whole rows (a power of two in 32..4096, rows * axis <= kShortTile floats) as ONE contiguous
 // span: it is loaded with coalesced float4s whatever the row length, parked in LDS at an odd
 // row stride (conflict-free), and then `256 / rows` lanes fold each row from LDS, in index
 // order within a lane.
@@ -474,6 +490,22 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     }
 }
 
+// ---------------------------------------------------------------- an axis of length 1
+
+// Every output folds exactly one input: an elementwise pass (SUM and MEAN still give 0 + x, which
+// turns -0 into +0 as the serial sum from 0f does; the arg reducers give 0).
+template <class R>
+__global__ __launch_bounds__(kBlock) void reduce_unit_axis_kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t n) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t n4 = n >> 2;
+    auto one = [](float x) { typename R::Acc a = R::init(); R::step(a, x, 0u); return R::finish(a, 1u); };
+    if (i < n4) {
+        const float4 v = ld4_stream(in + 4 * static_cast<size_t>(i));
+        *reinterpret_cast<float4*>(out + 4 * static_cast<size_t>(i)) = make_float4(one(v.x), one(v.y), one(v.z), one(v.w));
+    }
+    if (i < (n & 3u)) out[(static_cast<size_t>(n4) << 2) + i] = one(in[(static_cast<size_t>(n4) << 2) + i]);
+}
+
 // ---------------------------------------------------------------- second pass
 
 // Combines the `segments` partials of each output, always in the same order.
@@ -557,23 +589,38 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     Geom g{outer, axis, inner, 1, axis};
     const uint64_t n_out = static_cast<uint64_t>(outer) * inner;
 
-    if (inner == 1 && axis >= 8 && axis < 256) {
+    if (axis == 1) {
+        const uint32_t n = static_cast<uint32_t>(n_out);
+        hipError_t e;
+        {
+            LaunchScope scope("reduce_unit_axis_kernel", R::name, n_out * 8);
+            hipLaunchKernelGGL((reduce_unit_axis_kernel<R>), dim3(static_cast<uint32_t>(ceil_div((n >> 2) + 3, kBlock))), dim3(kBlock), 0, stream, in, out, n);
+            e = hipGetLastError();
+        }
+        if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+        return KTH_OK;
+    }
+
+    // Short rows, and rows up to 2048 floats that do not start on 16-byte boundaries (measured 3.7-3.8 TB/s
+    // when lanes peel such rows in place): whole rows staged through LDS as one aligned span.
+    if (inner == 1 && axis >= 2 && (axis < 256 || (axis % 4 != 0 && axis <= 2048))) {
         // rows per tile: the largest power of two with rows * axis <= kShortTile, at most kBlock
         ShortPlan pl{};
-        uint32_t rows = 4 * kBlock;
-        while (rows * axis > kShortTile) rows >>= 1;
+        uint32_t rows = 16 * kBlock;
+        while (rows * axis > kShortTile || rows * (axis | 1u) > kShortTile + kShortTile / 8) rows >>= 1;
         pl.outer = outer; pl.axis = axis; pl.rows = rows; pl.stride = axis | 1u; pl.aligned = 1;
         pl.axis_div = make_div(axis);
         const dim3 grid(static_cast<uint32_t>(ceil_div(outer, rows)));
         hipError_t e;
         {
             LaunchScope scope("reduce_short_rows_kernel", R::name, (static_cast<uint64_t>(outer) * axis + n_out) * 4);
+#define SHORT_LAUNCH(GG) hipLaunchKernelGGL((reduce_short_rows_kernel<R, GG>), grid, dim3(kBlock), 0, stream, in, out, pl)
             switch (rows >= kBlock ? 1 : kBlock / rows) {
-            case 1: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 1>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
-            case 2: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 2>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
-            case 4: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 4>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
-            default: hipLaunchKernelGGL((reduce_short_rows_kernel<R, 8>), grid, dim3(kBlock), 0, stream, in, out, pl); break;
+            case 1: SHORT_LAUNCH(1); break;   case 2: SHORT_LAUNCH(2); break;   case 4: SHORT_LAUNCH(4); break;
+            case 8: SHORT_LAUNCH(8); break;   case 16: SHORT_LAUNCH(16); break; case 32: SHORT_LAUNCH(32); break;
+            default: SHORT_LAUNCH(64); break;
             }
+#undef SHORT_LAUNCH
             e = hipGetLastError();
         }
         if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
