@@ -490,6 +490,56 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     }
 }
 
+// ---------------------------------------------------------------- few rows: axis of 2 ... 7 over wide columns
+
+// With so short an axis a column gives a thread only a handful of loads, so a thread takes four
+// columns (float4-wide with VEC = 4), 256 * VEC apart: 8 loads in flight (two axis positions of
+// its four columns), each a contiguous span across the workgroup. Axis positions in ascending order.
+template <class R, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_few_kernel(const float* __restrict__ in, float* __restrict__ out, Geom g, uint32_t tiles) {
+    using Acc = typename R::Acc;
+    constexpr int kCols = 4;
+    const uint32_t o = blockIdx.x / tiles;
+    const uint32_t col0 = ((blockIdx.x - o * tiles) * kCols * kBlock + threadIdx.x) * VEC;
+    const float* base = in + static_cast<size_t>(o) * g.axis * g.inner;
+    Acc acc[kCols][VEC];
+#pragma unroll
+    for (int u = 0; u < kCols; u++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[u][v] = R::init();
+    for (uint32_t a = 0; a < g.axis; a += 2) {
+        float w[2][kCols][VEC];
+#pragma unroll
+        for (uint32_t j = 0; j < 2; j++)
+#pragma unroll
+            for (int u = 0; u < kCols; u++) {
+                const uint32_t c = col0 + u * kBlock * VEC;
+                if (a + j < g.axis && c < g.inner) {
+                    const float* p = base + static_cast<size_t>(a + j) * g.inner + c;
+                    if (VEC == 4) { const float4 t = ld4_stream(p); w[j][u][0] = t.x; w[j][u][1 % VEC] = t.y; w[j][u][2 % VEC] = t.z; w[j][u][3 % VEC] = t.w; }
+                    else w[j][u][0] = ld1_stream(p);
+                }
+            }
+#pragma unroll
+        for (uint32_t j = 0; j < 2; j++)
+#pragma unroll
+            for (int u = 0; u < kCols; u++)
+                if (a + j < g.axis && col0 + u * kBlock * VEC < g.inner)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) R::step(acc[u][v], w[j][u][v], a + j);
+    }
+#pragma unroll
+    for (int u = 0; u < kCols; u++) {
+        const uint32_t c = col0 + u * kBlock * VEC;
+        if (c < g.inner) {
+            float* q = out + static_cast<size_t>(o) * g.inner + c;
+            if (VEC == 4) *reinterpret_cast<float4*>(q) = make_float4(R::finish(acc[u][0], g.axis), R::finish(acc[u][1 % VEC], g.axis),
+                                                                      R::finish(acc[u][2 % VEC], g.axis), R::finish(acc[u][3 % VEC], g.axis));
+            else *q = R::finish(acc[u][0], g.axis);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- an axis of length 1
 
 // Every output folds exactly one input: an elementwise pass (SUM and MEAN still give 0 + x, which
@@ -661,6 +711,23 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     // 3.3-6.1) and for float4 columns below 512; from there on the column kernel's 1 KiB spans win.
     const bool stream_fits = slab >= kStreamMinSlab && (inner < 256 || (inner < 512 && inner % 4 == 0)) &&
                              outer <= 0x7fffffffu / 64;
+    if ((axis <= 7 || (inner % 4 != 0 && axis <= 16)) && inner >= 1024 && !stream_fits && n_out >= 65536) {
+        // (slabs of such an axis that fit a tile were taken above)
+        const int vec = inner % 4 == 0 ? 4 : 1;
+        const uint32_t tiles = ceil_div(inner, 4u * kBlock * vec);
+        const uint64_t few_blocks = static_cast<uint64_t>(tiles) * outer;
+        if (few_blocks <= 0x7fffffffull) {
+            hipError_t e;
+            {
+                LaunchScope scope("reduce_few_kernel", R::name, (static_cast<uint64_t>(outer) * slab + n_out) * 4);
+                if (vec == 4) hipLaunchKernelGGL((reduce_few_kernel<R, 4>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
+                else          hipLaunchKernelGGL((reduce_few_kernel<R, 1>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
+                e = hipGetLastError();
+            }
+            if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+            return KTH_OK;
+        }
+    }
     enum { ROWS, COLS, STRIDED, STREAM } kind;
     int G = 1, VEC = 1, WY = 4, TW = 1;
     uint32_t stream_lanes = 0;

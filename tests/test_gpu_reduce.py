@@ -28,6 +28,8 @@ GEOMETRIES = [
     ([3, 7, 1001], 2), ([2, 300001], 1),
     # an axis of length 1 (elementwise pass) and unaligned rows of 256 ... 2048 floats through the row tiles
     ([1000, 1, 77], 1), ([5, 1], 1), ([1, 4099], 0), ([900, 261], 1), ([70, 555], 1), ([33, 2047], 1), ([9, 2049], 1),
+    # an axis of 2 ... 7 over wide columns: four columns per thread, float4 and scalar, ragged last tile
+    ([3, 2, 70001], 1), ([2, 3, 300000], 1), ([5, 7, 20000], 1), ([1, 5, 100003], 1), ([7, 66000], 0), ([2, 4, 40000, 2], 1),
     # short slabs, too few of them for the tiled kernel
     ([5000, 8, 8], 1), ([1000, 2, 2], 1), ([999, 3, 40], 1), ([257, 16, 16], 1), ([100, 4, 63], 1), ([70, 2, 3, 5], 2),    # slabs up to a whole tile for short axes: unaligned tiles, several lanes per output
     ([600, 8, 128], 1), ([300, 16, 64], 1), ([257, 3, 1024], 1), ([1100, 2, 300], 1), ([400, 4, 201], 1),
@@ -79,7 +81,7 @@ def test_axis_reductions(shape, axis, gc):
 @pytest.mark.parametrize("shape,axis", [([64, 40], 1), ([9, 1000], 1), ([3, 5000], 1), ([333, 1000], 0), ([4, 50, 64], 1),
                                         ([6, 3000, 5], 1), ([2, 70000], 1), ([70000, 64], 0), ([600, 100], 1), ([300, 12, 9], 1),
                                         ([2, 50000, 12], 1), ([700, 300, 7], 1), ([300, 16, 64], 1),
-                                        ([8000, 100, 3], 1), ([1500, 24, 80], 1), ([300, 1250], 1), ([5000, 3], 1), ([5, 100003], 1), ([600, 1, 33], 1), ([1, 5000], 0)],
+                                        ([8000, 100, 3], 1), ([1500, 24, 80], 1), ([300, 1250], 1), ([5000, 3], 1), ([5, 100003], 1), ([600, 1, 33], 1), ([1, 5000], 0), ([2, 3, 70001], 1), ([5, 80000], 0)],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
 def test_special_values_in_reductions(shape, axis, gc):
     """NaN propagation in max/min, NaN skipping in arg ops, signed zeros, lanes of -inf / +inf, ties."""
