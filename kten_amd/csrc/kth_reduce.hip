@@ -8,7 +8,9 @@
 //           take different rows and combine through LDS;
 //   stream  (1 < inner < 256, or < 512 in float4 columns; slab of 2048 floats or more): a workgroup per slab, threads stay on
 //           their column while the workgroup walks the slab as one contiguous span;
+//   few     (axis of 2 ... 7 over wide columns): four columns per thread;
 //   strided (other small inner): one thread per output element, serial walk down the axis.
+// An axis of length 1 is an elementwise pass.
 // When the output alone gives too few workgroups to fill 256 CUs, the axis is cut into
 // S segments; each (output, segment) writes a partial and a second kernel combines the
 // S partials in a fixed order. No atomics anywhere: the same input always gives the
