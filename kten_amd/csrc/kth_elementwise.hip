@@ -335,6 +335,20 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* _
     }
 }
 
+// Four values of an operand at offsets off, off + stride, ... (stride in elements).
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ void gather4(const float* __restrict__ p, uint32_t off, uint32_t stride, float (&v)[4]) {
+    if (stride == 0) {
+        const float x = p[off];
+        v[0] = x; v[1] = x; v[2] = x; v[3] = x;
+    } else if (stride == 1) {
+        const v4f_unaligned x = *reinterpret_cast<const v4f_unaligned*>(p + off);
+        v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+    } else {
+        v[0] = p[off]; v[1] = p[off + stride]; v[2] = p[off + 2 * stride]; v[3] = p[off + 3 * stride];
+    }
+}
+
 // Any shapes, four consecutive outputs per (thread, k): the output and every operand that
 // has the output's element count (AL / BL: it is then laid out exactly like the output) move
 // as float4; a broadcast operand is gathered element by element through the plan (dim 0 in
@@ -351,12 +365,25 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float*
             float va[4], vb[4];
             if (AL) { const float4 v = ld4(a, e0 >> 2); va[0] = v.x; va[1] = v.y; va[2] = v.z; va[3] = v.w; }
             if (BL) { const float4 v = ld4(b, e0 >> 2); vb[0] = v.x; vb[1] = v.y; vb[2] = v.z; vb[3] = v.w; }
+            // The four outputs are neighbours along dim 0 unless they cross its end. Then a broadcast
+            // operand that does not vary along dim 0 needs one load for all four, and one that is
+            // contiguous there one 16-byte load from a 4-byte aligned address: four single loads at
+            // lane stride 16 would each sweep the same eight cache lines.
+            uint32_t ao0, bo0;
+            decompose(pl, e0, ao0, bo0);
+            uint32_t r0 = e0;
+            if (pl.ndim > 1) r0 = e0 - ((__umulhi(e0, pl.div[0].mul) + e0) >> pl.div[0].shift) * pl.size[0];
+            if (pl.ndim == 1 || r0 + 3 < pl.size[0]) {
+                if (!AL) gather4(a, ao0, pl.astride[0], va);
+                if (!BL) gather4(b, bo0, pl.bstride[0], vb);
+            } else {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint32_t ao, bo;
-                decompose(pl, e0 + j, ao, bo);
-                if (!AL) va[j] = a[ao];
-                if (!BL) vb[j] = b[bo];
+                for (int j = 0; j < 4; j++) {
+                    uint32_t ao, bo;
+                    decompose(pl, e0 + j, ao, bo);
+                    if (!AL) va[j] = a[ao];
+                    if (!BL) vb[j] = b[bo];
+                }
             }
             float4 r;
             r.x = Op::apply(va[0], vb[0], eps); r.y = Op::apply(va[1], vb[1], eps);

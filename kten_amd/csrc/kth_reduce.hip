@@ -39,6 +39,14 @@ __device__ __forceinline__ float4 ld4_stream(const float* p) {
     return make_float4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ float ld1_stream(const float* p) { return __builtin_nontemporal_load(p); }
+// Four consecutive floats from an address that is only 4-byte aligned: the hardware takes a
+// 16-byte load from any dword address, and one such load per lane sweeps the cache lines a wave
+// touches once where four single loads at lane stride 16 would sweep them four times.
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ float4 ld4_stream_unaligned(const float* p) {
+    v4f_unaligned v = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
 
 // ---------------------------------------------------------------- reducers
 
@@ -120,7 +128,7 @@ __device__ __forceinline__ void emit(const Geom& g, uint32_t o, uint32_t s, uint
 
 // G lanes per row (G in {1, 2, 4, 16, 64}, or 256 = the whole workgroup).
 // VEC = 4 requires axis % 4 == 0 and seg_len % 4 == 0 so every row segment is 16-byte aligned;
-// VEC = 1 takes any row and peels it to 16-byte boundaries.
+// VEC = 1 takes any row with 16-byte loads from dword addresses.
 template <class R, int G, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                             typename R::Acc* __restrict__ partial, Geom g) {
@@ -139,44 +147,32 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
         // thread keeps kBatch requests in flight.
         constexpr uint32_t kBatch = 8;
         if (VEC == 4) {
-            uint32_t j = begin + lane * 4;
-            for (; j + (kBatch - 1) * G * 4 < end; j += kBatch * G * 4) {
+            // every pass issues its (up to) kBatch loads before consuming any; the last pass of a lane
+            // is predicated instead of falling back to one load at a time
+            for (uint32_t j = begin + lane * 4; j < end; j += kBatch * G * 4) {
                 float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + j + k * G * 4);
+                for (uint32_t k = 0; k < kBatch; k++) if (j + k * G * 4 < end) v[k] = ld4_stream(base + j + k * G * 4);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
                     const uint32_t jj = j + k * G * 4;
-                    R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3);
+                    if (jj < end) { R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3); }
                 }
-            }
-            for (; j < end; j += G * 4) {
-                float4 v = ld4_stream(base + j);
-                R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
             }
         } else {
-            // Rows that do not start on 16-byte boundaries: up to three single floats reach the next
-            // boundary, float4s cover the middle, up to three single floats finish the segment. A
-            // lane meets its elements in ascending index order, as the arg reducers require.
-            const uint32_t skew = static_cast<uint32_t>((static_cast<size_t>(row) * g.axis + begin) & 3u);
-            const uint32_t head = min((4u - skew) & 3u, end - begin);
-            for (uint32_t e = begin + lane; e < begin + head; e += G) R::step(acc, ld1_stream(base + e), e);
-            const uint32_t body = begin + head;
-            const uint32_t body_end = body + ((end - body) & ~3u);
-            uint32_t j = body + lane * 4;
-            for (; j + (kBatch - 1) * G * 4 < body_end; j += kBatch * G * 4) {
+            // Rows that do not start on 16-byte boundaries: 16-byte loads from dword addresses, then up
+            // to three single floats. A lane meets its elements in ascending index order, as the arg
+            // reducers require.
+            const uint32_t body_end = begin + ((end - begin) & ~3u);
+            for (uint32_t j = begin + lane * 4; j < body_end; j += kBatch * G * 4) {
                 float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + j + k * G * 4);
+                for (uint32_t k = 0; k < kBatch; k++) if (j + k * G * 4 < body_end) v[k] = ld4_stream_unaligned(base + j + k * G * 4);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
                     const uint32_t jj = j + k * G * 4;
-                    R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3);
+                    if (jj < body_end) { R::step(acc, v[k].x, jj); R::step(acc, v[k].y, jj + 1); R::step(acc, v[k].z, jj + 2); R::step(acc, v[k].w, jj + 3); }
                 }
-            }
-            for (; j < body_end; j += G * 4) {
-                float4 v = ld4_stream(base + j);
-                R::step(acc, v.x, j); R::step(acc, v.y, j + 1); R::step(acc, v.z, j + 2); R::step(acc, v.w, j + 3);
             }
             for (uint32_t e = body_end + lane; e < end; e += G) R::step(acc, ld1_stream(base + e), e);
         }
@@ -217,30 +213,14 @@ struct ShortPlan {
     FastDiv  axis_div, inner_div;
 };
 
-// Loads `floats` contiguous floats from `base` (16-byte aligned) and parks element e at
+// Loads `floats` contiguous floats from `base` (16-byte aligned if pl.aligned) and parks element e at
 // tile[(e / axis) * stride + e % axis].
 __device__ __forceinline__ void stage_short_tile(const float* __restrict__ base, uint32_t floats, const ShortPlan& pl, float* tile) {
-    if (!pl.aligned) {                       // tiles that start off a 16-byte boundary: coalesced scalar loads
-        for (uint32_t e0 = 0; e0 < floats; e0 += kBlock * 8) {
-            float w[8];
-#pragma unroll
-            for (uint32_t k = 0; k < 8; k++) { const uint32_t e = e0 + k * kBlock + threadIdx.x; if (e < floats) w[k] = ld1_stream(base + e); }
-#pragma unroll
-            for (uint32_t k = 0; k < 8; k++) {
-                const uint32_t e = e0 + k * kBlock + threadIdx.x;
-                if (e < floats) {
-                    const uint32_t r = (__umulhi(e, pl.axis_div.mul) + e) >> pl.axis_div.shift;
-                    tile[r * pl.stride + (e - r * pl.axis)] = w[k];
-                }
-            }
-        }
-        return;
-    }
     float4 v[kShortLoads];
 #pragma unroll
     for (uint32_t k = 0; k < kShortLoads; k++) {
         const uint32_t e = (k * kBlock + threadIdx.x) * 4;
-        if (e + 4 <= floats) v[k] = ld4_stream(base + e);
+        if (e + 4 <= floats) v[k] = pl.aligned ? ld4_stream(base + e) : ld4_stream_unaligned(base + e);
         else {
             v[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (e < floats) v[k].x = base[e];
@@ -352,34 +332,26 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
         const uint32_t begin = s * g.seg_len;
         const uint32_t end = min(begin + g.seg_len, g.axis);
         constexpr uint32_t kBatch = 8;          // loads in flight per thread
-        uint32_t r = begin + lane;
-        for (; r + (kBatch - 1) * WR < end; r += kBatch * WR) {
+        // every pass issues its (up to) kBatch loads before consuming any; the last pass is predicated
+        for (uint32_t r = begin + lane; r < end; r += kBatch * WR) {
             if (VEC == 4) {
                 float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * WR < end) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
                     const uint32_t rr = r + k * WR;
-                    R::step(acc[0], v[k].x, rr); R::step(acc[1 % VEC], v[k].y, rr);
-                    R::step(acc[2 % VEC], v[k].z, rr); R::step(acc[3 % VEC], v[k].w, rr);
+                    if (rr < end) {
+                        R::step(acc[0], v[k].x, rr); R::step(acc[1 % VEC], v[k].y, rr);
+                        R::step(acc[2 % VEC], v[k].z, rr); R::step(acc[3 % VEC], v[k].w, rr);
+                    }
                 }
             } else {
                 float v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) v[k] = ld1_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * WR < end) v[k] = ld1_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], v[k], r + k * WR);
-            }
-        }
-        for (; r < end; r += WR) {
-            const float* p = base + static_cast<size_t>(r) * g.inner;
-            if (VEC == 4) {
-                float4 v = ld4_stream(p);
-                R::step(acc[0], v.x, r); R::step(acc[1 % VEC], v.y, r);
-                R::step(acc[2 % VEC], v.z, r); R::step(acc[3 % VEC], v.w, r);
-            } else {
-                R::step(acc[0], ld1_stream(p), r);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * WR < end) R::step(acc[0], v[k], r + k * WR);
             }
         }
     }
@@ -453,32 +425,27 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     if (lane < lanes) {
         const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + c * VEC;
         constexpr uint32_t kBatch = VEC == 4 ? 4 : 8;
-        uint32_t r = begin + lane;
-        if (VEC == 4) {
-            for (; r + (kBatch - 1) * lanes < end; r += kBatch * lanes) {
+        // every pass issues its (up to) kBatch loads before consuming any; the last pass is predicated
+        for (uint32_t r = begin + lane; r < end; r += kBatch * lanes) {
+            if (VEC == 4) {
                 float4 w[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) w[k] = ld4_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * lanes < end) w[k] = ld4_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
-                    R::step(acc[0], w[k].x, r + k * lanes); R::step(acc[VEC > 1 ? 1 : 0], w[k].y, r + k * lanes);
-                    R::step(acc[VEC > 2 ? 2 : 0], w[k].z, r + k * lanes); R::step(acc[VEC > 3 ? 3 : 0], w[k].w, r + k * lanes);
+                    const uint32_t rr = r + k * lanes;
+                    if (rr < end) {
+                        R::step(acc[0], w[k].x, rr); R::step(acc[VEC > 1 ? 1 : 0], w[k].y, rr);
+                        R::step(acc[VEC > 2 ? 2 : 0], w[k].z, rr); R::step(acc[VEC > 3 ? 3 : 0], w[k].w, rr);
+                    }
                 }
-            }
-            for (; r < end; r += lanes) {
-                const float4 w = ld4_stream(base + static_cast<size_t>(r) * g.inner);
-                R::step(acc[0], w.x, r); R::step(acc[VEC > 1 ? 1 : 0], w.y, r);
-                R::step(acc[VEC > 2 ? 2 : 0], w.z, r); R::step(acc[VEC > 3 ? 3 : 0], w.w, r);
-            }
-        } else {
-            for (; r + (kBatch - 1) * lanes < end; r += kBatch * lanes) {
+            } else {
                 float w[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) w[k] = ld1_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * lanes < end) w[k] = ld1_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) R::step(acc[0], w[k], r + k * lanes);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * lanes < end) R::step(acc[0], w[k], r + k * lanes);
             }
-            for (; r < end; r += lanes) R::step(acc[0], ld1_stream(base + static_cast<size_t>(r) * g.inner), r);
         }
     }
     // fold[lane][column]: thread t owns columns c * VEC .. c * VEC + VEC - 1 of lane t / cols
@@ -653,9 +620,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         return KTH_OK;
     }
 
-    // Short rows, and rows up to 2048 floats that do not start on 16-byte boundaries (measured 3.7-3.8 TB/s
-    // when lanes peel such rows in place): whole rows staged through LDS as one aligned span.
-    if (inner == 1 && axis >= 2 && (axis < 256 || (axis % 4 != 0 && axis <= 2048))) {
+    if (inner == 1 && axis >= 2 && axis < 256) {
         // rows per tile: the largest power of two with rows * axis <= kShortTile, at most kBlock
         ShortPlan pl{};
         uint32_t rows = 16 * kBlock;
@@ -738,7 +703,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     if (inner == 1) {
         kind = ROWS;
         VEC = (axis % 4 == 0) ? 4 : 1;
-        const uint32_t per_lane = axis / VEC;          // loads per row
+        const uint32_t per_lane = axis / 4;            // 16-byte loads per row
         G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : per_lane >= 2 ? 2 : 1;
         const uint64_t base_blocks = ceil_div(outer, kBlock / G);
         plan_segments(&g, base_blocks, target / 2, G * VEC, G * VEC * 16);
