@@ -88,31 +88,42 @@ __global__ __launch_bounds__(kBlock) void move_kernel(const float* __restrict__ 
 }
 
 // The same moves when the strided side cannot take float4s (odd run lengths or offsets): the
-// dense side still moves as float4s, 16-byte aligned from the start of its store, and the four
-// floats of each meet the strided side one by one. Lanes next to each other stay next to each
-// other on both sides, so the scalar accesses coalesce. `n` counts floats; MODE 0 and 1 only.
+// dense side still moves as float4s, 16-byte aligned from the start of its store. Where its four
+// floats are neighbours on the strided side as well they move there as one 16-byte access at a
+// dword address, otherwise one by one. `n` counts floats; MODE 0 and 1 only.
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restrict__ src, float* __restrict__ dst,
                                                            uint32_t n, MovePlan pl) {
     const uint32_t base = blockIdx.x * (kBlock * kMoveUnroll) + threadIdx.x;
     uint32_t at[kMoveUnroll][4];
+    bool run4[kMoveUnroll];                  // the four floats lie next to each other on the strided side too
     v4f v[kMoveUnroll];
 #pragma unroll
     for (int k = 0; k < kMoveUnroll; k++) {
         const uint32_t i = (base + k * kBlock) * 4u;
+        run4[k] = false;
         if (i >= n) continue;
         // position inside the innermost run decides whether the four floats share it
         const uint32_t q0 = (__umulhi(i, pl.div[0].mul) + i) >> pl.div[0].shift;
         const uint32_t r0 = i - q0 * pl.size[0];
         at[k][0] = strided_offset(pl, i);
+        const bool together = pl.ndim == 1 || r0 + 3 < pl.size[0];
+        run4[k] = together && pl.stride[0] == 1 && i + 3 < n;
 #pragma unroll
         for (int j = 1; j < 4; j++)
             at[k][j] = (pl.ndim == 1 || r0 + j < pl.size[0]) ? at[k][0] + j * pl.stride[0] : (i + j < n ? strided_offset(pl, i + j) : at[k][0]);
         if (MODE == 0) {
-            v[k].x = src[at[k][0]];
-            v[k].y = i + 1 < n ? src[at[k][1]] : 0.0f;
-            v[k].z = i + 2 < n ? src[at[k][2]] : 0.0f;
-            v[k].w = i + 3 < n ? src[at[k][3]] : 0.0f;
+            if (run4[k]) {                   // one 16-byte load from a dword address
+                const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(src + at[k][0]);
+                v[k] = v4f{t.x, t.y, t.z, t.w};
+            } else {
+                v[k].x = src[at[k][0]];
+                v[k].y = i + 1 < n ? src[at[k][1]] : 0.0f;
+                v[k].z = i + 2 < n ? src[at[k][2]] : 0.0f;
+                v[k].w = i + 3 < n ? src[at[k][3]] : 0.0f;
+            }
         } else if (i + 3 < n) {
             v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + i));
         } else {
@@ -126,6 +137,8 @@ __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restr
         if (MODE == 0) {
             if (i + 3 < n) *reinterpret_cast<v4f*>(dst + i) = v[k];
             else { dst[i] = v[k].x; if (i + 1 < n) dst[i + 1] = v[k].y; if (i + 2 < n) dst[i + 2] = v[k].z; }
+        } else if (run4[k]) {
+            *reinterpret_cast<v4f_unaligned*>(dst + at[k][0]) = v4f_unaligned{v[k].x, v[k].y, v[k].z, v[k].w};
         } else {
             dst[at[k][0]] = v[k].x;
             if (i + 1 < n) dst[at[k][1]] = v[k].y;
