@@ -57,13 +57,17 @@ __device__ __forceinline__ void block_fold2(double& a, double& b, double* lds) {
 
 // ---------------------------------------------------------------- stats, long runs (inner >= 64)
 
-// Work of one channel: outer runs of `inner` contiguous floats, cut into chunks of
-// kBlock * W floats (W = 4 with float4 loads); a workgroup takes the chunks
+// Work of one channel: outer runs of `inner` contiguous floats, numbered through as units of W
+// floats (W = 4 with float4 loads) and cut into chunks of kBlock units, so every lane has a unit
+// whatever the run length; a workgroup takes the chunks
 // [seg * chunks_per_seg, (seg + 1) * chunks_per_seg) of channel blockIdx.x / segments.
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
 struct RunPlan {
     Geometry g;
-    uint32_t segments, chunks_per_seg, total_chunks, chunks_per_run;
-    FastDiv  run_div, seg_div;
+    uint32_t segments, chunks_per_seg, total_chunks;
+    uint32_t units_per_run, total_units;
+    FastDiv  run_div, seg_div;               // run_div divides by units_per_run
 };
 
 // BACKWARD false: (sum of d, sum of d*d), d = x - k. BACKWARD true: (sum of g, sum of (x - mean) g).
@@ -71,7 +75,7 @@ template <bool BACKWARD, bool VEC>
 __global__ __launch_bounds__(kBlock) void bn_stats_runs_kernel(const float* __restrict__ x, const float* __restrict__ go,
                                                               const float* __restrict__ mean, double* __restrict__ partial, RunPlan pl) {
     __shared__ double lds[2 * kBlock / 64];
-    constexpr uint32_t W = VEC ? 4 : 1;
+    constexpr uint32_t W = 4;                // !VEC: runs of any length, 16-byte loads from dword addresses, ragged last unit
     const uint32_t b = blockIdx.x;
     const uint32_t c = (__umulhi(b, pl.seg_div.mul) + b) >> pl.seg_div.shift;
     const uint32_t seg = b - c * pl.segments;
@@ -83,25 +87,33 @@ __global__ __launch_bounds__(kBlock) void bn_stats_runs_kernel(const float* __re
     for (uint32_t q0 = first; q0 < last; q0 += kBatch) {
         v4f vx[kBatch], vg[kBatch];
         bool ok[kBatch];
-        uint32_t valid[kBatch];
+        uint32_t valid[kBatch], skip[kBatch];
 #pragma unroll
         for (int k = 0; k < kBatch; k++) {
             const uint32_t q = q0 + k;
             ok[k] = q < last;
-            valid[k] = 0;
+            valid[k] = 0; skip[k] = 0;
             if (ok[k]) {
-                const uint32_t o = (__umulhi(q, pl.run_div.mul) + q) >> pl.run_div.shift;
-                const uint32_t off = (q - o * pl.chunks_per_run) * (kBlock * W) + threadIdx.x * W;
-                if (off < pl.g.inner) {
+                const uint32_t u = q * kBlock + threadIdx.x;
+                if (u < pl.total_units) {
+                    const uint32_t o = (__umulhi(u, pl.run_div.mul) + u) >> pl.run_div.shift;
+                    const uint32_t off = (u - o * pl.units_per_run) * W;
                     const uint64_t at = (static_cast<uint64_t>(o) * pl.g.channels + c) * pl.g.inner + off;
                     if (VEC) {
                         valid[k] = 4;
                         vx[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x + at));
                         if (BACKWARD) vg[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(go + at));
                     } else {
-                        valid[k] = 1;
-                        vx[k].x = x[at];
-                        if (BACKWARD) vg[k].x = go[at];
+                        // the last unit of a run is read as the run's last four floats; the ones a
+                        // neighbouring unit already counted are skipped
+                        const uint32_t back = off + 4 > pl.g.inner ? off + 4 - pl.g.inner : 0u;
+                        valid[k] = 4; skip[k] = back;
+                        const v4f_unaligned tx = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(x + at - back));
+                        vx[k] = v4f{tx.x, tx.y, tx.z, tx.w};
+                        if (BACKWARD) {
+                            const v4f_unaligned tg = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(go + at - back));
+                            vg[k] = v4f{tg.x, tg.y, tg.z, tg.w};
+                        }
                     }
                 }
             }
@@ -111,6 +123,7 @@ __global__ __launch_bounds__(kBlock) void bn_stats_runs_kernel(const float* __re
             if (valid[k] == 0) continue;
 #pragma unroll
             for (int e = 0; e < static_cast<int>(W); e++) {
+                if (static_cast<uint32_t>(e) < skip[k]) continue;
                 const double d = static_cast<double>(vx[k][e]) - shift;
                 if (BACKWARD) { const double g = static_cast<double>(vg[k][e]); s1 += g; s2 += d * g; }
                 else { s1 += d; s2 += d * d; }
@@ -242,7 +255,7 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
                                                                     float momentum, float epsilon, float* running_mean, float* running_var,
                                                                     const float* __restrict__ gamma, const float* __restrict__ beta,
                                                                     float* __restrict__ current_mean, float* __restrict__ current_std,
-                                                                    ForwardParams* __restrict__ params) {
+                                                                    ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch) {
     const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
     if (c >= g.channels) return;
     float mean, stdev = 0.0f;
@@ -277,6 +290,8 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
     p.gamma = gamma != nullptr ? gamma[c] : 1.0f;                               // :84-85
     p.beta = beta != nullptr ? beta[c] : 0.0f;
     params[c] = p;
+    // the same by parameter, for layouts where neighbouring elements belong to neighbouring channels
+    soa[c] = p.mean; soa[pitch + c] = p.stdev; soa[2 * pitch + c] = p.gamma; soa[3 * pitch + c] = p.beta;
 }
 
 __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const double* __restrict__ partial, Geometry g, uint32_t segments,
@@ -284,7 +299,8 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
                                                                      const float* __restrict__ running_mean, const float* __restrict__ running_var,
                                                                      const float* __restrict__ current_mean, const float* __restrict__ current_std,
                                                                      const float* __restrict__ gamma, float* __restrict__ grad_gamma,
-                                                                     float* __restrict__ grad_beta, BackwardParams* __restrict__ params) {
+                                                                     float* __restrict__ grad_beta, BackwardParams* __restrict__ params,
+                                                                     float* __restrict__ soa, uint32_t pitch) {
     const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
     if (c >= g.channels) return;
     double s1 = 0.0, s2 = 0.0;
@@ -309,6 +325,7 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
     p.grad_mean = sum / count;                                                  // :152
     p.pad0 = p.pad1 = p.pad2 = 0.0f;
     params[c] = p;
+    soa[c] = p.mean; soa[pitch + c] = p.stdev; soa[2 * pitch + c] = p.gamma; soa[3 * pitch + c] = p.dot_std_sq; soa[4 * pitch + c] = p.grad_mean;
     if (grad_gamma != nullptr) grad_gamma[c] = dot * stdev;                     // :171-173
     if (grad_beta != nullptr) grad_beta[c] = sum;                               // :175-177
 }
@@ -318,6 +335,9 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
 struct ApplyPlan {
     uint32_t units;                 // float4s (VEC) or floats
     uint32_t channels;
+    const float* soa;               // parameters by kind, [kind][pitch]; used when by_channel4
+    uint32_t pitch;
+    uint32_t by_channel4;           // inner == 1 and channels % 4 == 0: a float4 holds four consecutive channels
     FastDiv  inner_div, channel_div;   // inner counted in the kernel's units
 };
 
@@ -362,6 +382,27 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float* __restric
             const uint32_t i = base + k * kBlock;
             if (i < pl.units) {
                 v4f r;
+                if (!UNIFORM && pl.by_channel4) {
+                    // four consecutive channels: one float4 per parameter kind instead of four structs,
+                    // whose lane stride would sweep 32 or 64 cache lines per load
+                    const uint32_t c0 = channel_of(pl, i * 4);
+                    const v4f mean = *reinterpret_cast<const v4f*>(pl.soa + c0);
+                    const v4f stdev = *reinterpret_cast<const v4f*>(pl.soa + pl.pitch + c0);
+                    const v4f gamma = *reinterpret_cast<const v4f*>(pl.soa + 2 * pl.pitch + c0);
+                    const v4f p3 = *reinterpret_cast<const v4f*>(pl.soa + 3 * pl.pitch + c0);      // beta | dot_std_sq
+                    v4f p4 = p3;
+                    if (MODE == 1) p4 = *reinterpret_cast<const v4f*>(pl.soa + 4 * pl.pitch + c0);  // grad_mean
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (MODE == 0) { ForwardParams q; q.mean = mean[e]; q.stdev = stdev[e]; q.gamma = gamma[e]; q.beta = p3[e]; r[e] = bn_forward(vx[k][e], q); }
+                        else {
+                            BackwardParams q; q.mean = mean[e]; q.stdev = stdev[e]; q.gamma = gamma[e]; q.dot_std_sq = p3[e]; q.grad_mean = p4[e];
+                            r[e] = MODE == 1 ? bn_backward_training(vx[k][e], vg[k][e], q) : bn_backward_inference(vg[k][e], q);
+                        }
+                    }
+                    reinterpret_cast<v4f*>(out)[i] = r;
+                    continue;
+                }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const uint32_t c = UNIFORM ? channel_of(pl, i) : channel_of(pl, i * 4 + e);
@@ -434,18 +475,18 @@ StatsLaunch plan_stats(const Geometry& g) {
     if (g.inner >= 64) {
         st.by_cols = false;
         st.vec = g.inner % 4 == 0;
-        const uint32_t chunk = kBlock * (st.vec ? 4 : 1);
         RunPlan& p = st.run;
         p.g = g;
-        p.chunks_per_run = (g.inner + chunk - 1) / chunk;
-        p.total_chunks = g.outer * p.chunks_per_run;
+        p.units_per_run = (g.inner + 3) / 4;
+        p.total_units = g.outer * p.units_per_run;
+        p.total_chunks = (p.total_units + kBlock - 1) / kBlock;
         uint32_t segments = (target + g.channels - 1) / g.channels;
         const uint32_t max_segments = (p.total_chunks + kBatch - 1) / kBatch;      // at least one batch of chunks each
         if (segments > max_segments) segments = max_segments;
         if (segments < 1) segments = 1;
         p.chunks_per_seg = (p.total_chunks + segments - 1) / segments;
         p.segments = (p.total_chunks + p.chunks_per_seg - 1) / p.chunks_per_seg;
-        p.run_div = make_div(p.chunks_per_run);
+        p.run_div = make_div(p.units_per_run);
         p.seg_div = make_div(p.segments);
         st.segments = p.segments;
         st.partial_doubles = static_cast<uint64_t>(g.channels) * p.segments * 2;
@@ -489,9 +530,12 @@ void launch_stats(const StatsLaunch& st, const float* x, const float* go, const 
 }
 
 template <int MODE>
-void launch_apply(const Geometry& g, uint64_t n, const float* x, const float* go, float* out, const ForwardParams* fp, const BackwardParams* bp) {
+void launch_apply(const Geometry& g, uint64_t n, const float* x, const float* go, float* out, const ForwardParams* fp, const BackwardParams* bp,
+                  const float* soa, uint32_t pitch) {
     ApplyPlan pl{};
     const bool vec = n % 4 == 0, uniform = g.inner % 4 == 0;
+    pl.soa = soa; pl.pitch = pitch;
+    pl.by_channel4 = (g.inner == 1 && g.channels % 4 == 0) ? 1u : 0u;
     pl.units = static_cast<uint32_t>(vec ? n / 4 : n);
     pl.channels = g.channels;
     pl.inner_div = make_div(uniform ? g.inner / 4 : g.inner);
@@ -537,20 +581,23 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     if (!cm || !cs) return fail(KTH_E_ARGUMENT, "kth_batch_norm_forward: current_mean and current_std are outputs and must be given");
 
     const StatsLaunch st = training ? plan_stats(g) : StatsLaunch{};
-    const uint64_t params_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(ForwardParams));
+    const uint32_t pitch = (g.channels + 3u) & ~3u;
+    const uint64_t aos_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(ForwardParams));
+    const uint64_t params_bytes = aos_bytes + align256(4ull * pitch * sizeof(float));
     const uint64_t ws_bytes = params_bytes + st.partial_doubles * sizeof(double);
     uint64_t cap;
     char* ws = reinterpret_cast<char*>(workspace_acquire(ws_bytes, &cap));
     if (!ws) return fail(KTH_E_MEMORY, "kth_batch_norm_forward: no workspace of %llu bytes", static_cast<unsigned long long>(ws_bytes));
     ForwardParams* params = reinterpret_cast<ForwardParams*>(ws);
+    float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
     if (training) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
     {
         LaunchScope scope("bn_finalize_forward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
         hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
-                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params);
+                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params, soa, pitch);
     }
-    launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr);
+    launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr, soa, pitch);
     workspace_release(reinterpret_cast<float*>(ws), cap);
     KTH_LAUNCH_CHECK("batch_norm_forward");
     return KTH_OK;
@@ -587,22 +634,25 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     // inference-mode input gradient does not use them.
     const bool need_sums = training || gg != nullptr || gb != nullptr;
     const StatsLaunch st = need_sums ? plan_stats(g) : StatsLaunch{};
-    const uint64_t params_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(BackwardParams));
+    const uint32_t pitch = (g.channels + 3u) & ~3u;
+    const uint64_t aos_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(BackwardParams));
+    const uint64_t params_bytes = aos_bytes + align256(5ull * pitch * sizeof(float));
     const uint64_t ws_bytes = params_bytes + st.partial_doubles * sizeof(double);
     uint64_t cap;
     char* ws = reinterpret_cast<char*>(workspace_acquire(ws_bytes, &cap));
     if (!ws) return fail(KTH_E_MEMORY, "kth_batch_norm_backward: no workspace of %llu bytes", static_cast<unsigned long long>(ws_bytes));
     BackwardParams* params = reinterpret_cast<BackwardParams*>(ws);
+    float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
     if (need_sums) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
     {
         LaunchScope scope("bn_finalize_backward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
         hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
-                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params);
+                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch);
     }
     if (sgi) {
-        if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params);
-        else launch_apply<2>(g, n, nullptr, sg->ptr, sgi->ptr, nullptr, params);
+        if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
+        else launch_apply<2>(g, n, nullptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
     }
     workspace_release(reinterpret_cast<float*>(ws), cap);
     KTH_LAUNCH_CHECK("batch_norm_backward");

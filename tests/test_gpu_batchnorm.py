@@ -40,7 +40,10 @@ def channel_sums64(a, axis):
 # more channels than workgroup columns, a single row
 LAYOUTS = [([10, 3, 4, 5], 1), ([8, 16, 32, 32], 1), ([4, 6, 67], 1), ([4, 5, 257], 1), ([64, 33, 7], 1), ([512, 40], 1),
            ([300, 129], 1), ([40, 512], 0), ([3, 2000], 0), ([2, 3, 4, 5], 3), ([6, 1, 300], 1), ([1, 8, 4096], 1),
-           ([9, 4, 1024], 1), ([10, 3, 4, 5], 2)]
+           ([9, 4, 1024], 1), ([10, 3, 4, 5], 2),
+           # runs whose length is 1, 2, 3 past a multiple of 4 (the last unit overlaps its neighbour), channels innermost
+           # with a multiple of 4 channels (parameters read four channels at a time)
+           ([20, 12, 13, 13], 1), ([7, 8, 65], 1), ([5, 4, 66], 1), ([3, 5, 71], 1), ([1000, 256], 1), ([33, 4, 7, 12], 3)]
 
 
 @pytest.mark.parametrize("affine,running", [(True, True), (False, False)])
