@@ -55,6 +55,29 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict_
     out[e] = in[ao + static_cast<uint32_t>(sel) * pl.a_axis_stride];
 }
 
+// A contiguous row between global memory and LDS, 16 bytes per lane (the global side may start at
+// any dword address), the last 1 ... 3 floats one by one.
+typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+typedef float v4f_lds __attribute__((ext_vector_type(4)));
+template <int THREADS>
+__device__ __forceinline__ void row_to_lds(const float* __restrict__ row, float* tile, uint32_t len) {
+    const uint32_t body = len & ~3u;
+    for (uint32_t j = threadIdx.x * 4; j < body; j += THREADS * 4) {
+        const v4f_unaligned v = *reinterpret_cast<const v4f_unaligned*>(row + j);
+        *reinterpret_cast<v4f_lds*>(tile + j) = v4f_lds{v.x, v.y, v.z, v.w};
+    }
+    if (threadIdx.x < len - body) tile[body + threadIdx.x] = row[body + threadIdx.x];
+}
+template <int THREADS>
+__device__ __forceinline__ void lds_to_row(const float* tile, float* __restrict__ row, uint32_t len) {
+    const uint32_t body = len & ~3u;
+    for (uint32_t j = threadIdx.x * 4; j < body; j += THREADS * 4) {
+        const v4f_lds v = *reinterpret_cast<const v4f_lds*>(tile + j);
+        *reinterpret_cast<v4f_unaligned*>(row + j) = v4f_unaligned{v.x, v.y, v.z, v.w};
+    }
+    if (threadIdx.x < len - body) row[body + threadIdx.x] = tile[body + threadIdx.x];
+}
+
 // gather along the innermost axis when the index rows are long: one workgroup per position reads
 // the input row into LDS as one contiguous span and serves out[r] = row[index[r]] from there, so
 // both the reads and the writes of global memory are contiguous. The plan is the scatter form:
@@ -63,14 +86,14 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const float* __restrict_
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void gather_rows_lds_kernel(const float* __restrict__ in, const float* __restrict__ index,
                                                                  float* __restrict__ out, IndexPlan pl, int* bad) {
-    extern __shared__ float gather_row[];
+    extern __shared__ __attribute__((aligned(16))) float gather_row[];
     const uint32_t tid = threadIdx.x;
     uint32_t io, ao, bo;
     locate(pl, blockIdx.x, io, ao, bo);
     const float* arow = in + ao;
     const float* irow = index + io;
     float* orow = out + bo;
-    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) gather_row[j] = arow[j];
+    row_to_lds<THREADS>(arow, gather_row, pl.a_axis_len);
     __syncthreads();
     constexpr uint32_t kBatch = 4;
     for (uint32_t r0 = tid; r0 < pl.i_axis_len; r0 += kBatch * THREADS) {
@@ -138,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 template <int MODE, int THREADS>
 __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __restrict__ target, const float* __restrict__ index,
                                                                  const float* __restrict__ src, float value, IndexPlan pl, int* bad) {
-    extern __shared__ float row_lds[];
+    extern __shared__ __attribute__((aligned(16))) float row_lds[];
     float* tile = row_lds;
     uint32_t* tile_bits = reinterpret_cast<uint32_t*>(row_lds);
     uint32_t* tag = reinterpret_cast<uint32_t*>(row_lds) + pl.a_axis_len;     // MODE 1 only
@@ -148,10 +171,8 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
     float* trow = target + ao;
     const float* irow = index + io;
     const float* srow = src + bo;
-    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) {
-        tile[j] = trow[j];
-        if (MODE == 1) tag[j] = 0xffffffffu;
-    }
+    row_to_lds<THREADS>(trow, tile, pl.a_axis_len);
+    if (MODE == 1) for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) tag[j] = 0xffffffffu;
     // the first chunk's entries are fetched while the row arrives
     float next_i = 0.0f, next_v = value;
     if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
@@ -190,7 +211,7 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         }
     }
     __syncthreads();
-    for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) trow[j] = tile[j];
+    lds_to_row<THREADS>(tile, trow, pl.a_axis_len);
 }
 
 // indexSelect / indexAdd (JVMRawTensor.kt:484-516): the index is one list of k rows along the
