@@ -237,6 +237,25 @@ __global__ __launch_bounds__(kBlock) void index_select_kernel(const float* __res
     else out[e] = in[from];
 }
 
+// The same for rows whose length is not a multiple of 4 (but at least 4): a row is covered by
+// ceil(inner / 4) units of four floats at dword addresses, the last one moved back so that it ends
+// with the row (it rewrites up to three floats with the values they already have). pl.inner counts units.
+__global__ __launch_bounds__(kBlock) void index_select_ragged_kernel(const float* __restrict__ in, const float* __restrict__ index,
+                                                                    float* __restrict__ out, uint32_t units, uint32_t row_floats,
+                                                                    RowsPlan pl, int* bad) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= units) return;
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t unit = e - row * pl.inner;
+    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
+    const int sel = static_cast<int>(index[row - o * pl.k]);
+    if (sel < 0 || static_cast<uint32_t>(sel) >= pl.axis_len) { *bad = 1; return; }
+    const uint32_t off = min(unit * 4u, row_floats - 4u);
+    const size_t from = (static_cast<size_t>(o) * pl.axis_len + static_cast<uint32_t>(sel)) * row_floats + off;
+    const size_t to = static_cast<size_t>(row) * row_floats + off;
+    *reinterpret_cast<v4f_unaligned*>(out + to) = *reinterpret_cast<const v4f_unaligned*>(in + from);
+}
+
 // One thread per position (o, column): target[o, index[i], column] += src[o, i, column] * alpha
 // for i ascending, so repeated indices accumulate in index order as on the JVM.
 __global__ __launch_bounds__(kBlock) void index_add_kernel(float* __restrict__ target, const float* __restrict__ index,
@@ -281,23 +300,33 @@ __global__ __launch_bounds__(kBlock) void index_keys_kernel(const float* __restr
     vals[i] = i;
 }
 
-// One thread per unit (float or float4) of [outer, k, inner] in sorted order. The thread at the
-// head of a run of equal keys owns that target row's unit: it adds the run's source rows in
-// order, target = target + src * alpha each time (two roundings, as JVMRawTensor.kt:515);
-// the other threads of the run have nothing to do. No two threads write the same element.
+// flags[i] = 1 where a run of equal, valid keys starts in the sorted list.
+__global__ __launch_bounds__(kBlock) void index_heads_kernel(const uint32_t* __restrict__ keys, uint32_t k, uint32_t axis_len, uint8_t* __restrict__ flags) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= k) return;
+    const uint32_t key = keys[i];
+    flags[i] = (key < axis_len && (i == 0 || keys[i - 1] != key)) ? 1 : 0;
+}
+
+// The runs of equal keys are the touched target rows; their first positions (`heads`, *head_count
+// of them) come from a compaction of the sorted list. One thread per unit (float or float4) of
+// [outer, touched row, inner]: it adds the run's source rows in order, target = target + src * alpha
+// each time (two roundings, as JVMRawTensor.kt:515). The grid covers k rows per outer index; threads
+// past the number of touched rows leave at once. No two threads write the same element.
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                  const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                                                                 const uint32_t* __restrict__ heads, const uint32_t* __restrict__ head_count,
                                                                  float alpha, uint32_t units, RowsPlan pl) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
     const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
     const uint32_t col = e - row * pl.inner;
     const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
-    const uint32_t i = row - o * pl.k;
+    const uint32_t h = row - o * pl.k;                     // the h-th touched target row
+    if (h >= *head_count) return;
+    const uint32_t i = heads[h];
     const uint32_t key = keys[i];
-    if (key >= pl.axis_len) return;
-    if (i > 0 && keys[i - 1] == key) return;
     const size_t t_at = (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
     const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
     if (VEC) {
@@ -331,6 +360,40 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restr
         }
         *t = acc;
     }
+}
+
+// The same for rows whose length is not a multiple of 4 (but more than 4): a row is ceil(inner / 4)
+// units; a full unit moves as 16 bytes at a dword address, the last one as its 1 ... 3 floats.
+// pl.inner counts units, row_floats the floats of a row.
+__global__ __launch_bounds__(kBlock) void index_add_sorted_ragged_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                        const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                                                                        const uint32_t* __restrict__ heads, const uint32_t* __restrict__ head_count,
+                                                                        float alpha, uint32_t units, uint32_t row_floats, RowsPlan pl) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= units) return;
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t off = (e - row * pl.inner) * 4u;
+    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
+    const uint32_t h = row - o * pl.k;                     // the h-th touched target row
+    if (h >= *head_count) return;
+    const uint32_t i = heads[h];
+    const uint32_t key = keys[i];
+    float* t = target + (static_cast<size_t>(o) * pl.axis_len + key) * row_floats + off;
+    const float* s = src + static_cast<size_t>(o) * pl.k * row_floats + off;
+    const uint32_t cnt = min(4u, row_floats - off);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (cnt == 4) { const v4f_unaligned v = *reinterpret_cast<const v4f_unaligned*>(t); acc[0] = v.x; acc[1] = v.y; acc[2] = v.z; acc[3] = v.w; }
+    else for (uint32_t j = 0; j < cnt; j++) acc[j] = t[j];
+    for (uint32_t r = i; r < pl.k && keys[r] == key; r++) {
+        const float* p = s + static_cast<size_t>(vals[r]) * row_floats;
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (cnt == 4) { const v4f_unaligned w = *reinterpret_cast<const v4f_unaligned*>(p); v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w; }
+        else for (uint32_t j = 0; j < cnt; j++) v[j] = p[j];
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = acc[j] + v[j] * alpha;
+    }
+    if (cnt == 4) *reinterpret_cast<v4f_unaligned*>(t) = v4f_unaligned{acc[0], acc[1], acc[2], acc[3]};
+    else for (uint32_t j = 0; j < cnt; j++) t[j] = acc[j];
 }
 
 __global__ void clear_int_kernel(int* p) { *p = 0; }
@@ -665,6 +728,21 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
                 hipLaunchKernelGGL((gather_rows_lds_kernel<256>), grid, dim3(256), lds_bytes, state().stream, si->ptr, sx->ptr, so->ptr, rp, flag);
         });
     }
+    if (inner % 4 != 0 && inner > 4) {
+        RowsPlan rp{};
+        rp.axis_len = static_cast<uint32_t>(shape[axis]); rp.k = static_cast<uint32_t>(k);
+        rp.inner = static_cast<uint32_t>((inner + 3) / 4);
+        rp.inner_div = make_div(rp.inner); rp.k_div = make_div(rp.k);
+        const uint64_t units64 = outer * k * rp.inner;
+        if (units64 <= kMaxElements) {
+            const uint32_t units = static_cast<uint32_t>(units64);
+            return with_index_check("Index select", [&](int* flag) {
+                LaunchScope scope("index_select_kernel", "float4 at dword addresses", 2 * n_out * 4 + k * 4);
+                hipLaunchKernelGGL(index_select_ragged_kernel, dim3((units + kBlock - 1) / kBlock), dim3(kBlock), 0, state().stream,
+                                   si->ptr, sx->ptr, so->ptr, units, static_cast<uint32_t>(inner), rp, flag);
+            });
+        }
+    }
     const bool vec = inner % 4 == 0;
     RowsPlan pl{};
     pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k);
@@ -732,9 +810,15 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     int end_bit = 1;
     while (end_bit < 32 && (1ull << end_bit) <= pl.axis_len) end_bit++;      // keys run up to axis_len inclusive
     const uint64_t k_pad = (k + 63) & ~63ull;                                // keeps the four arrays 256-byte aligned
+    size_t select_bytes = 0;
     if (k >= kSortedFrom &&
-        sort_pairs_u32(nullptr, &temp_bytes, nullptr, nullptr, nullptr, nullptr, pl.k, end_bit, stream) == hipSuccess)
-        keys = reinterpret_cast<uint32_t*>(workspace_acquire(4 * k_pad * 4 + temp_bytes, &cap));
+        sort_pairs_u32(nullptr, &temp_bytes, nullptr, nullptr, nullptr, nullptr, pl.k, end_bit, stream) == hipSuccess &&
+        select_flagged_positions(nullptr, &select_bytes, nullptr, nullptr, nullptr, pl.k, stream) == hipSuccess) {
+        if (select_bytes > temp_bytes) temp_bytes = select_bytes;           // the two passes share their scratch
+        temp_bytes = (temp_bytes + 255) & ~static_cast<size_t>(255);
+        // keys, vals, sorted keys, sorted vals, heads: k_pad each; count: 64; flags: k_pad bytes
+        keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 64 * 4 + k_pad + temp_bytes, &cap));
+    }
     if (!keys) {
         (void)hipGetLastError();
         const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
@@ -747,23 +831,36 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     uint32_t* vals = keys + k_pad;
     uint32_t* keys_sorted = vals + k_pad;
     uint32_t* vals_sorted = keys_sorted + k_pad;
-    void* temp = vals_sorted + k_pad;
+    uint32_t* heads = vals_sorted + k_pad;
+    uint32_t* head_count = heads + k_pad;
+    void* temp = head_count + 64;
+    uint8_t* flags = reinterpret_cast<uint8_t*>(temp) + temp_bytes;
     const bool vec = inner % 4 == 0;
+    const bool ragged = !vec && inner > 4 && outer * k * ((inner + 3) / 4) <= kMaxElements;
     if (vec) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }
-    const uint32_t units = static_cast<uint32_t>(vec ? n_src / 4 : n_src);
+    if (ragged) { pl.inner = static_cast<uint32_t>((inner + 3) / 4); pl.inner_div = make_div(pl.inner); }
+    const uint32_t units = static_cast<uint32_t>(vec ? n_src / 4 : ragged ? outer * k * pl.inner : n_src);
     hipError_t sort_status = hipSuccess;
     int rc = with_index_check("Index Add", [&](int* flag) {
         {
-            LaunchScope scope("index_sort", "", k * 4 * 5);
+            LaunchScope scope("index_sort", "", k * 4 * 7);
             hipLaunchKernelGGL(index_keys_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, sx->ptr, pl.k,
                                pl.axis_len, keys, vals, flag);
-            sort_status = sort_pairs_u32(temp, &temp_bytes, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
+            size_t scratch = temp_bytes;
+            sort_status = sort_pairs_u32(temp, &scratch, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
+            if (sort_status == hipSuccess) {
+                hipLaunchKernelGGL(index_heads_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, flags);
+                scratch = temp_bytes;
+                sort_status = select_flagged_positions(temp, &scratch, flags, heads, head_count, pl.k, stream);
+            }
         }
         if (sort_status != hipSuccess) return;
-        LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : "float", 3 * n_src * 4 + k * 4);
+        LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : ragged ? "float4 at dword addresses" : "float", 3 * n_src * 4 + k * 4);
         const dim3 grid((units + kBlock - 1) / kBlock);
-        if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, alpha, units, pl);
-        else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, alpha, units, pl);
+        if (ragged) hipLaunchKernelGGL(index_add_sorted_ragged_kernel, grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units,
+                                       static_cast<uint32_t>(inner), pl);
+        else if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
+        else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
     });
     workspace_release(reinterpret_cast<float*>(keys), cap);
     if (sort_status != hipSuccess) return fail(KTH_E_DEVICE, "kth_index_add: sorting the index list failed: %s", hipGetErrorString(sort_status));

@@ -81,6 +81,11 @@ Store* lookup(uint64_t handle, const char* what);
 float* workspace_acquire(uint64_t bytes, uint64_t* cap_bytes);
 void   workspace_release(float* p, uint64_t cap_bytes);
 
+// The ascending positions i in [0, n) with flags[i] != 0 and their number, on `stream` (kth_sort.hip).
+// With temp == nullptr only *temp_bytes is set, to the scratch size needed.
+hipError_t select_flagged_positions(void* temp, size_t* temp_bytes, const uint8_t* flags, uint32_t* positions, uint32_t* count,
+                                    uint32_t n, hipStream_t stream);
+
 // out = in with its dims reordered: out dim d is in dim axes[d] (kth_layout.hip). Device pointers
 // to dense tensors of the same, non-zero element count; `axes` names every dim once.
 int permute_device(const char* what, const float* in, float* out, const int32_t* shape, int dims, const int32_t* axes);
