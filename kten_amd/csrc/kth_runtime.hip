@@ -357,6 +357,25 @@ __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ src
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) dst[(n4 << 2) + threadIdx.x] = src[(n4 << 2) + threadIdx.x];
 }
 
+// The same between any two dword addresses: 16-byte accesses on both sides (the hardware takes them
+// at any dword address); the destination side is brought to a 16-byte boundary first so that its
+// stores are the aligned ones. `head` = floats before that boundary (0 ... 3), moved by workgroup 0
+// together with the tail.
+typedef float copy_v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+__global__ __launch_bounds__(256) void copy_any_kernel(const float* __restrict__ src, float* __restrict__ dst, uint32_t n, uint32_t head) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t body = (n - head) >> 2;
+    if (i < body) {
+        const copy_v4f_unaligned v = __builtin_nontemporal_load(reinterpret_cast<const copy_v4f_unaligned*>(src + head) + i);
+        reinterpret_cast<copy_v4f*>(dst + head)[i] = copy_v4f{v.x, v.y, v.z, v.w};
+    }
+    if (blockIdx.x == 0) {
+        if (threadIdx.x < head) dst[threadIdx.x] = src[threadIdx.x];
+        const uint32_t done = head + (body << 2);
+        if (threadIdx.x >= 64 && threadIdx.x - 64 < n - done) dst[done + threadIdx.x - 64] = src[done + threadIdx.x - 64];
+    }
+}
+
 }  // namespace
 
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n) {
@@ -380,6 +399,16 @@ int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offse
         const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + 255) / 256);
         hipLaunchKernelGGL(copy_kernel, dim3(blocks == 0 ? 1 : blocks), dim3(256), 0, s.stream, sst->ptr + src_offset,
                            d->ptr + dst_offset, static_cast<uint32_t>(n));
+        KTH_LAUNCH_CHECK("copy_kernel");
+        return KTH_OK;
+    }
+    if (n <= kMaxElements) {
+        uint32_t head = static_cast<uint32_t>((4 - dst_offset % 4) % 4);
+        if (head > n) head = static_cast<uint32_t>(n);
+        LaunchScope scope("copy_kernel", "dword addresses", n * 8);
+        const uint32_t blocks = static_cast<uint32_t>((((n - head) >> 2) + 255) / 256);
+        hipLaunchKernelGGL(copy_any_kernel, dim3(blocks == 0 ? 1 : blocks), dim3(256), 0, s.stream, sst->ptr + src_offset,
+                           d->ptr + dst_offset, static_cast<uint32_t>(n), head);
         KTH_LAUNCH_CHECK("copy_kernel");
         return KTH_OK;
     }

@@ -233,3 +233,31 @@ def test_inplace_resize_parity(old, new, gc):
     assert_bits_equal(shared.toArray().reshape(-1), x.reshape(-1), "the shallow copy keeps the old store")
     g.plusAssign(1.0); c.plusAssign(1.0)                      # the new store is an ordinary store
     assert_bits_equal(g.toArray().reshape(-1), c.toArray().reshape(-1), "arithmetic on the resized tensor")
+
+
+def test_copy_between_any_offsets(hip):
+    """kth_copy for every combination of source and destination offsets modulo 4 and lengths around
+    the 16-byte units: the range arrives bit for bit and nothing next to it is touched."""
+    import ctypes
+    from kten_amd import abi
+    lib = hip.lib
+    size = 6000
+    src_host = np.random.default_rng(9).standard_normal(size).astype(np.float32)
+    hs, hd = ctypes.c_uint64(), ctypes.c_uint64()
+    abi.check(lib.kth_alloc(size, ctypes.byref(hs))); abi.check(lib.kth_alloc(size, ctypes.byref(hd)))
+    abi.check(lib.kth_upload(hs, 0, src_host.ctypes.data_as(ctypes.c_void_p), size))
+    out = np.empty(size, np.float32)
+    try:
+        for n in (0, 1, 2, 3, 4, 5, 7, 8, 9, 255, 1023, 1024, 1025, 4099):
+            for so in range(5):
+                for do in range(5):
+                    abi.check(lib.kth_fill(hd, 0, size, -7.0))
+                    abi.check(lib.kth_copy(hd, 10 + do, hs, 20 + so, n))
+                    abi.check(lib.kth_download(out.ctypes.data_as(ctypes.c_void_p), hd, 0, size))
+                    want = np.full(size, -7.0, np.float32)
+                    want[10 + do:10 + do + n] = src_host[20 + so:20 + so + n]
+                    assert_bits_equal(out, want, f"copy of {n} floats from offset {20 + so} to offset {10 + do}")
+        assert lib.kth_copy(hd, 0, hd, 2, 10) == abi.KTH_E_ARGUMENT          # overlapping ranges in one store
+        assert lib.kth_copy(hd, size - 3, hs, 0, 4) == abi.KTH_E_ARGUMENT    # past the end of the destination
+    finally:
+        abi.check(lib.kth_release(hs)); abi.check(lib.kth_release(hd))
