@@ -156,62 +156,71 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 //   add:    contenders lower the element's tag to their lane number with an atomic min; the
 //           lowest lane adds its value and leaves, and the round repeats until nobody is left
 //           (as many rounds as the most frequent index of the chunk occurs).
-// LDS: a_axis_len floats, plus a_axis_len tags for MODE 1. THREADS = 1024 for rows above 32 KiB of
+// LDS: band_len floats (the whole row when it fits), plus band_len tags for MODE 1. THREADS = 1024 for rows above 32 KiB of
 // LDS, which leave room for few workgroups on a CU: the chunk is then 1024 entries.
 template <int MODE, int THREADS>
 __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __restrict__ target, const float* __restrict__ index,
-                                                                 const float* __restrict__ src, float value, IndexPlan pl, int* bad) {
+                                                                 const float* __restrict__ src, float value, IndexPlan pl, int* bad,
+                                                                 uint32_t band_len) {
     extern __shared__ __attribute__((aligned(16))) float row_lds[];
     float* tile = row_lds;
     uint32_t* tile_bits = reinterpret_cast<uint32_t*>(row_lds);
-    uint32_t* tag = reinterpret_cast<uint32_t*>(row_lds) + pl.a_axis_len;     // MODE 1 only
+    uint32_t* tag = reinterpret_cast<uint32_t*>(row_lds) + band_len;          // MODE 1 only
     const uint32_t tid = threadIdx.x;
     uint32_t io, ao, bo;
     locate(pl, blockIdx.x, io, ao, bo);
-    float* trow = target + ao;
     const float* irow = index + io;
     const float* srow = src + bo;
-    row_to_lds<THREADS>(trow, tile, pl.a_axis_len);
-    if (MODE == 1) for (uint32_t j = tid; j < pl.a_axis_len; j += THREADS) tag[j] = 0xffffffffu;
-    // the first chunk's entries are fetched while the row arrives
-    float next_i = 0.0f, next_v = value;
-    if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
-    __syncthreads();
-    for (uint32_t r0 = 0; r0 < pl.i_axis_len; r0 += THREADS) {
-        const uint32_t r = r0 + tid;
-        bool have = r < pl.i_axis_len;
-        const int sel_raw = static_cast<int>(next_i);
-        const float v = MODE == 1 ? next_v * value : next_v;      // add form: value is the factor on the source (1 for scatterAdd)
-        if (r + THREADS < pl.i_axis_len) { next_i = irow[r + THREADS]; if (MODE != 2) next_v = srow[r + THREADS]; }
-        if (have && (sel_raw < 0 || static_cast<uint32_t>(sel_raw) >= pl.a_axis_len)) { *bad = 1; have = false; }
-        const uint32_t sel = have ? static_cast<uint32_t>(sel_raw) : 0u;
-        if (MODE == 2) {
-            if (have) tile[sel] = value;                   // equal values: the order of the stores is immaterial
-        } else if (MODE == 0) {
-            if (have) tile_bits[sel] = 0u;
-            __syncthreads();
-            if (have) atomicMax(&tile_bits[sel], tid + 1u);
-            __syncthreads();
-            const bool last = have && tile_bits[sel] == tid + 1u;
-            __syncthreads();
-            if (last) tile[sel] = v;
-            __syncthreads();
-        } else {
-            bool pending = have;
-            while (true) {
-                if (pending) atomicMin(&tag[sel], tid);
+    // A target row longer than the LDS holds is taken in bands of band_len elements (a multiple of 4):
+    // each band walks the whole index row and applies the entries that fall into it. Entries for one
+    // element are all in the same band, so their order is kept.
+    for (uint32_t band0 = 0; band0 < pl.a_axis_len; band0 += band_len) {
+        const uint32_t band = min(band_len, pl.a_axis_len - band0);
+        float* trow = target + ao + band0;
+        if (band0 > 0) __syncthreads();                       // the previous band has left the tile
+        row_to_lds<THREADS>(trow, tile, band);
+        if (MODE == 1) for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
+        // the first chunk's entries are fetched while the row arrives
+        float next_i = 0.0f, next_v = value;
+        if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
+        __syncthreads();
+        for (uint32_t r0 = 0; r0 < pl.i_axis_len; r0 += THREADS) {
+            const uint32_t r = r0 + tid;
+            bool have = r < pl.i_axis_len;
+            const int sel_raw = static_cast<int>(next_i);
+            const float v = MODE == 1 ? next_v * value : next_v;  // add form: value is the factor on the source (1 for scatterAdd)
+            if (r + THREADS < pl.i_axis_len) { next_i = irow[r + THREADS]; if (MODE != 2) next_v = srow[r + THREADS]; }
+            if (have && (sel_raw < 0 || static_cast<uint32_t>(sel_raw) >= pl.a_axis_len)) { *bad = 1; have = false; }
+            if (have && (static_cast<uint32_t>(sel_raw) < band0 || static_cast<uint32_t>(sel_raw) >= band0 + band)) have = false;
+            const uint32_t sel = have ? static_cast<uint32_t>(sel_raw) - band0 : 0u;
+            if (MODE == 2) {
+                if (have) tile[sel] = value;               // equal values: the order of the stores is immaterial
+            } else if (MODE == 0) {
+                if (have) tile_bits[sel] = 0u;
                 __syncthreads();
-                if (pending && tag[sel] == tid) {          // one lane per element gets here
-                    tile[sel] = tile[sel] + v;
-                    tag[sel] = 0xffffffffu;
-                    pending = false;
+                if (have) atomicMax(&tile_bits[sel], tid + 1u);
+                __syncthreads();
+                const bool last = have && tile_bits[sel] == tid + 1u;
+                __syncthreads();
+                if (last) tile[sel] = v;
+                __syncthreads();
+            } else {
+                bool pending = have;
+                while (true) {
+                    if (pending) atomicMin(&tag[sel], tid);
+                    __syncthreads();
+                    if (pending && tag[sel] == tid) {      // one lane per element gets here
+                        tile[sel] = tile[sel] + v;
+                        tag[sel] = 0xffffffffu;
+                        pending = false;
+                    }
+                    if (!__syncthreads_or(pending ? 1 : 0)) break;
                 }
-                if (!__syncthreads_or(pending ? 1 : 0)) break;
             }
         }
+        __syncthreads();
+        lds_to_row<THREADS>(tile, trow, band);
     }
-    __syncthreads();
-    lds_to_row<THREADS>(tile, trow, pl.a_axis_len);
 }
 
 // indexSelect / indexAdd (JVMRawTensor.kt:484-516): the index is one list of k rows along the
@@ -464,9 +473,8 @@ static bool gather_rows_fit_lds(uint32_t a_axis_len, uint32_t i_axis_len) {
     return static_cast<uint64_t>(a_axis_len) * 4u <= rows_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
 }
 
-static bool scatter_rows_fit_lds(int mode, uint32_t a_axis_len, uint32_t i_axis_len) {
-    const uint64_t lds_bytes = static_cast<uint64_t>(a_axis_len) * (mode == 1 ? 8u : 4u);
-    return lds_bytes <= rows_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
+static bool scatter_rows_fit_lds(int /*mode*/, uint32_t a_axis_len, uint32_t i_axis_len) {
+    return i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;      // longer target rows go in bands
 }
 
 }  // namespace
@@ -560,14 +568,18 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
     const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
     const uint64_t bytes = (mode == 2 ? 2 : mode == 1 ? 4 : 3) * idx_n * 4;
     if (axis == dims - 1 && scatter_rows_fit_lds(mode, pl.a_axis_len, pl.i_axis_len) && positions <= 0x7fffffffull) {
-        const uint32_t lds_bytes = pl.a_axis_len * (mode == 1 ? 8u : 4u);
-        const uint64_t row_bytes = (2ull * pl.a_axis_len * positions + (mode == 2 ? 1 : 2) * idx_n) * 4;
+        const uint32_t per_element = mode == 1 ? 8u : 4u;
+        uint32_t band_len = pl.a_axis_len;
+        if (static_cast<uint64_t>(band_len) * per_element > rows_lds_limit()) band_len = (rows_lds_limit() / per_element) & ~3u;
+        const uint32_t lds_bytes = band_len * per_element;
+        const uint64_t bands = (pl.a_axis_len + band_len - 1) / band_len;
+        const uint64_t row_bytes = (2ull * pl.a_axis_len * positions + bands * (mode == 2 ? 1 : 2) * idx_n) * 4;
         return with_index_check("Scatter", [&](int* flag) {
             LaunchScope scope("scatter_rows_lds_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", row_bytes);
             const dim3 grid(static_cast<uint32_t>(positions));
             hipStream_t stream = state().stream;
             const float factor = mode == 1 ? 1.0f : value;
-#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag)
+#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag, band_len)
             if (lds_bytes > 32768u) { if (mode == 0) ROWS_LAUNCH(0, 1024); else if (mode == 1) ROWS_LAUNCH(1, 1024); else ROWS_LAUNCH(2, 1024); }
             else                    { if (mode == 0) ROWS_LAUNCH(0, 256);  else if (mode == 1) ROWS_LAUNCH(1, 256);  else ROWS_LAUNCH(2, 256); }
 #undef ROWS_LAUNCH
@@ -789,14 +801,16 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
         rp.i_stride[0] = 0; rp.a_stride[0] = pl.axis_len; rp.b_stride[0] = pl.k;
         rp.i_axis_stride = rp.a_axis_stride = rp.b_axis_stride = 1;
         rp.i_axis_len = pl.k; rp.a_axis_len = pl.axis_len;
-        const uint32_t lds_bytes = rp.a_axis_len * 8u;
+        uint32_t band_len = rp.a_axis_len;
+        if (static_cast<uint64_t>(band_len) * 8u > rows_lds_limit()) band_len = (rows_lds_limit() / 8u) & ~3u;
+        const uint32_t lds_bytes = band_len * 8u;
         return with_index_check("Index Add", [&](int* flag) {
             LaunchScope scope("scatter_rows_lds_kernel", "indexAdd", (2 * total + n_src + k) * 4);
             const dim3 grid(static_cast<uint32_t>(outer));
             if (lds_bytes > 32768u)
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len);
             else
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len);
         });
     }
 

@@ -18,7 +18,7 @@ CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([
          # rows along the innermost axis that are scattered inside LDS: the size limits of the assign and add forms
          # and one past them, index dims smaller than the target's, one index value for a whole row
          ([3, 16384], [3, 5000], 1), ([3, 8192], [3, 3000], 1), ([2, 8193], [2, 2000], 1), ([2, 16385], [2, 4000], 1),
-         ([2, 32768], [2, 5000], 1), ([2, 32769], [2, 5000], 1),
+         ([2, 32768], [2, 5000], 1), ([2, 32769], [2, 5000], 1), ([3, 100001], [3, 40000], 1), ([70001, 6], [30000, 5], 0),
          ([10, 6, 300], [7, 4, 100], 2), ([5, 1], [5, 700], 1), ([1, 4096], [1, 4096], 1),
          # a long axis that is not the innermost: scattered as rows between two permutes
          ([4096, 96], [4096, 96], 0), ([2, 3000, 40], [2, 2500, 33], 1), ([8192, 3, 5], [8000, 2, 5], 0), ([5000, 7], [700, 7], 0)]
