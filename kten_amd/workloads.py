@@ -266,7 +266,84 @@ def _bytes_bn(d):
     return 4 * (8 * full + 14 * c)
 
 
+# ---- reductions over the geometries that have kernels of their own ------------------------------
+
+# (shape at scale 1, axis, op): slabs staged in LDS, a streamed slab, a few rows over wide columns,
+# rows that start off 16-byte boundaries, short rows
+_REDUCE_SHAPES = [([65536, 16, 64], 1, "sum"), ([6710, 1000, 10], 1, "sum"), ([23, 2, 1456699], 1, "max"),
+                  ([32752, 2049], 1, "argMax"), ([262144, 255], 1, "mean")]
+
+
+def reduce_shapes_at(d):
+    """The (shape, axis, op) list of the reduce_shapes workload at dims `d`."""
+    return [([max(1, shape[0] // d["scale"])] + shape[1:], axis, op) for shape, axis, op in _REDUCE_SHAPES]
+
+
+def _in_red(d):
+    g = SplitMix64(11)
+    return {f"x{i}": g.normal(shape) for i, (shape, _, _) in enumerate(reduce_shapes_at(d))}
+
+
+def _run_red(ops, inp):
+    out = {}
+    for i, (shape, axis, op) in enumerate(_REDUCE_SHAPES):
+        x = ops.create(list(inp[f"x{i}"].shape), False, inp[f"x{i}"])
+        out[f"{op}{i}"] = getattr(x, op)(axis)
+    return out
+
+
+def _bytes_red(d):
+    total = 0
+    for shape, axis, _ in reduce_shapes_at(d):
+        n = int(np.prod(shape, dtype=np.int64))
+        total += 4 * (n + n // shape[axis])
+    return total
+
+
+# ---- indexed moves with index tensors as large as the data ---------------------------------------
+
+def _in_idx(d):
+    g = SplitMix64(12)
+    rows, cols = d["rows"], d["cols"]
+    def ints(shape, limit):
+        return np.minimum(np.floor(g.uniform(shape, 0.0, float(limit))), np.float32(limit - 1)).astype(np.float32)
+    return {"x": g.normal([rows, cols]), "along_cols": ints([rows, cols], cols), "along_rows": ints([rows, cols], rows),
+            "row_list": ints([rows], rows)}
+
+
+def _run_idx(ops, inp):
+    from .autograd import NoGradVariable
+    raw = {k: ops.create(list(v.shape), False, v).getRawValue() for k, v in inp.items()}
+    x = raw["x"]
+    gathered = x.gather(1, raw["along_cols"])
+    assigned = ops.zerosLike(x)
+    assigned.inplaceScatter(1, raw["along_cols"], x)
+    added = ops.zerosLike(x)
+    added.inplaceScatterAdd(0, raw["along_rows"], x)
+    selected = x.indexSelect(0, raw["row_list"])
+    summed = ops.zerosLike(x)
+    summed.indexAdd(0, raw["row_list"], selected, 1.0)
+    res = {"gathered": gathered, "assigned": assigned, "added": added, "selected": selected, "summed": summed}
+    return {k: NoGradVariable(ops, v) for k, v in res.items()}
+
+
+def _bytes_idx(d):
+    n, rows = d["rows"] * d["cols"], d["rows"]
+    # gather 12 N; three zerosLike 4 N each; assign 12 N; add 16 N; indexSelect 8 N + list; indexAdd 12 N + list
+    return 72 * n + 8 * rows
+
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "reduce_shapes": Workload("reduce_shapes", "axis reductions over a middle or last axis on five geometries of 2^26 elements each: "
+                                               "[65536,16,64] sum, [6710,1000,10] sum, [23,2,1456699] max, [32752,2049] argMax, "
+                                               "[262144,255] mean; N(0,1), seed 11",
+                              {"scale": 1}, _in_red, _run_red, _bytes_red),
+    "indexed_moves": Workload("indexed_moves", "x[16384,4096] with index tensors of its own size: gather along axis 1, inplaceScatter "
+                                               "along axis 1, inplaceScatterAdd along axis 0 (each into zerosLike(x)), indexSelect and "
+                                               "indexAdd of 16384 rows; seed 12",
+                              {"rows": 16384, "cols": 4096}, _in_idx, _run_idx, _bytes_idx),
+
     "batch_norm": Workload("batch_norm", "BatchNormOperation over axis 1 of NCHW [64,128,56,56], training mode: calculateOutput "
                                          "then calculateGrads (input, gamma and beta gradients); seed 10",
                            {"n": 64, "c": 128, "h": 56, "w": 56}, _in_bn, _run_bn, _bytes_bn),

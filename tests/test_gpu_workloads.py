@@ -8,7 +8,7 @@ argmax against numpy on tie-free data."""
 import numpy as np
 import pytest
 
-from kten_amd.workloads import WORKLOADS
+from kten_amd.workloads import WORKLOADS, reduce_shapes_at
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal, assert_reduction_close, assert_ulp_close, ulp_distance
 
@@ -207,3 +207,49 @@ def test_cfg5_full(gc):
     assert_reduction_close(got["grad_w"], gw_ref, jvm_gw, "grad w")
     assert_reduction_close(got["grad_b"], [gb_ref], jvm_gb, "grad b")
     assert abs(float(got["loss"][0]) - loss_ref) <= 1e-5 * loss_ref
+
+
+def _check_reduce_shapes(inp, got, scale):
+    for i, (shape, axis, op) in enumerate(reduce_shapes_at({"scale": scale})):
+        x = inp[f"x{i}"]
+        res = got[f"{op}{i}"]
+        if op in ("sum", "mean"):
+            ref, _ = jo.axis_sum_f64(x, axis)
+            want = jo.aggregate(op, x, axis).reshape(-1)
+            assert_reduction_close(res.reshape(-1), ref / (shape[axis] if op == "mean" else 1), want, f"{op} {shape}")
+        else:
+            code = {"max": "max", "argMax": "arg_max"}[op]
+            assert_bits_equal(res.reshape(-1), jo.aggregate(code, x, axis).reshape(-1), f"{op} {shape}")
+
+
+def test_reduce_shapes_small(gc):
+    wl = WORKLOADS["reduce_shapes"]
+    inp = wl.make_inputs({"scale": 64})
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    _check_reduce_shapes(inp, got, 64)
+
+
+def test_reduce_shapes_full(gc):
+    """The five geometries at 2^26 elements each against the checker running on 16 threads."""
+    wl = WORKLOADS["reduce_shapes"]
+    inp = wl.make_inputs(wl.full_dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    jo.set_threads(16)
+    try:
+        _check_reduce_shapes(inp, got, 1)
+    finally:
+        jo.set_threads(1)
+
+
+@pytest.mark.parametrize("dims", [{"rows": 300, "cols": 520}, {"rows": 16384, "cols": 4096}], ids=["small", "full"])
+def test_indexed_moves(dims, gc):
+    """Bit-exact against the checker, full size included: gather, assignment with the last entry
+    winning, adds in index order, row selection and row accumulation."""
+    wl = WORKLOADS["indexed_moves"]
+    inp = wl.make_inputs(dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    want = {k: v.toArray() for k, v in wl.run(jo.JvmOracleOperations(), inp).items()}
+    for k in ("gathered", "assigned", "added", "selected", "summed"):
+        assert_bits_equal(got[k], want[k], k)
+    assert_bits_equal(got["gathered"], np.take_along_axis(inp["x"], inp["along_cols"].astype(np.int64), 1), "gather vs numpy")
+    assert_bits_equal(got["selected"], inp["x"][inp["row_list"].astype(np.int64)], "indexSelect vs numpy")
