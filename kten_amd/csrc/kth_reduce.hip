@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const float* __rest
 // span: it is loaded with coalesced float4s whatever the row length, parked in LDS at an odd
 // row stride (conflict-free), and then `256 / rows` lanes fold each row from LDS, in index
 // order within a lane.
-constexpr uint32_t kShortTile = 8192;        // floats per tile: 32 KiB of LDS (+ padding)
+constexpr uint32_t kShortTile = 4096;        // floats per tile: 16 KiB of LDS (+ padding); measured against 8 and 32 KiB
 constexpr uint32_t kShortLoads = kShortTile / 4 / kBlock;
 
 struct ShortPlan {
