@@ -1,7 +1,7 @@
 """The five benchmark configurations through the `Tensor` API on the HIP backend.
 
 Scaled-down shapes are compared with the CPU checker running the very same graph.
-Full BASELINE shapes are checked through what does not need the serial CPU restatement
+Full benchmark shapes are checked through what does not need the serial CPU restatement
 of every pass: numpy closed forms for single-rounding ops, float64 references for the
 reductions (plus the checker's own error on the reductions, which it can do in seconds),
 argmax against numpy on tie-free data."""
@@ -105,7 +105,7 @@ def test_cfg5_gradient_accumulates_over_two_backward_passes(gc):
     assert not w.grad().toArray().any()
 
 
-# ---------------------------------------------------------------- full BASELINE shapes
+# ---------------------------------------------------------------- full benchmark shapes
 
 def test_cfg1_full(gc):
     wl = WORKLOADS["cfg1"]
