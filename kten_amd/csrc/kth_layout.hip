@@ -93,36 +93,46 @@ __global__ __launch_bounds__(kBlock) void move_kernel(const float* __restrict__ 
 // dword address, otherwise one by one. `n` counts floats; MODE 0 and 1 only.
 typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
+// Offsets on the strided side of dense floats i+1 .. i+3, given float i's (`first`, at place r0 of
+// its innermost run). Floats past `n` get `first`; their lanes are never moved.
+__device__ __forceinline__ void straddling_offsets(const MovePlan& pl, uint32_t i, uint32_t n, uint32_t r0, uint32_t first,
+                                                   uint32_t at[4]) {
+    at[0] = first;
+#pragma unroll
+    for (int j = 1; j < 4; j++)
+        at[j] = (pl.ndim == 1 || r0 + j < pl.size[0]) ? first + j * pl.stride[0] : (i + j < n ? strided_offset(pl, i + j) : first);
+}
+
+constexpr int kMixedUnroll = 1;
+
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restrict__ src, float* __restrict__ dst,
                                                            uint32_t n, MovePlan pl) {
-    const uint32_t base = blockIdx.x * (kBlock * kMoveUnroll) + threadIdx.x;
-    uint32_t at[kMoveUnroll][4];
-    bool run4[kMoveUnroll];                  // the four floats lie next to each other on the strided side too
-    v4f v[kMoveUnroll];
+    const uint32_t base = blockIdx.x * (kBlock * kMixedUnroll) + threadIdx.x;
+    uint32_t first[kMixedUnroll], place[kMixedUnroll];
+    bool run4[kMixedUnroll];                  // the four floats lie next to each other on the strided side too
+    v4f v[kMixedUnroll];
 #pragma unroll
-    for (int k = 0; k < kMoveUnroll; k++) {
+    for (int k = 0; k < kMixedUnroll; k++) {
         const uint32_t i = (base + k * kBlock) * 4u;
         run4[k] = false;
         if (i >= n) continue;
         // position inside the innermost run decides whether the four floats share it
         const uint32_t q0 = (__umulhi(i, pl.div[0].mul) + i) >> pl.div[0].shift;
-        const uint32_t r0 = i - q0 * pl.size[0];
-        at[k][0] = strided_offset(pl, i);
-        const bool together = pl.ndim == 1 || r0 + 3 < pl.size[0];
-        run4[k] = together && pl.stride[0] == 1 && i + 3 < n;
-#pragma unroll
-        for (int j = 1; j < 4; j++)
-            at[k][j] = (pl.ndim == 1 || r0 + j < pl.size[0]) ? at[k][0] + j * pl.stride[0] : (i + j < n ? strided_offset(pl, i + j) : at[k][0]);
+        place[k] = i - q0 * pl.size[0];
+        first[k] = strided_offset(pl, i);
+        run4[k] = pl.stride[0] == 1 && (pl.ndim == 1 || place[k] + 3 < pl.size[0]) && i + 3 < n;
         if (MODE == 0) {
             if (run4[k]) {                   // one 16-byte load from a dword address
-                const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(src + at[k][0]);
+                const v4f_unaligned t = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(src + first[k]));
                 v[k] = v4f{t.x, t.y, t.z, t.w};
             } else {
-                v[k].x = src[at[k][0]];
-                v[k].y = i + 1 < n ? src[at[k][1]] : 0.0f;
-                v[k].z = i + 2 < n ? src[at[k][2]] : 0.0f;
-                v[k].w = i + 3 < n ? src[at[k][3]] : 0.0f;
+                uint32_t at[4];
+                straddling_offsets(pl, i, n, place[k], first[k], at);
+                v[k].x = src[at[0]];
+                v[k].y = i + 1 < n ? src[at[1]] : 0.0f;
+                v[k].z = i + 2 < n ? src[at[2]] : 0.0f;
+                v[k].w = i + 3 < n ? src[at[3]] : 0.0f;
             }
         } else if (i + 3 < n) {
             v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + i));
@@ -131,19 +141,21 @@ __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restr
         }
     }
 #pragma unroll
-    for (int k = 0; k < kMoveUnroll; k++) {
+    for (int k = 0; k < kMixedUnroll; k++) {
         const uint32_t i = (base + k * kBlock) * 4u;
         if (i >= n) continue;
         if (MODE == 0) {
             if (i + 3 < n) *reinterpret_cast<v4f*>(dst + i) = v[k];
             else { dst[i] = v[k].x; if (i + 1 < n) dst[i + 1] = v[k].y; if (i + 2 < n) dst[i + 2] = v[k].z; }
         } else if (run4[k]) {
-            *reinterpret_cast<v4f_unaligned*>(dst + at[k][0]) = v4f_unaligned{v[k].x, v[k].y, v[k].z, v[k].w};
+            *reinterpret_cast<v4f_unaligned*>(dst + first[k]) = v4f_unaligned{v[k].x, v[k].y, v[k].z, v[k].w};
         } else {
-            dst[at[k][0]] = v[k].x;
-            if (i + 1 < n) dst[at[k][1]] = v[k].y;
-            if (i + 2 < n) dst[at[k][2]] = v[k].z;
-            if (i + 3 < n) dst[at[k][3]] = v[k].w;
+            uint32_t at[4];
+            straddling_offsets(pl, i, n, place[k], first[k], at);
+            dst[at[0]] = v[k].x;
+            if (i + 1 < n) dst[at[1]] = v[k].y;
+            if (i + 2 < n) dst[at[2]] = v[k].z;
+            if (i + 3 < n) dst[at[3]] = v[k].w;
         }
     }
 }
@@ -222,7 +234,9 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
 struct RunsPlan {
     TilePlan t;
     uint32_t run, tile, pitch;               // elements per run, runs per tile side, LDS elements per x
+    uint32_t tiles;                          // the grid holds this many rounded up to a multiple of 8
     FastDiv  in_row_div, run_div, out_row_div;
+    FastDiv  unit_row_div;                   // by the 16-byte units of one span (float runs only)
 };
 
 template <class V>
@@ -230,7 +244,10 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
     constexpr uint32_t kElems = kTileElems * sizeof(float) / sizeof(V);      // 16 KiB of elements
     __shared__ V tile[kElems + 64];
     const TilePlan& pl = rp.t;
-    uint32_t t = blockIdx.x;
+    // Workgroups go to the eight XCDs in turn: give each XCD one contiguous eighth of the tiles, so
+    // that the cache lines two neighbouring tiles share are fetched into one L2 and not into two.
+    uint32_t t = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (t >= rp.tiles) return;
     uint32_t q = (__umulhi(t, pl.x_tiles_div.mul) + t) >> pl.x_tiles_div.shift;
     const uint32_t x0 = (t - q * pl.x_tiles) * rp.tile;
     t = q;
@@ -251,37 +268,103 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
     V* dst = out + (static_cast<size_t>(out_off) + y0) * rp.run;
     const uint32_t x_floats = min(rp.tile, pl.x_len - x0) * rp.run;   // valid part of an input span
     const uint32_t y_floats = min(rp.tile, pl.y_len - y0) * rp.run;   // valid part of an output span
-    constexpr uint32_t kPasses = kElems / kBlock;
-    V v[kPasses];
+    if constexpr (sizeof(V) == sizeof(float)) {
+        // Runs of floats: a span (a whole number of runs, a multiple of 8 floats) moves as 16-byte
+        // units at dword addresses on both sides; only a unit over the valid end of a span at the
+        // tensor's edge moves float by float.
+        const uint32_t upr = row >> 2;
+        const uint32_t units = rp.tile * upr;
+        constexpr uint32_t kUnitPasses = kElems / 4 / kBlock;
+        v4f v[kUnitPasses];
 #pragma unroll
-    for (uint32_t k = 0; k < kPasses; k++) {
-        const uint32_t f = k * kBlock + threadIdx.x;
-        if (f < floats) {
-            const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
-            const uint32_t p = f - y * row;
-            if (y0 + y < pl.y_len && p < x_floats)
-                v[k] = __builtin_nontemporal_load(src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p);
+        for (uint32_t k = 0; k < kUnitPasses; k++) {
+            const uint32_t u = k * kBlock + threadIdx.x;
+            if (u < units) {
+                const uint32_t y = (__umulhi(u, rp.unit_row_div.mul) + u) >> rp.unit_row_div.shift;
+                const uint32_t p = (u - y * upr) * 4u;
+                if (y0 + y < pl.y_len && p < x_floats) {
+                    const float* g = src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p;
+                    if (p + 4 <= x_floats) {
+                        const v4f_unaligned t4 = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(g));
+                        v[k] = v4f{t4.x, t4.y, t4.z, t4.w};
+                    } else {
+                        v[k].x = g[0];
+                        v[k].y = p + 1 < x_floats ? g[1] : 0.0f;
+                        v[k].z = p + 2 < x_floats ? g[2] : 0.0f;
+                        v[k].w = 0.0f;
+                    }
+                }
+            }
         }
-    }
 #pragma unroll
-    for (uint32_t k = 0; k < kPasses; k++) {
-        const uint32_t f = k * kBlock + threadIdx.x;
-        if (f < floats) {
-            const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
-            const uint32_t p = f - y * row;
-            const uint32_t x = (__umulhi(p, rp.run_div.mul) + p) >> rp.run_div.shift;
-            tile[x * rp.pitch + y * rp.run + (p - x * rp.run)] = v[k];
+        for (uint32_t k = 0; k < kUnitPasses; k++) {
+            const uint32_t u = k * kBlock + threadIdx.x;
+            if (u < units) {
+                const uint32_t y = (__umulhi(u, rp.unit_row_div.mul) + u) >> rp.unit_row_div.shift;
+                const uint32_t p = (u - y * upr) * 4u;
+                const uint32_t x = (__umulhi(p, rp.run_div.mul) + p) >> rp.run_div.shift;
+                uint32_t r = p - x * rp.run, at = x * rp.pitch + y * rp.run;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    tile[at + r] = v[k][j];
+                    if (++r == rp.run) { r = 0; at += rp.pitch; }
+                }
+            }
         }
-    }
-    __syncthreads();
+        __syncthreads();
 #pragma unroll
-    for (uint32_t k = 0; k < kPasses; k++) {
-        const uint32_t f = k * kBlock + threadIdx.x;
-        if (f < floats) {
-            const uint32_t x = (__umulhi(f, rp.out_row_div.mul) + f) >> rp.out_row_div.shift;
-            const uint32_t p = f - x * row;
-            if (x0 + x < pl.x_len && p < y_floats)
-                dst[static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p] = tile[x * rp.pitch + p];
+        for (uint32_t k = 0; k < kUnitPasses; k++) {
+            const uint32_t u = k * kBlock + threadIdx.x;
+            if (u < units) {
+                const uint32_t x = (__umulhi(u, rp.unit_row_div.mul) + u) >> rp.unit_row_div.shift;
+                const uint32_t p = (u - x * upr) * 4u;
+                if (x0 + x < pl.x_len && p < y_floats) {
+                    const float* l = tile + x * rp.pitch + p;
+                    float* g = dst + static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p;
+                    if (p + 4 <= y_floats) {
+                        *reinterpret_cast<v4f_unaligned*>(g) = v4f_unaligned{l[0], l[1], l[2], l[3]};
+                    } else {
+                        g[0] = l[0];
+                        if (p + 1 < y_floats) g[1] = l[1];
+                        if (p + 2 < y_floats) g[2] = l[2];
+                    }
+                }
+            }
+        }
+        return;
+    } else {
+        constexpr uint32_t kPasses = kElems / kBlock;
+        V v[kPasses];
+#pragma unroll
+        for (uint32_t k = 0; k < kPasses; k++) {
+            const uint32_t f = k * kBlock + threadIdx.x;
+            if (f < floats) {
+                const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
+                const uint32_t p = f - y * row;
+                if (y0 + y < pl.y_len && p < x_floats)
+                    v[k] = __builtin_nontemporal_load(src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p);
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < kPasses; k++) {
+            const uint32_t f = k * kBlock + threadIdx.x;
+            if (f < floats) {
+                const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
+                const uint32_t p = f - y * row;
+                const uint32_t x = (__umulhi(p, rp.run_div.mul) + p) >> rp.run_div.shift;
+                tile[x * rp.pitch + y * rp.run + (p - x * rp.run)] = v[k];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t k = 0; k < kPasses; k++) {
+            const uint32_t f = k * kBlock + threadIdx.x;
+            if (f < floats) {
+                const uint32_t x = (__umulhi(f, rp.out_row_div.mul) + f) >> rp.out_row_div.shift;
+                const uint32_t p = f - x * row;
+                if (x0 + x < pl.x_len && p < y_floats)
+                    dst[static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p] = tile[x * rp.pitch + p];
+            }
         }
     }
 }
@@ -400,7 +483,8 @@ void launch_move(const char* family, const float* src, float* dst, uint64_t coun
     for (int d = 0; d < dims.n; d++) pl.div[d] = make_div(pl.size[d]);
     const uint32_t per_block = kBlock * kMoveUnroll;
     if constexpr (MODE != 2) if (!vec && count >= 1024) {
-        const uint32_t blocks4 = static_cast<uint32_t>(((count + 3) / 4 + per_block - 1) / per_block);
+        const uint32_t per_block4 = kBlock * kMixedUnroll;
+        const uint32_t blocks4 = static_cast<uint32_t>(((count + 3) / 4 + per_block4 - 1) / per_block4);
         LaunchScope scope(family, "float4 dense side", bytes);
         hipLaunchKernelGGL((move_mixed_kernel<MODE>), dim3(blocks4), dim3(kBlock), 0, state().stream, src, dst,
                            static_cast<uint32_t>(count), pl);
@@ -500,6 +584,7 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
         rp.tile = elem <= 4 ? 32u : elem <= 16 ? 16u : 8u;
         rp.pitch = (rp.tile * rp.run) | 1u;
         rp.in_row_div = make_div(rp.tile * rp.run); rp.out_row_div = rp.in_row_div; rp.run_div = make_div(rp.run);
+        rp.unit_row_div = make_div(rp.tile * rp.run / 4);
         pl.x_tiles = (pl.x_len + rp.tile - 1) / rp.tile;
         pl.y_tiles = (pl.y_len + rp.tile - 1) / rp.tile;
         pl.x_tiles_div = make_div(pl.x_tiles);
@@ -509,10 +594,12 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
         rp.t = pl;
         const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
         if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+        rp.tiles = static_cast<uint32_t>(blocks);
+        const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
         LaunchScope scope("permute_runs_kernel", vec ? "float4" : "float", n * 8);
-        if (vec) hipLaunchKernelGGL((permute_runs_kernel<v4f>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream,
+        if (vec) hipLaunchKernelGGL((permute_runs_kernel<v4f>), grid, dim3(kBlock), 0, stream,
                                     reinterpret_cast<const v4f*>(in), reinterpret_cast<v4f*>(out), rp);
-        else     hipLaunchKernelGGL((permute_runs_kernel<float>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, stream, in, out, rp);
+        else     hipLaunchKernelGGL((permute_runs_kernel<float>), grid, dim3(kBlock), 0, stream, in, out, rp);
         return KTH_OK;
     }
     // Tile shape: narrow along a dim shorter than 64 (the smallest power of two that holds it), square

@@ -334,7 +334,53 @@ def _bytes_idx(d):
 
 
 
+# ---- layout moves on shapes that are not multiples of anything convenient --------------------------
+
+# (shape at scale 1, permutation): a run of 8 floats kept innermost, a run of 3, a run of 33, a long
+# odd run (one 16-byte side); then a range get whose box starts one float into every row
+_LAYOUT_SHAPES = [([64, 512, 256, 8], [0, 2, 1, 3]), ([4096, 5461, 3], [1, 0, 2]), ([2048, 1024, 33], [1, 0, 2]),
+                  ([4096, 5, 3277], [1, 0, 2])]
+_LAYOUT_BOX = [8192, 8192]
+
+
+def layout_shapes_at(d):
+    """The (shape, permutation) list and the [rows, cols] of the boxed tensor at dims `d`."""
+    return ([([max(1, shape[0] // d["scale"])] + shape[1:], perm) for shape, perm in _LAYOUT_SHAPES],
+            [max(2, _LAYOUT_BOX[0] // d["scale"]), _LAYOUT_BOX[1]])
+
+
+def _in_lay(d):
+    g = SplitMix64(13)
+    shapes, box = layout_shapes_at(d)
+    inp = {f"x{i}": g.uniform(shape, -1.0, 1.0) for i, (shape, _) in enumerate(shapes)}
+    inp["boxed"] = g.uniform(box, -1.0, 1.0)
+    return inp
+
+
+def _run_lay(ops, inp):
+    from .shape_functions import ALL
+    out = {}
+    for i, (_, perm) in enumerate(_LAYOUT_SHAPES):
+        x = ops.create(list(inp[f"x{i}"].shape), False, inp[f"x{i}"])
+        out[f"permuted{i}"] = x.permute(*perm)
+    boxed = ops.create(list(inp["boxed"].shape), False, inp["boxed"])
+    out["box"] = boxed[ALL, (1, inp["boxed"].shape[1] - 3)]
+    return out
+
+
+def _bytes_lay(d):
+    shapes, box = layout_shapes_at(d)
+    total = sum(8 * int(np.prod(shape, dtype=np.int64)) for shape, _ in shapes)
+    return total + 8 * box[0] * (box[1] - 3)
+
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "layout_shapes": Workload("layout_shapes", "permutes that keep an innermost run of 8, 3, 33 and 3277 floats ([64,512,256,8], "
+                                               "[4096,5461,3], [2048,1024,33], [4096,5,3277]) and a range get x[:, 1:8190] of "
+                                               "[8192,8192]; U(-1,1), seed 13",
+                              {"scale": 1}, _in_lay, _run_lay, _bytes_lay),
+
     "reduce_shapes": Workload("reduce_shapes", "axis reductions over a middle or last axis on five geometries of 2^26 elements each: "
                                                "[65536,16,64] sum, [6710,1000,10] sum, [23,2,1456699] max, [32752,2049] argMax, "
                                                "[262144,255] mean; N(0,1), seed 11",

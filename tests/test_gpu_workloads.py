@@ -8,7 +8,7 @@ argmax against numpy on tie-free data."""
 import numpy as np
 import pytest
 
-from kten_amd.workloads import WORKLOADS, reduce_shapes_at
+from kten_amd.workloads import WORKLOADS, layout_shapes_at, reduce_shapes_at
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal, assert_reduction_close, assert_ulp_close, ulp_distance
 
@@ -253,3 +253,16 @@ def test_indexed_moves(dims, gc):
         assert_bits_equal(got[k], want[k], k)
     assert_bits_equal(got["gathered"], np.take_along_axis(inp["x"], inp["along_cols"].astype(np.int64), 1), "gather vs numpy")
     assert_bits_equal(got["selected"], inp["x"][inp["row_list"].astype(np.int64)], "indexSelect vs numpy")
+
+
+@pytest.mark.parametrize("scale", [64, 1], ids=["small", "full"])
+def test_layout_shapes(scale, gc):
+    """Permutes and the range get against numpy (which the checker is pinned to for these moves), bit for bit."""
+    wl = WORKLOADS["layout_shapes"]
+    dims = {"scale": scale}
+    inp = wl.make_inputs(dims)
+    got = wl.run(gc, inp)
+    shapes, _ = layout_shapes_at(dims)
+    for i, (shape, perm) in enumerate(shapes):
+        assert_bits_equal(got[f"permuted{i}"].toArray(), np.transpose(inp[f"x{i}"], perm), f"permute {shape} {perm}")
+    assert_bits_equal(got["box"].toArray(), inp["boxed"][:, 1:inp["boxed"].shape[1] - 2], "range get")
