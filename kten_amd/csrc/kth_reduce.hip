@@ -653,6 +653,10 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     if (inner > 1 && axis >= 2 && (slab < kStreamMinSlab || (axis <= 16 && slab <= kShortTile))) {
         slab_rows = static_cast<uint32_t>(kShortTile / slab);
         if (slab_rows > 4 * kBlock) slab_rows = 4 * kBlock;
+        // the tile parks a slab at the odd pitch slab | 1: slabs of 4 and 6 floats grow by more than the
+        // tile's padding of an eighth, so fewer of them fit (kept a multiple of 4: tiles stay 16-byte aligned)
+        const uint32_t padded_rows = static_cast<uint32_t>((kShortTile + kShortTile / 8) / (slab | 1u));
+        if (slab_rows > padded_rows) slab_rows = padded_rows >= 8 ? (padded_rows & ~3u) : padded_rows;
         if (ceil_div(outer, slab_rows) < static_cast<uint64_t>(st.compute_units)) slab_rows = 0;
     }
     if (slab_rows > 0) {

@@ -36,6 +36,8 @@ GEOMETRIES = [
     # slabs of up to 2047 floats with any axis length, enough of them to take the tiled kernel
     ([8000, 17, 17], 1), ([7000, 40, 8], 1), ([8000, 100, 3], 1), ([3000, 500, 2], 1), ([1500, 24, 80], 1),
     ([1500, 19, 100], 1), ([1500, 128, 13], 1),
+    # the smallest slabs (4 ... 10 floats) in numbers that take the tiled kernel: the odd LDS pitch adds a quarter to a slab of 4
+    ([300000, 2, 2], 1), ([250000, 3, 2], 1), ([250000, 2, 3], 1), ([140000, 2, 4], 1), ([200000, 3, 3], 1), ([120000, 2, 5], 1),
     # a slab (or a segment of it) streamed by one workgroup: scalar and float4 columns, with and without segments
     ([300, 700, 3], 1), ([2, 50000, 12], 1), ([2000, 64, 33], 1), ([1500, 100, 40], 1), ([5, 2049, 1, 63], 1),
     ([3, 40000, 2], 1), ([1, 100000, 7], 1),
