@@ -117,3 +117,48 @@ def test_random_indexed_moves(seed, gc):
         gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
         gt.indexAdd(axis, gr, ga, 0.7); ct.indexAdd(axis, cr, ca, 0.7)
         assert_bits_equal(gt.toArray(), ct.toArray(), f"indexAdd {shape} axis {axis} k {n_rows}")
+
+
+def tiny_and_large(rng, total, k):
+    """k dims: one large, the others drawn from 1..12, in random order; product about `total`."""
+    small = [int(rng.integers(1, 13)) for _ in range(k - 1)]
+    big = max(1, total // int(np.prod(small)))
+    dims = small + [big]
+    return [dims[i] for i in rng.permutation(k)]
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_tiny_dims(seed, gc):
+    """Tiny dims around one large dim: the smallest slabs, rows and runs of the tiled kernels, whose tile
+    paddings and ragged last units differ from those of the mid-sized cases."""
+    rng = np.random.default_rng(5000 + seed)
+    cpu = jo.JvmOracleOperations()
+    for _ in range(8):
+        k = int(rng.integers(2, 5))
+        shape = tiny_and_large(rng, int(rng.integers(1 << 19, 1 << 21)), k)
+        x = (np.round(rng.standard_normal(shape) * 8) / 8).astype(np.float32)
+        t = gc.createRaw(shape, x)
+        ref = cpu.createRaw(shape, x)
+        for axis in range(k):
+            for op, code in (("max", "max"), ("argMax", "arg_max"), ("min", "min")):
+                assert_bits_equal(getattr(t, op)(axis).toArray().reshape(-1), jo.aggregate(code, x, axis).reshape(-1),
+                                  f"{op} {shape} axis {axis}")
+            ref64, _ = jo.axis_sum_f64(x, axis)
+            assert_reduction_close(t.sum(axis).toArray().reshape(-1), ref64, jo.aggregate("sum", x, axis).reshape(-1),
+                                   f"sum {shape} axis {axis}")
+        perm = [int(v) for v in rng.permutation(k)]
+        assert_bits_equal(t.permute(perm).toArray(), np.transpose(x, perm), f"permute {shape} {perm}")
+        # a broadcast partner that keeps a random subset of the dims
+        b_shape = [d if rng.random() < 0.5 else 1 for d in shape]
+        b = rng.uniform(0.5, 2.0, b_shape).astype(np.float32)
+        tb = gc.createRaw(b_shape, b)
+        assert_bits_equal(t._binary("times", tb).toArray(), x * b, f"times {shape} {b_shape}")
+        assert_bits_equal(tb._binary("minus", t).toArray(), b - x, f"minus {b_shape} {shape}")
+        # a box with ragged ends in every dim
+        ranges = []
+        for d in shape:
+            lo = int(rng.integers(0, d)); hi = int(rng.integers(lo, d))
+            ranges.append((lo, hi))
+        want = x[tuple(slice(lo, hi + 1) for lo, hi in ranges)]
+        assert_bits_equal(t.get(ranges).toArray().reshape(-1), want.reshape(-1), f"get {shape} {ranges}")
+        assert_bits_equal(ref.get(ranges).toArray().reshape(-1), want.reshape(-1), f"checker get {shape} {ranges}")
