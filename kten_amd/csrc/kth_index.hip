@@ -152,10 +152,12 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 // order; inside such a chunk, entries that name the same target element are put in order
 // through an LDS tag per element:
 //   assign: the element is cleared, every contender raises it to its lane number + 1 with an
-//           atomic max, and the highest lane (the last entry) then stores its value there;
-//   add:    contenders lower the element's tag to their lane number with an atomic min; the
+//           atomic max, and the highest lane (the last entry) then stores its value there (the
+//           same scheme with tags of their own and one barrier per chunk measured 20 % slower:
+//           twice the LDS per workgroup);
+//   add:    contenders lower the element's tag to (round number, lane) with an atomic min; the
 //           lowest lane adds its value and leaves, and the round repeats until nobody is left
-//           (as many rounds as the most frequent index of the chunk occurs).
+//           (as many rounds as the most frequent index of the chunk occurs), one barrier a round.
 // LDS: band_len floats (the whole row when it fits), plus band_len tags for MODE 1. THREADS = 1024 for rows above 32 KiB of
 // LDS, which leave room for few workgroups on a CU: the chunk is then 1024 entries.
 template <int MODE, int THREADS>
@@ -163,6 +165,9 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                                                                  const float* __restrict__ src, float value, IndexPlan pl, int* bad,
                                                                  uint32_t band_len) {
     extern __shared__ __attribute__((aligned(16))) float row_lds[];
+    constexpr uint32_t kFirstEpoch = 0x3ffffeu;               // 22 bits above the 10 bits of a thread id
+    static_assert(THREADS <= 1024, "a bid keeps the thread id in 10 bits");
+    __shared__ uint32_t any_pending[3];
     float* tile = row_lds;
     uint32_t* tile_bits = reinterpret_cast<uint32_t*>(row_lds);
     uint32_t* tag = reinterpret_cast<uint32_t*>(row_lds) + band_len;          // MODE 1 only
@@ -180,6 +185,8 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         if (band0 > 0) __syncthreads();                       // the previous band has left the tile
         row_to_lds<THREADS>(trow, tile, band);
         if (MODE == 1) for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
+        if (MODE == 1 && tid < 3) any_pending[tid] = 0u;
+        uint32_t epoch = kFirstEpoch;                         // MODE 1: the round counter, uniform over the workgroup
         // the first chunk's entries are fetched while the row arrives
         float next_i = 0.0f, next_v = value;
         if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
@@ -205,16 +212,42 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                 if (last) tile[sel] = v;
                 __syncthreads();
             } else {
-                bool pending = have;
-                while (true) {
-                    if (pending) atomicMin(&tag[sel], tid);
+                // Entries for one element are added in index order, one per round: every pending entry
+                // bids (round, tid) for its element with atomicMin, the lowest tid of the round wins and
+                // adds. Rounds count down, so a bid of a later round always beats what earlier rounds
+                // left in the tag and the tags are never reset; one barrier per round, with a flag that tells
+                // whether anything was pending. A winner that reads its tag after a faster loser has
+                // already bid for the next round sees that bid, stays pending and wins the next round
+                // (same round, lower tid): the order is kept.
+                if (epoch < 2u * THREADS + 4u) {              // (only after millions of rounds on one band)
                     __syncthreads();
-                    if (pending && tag[sel] == tid) {      // one lane per element gets here
+                    for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
+                    if (tid < 3) any_pending[tid] = 0u;
+                    epoch = kFirstEpoch;
+                    __syncthreads();
+                }
+                bool pending = have;
+                for (uint32_t rounds = 0;; rounds++) {
+                    const uint32_t bid = (epoch << 10) | tid;
+                    const uint32_t slot = epoch % 3u;
+                    if (pending) { atomicMin(&tag[sel], bid); any_pending[slot] = 1u; }
+                    // three flags in turn: this round's is read after the barrier; the next round's, last
+                    // read two rounds ago (before the previous barrier), is cleared now. The last round's may
+                    // still be being read by a slow thread and is left alone. Every round, the last one of a
+                    // chunk included, moves on to the next flag.
+                    if (tid == 0) any_pending[(slot + 2u) % 3u] = 0u;
+                    __syncthreads();
+                    const bool more = any_pending[slot] != 0u;
+                    epoch--;
+                    if (!more) break;
+                    if (pending && tag[sel] == bid) {      // one lane per element gets here
                         tile[sel] = tile[sel] + v;
-                        tag[sel] = 0xffffffffu;
                         pending = false;
                     }
-                    if (!__syncthreads_or(pending ? 1 : 0)) break;
+                    // A chunk of THREADS entries needs at most THREADS rounds unless winners keep missing their
+                    // tags; from there on a second barrier keeps the next round's bids behind the winners' reads,
+                    // and every round retires an entry of every element that still has one.
+                    if (rounds >= THREADS) __syncthreads();
                 }
             }
         }

@@ -209,3 +209,30 @@ def test_scatter_rows_with_a_larger_source_and_bad_values(gc):
     for r in range(4):
         want[r, idx[r].astype(int)] = 2.0
     assert_bits_equal(ok.toArray(), want, "fill after a reported error")
+
+
+@pytest.mark.parametrize("shape,ishape", [([4, 4096], [4, 6000]), ([2, 12000], [2, 9000]), ([1, 12000], [1, 3000]), ([3, 40000], [3, 20000])],
+                         ids=lambda v: "x".join(map(str, v)))
+def test_scatter_add_with_hot_elements(shape, ishape, gc):
+    """Index rows in which a few elements take most of the entries (and one row that names a single element):
+    the adds of one element happen one per round in index order, over hundreds of rounds per chunk, in the
+    256- and the 1024-thread form and in bands. Bit-exact against the serial order of the checker."""
+    rng = np.random.default_rng(shape[1])
+    x = rng.standard_normal(shape).astype(np.float32)
+    hot = rng.integers(0, shape[1], size=4)
+    idx = np.where(rng.random(ishape) < 0.7, hot[rng.integers(0, 4, size=ishape)], rng.integers(0, shape[1], size=ishape)).astype(np.float32)
+    idx[0, :] = float(hot[0]) if shape[0] > 1 else idx[0, :]
+    if shape[0] == 1:
+        idx[0, : ishape[1] // 2] = 7.0
+    src = (rng.standard_normal(ishape) * 100).astype(np.float32)          # large spread: the order of the adds shows in the last bits
+    for name in ("inplaceScatterAdd", "inplaceScatter"):
+        gt, ct = both(gc, shape, x)
+        gi, ci = both(gc, ishape, idx); gs, cs = both(gc, ishape, src)
+        getattr(gt, name)(1, gi, gs); getattr(ct, name)(1, ci, cs)
+        assert_bits_equal(gt.toArray(), ct.toArray(), name)
+    # the same list of hot rows through indexAdd on a vector (inner size 1: the same rounds, with a factor)
+    rows = idx[0]
+    add = src[0]
+    gt, ct = both(gc, [shape[1]], x[0]); gr, cr = both(gc, [ishape[1]], rows); ga, ca = both(gc, [ishape[1]], add)
+    gt.indexAdd(0, gr, ga, 0.3); ct.indexAdd(0, cr, ca, 0.3)
+    assert_bits_equal(gt.toArray(), ct.toArray(), "indexAdd on a vector")
