@@ -593,7 +593,7 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
         for (int d = 0; d < nb; d++) { pl.bsize[d] = bsize[d]; pl.bdiv[d] = make_div(bsize[d]); pl.b_in[d] = b_in[d]; pl.b_out[d] = b_out[d]; }
         rp.t = pl;
         const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
-        if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+        if (blocks > kMaxElements - 8) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);   // (the grid is rounded up to 8)
         rp.tiles = static_cast<uint32_t>(blocks);
         const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
         LaunchScope scope("permute_runs_kernel", vec ? "float4" : "float", n * 8);
