@@ -375,7 +375,33 @@ def _bytes_lay(d):
 
 
 
+# ---- the transcendental maps that cfg2 does not use ----------------------------------------------
+
+_UNARY_MAPS = ["tanh", "sigmoid", "sinh", "cosh", "sin", "cos", "tan", "asin", "acos", "atan"]
+
+
+def _in_maps(d):
+    g = SplitMix64(14)
+    return {"x": g.uniform([d["n"]], -1.0, 1.0), "p": g.uniform([d["n"]], 0.01, 2.0)}
+
+
+def _run_maps(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    p = ops.create(list(inp["p"].shape), False, inp["p"])
+    out = {name: getattr(x, name)() for name in _UNARY_MAPS}
+    out["pow1.5"] = p ** 1.5
+    return out
+
+
+def _bytes_maps(d):
+    return 8 * d["n"] * (len(_UNARY_MAPS) + 1)
+
+
 WORKLOADS: Dict[str, Workload] = {
+    "unary_maps": Workload("unary_maps", "tanh sigmoid sinh cosh sin cos tan asin acos atan of x[2^26] in U(-1,1) and p pow 1.5 "
+                                         "of p[2^26] in U(0.01,2), seed 14: one map per launch",
+                           {"n": 1 << 26}, _in_maps, _run_maps, _bytes_maps),
+
     "layout_shapes": Workload("layout_shapes", "permutes that keep an innermost run of 8, 3, 33 and 3277 floats ([64,512,256,8], "
                                                "[4096,5461,3], [2048,1024,33], [4096,5,3277]) and a range get x[:, 1:8190] of "
                                                "[8192,8192]; U(-1,1), seed 13",

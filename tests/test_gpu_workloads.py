@@ -266,3 +266,25 @@ def test_layout_shapes(scale, gc):
     for i, (shape, perm) in enumerate(shapes):
         assert_bits_equal(got[f"permuted{i}"].toArray(), np.transpose(inp[f"x{i}"], perm), f"permute {shape} {perm}")
     assert_bits_equal(got["box"].toArray(), inp["boxed"][:, 1:inp["boxed"].shape[1] - 2], "range get")
+
+
+@pytest.mark.parametrize("n", [70001, 1 << 26], ids=["small", "full"])
+def test_unary_maps(n, gc):
+    """The transcendental maps at the benchmark size: at most 2 ulp from the checker on a slice (or the whole
+    small tensor), and on the whole tensor from numpy's float64 routines rounded once, which agree with the
+    checker's libm to the last float64 bit or nearly so."""
+    wl = WORKLOADS["unary_maps"]
+    inp = wl.make_inputs({"n": n})
+    got = wl.run(gc, inp)
+    x, p = inp["x"], inp["p"]
+    sl = slice(0, n) if n < (1 << 20) else slice(54321, 54321 + (1 << 20))
+    f64 = {"tanh": np.tanh, "sinh": np.sinh, "cosh": np.cosh, "sin": np.sin, "cos": np.cos, "tan": np.tan,
+           "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan, "sigmoid": lambda v: 1.0 / (1.0 + np.exp(-v))}
+    for name, fn in f64.items():
+        res = got[name].toArray()
+        assert_ulp_close(res[sl], jo.unary(name, x[sl]), 2, name + " against the checker")
+        assert ulp_distance(res, fn(x.astype(np.float64)).astype(np.float32)).max() <= 2, name + " against float64"
+        gc.release(got[name])
+    res = got["pow1.5"].toArray()
+    assert_ulp_close(res[sl], jo.binary("pow", p[sl], np.float32(1.5)), 2, "pow against the checker")
+    assert ulp_distance(res, np.power(p.astype(np.float64), 1.5).astype(np.float32)).max() <= 2, "pow against float64"
