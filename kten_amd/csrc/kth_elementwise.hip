@@ -653,10 +653,16 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
     const float eps = state().epsilon;
     const bool rev = reverse != 0;
-    // pow with an exponent whose f64 result is exact needs no transcendental:
-    // pow(x, 2) is the exact product x*x (48 bits fit a double), pow(x, 1) is x.
+    // pow with an exponent whose f64 result is exact or one correctly rounded operation needs no
+    // transcendental: pow(x, 2) is the exact product x*x (48 bits fit a double), pow(x, 1) is x;
+    // 3, 4, -1, -2 and 0.5 likewise.
     if (op == KTH_POW && !rev && c == 2.0f)      launch_unary<OpSquare>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == 1.0f) launch_unary<OpIdentity>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == 3.0f)  launch_unary<OpPowCube>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == 4.0f)  launch_unary<OpPowFourth>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == -1.0f) launch_unary<OpPowInverse>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == 0.5f)  launch_unary<OpPowHalf>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW && !rev && c == -2.0f) launch_unary<OpPowInverseSquare>(pa, po, n32, 0.0f, 0.0f);
     else {
 #define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
         KTH_BINARY_DISPATCH(op, S)

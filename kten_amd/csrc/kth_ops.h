@@ -77,6 +77,21 @@ KTH_UNARY(OpTrunc,      truncf(x))                                      // :433 
 KTH_UNARY(OpRsqrt,      1.0f / sqrtf(x))                                // :435 two roundings, not a hardware rsq
 KTH_UNARY(OpSquare,     x * x)                                          // pow(x, 2f): the exact product is representable in f64
 KTH_UNARY(OpIdentity,   x)                                              // pow(x, 1f)
+// pow(x, c) for the exponents whose correctly rounded f64 result is one f64 operation away (Math.pow is
+// within one f64 ulp of it and rounds to the same float): x^3 = (x*x)*x and x^4 = (x*x)*(x*x) with x*x exact,
+// x^-1 = 1/x, x^-2 = 1/(x*x), x^0.5 = sqrt(x) except that pow(-0, 0.5) = +0 and pow(-inf, 0.5) = +inf.
+__device__ __forceinline__ float pow_cube(float x)   { const double d = static_cast<double>(x); return static_cast<float>((d * d) * d); }
+__device__ __forceinline__ float pow_fourth(float x) { const double d = static_cast<double>(x), q = d * d; return static_cast<float>(q * q); }
+__device__ __forceinline__ float pow_half(float x) {
+    if (x == 0.0f) return 0.0f;
+    if (x == -INFINITY) return INFINITY;
+    return static_cast<float>(sqrt(static_cast<double>(x)));
+}
+KTH_UNARY(OpPowCube,    pow_cube(x))
+KTH_UNARY(OpPowFourth,  pow_fourth(x))
+KTH_UNARY(OpPowInverse, static_cast<float>(1.0 / static_cast<double>(x)))
+KTH_UNARY(OpPowHalf,    pow_half(x))
+KTH_UNARY(OpPowInverseSquare, static_cast<float>(1.0 / (static_cast<double>(x) * static_cast<double>(x))))
 #undef KTH_UNARY
 
 // sigmoid = 1f / (1f + exp(-1f * x)) with exp rounded to float first. (:399)

@@ -54,12 +54,12 @@ def test_clamp(gc, samples):
 @pytest.mark.parametrize("op", ["plus", "minus", "times", "div", "pow", "lt", "lte", "gt", "gte", "eq", "neq"])
 def test_scalar_ops(op, gc, samples):
     x = samples[:50000]
-    for c in (2.0, -0.75, 1e-3, 0.0, 3.0, -0.5, 1.0):
+    for c in (2.0, -0.75, 1e-3, 0.0, 3.0, -0.5, 1.0, 4.0, -1.0, -2.0, 0.5):
         got = raw(gc, x)._scalar(op, c).toArray()
         want = jo.scalar(op, x, c)
         if op == "pow":
             assert_ulp_close(got, want, what=f"pow {c}")
-            if c in (0.0, 1.0, 2.0):
+            if c in (0.0, 1.0, 2.0, 3.0, 4.0, -1.0, -2.0, 0.5):     # exponents computed without the transcendental routine
                 assert_bits_equal(got, want, f"pow {c}")
         else:
             assert_bits_equal(got, want, f"{op} {c}")
@@ -248,3 +248,11 @@ def test_gc_scope_keeps_referenced_tensors(hip):
         drop.getSingleValue([0])
     keep.release()
     assert not keep.referenced()
+
+
+@pytest.mark.parametrize("c", [3.0, 4.0, -1.0, -2.0, 0.5])
+def test_pow_with_exact_exponents_over_the_float_space(c, gc):
+    """Every 509th bit pattern (all exponents, signs and specials): the products, the quotient and the square root
+    that stand in for pow at these exponents give the checker's pow bit for bit, -0, infinities and NaN included."""
+    x = np.arange(0, 1 << 32, 509, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    assert_bits_equal(raw(gc, x)._scalar("pow", c).toArray(), jo.scalar("pow", x, c), f"pow {c}")
