@@ -239,13 +239,27 @@ __device__ __forceinline__ double atan_unit(double a, const double* tab) {
     return tab[static_cast<int>(id)] + fma(t * z, p, t);
 }
 
+// atan(num / den) for 0 <= num <= den, den in [1, 1e300], without forming the quotient: with u = num / den the
+// same t is (num - c den) / (den + num c), so the division by den and the one inside atan_unit become one.
+// c only has to be near u: the hardware's reciprocal estimate picks it.
+__device__ __forceinline__ double atan_ratio(double num, double den, const double* tab) {
+    const double id = rint(num * __builtin_amdgcn_rcp(den) * 64.0);
+    const double c = id * 0.015625;
+    const double t = fma(-c, den, num) * newton_rcp_any(fma(num, c, den));
+    const double z = t * t;
+    double p = fma(z, 1.0 / 9.0, -1.0 / 7.0);
+    p = fma(z, p, 1.0 / 5.0);
+    p = fma(z, p, -1.0 / 3.0);
+    return tab[static_cast<int>(id)] + fma(t * z, p, t);
+}
+
 constexpr double kPio2Hi = 0x1.921fb54442d18p+0, kPio2Lo = 0x1.1a62633145c07p-54;
 
 // atan of a >= 0 (finite or inf).
 __device__ __forceinline__ double atan_positive(double a, const double* tab) {
     if (a <= 1.0) return atan_unit(a, tab);
-    const double inv = a > 1.0e300 ? 0.0 : newton_rcp_any(a);
-    return (kPio2Hi - atan_unit(inv, tab)) + kPio2Lo;
+    const double small = a > 1.0e300 ? 0.0 : atan_ratio(1.0, a, tab);
+    return (kPio2Hi - small) + kPio2Lo;
 }
 
 __device__ __forceinline__ float table_atan(float x, const double* tab) {
@@ -254,22 +268,35 @@ __device__ __forceinline__ float table_atan(float x, const double* tab) {
     return res;
 }
 
+// 1 / sqrt(w) for w in [2^-30, 2]: the hardware estimate and two Newton steps on the residual 1 - w y^2.
+__device__ __forceinline__ double newton_rsqrt_unit(double w) {
+    double y = __builtin_amdgcn_rsq(w);
+    double e = fma(-w * y, y, 1.0);
+    y = fma(y * e, 0.5, y);
+    e = fma(-w * y, y, 1.0);
+    return fma(y * e, 0.5, y);
+}
+
 // asin a = 2 atan(a / (1 + sqrt((1 - a)(1 + a)))) on [0, 1]; NaN outside [-1, 1] (Math.asin).
 __device__ __forceinline__ float table_asin(float x, const double* tab) {
     const double a = fabs(static_cast<double>(x));
     if (!(a <= 1.0)) return __uint_as_float(0x7fc00000u);
-    const double w = sqrt((1.0 - a) * (1.0 + a));
-    const double u = a * newton_rcp_any(1.0 + w);
-    return copysignf(static_cast<float>(2.0 * atan_unit(u, tab)), x);
+    const double w = (1.0 - a) * (1.0 + a);
+    const double root = w > 0.0 ? w * newton_rsqrt_unit(w) : 0.0;       // sqrt(w)
+    return copysignf(static_cast<float>(2.0 * atan_ratio(a, 1.0 + root, tab)), x);
 }
 
 // acos x = 2 atan(sqrt((1 - x) / (1 + x))) on (-1, 1], pi at -1; NaN outside [-1, 1] (Math.acos).
+// acos |x| = 2 atan(sqrt((1 - |x|) / (1 + |x|))), whose argument stays in [0, 1]; acos x = pi - acos |x| below zero.
 __device__ __forceinline__ float table_acos(float x, const double* tab) {
     const double d = static_cast<double>(x);
-    if (!(fabs(d) <= 1.0)) return __uint_as_float(0x7fc00000u);
-    if (d == -1.0) return static_cast<float>(2.0 * kPio2Hi);
-    const double ratio = (1.0 - d) * newton_rcp_any(1.0 + d);
-    return static_cast<float>(2.0 * atan_positive(sqrt(ratio), tab));
+    const double a = fabs(d);
+    if (!(a <= 1.0)) return __uint_as_float(0x7fc00000u);
+    // sqrt((1 - a) / (1 + a)) = (1 - a) / sqrt((1 - a)(1 + a)); both factors are exact for a float a >= 2^-29
+    const double w = (1.0 - a) * (1.0 + a);
+    const double root = w > 0.0 ? (1.0 - a) * newton_rsqrt_unit(w) : 0.0;
+    const double r = 2.0 * atan_unit(root, tab);
+    return static_cast<float>(d < 0.0 ? (2.0 * kPio2Hi - r) + 2.0 * kPio2Lo : r);
 }
 
 }  // namespace kth
