@@ -144,13 +144,14 @@ struct OpTanT { static constexpr const char* name = "OpTan"; static __device__ _
 // pow(tensor | Float): the common operands (finite non-zero base, finite exponent) go through
 // the exp / log tables, read from global memory (3 KiB, cache resident); zeros, infinities
 // and NaNs take jpow's spelled-out Java rules over the library routine.
+__device__ __forceinline__ float pow_with_tables(float a, float b, const LogEntry* log_tab, const double* exp_tab) {
+    const bool common = (a != 0.0f) && (fabsf(a) < INFINITY) && (fabsf(b) < INFINITY) && (b != 0.0f);
+    if (common) return table_pow_finite(a, b, log_tab, exp_tab);
+    return jpow(a, b);
+}
 struct OpPowT {
     static constexpr const char* name = "OpPow";
-    static __device__ __forceinline__ float apply(float a, float b, float) {
-        const bool common = (a != 0.0f) && (fabsf(a) < INFINITY) && (fabsf(b) < INFINITY) && (b != 0.0f);
-        if (common) return table_pow_finite(a, b, g_log_table, g_exp_table);
-        return jpow(a, b);
-    }
+    static __device__ __forceinline__ float apply(float a, float b, float) { return pow_with_tables(a, b, g_log_table, g_exp_table); }
 };
 
 // Unary map whose op reads a small f64 table through LDS. The data loads of the tile are
@@ -183,6 +184,46 @@ __global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
         uint32_t i = (n4 << 2) + threadIdx.x;
         out[i] = Op::apply(a[i], tab);
+    }
+}
+
+// out[i] = REV ? pow(c, a[i]) : pow(a[i], c) with both tables (3 KiB) in LDS: the lookups of 64 lanes go to
+// 64 different entries, which as loads from global memory cost more than the arithmetic.
+template <bool REV>
+__global__ __launch_bounds__(kBlock) void pow_scalar_lds_kernel(const float* a, float* out, uint32_t n, float c) {
+    constexpr int kLogDoubles = 2 * kLogTableEntries;
+    __shared__ double tab[kLogDoubles + kExpTableEntries];
+    const uint32_t n4 = n >> 2;
+    const uint32_t base = blockIdx.x * (kBlock * kLdsUnroll) + threadIdx.x;
+    float4 v[kLdsUnroll];
+#pragma unroll
+    for (int k = 0; k < kLdsUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) v[k] = ld4(a, i);
+    }
+    for (int i = threadIdx.x; i < kLogDoubles + kExpTableEntries; i += kBlock)
+        tab[i] = i < kLogDoubles ? reinterpret_cast<const double*>(g_log_table)[i] : g_exp_table[i - kLogDoubles];
+    __syncthreads();
+    const LogEntry* log_tab = reinterpret_cast<const LogEntry*>(tab);
+    const double* exp_tab = tab + kLogDoubles;
+#pragma unroll
+    for (int k = 0; k < kLdsUnroll; k++) {
+        uint32_t i = base + k * kBlock;
+        if (i < n4) {
+            float4 r;
+            if (REV) {
+                r.x = pow_with_tables(c, v[k].x, log_tab, exp_tab); r.y = pow_with_tables(c, v[k].y, log_tab, exp_tab);
+                r.z = pow_with_tables(c, v[k].z, log_tab, exp_tab); r.w = pow_with_tables(c, v[k].w, log_tab, exp_tab);
+            } else {
+                r.x = pow_with_tables(v[k].x, c, log_tab, exp_tab); r.y = pow_with_tables(v[k].y, c, log_tab, exp_tab);
+                r.z = pow_with_tables(v[k].z, c, log_tab, exp_tab); r.w = pow_with_tables(v[k].w, c, log_tab, exp_tab);
+            }
+            st4(out, i, r);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
+        uint32_t i = (n4 << 2) + threadIdx.x;
+        out[i] = REV ? pow_with_tables(c, a[i], log_tab, exp_tab) : pow_with_tables(a[i], c, log_tab, exp_tab);
     }
 }
 
@@ -514,6 +555,15 @@ void launch_scalar(bool rev, const float* a, float* out, uint32_t n, float c, fl
     else     hipLaunchKernelGGL((scalar_kernel<Op, false>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
 }
 
+void launch_pow_scalar(bool rev, const float* a, float* out, uint32_t n, float c) {
+    LaunchScope scope(rev ? "pow_scalar_lds_kernel_rev" : "pow_scalar_lds_kernel", "OpPow", static_cast<uint64_t>(n) * 8);
+    const uint64_t tile = static_cast<uint64_t>(kBlock) * kLdsUnroll;
+    const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + tile - 1) / tile);
+    const dim3 grid(blocks == 0 ? 1 : blocks);
+    if (rev) hipLaunchKernelGGL((pow_scalar_lds_kernel<true>), grid, dim3(kBlock), 0, state().stream, a, out, n, c);
+    else     hipLaunchKernelGGL((pow_scalar_lds_kernel<false>), grid, dim3(kBlock), 0, state().stream, a, out, n, c);
+}
+
 template <class Op>
 void launch_binary_same(const float* a, const float* b, float* out, uint32_t n, float eps) {
     LaunchScope scope("binary_same_kernel", Op::name, static_cast<uint64_t>(n) * 12);
@@ -663,6 +713,7 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     else if (op == KTH_POW && !rev && c == -1.0f) launch_unary<OpPowInverse>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == 0.5f)  launch_unary<OpPowHalf>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == -2.0f) launch_unary<OpPowInverseSquare>(pa, po, n32, 0.0f, 0.0f);
+    else if (op == KTH_POW) launch_pow_scalar(rev, pa, po, n32, c);
     else {
 #define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
         KTH_BINARY_DISPATCH(op, S)

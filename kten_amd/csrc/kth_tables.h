@@ -221,7 +221,8 @@ __device__ __forceinline__ float table_tan(float x) {
     double s, c; int k;
     sincos_reduced(d, s, c, k);
     // cos r >= 0.7 on the reduced range; sin r of an odd quadrant is at least 1e-9 for a float argument
-    return static_cast<float>((k & 1) ? -c * newton_rcp_any(s) : s * newton_rcp_any(c));
+    const bool odd = (k & 1) != 0;                               // one reciprocal for either quadrant
+    return static_cast<float>((odd ? -c : s) * newton_rcp_any(odd ? s : c));
 }
 
 // ---------------------------------------------------------------- atan / asin / acos
