@@ -85,7 +85,7 @@ __device__ __forceinline__ float pow_fourth(float x) { const double d = static_c
 __device__ __forceinline__ float pow_half(float x) {
     if (x == 0.0f) return 0.0f;
     if (x == -INFINITY) return INFINITY;
-    return static_cast<float>(sqrt(static_cast<double>(x)));
+    return sqrtf(x);                                            // (the f64 square root rounds to the same float)
 }
 KTH_UNARY(OpPowCube,    pow_cube(x))
 KTH_UNARY(OpPowFourth,  pow_fourth(x))
