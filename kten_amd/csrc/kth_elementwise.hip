@@ -187,43 +187,42 @@ __global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float
     }
 }
 
-// out[i] = REV ? pow(c, a[i]) : pow(a[i], c) with both tables (3 KiB) in LDS: the lookups of 64 lanes go to
-// 64 different entries, which as loads from global memory cost more than the arithmetic.
-template <bool REV>
-__global__ __launch_bounds__(kBlock) void pow_scalar_lds_kernel(const float* a, float* out, uint32_t n, float c) {
+// pow with both tables (3 KiB) in LDS: the lookups of 64 lanes go to 64 different entries, which as loads from
+// global memory cost more than the arithmetic. MODE 0: out[i] = pow(a[i], c); 1: pow(c, a[i]); 2: pow(a[i], b[i]).
+// out may alias a or b.
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const float* b, float* out, uint32_t n, float c) {
     constexpr int kLogDoubles = 2 * kLogTableEntries;
     __shared__ double tab[kLogDoubles + kExpTableEntries];
     const uint32_t n4 = n >> 2;
     const uint32_t base = blockIdx.x * (kBlock * kLdsUnroll) + threadIdx.x;
-    float4 v[kLdsUnroll];
+    float4 v[kLdsUnroll], w[kLdsUnroll];
 #pragma unroll
     for (int k = 0; k < kLdsUnroll; k++) {
         uint32_t i = base + k * kBlock;
-        if (i < n4) v[k] = ld4(a, i);
+        if (i < n4) { v[k] = ld4(a, i); if (MODE == 2) w[k] = ld4(b, i); }
     }
     for (int i = threadIdx.x; i < kLogDoubles + kExpTableEntries; i += kBlock)
         tab[i] = i < kLogDoubles ? reinterpret_cast<const double*>(g_log_table)[i] : g_exp_table[i - kLogDoubles];
     __syncthreads();
     const LogEntry* log_tab = reinterpret_cast<const LogEntry*>(tab);
     const double* exp_tab = tab + kLogDoubles;
+    auto one = [&](float x, float y) {
+        return MODE == 1 ? pow_with_tables(c, x, log_tab, exp_tab) : pow_with_tables(x, MODE == 2 ? y : c, log_tab, exp_tab);
+    };
 #pragma unroll
     for (int k = 0; k < kLdsUnroll; k++) {
         uint32_t i = base + k * kBlock;
         if (i < n4) {
             float4 r;
-            if (REV) {
-                r.x = pow_with_tables(c, v[k].x, log_tab, exp_tab); r.y = pow_with_tables(c, v[k].y, log_tab, exp_tab);
-                r.z = pow_with_tables(c, v[k].z, log_tab, exp_tab); r.w = pow_with_tables(c, v[k].w, log_tab, exp_tab);
-            } else {
-                r.x = pow_with_tables(v[k].x, c, log_tab, exp_tab); r.y = pow_with_tables(v[k].y, c, log_tab, exp_tab);
-                r.z = pow_with_tables(v[k].z, c, log_tab, exp_tab); r.w = pow_with_tables(v[k].w, c, log_tab, exp_tab);
-            }
+            r.x = one(v[k].x, MODE == 2 ? w[k].x : 0.0f); r.y = one(v[k].y, MODE == 2 ? w[k].y : 0.0f);
+            r.z = one(v[k].z, MODE == 2 ? w[k].z : 0.0f); r.w = one(v[k].w, MODE == 2 ? w[k].w : 0.0f);
             st4(out, i, r);
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
         uint32_t i = (n4 << 2) + threadIdx.x;
-        out[i] = REV ? pow_with_tables(c, a[i], log_tab, exp_tab) : pow_with_tables(a[i], c, log_tab, exp_tab);
+        out[i] = one(a[i], MODE == 2 ? b[i] : 0.0f);
     }
 }
 
@@ -555,13 +554,16 @@ void launch_scalar(bool rev, const float* a, float* out, uint32_t n, float c, fl
     else     hipLaunchKernelGGL((scalar_kernel<Op, false>), dim3(blocks_for(n >> 2)), dim3(kBlock), 0, state().stream, a, out, n, c, eps);
 }
 
-void launch_pow_scalar(bool rev, const float* a, float* out, uint32_t n, float c) {
-    LaunchScope scope(rev ? "pow_scalar_lds_kernel_rev" : "pow_scalar_lds_kernel", "OpPow", static_cast<uint64_t>(n) * 8);
+// mode 0: a ^ c, 1: c ^ a, 2: a ^ b (see pow_lds_kernel)
+void launch_pow(int mode, const float* a, const float* b, float* out, uint32_t n, float c) {
+    LaunchScope scope(mode == 0 ? "pow_lds_kernel_scalar" : mode == 1 ? "pow_lds_kernel_scalar_rev" : "pow_lds_kernel", "OpPow",
+                      static_cast<uint64_t>(n) * (mode == 2 ? 12 : 8));
     const uint64_t tile = static_cast<uint64_t>(kBlock) * kLdsUnroll;
     const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + tile - 1) / tile);
     const dim3 grid(blocks == 0 ? 1 : blocks);
-    if (rev) hipLaunchKernelGGL((pow_scalar_lds_kernel<true>), grid, dim3(kBlock), 0, state().stream, a, out, n, c);
-    else     hipLaunchKernelGGL((pow_scalar_lds_kernel<false>), grid, dim3(kBlock), 0, state().stream, a, out, n, c);
+    if (mode == 0)      hipLaunchKernelGGL((pow_lds_kernel<0>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+    else if (mode == 1) hipLaunchKernelGGL((pow_lds_kernel<1>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+    else                hipLaunchKernelGGL((pow_lds_kernel<2>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
 }
 
 template <class Op>
@@ -713,7 +715,7 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     else if (op == KTH_POW && !rev && c == -1.0f) launch_unary<OpPowInverse>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == 0.5f)  launch_unary<OpPowHalf>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == -2.0f) launch_unary<OpPowInverseSquare>(pa, po, n32, 0.0f, 0.0f);
-    else if (op == KTH_POW) launch_pow_scalar(rev, pa, po, n32, c);
+    else if (op == KTH_POW) launch_pow(rev ? 1 : 0, pa, nullptr, po, n32, c);
     else {
 #define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
         KTH_BINARY_DISPATCH(op, S)
@@ -737,9 +739,12 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
     if (n == 0) return KTH_OK;
     float* pa = sa->ptr; const float* pb = sb->ptr; uint32_t n32 = static_cast<uint32_t>(n);
     const float eps = state().epsilon;
+    if (op == KTH_POW) launch_pow(2, pa, pb, pa, n32, 0.0f);
+    else {
 #define B(OP) launch_binary_same<OP>(pa, pb, pa, n32, eps)
-    KTH_BINARY_DISPATCH(op, B)
+        KTH_BINARY_DISPATCH(op, B)
 #undef B
+    }
     KTH_LAUNCH_CHECK("binary_inplace");
     return KTH_OK;
 }
@@ -776,7 +781,9 @@ int kth_binary(int op,
     const float* pa = sa->ptr; const float* pb = sb->ptr; float* po = so->ptr;
     const uint32_t n32 = static_cast<uint32_t>(on);
     const float eps = state().epsilon;
-    if (all_same) {
+    if (all_same && op == KTH_POW) {
+        launch_pow(2, pa, pb, po, n32, 0.0f);
+    } else if (all_same) {
 #define B(OP) launch_binary_same<OP>(pa, pb, po, n32, eps)
         KTH_BINARY_DISPATCH(op, B)
 #undef B
