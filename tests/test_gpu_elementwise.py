@@ -256,3 +256,15 @@ def test_pow_with_exact_exponents_over_the_float_space(c, gc):
     that stand in for pow at these exponents give the checker's pow bit for bit, -0, infinities and NaN included."""
     x = np.arange(0, 1 << 32, 509, dtype=np.uint64).astype(np.uint32).view(np.float32)
     assert_bits_equal(raw(gc, x)._scalar("pow", c).toArray(), jo.scalar("pow", x, c), f"pow {c}")
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 1023, 1027, 262147, 3000001])
+def test_contains_nan_at_every_kind_of_position(n, gc):
+    """A single NaN in the float4 body, in the tail of n mod 4 elements, at either end; infinities are not NaN."""
+    x = np.random.default_rng(n).standard_normal(n).astype(np.float32)
+    x[n // 3] = np.inf
+    assert not raw(gc, x).containsNan()
+    for pos in sorted({0, n // 2, max(0, n - 4), max(0, n - 3), max(0, n - 2), n - 1}):
+        y = x.copy()
+        y[pos] = np.nan
+        assert raw(gc, y).containsNan(), f"NaN at {pos} of {n}"
