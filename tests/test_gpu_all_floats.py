@@ -2,8 +2,8 @@
 
 By default every 509th bit pattern of the 2^32 (8.4 M inputs per op, every exponent and
 sign, all specials) is checked. With KTEN_ALL_FLOATS=1 all 2^32 patterns are checked,
-64 Mi at a time (about a minute of CPU time per op for the checker): run by hand, results
-recorded in the design notes.
+64 Mi at a time (about a minute of CPU time per op for the checker): run by hand after a
+change to one of these routines.
 Bars: exact ops bit-exact; f64-libm-then-round ops at most 2 ulp (NaN matches NaN)."""
 import os
 from concurrent.futures import ThreadPoolExecutor
