@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from kten_amd.shape_functions import ALL
+from oracle import jvm_oracle as jo
 
 pytestmark = pytest.mark.gpu
 
@@ -82,3 +83,101 @@ def test_flat_tensor_of_exactly_int_max_elements(gc):
     assert x.containsNan()
     with pytest.raises((ValueError, MemoryError)):
         gc.createRaw([2, 2 ** 30])                                       # 2^31 elements: one past the limit
+
+
+def test_three_dimensional_tensor_near_the_limit(gc):
+    """x[i, j, k] = r[i] + s[j] + c[k] on [2047, 1024, 1024] (2 146 435 072 elements): the kernels that the
+    two-dimensional case does not reach -- reductions over a middle axis in their streamed, tiled and few-rows
+    forms, a permute that keeps an innermost run, gather and scatter-add of rows inside LDS, indexSelect, the
+    sorted indexAdd and the fused batch-norm -- with offsets at the top of the 32-bit range. Values are multiples
+    of 1/8, so every expected value is exact in float32 or float64."""
+    A, B, C = 2047, 1024, 1024
+    rng = np.random.default_rng(2)
+    eighths = lambda n: (rng.integers(-256, 256, n) / 8.0).astype(np.float32)
+    r, s, c = eighths(A), eighths(B), eighths(C)
+    rs = gc.createRaw([A, 1, 1], r).plus(gc.createRaw([B, 1], s))
+    x = rs.plus(gc.createRaw([C], c))
+    assert x.shape == [A, B, C]
+    gc.release(rs)
+    pos = [(0, 0, 0), (A - 1, B - 1, C - 1), (A - 1, 0, C - 1), (1023, 512, 7)]
+    pos += [(int(rng.integers(0, A)), int(rng.integers(0, B)), int(rng.integers(0, C))) for _ in range(30)]
+    val = lambda i, j, k: np.float32(np.float32(r[i] + s[j]) + c[k])
+    for i, j, k in pos:
+        assert x.getSingleValue([i, j, k]) == val(i, j, k)
+    r64, s64, c64 = r.astype(np.float64), s.astype(np.float64), c.astype(np.float64)
+
+    # a middle axis streamed by a workgroup per slab segment: [A, B * 4, 256] over axis 1
+    got = x.view([A, B * 4, 256]).sum(1).toArray().astype(np.float64)
+    want = 4 * B * r64[:, None] + 4 * s64.sum() + B * c64.reshape(4, 256).sum(0)[None, :]
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    # small slabs through LDS tiles: [A * B, 64, 16] over axis 1
+    got = x.view([A * B, 64, 16]).sum(1).toArray().astype(np.float64).reshape(A, B, 16)
+    want = 64 * (r64[:, None, None] + s64[None, :, None]) + c64.reshape(64, 16).sum(0)[None, None, :]
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    # an axis of two over wide columns: [A * B / 8, 2, 4096]; the maximum of x[.., j, :] and x[.., j + 1, :] for even j,
+    # seen as rows of four (i, j) pairs
+    got = x.view([A * B // 8, 2, 4096]).max(1).toArray().reshape(A, B // 8, 4, C)
+    for i, j, k in pos:
+        g, q = divmod(j, 8)                       # q 0..3 pairs with q + 4
+        if q < 4:
+            assert got[i, g, q, k] == max(val(i, j, k), val(i, j + 4, k))
+    del got
+
+    # a permute that keeps the innermost run of 8 floats: [A, B, 128, 8] -> [A, 128, B, 8]
+    p = x.view([A, B, 128, 8]).permute([0, 2, 1, 3])
+    assert p.shape == [A, 128, B, 8]
+    for i, j, k in pos:
+        assert p.getSingleValue([i, k // 8, j, k % 8]) == val(i, j, k)
+    gc.release(p)
+
+    # gather and scatter-add along the innermost axis with rows of 128 indices (the row lives in LDS)
+    cols = rng.integers(0, C, 128)
+    zeros = gc.createRawFill([A, B, 1], 0.0)
+    index = zeros.plus(gc.createRaw([128], cols.astype(np.float32)))
+    assert index.shape == [A, B, 128]
+    g = x.gather(2, index)
+    for i, j, k in pos:
+        m = k % 128
+        assert g.getSingleValue([i, j, m]) == val(i, j, int(cols[m]))
+    gc.release(g)
+    ones = gc.createRawFill([A, B, 128], 1.0)
+    x.inplaceScatterAdd(2, index, ones)
+    hits = np.bincount(cols, minlength=C).astype(np.float32)
+    for i, j, k in pos:
+        assert x.getSingleValue([i, j, k]) == np.float32(val(i, j, k) + hits[k])      # small integers added to eighths: exact
+    minus = gc.createRawFill([A, B, 128], -1.0)
+    x.inplaceScatterAdd(2, index, minus)                                               # and taken off again
+    for i, j, k in pos:
+        assert x.getSingleValue([i, j, k]) == val(i, j, k)
+    gc.release(index, ones, minus, zeros)
+
+    # indexSelect and the sorted indexAdd along axis 0, the last rows of the tensor among them
+    rows = np.concatenate([[A - 1, 0, A - 1], rng.integers(0, A, 61)]).astype(np.float32)
+    sel = x.indexSelect(0, gc.createRaw([64], rows))
+    assert sel.shape == [64, B, C]
+    for m in (0, 1, 2, 40, 63):
+        for _, j, k in pos[:8]:
+            assert sel.getSingleValue([m, j, k]) == val(int(rows[m]), j, k)
+    x.indexAdd(0, gc.createRaw([64], rows), sel, -1.0)          # x[row] -= x[row], once per occurrence of the row
+    times = np.bincount(rows.astype(np.int64), minlength=A)
+    for i, j, k in pos:
+        v = val(i, j, k)
+        want = v
+        for _ in range(int(times[i])):
+            want = np.float32(want + np.float32(v * np.float32(-1.0)))
+        assert x.getSingleValue([i, j, k]) == want
+    gc.release(sel)
+
+    # the fused batch-norm over axis 1: statistics of 2 M elements per channel at offsets up to 2^31
+    y = gc.createRaw([A, 1, 1], r).plus(gc.createRaw([B, 1], s)).plus(gc.createRaw([C], c))          # x again, untouched
+    op = gc.batchNorm(1, 0.1, 1e-3, True)
+    out, mean, std = op.calculateOutput(y, gc.createRawFill([B], 0.0), gc.createRawFill([B], 1.0), None, None)
+    mean64 = s64 + r64.mean() + c64.mean()
+    var64 = r64.var() + c64.var()                                  # r and c vary independently over a channel's elements
+    assert np.abs(mean.toArray() - mean64).max() <= 1e-5 * np.abs(mean64).max() + 1e-6
+    assert np.abs(std.toArray() - 1.0 / np.sqrt(var64 + 1e-3)).max() <= 1e-5 / np.sqrt(var64 + 1e-3)
+    dm, ds = mean.toArray(), std.toArray()
+    chan = np.array([j for _, j, _ in pos])
+    want = jo.batch_norm_apply(np.array([val(i, j, k) for i, j, k in pos], np.float32), 0, dm[chan], ds[chan])
+    for (i, j, k), w in zip(pos, want):
+        assert out.getSingleValue([i, j, k]) == w
