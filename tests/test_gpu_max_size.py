@@ -181,3 +181,23 @@ def test_three_dimensional_tensor_near_the_limit(gc):
     want = jo.batch_norm_apply(np.array([val(i, j, k) for i, j, k in pos], np.float32), 0, dm[chan], ds[chan])
     for (i, j, k), w in zip(pos, want):
         assert out.getSingleValue([i, j, k]) == w
+
+    # gather and scatter along axis 0 with 256 index rows: the scatter goes through the transposed copies
+    # (target, index and source permuted to axis-innermost layout, scattered as rows, permuted back)
+    perm = rng.permutation(A)[:256]
+    perm[0], perm[1] = A - 1, 0
+    q = eighths(256)
+    plane = gc.createRawFill([B, C], 0.0)
+    index0 = gc.createRaw([256, 1, 1], perm.astype(np.float32)).plus(plane)
+    src0 = gc.createRaw([256, 1, 1], q).plus(plane)
+    assert index0.shape == [256, B, C]
+    g0 = y.gather(0, index0)
+    for m in (0, 1, 2, 100, 255):
+        for _, j, k in pos[:8]:
+            assert g0.getSingleValue([m, j, k]) == val(int(perm[m]), j, k)
+    gc.release(g0)
+    y.inplaceScatter(0, index0, src0)
+    row_of = {int(p): m for m, p in enumerate(perm)}
+    for i, j, k in pos + [(A - 1, 5, 9), (0, B - 1, C - 1)]:
+        want = q[row_of[i]] if i in row_of else val(i, j, k)
+        assert y.getSingleValue([i, j, k]) == want
