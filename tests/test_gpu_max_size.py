@@ -93,6 +93,7 @@ def test_three_dimensional_tensor_near_the_limit(gc):
     of 1/8, so every expected value is exact in float32 or float64."""
     A, B, C = 2047, 1024, 1024
     rng = np.random.default_rng(2)
+    gc.profileBegin()                             # the names of the kernels launched are checked at the end
     eighths = lambda n: (rng.integers(-256, 256, n) / 8.0).astype(np.float32)
     r, s, c = eighths(A), eighths(B), eighths(C)
     rs = gc.createRaw([A, 1, 1], r).plus(gc.createRaw([B, 1], s))
@@ -182,8 +183,7 @@ def test_three_dimensional_tensor_near_the_limit(gc):
     for (i, j, k), w in zip(pos, want):
         assert out.getSingleValue([i, j, k]) == w
 
-    # gather and scatter along axis 0 with 256 index rows: the scatter goes through the transposed copies
-    # (target, index and source permuted to axis-innermost layout, scattered as rows, permuted back)
+    # gather and scatter along axis 0 with 256 index rows (a million positions walk them side by side)
     perm = rng.permutation(A)[:256]
     perm[0], perm[1] = A - 1, 0
     q = eighths(256)
@@ -201,3 +201,35 @@ def test_three_dimensional_tensor_near_the_limit(gc):
     for i, j, k in pos + [(A - 1, 5, 9), (0, B - 1, C - 1)]:
         want = q[row_of[i]] if i in row_of else val(i, j, k)
         assert y.getSingleValue([i, j, k]) == want
+
+    launched = " ".join(gc.profileEnd().keys())
+    for kernel in ("reduce_stream_kernel", "reduce_short_slabs_kernel", "reduce_few_kernel", "permute_runs_kernel",
+                   "gather_rows_lds_kernel", "scatter_rows_lds_kernel<add>", "scatter_kernel<set>", "index_select_kernel",
+                   "index_add_sorted_kernel", "bn_stats", "bn_apply"):
+        assert kernel in launched, f"{kernel} was not reached: {launched}"
+
+
+def test_scatter_along_a_long_axis_near_the_limit(gc):
+    """inplaceScatter along axis 0 of [1 048 575, 2047] with an index of the same shape: target, index and source
+    are permuted to axis-innermost layout (rows of a million elements, scattered in bands through LDS) and the
+    target is permuted back; every copy holds 2 146 433 025 elements."""
+    R, W = 1048575, 2047
+    rng = np.random.default_rng(3)
+    perm = rng.permutation(R)
+    q = (rng.integers(-1024, 1024, R) / 8.0).astype(np.float32)
+    zeros = gc.createRawFill([W], 0.0)
+    index = gc.createRaw([R, 1], perm.astype(np.float32)).plus(zeros)
+    src = gc.createRaw([R, 1], q).plus(gc.createRaw([W], np.arange(W, dtype=np.float32)))      # src[i, j] = q[i] + j, exact
+    x = gc.createRawFill([R, W], -5.0)
+    gc.profileBegin()
+    x.inplaceScatter(0, index, src)
+    launched = " ".join(gc.profileEnd().keys())
+    assert "scatter_rows_lds_kernel<set>" in launched and "permute_tile_kernel" in launched, launched
+    where = np.empty(R, np.int64); where[perm] = np.arange(R)          # x[perm[i], j] = src[i, j]
+    rows = [0, R - 1, int(perm[0]), int(perm[-1])] + [int(v) for v in rng.integers(0, R, 30)]
+    for row in rows:
+        for j in (0, 1, W // 2, W - 1):
+            assert x.getSingleValue([row, j]) == np.float32(q[where[row]] + np.float32(j))
+    # the index survives the call untouched
+    for i in (0, R - 1, 12345):
+        assert index.getSingleValue([i, W - 1]) == float(perm[i])
