@@ -233,3 +233,62 @@ def test_scatter_along_a_long_axis_near_the_limit(gc):
     # the index survives the call untouched
     for i in (0, R - 1, 12345):
         assert index.getSingleValue([i, W - 1]) == float(perm[i])
+
+
+def test_odd_shaped_tensor_near_the_limit(gc):
+    """x[i, j] = r[i] + c[j] on [46339, 46337] (2 147 210 243 elements, rows that start off 16-byte boundaries):
+    the forms the kernels take when nothing is a multiple of four -- element gathers in the broadcast, rows read
+    from dword addresses in the reductions, scalar columns, ragged tile edges in the transpose, the mixed range
+    moves, concat."""
+    R, W = 46339, 46337
+    rng = np.random.default_rng(4)
+    r = (rng.integers(-512, 512, R) / 8.0).astype(np.float32)
+    c = (rng.integers(-512, 512, W) / 8.0).astype(np.float32)
+    gc.profileBegin()
+    gcol = gc.createRaw([W], c)
+    x = gc.createRaw([R, 1], r).plus(gcol)
+    assert x.shape == [R, W]
+    pos = [(0, 0), (R - 1, W - 1), (R - 1, 0), (0, W - 1), (R - 2, W - 3)]
+    pos += [(int(rng.integers(0, R)), int(rng.integers(0, W))) for _ in range(30)]
+    val = lambda i, j: np.float32(r[i] + c[j])
+    for i, j in pos:
+        assert x.getSingleValue([i, j]) == val(i, j)
+    y = x.plus(gcol)                                                     # full-size operand and a row vector
+    for i, j in pos:
+        assert y.getSingleValue([i, j]) == np.float32(val(i, j) + c[j])
+    gc.release(y)
+    r64, c64 = r.astype(np.float64), c.astype(np.float64)
+    got = x.sum(1).toArray().astype(np.float64)
+    want = W * r64 + c64.sum()
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    got = x.sum(0).toArray().astype(np.float64)
+    want = r64.sum() + R * c64
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    arg = x.argMax(1).toArray()
+    assert arg[0] == np.argmax(c) and arg[-1] == np.argmax(c) and np.all(c[arg.astype(np.int64)] == c.max())
+    arg = x.argMin(0).toArray()
+    assert arg[0] == np.argmin(r) and arg[-1] == np.argmin(r)
+
+    t = x.transpose(0, 1)
+    for i, j in pos:
+        assert t.getSingleValue([j, i]) == val(i, j)
+    gc.release(t)
+    box = x.get([(1, R - 2), (3, W - 2)])                                # rows of W - 4 floats cut out of rows of W
+    assert box.shape == [R - 2, W - 4]
+    for i, j in pos:
+        if 1 <= i <= R - 2 and 3 <= j <= W - 2:
+            assert box.getSingleValue([i - 1, j - 3]) == val(i, j)
+    assert box.getSingleValue([R - 3, W - 5]) == val(R - 2, W - 2)
+    gc.release(box)
+    wide = gc.concat(1, [x, gc.createRaw([R, 3], np.tile(np.array([1.0, 2.0, 3.0], np.float32), (R, 1)))])
+    assert wide.shape == [R, W + 3]
+    for i, j in pos:
+        assert wide.getSingleValue([i, j]) == val(i, j)
+    assert wide.getSingleValue([R - 1, W + 2]) == 3.0 and wide.getSingleValue([0, W]) == 1.0
+    gc.release(wide)
+    x.set([(5, R - 1), (1, W - 1)], 9.0)
+    for i, j in pos:
+        assert x.getSingleValue([i, j]) == (9.0 if i >= 5 and j >= 1 else val(i, j))
+    launched = " ".join(gc.profileEnd().keys())
+    for kernel in ("binary_bcast_mixed_kernel", "reduce_rows_kernel", "reduce_cols_kernel", "permute_tile_kernel", "float4 dense side"):
+        assert kernel in launched, f"{kernel} was not reached: {launched}"
