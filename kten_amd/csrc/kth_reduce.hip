@@ -232,13 +232,14 @@ __device__ __forceinline__ void stage_short_tile(const float* __restrict__ base,
     for (uint32_t k = 0; k < kShortLoads; k++) {
         const uint32_t e = (k * kBlock + threadIdx.x) * 4;
         const float vals[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        // one division for the first of the four, the others step along the row and over its end
+        const uint32_t r = (__umulhi(e, pl.axis_div.mul) + e) >> pl.axis_div.shift;
+        uint32_t col = e - r * pl.axis, at = r * pl.stride + col;
 #pragma unroll
         for (uint32_t j = 0; j < 4; j++) {
-            const uint32_t ee = e + j;
-            if (ee < floats) {
-                const uint32_t r = (__umulhi(ee, pl.axis_div.mul) + ee) >> pl.axis_div.shift;
-                tile[r * pl.stride + (ee - r * pl.axis)] = vals[j];
-            }
+            if (e + j < floats) tile[at] = vals[j];
+            at++;
+            if (++col == pl.axis) { col = 0; at += pl.stride - pl.axis; }
         }
     }
 }
