@@ -401,32 +401,70 @@ __global__ __launch_bounds__(kBlock) void permute_slabs_kernel(const float* __re
     }
     const uint32_t slabs = min(pl.group, pl.batch0 - first);
     const uint32_t floats = slabs * pl.slab, lds_slab = pl.y_len * pl.pitch;
-    constexpr uint32_t kLoads = kSlabTile / kBlock;
-    float v[kLoads];
+    // The span moves as 16-byte units at dword addresses on both sides. A unit's first element is placed by two
+    // divisions, the other three step from it: along x and over the ends of rows and slabs on the way in (the LDS
+    // position just grows: a slab's rows follow each other at the row pitch, and so do the slabs), along y and over
+    // the ends of columns and slabs on the way out.
+    constexpr uint32_t kUnits = kSlabTile / 4 / kBlock;
+    const float* src = in + in_off;
+    float* dst = out + out_off;
+    v4f v[kUnits];
 #pragma unroll
-    for (uint32_t k = 0; k < kLoads; k++) {
-        const uint32_t e = k * kBlock + threadIdx.x;
-        if (e < floats) v[k] = __builtin_nontemporal_load(in + in_off + e);
+    for (uint32_t k = 0; k < kUnits; k++) {
+        const uint32_t e = (k * kBlock + threadIdx.x) * 4u;
+        if (e + 4 <= floats) {
+            const v4f_unaligned t4 = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(src + e));
+            v[k] = v4f{t4.x, t4.y, t4.z, t4.w};
+        } else if (e < floats) {
+            v[k].x = src[e];
+            v[k].y = e + 1 < floats ? src[e + 1] : 0.0f;
+            v[k].z = e + 2 < floats ? src[e + 2] : 0.0f;
+            v[k].w = 0.0f;
+        }
     }
 #pragma unroll
-    for (uint32_t k = 0; k < kLoads; k++) {
-        const uint32_t e = k * kBlock + threadIdx.x;
+    for (uint32_t k = 0; k < kUnits; k++) {
+        const uint32_t e = (k * kBlock + threadIdx.x) * 4u;
         if (e < floats) {                                     // input order inside a slab: (y, x), x fastest
             const uint32_t g = (__umulhi(e, pl.slab_div.mul) + e) >> pl.slab_div.shift;
             const uint32_t r = e - g * pl.slab;
             const uint32_t y = (__umulhi(r, pl.x_div.mul) + r) >> pl.x_div.shift;
-            tile[g * lds_slab + y * pl.pitch + (r - y * pl.x_len)] = v[k];
+            uint32_t x = r - y * pl.x_len;
+            uint32_t at = g * lds_slab + y * pl.pitch + x;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++) {
+                if (e + j < floats) tile[at] = v[k][j];
+                at++;
+                if (++x == pl.x_len) { x = 0; at += pl.pitch - pl.x_len; }
+            }
         }
     }
     __syncthreads();
 #pragma unroll
-    for (uint32_t k = 0; k < kLoads; k++) {
-        const uint32_t e = k * kBlock + threadIdx.x;
+    for (uint32_t k = 0; k < kUnits; k++) {
+        const uint32_t e = (k * kBlock + threadIdx.x) * 4u;
         if (e < floats) {                                     // output order inside a slab: (x, y), y fastest
             const uint32_t g = (__umulhi(e, pl.slab_div.mul) + e) >> pl.slab_div.shift;
             const uint32_t r = e - g * pl.slab;
-            const uint32_t x = (__umulhi(r, pl.y_div.mul) + r) >> pl.y_div.shift;
-            out[out_off + e] = tile[g * lds_slab + (r - x * pl.y_len) * pl.pitch + x];
+            uint32_t x = (__umulhi(r, pl.y_div.mul) + r) >> pl.y_div.shift;
+            uint32_t y = r - x * pl.y_len;
+            uint32_t column = g * lds_slab + x;               // LDS position of (y = 0, x) of this slab
+            float w[4];
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++) {
+                w[j] = e + j < floats ? tile[column + y * pl.pitch] : 0.0f;
+                if (++y == pl.y_len) {
+                    y = 0; column++;
+                    if (++x == pl.x_len) { x = 0; column += lds_slab - pl.x_len; }
+                }
+            }
+            if (e + 4 <= floats) {
+                *reinterpret_cast<v4f_unaligned*>(dst + e) = v4f_unaligned{w[0], w[1], w[2], w[3]};
+            } else {
+                dst[e] = w[0];
+                if (e + 1 < floats) dst[e + 1] = w[1];
+                if (e + 2 < floats) dst[e + 2] = w[2];
+            }
         }
     }
 }
