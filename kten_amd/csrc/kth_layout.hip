@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kBlock) void move_kernel(const float* __restrict__ 
 // The same moves when the strided side cannot take float4s (odd run lengths or offsets): the
 // dense side still moves as float4s, 16-byte aligned from the start of its store. Where its four
 // floats are neighbours on the strided side as well they move there as one 16-byte access at a
-// dword address, otherwise one by one. `n` counts floats; MODE 0 and 1 only.
+// dword address, otherwise one by one. `n` counts floats; for MODE 2 the dense side is the fill value.
 typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
 // Offsets on the strided side of dense floats i+1 .. i+3, given float i's (`first`, at place r0 of
@@ -107,7 +107,7 @@ constexpr int kMixedUnroll = 1;              // units of four floats per thread 
 
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                           uint32_t n, MovePlan pl) {
+                                                           uint32_t n, float value, MovePlan pl) {
     const uint32_t base = blockIdx.x * (kBlock * kMixedUnroll) + threadIdx.x;
     uint32_t first[kMixedUnroll], place[kMixedUnroll];
     bool run4[kMixedUnroll];                  // the four floats lie next to each other on the strided side too
@@ -134,6 +134,8 @@ __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restr
                 v[k].z = i + 2 < n ? src[at[2]] : 0.0f;
                 v[k].w = i + 3 < n ? src[at[3]] : 0.0f;
             }
+        } else if (MODE == 2) {
+            v[k] = v4f{value, value, value, value};
         } else if (i + 3 < n) {
             v[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + i));
         } else {
@@ -520,12 +522,12 @@ void launch_move(const char* family, const float* src, float* dst, uint64_t coun
     if (vec) { pl.size[0] /= 4; pl.stride[0] = 4; units = count / 4; }
     for (int d = 0; d < dims.n; d++) pl.div[d] = make_div(pl.size[d]);
     const uint32_t per_block = kBlock * kMoveUnroll;
-    if constexpr (MODE != 2) if (!vec && count >= 1024) {
+    if (!vec && count >= 1024) {
         const uint32_t per_block4 = kBlock * kMixedUnroll;
         const uint32_t blocks4 = static_cast<uint32_t>(((count + 3) / 4 + per_block4 - 1) / per_block4);
         LaunchScope scope(family, "float4 dense side", bytes);
         hipLaunchKernelGGL((move_mixed_kernel<MODE>), dim3(blocks4), dim3(kBlock), 0, state().stream, src, dst,
-                           static_cast<uint32_t>(count), pl);
+                           static_cast<uint32_t>(count), value, pl);
         return;
     }
     const uint32_t blocks = static_cast<uint32_t>((units + per_block - 1) / per_block);
