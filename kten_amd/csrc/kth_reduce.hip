@@ -310,7 +310,7 @@ __global__ __launch_bounds__(kBlock) void reduce_short_slabs_kernel(const float*
 
 // Workgroup = 64 x WY threads over a tile of TW * 64 * VEC columns: lane x of wave y owns VEC
 // adjacent columns of sub-tile y % TW (so TW waves side by side read one contiguous span of a
-// row), and takes rows y / TW, y / TW + WY / TW, ... of the segment.
+// row), and takes rows y / TW, y / TW + WY / TW, ... of the segment. In use: VEC = 4, TW = 1.
 template <class R, int VEC, int WY, int TW>
 __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                                  typename R::Acc* __restrict__ partial, Geom g, uint32_t tiles) {
@@ -323,8 +323,11 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
     const uint32_t o = rest / g.segments;
     const uint32_t tx = threadIdx.x, ty = threadIdx.y;
     const uint32_t sub = ty % TW, lane = ty / TW;
-    const uint32_t col = ((tile * TW + sub) * kWave + tx) * VEC;
-    const bool active = col < g.inner;          // inner % VEC == 0, so a float4 is all in or all out
+    const uint32_t own = ((tile * TW + sub) * kWave + tx) * VEC;       // first column this thread answers for
+    const bool active = own < g.inner;
+    // float4 columns of an inner size that is not a multiple of 4: the last group starts at inner - 4 and
+    // overlaps its neighbour (the loads are 16 bytes from a dword address anyway); it emits only its own columns
+    const uint32_t col = (VEC == 4 && active && own + 4 > g.inner) ? g.inner - 4 : own;
     Acc acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; v++) acc[v] = R::init();
@@ -338,7 +341,7 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
             if (VEC == 4) {
                 float4 v[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) if (r + k * WR < end) v[k] = ld4_stream(base + static_cast<size_t>(r + k * WR) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * WR < end) v[k] = ld4_stream_unaligned(base + static_cast<size_t>(r + k * WR) * g.inner);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
                     const uint32_t rr = r + k * WR;
@@ -365,7 +368,7 @@ __global__ __launch_bounds__(kWave * WY) void reduce_cols_kernel(const float* __
         for (int v = 0; v < VEC; v++) {
             Acc t = lds[sub][tx * VEC + v];
             for (uint32_t w = 1; w < WR; w++) t = R::merge(t, lds[w * TW + sub][tx * VEC + v]);
-            emit<R>(g, o, s, col + v, t, out, partial);
+            if (col + v >= own) emit<R>(g, o, s, col + v, t, out, partial);
         }
     }
 }
@@ -715,10 +718,10 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         blocks = base_blocks * g.segments;
     } else if (inner >= 64 && !stream_fits) {
         kind = COLS;
-        VEC = (inner % 4 == 0) ? 4 : 1;
-        // Scalar columns: four waves side by side make a row's span 1 KiB instead of 256 B
-        // (measured 51 us against 60 on [4,16384,1001]); with float4 columns the narrow tile is faster.
-        TW = (VEC == 1 && inner >= 256) ? 4 : 1;
+        VEC = 4;                                       // (inner >= 64; an inner size off a multiple of 4 overlaps its last group)
+        // (scalar columns with four waves side by side measured 51 us on [4,16384,1001], the overlapping
+        // float4 groups 46.6 us; with float4 columns the tile one wave wide is the faster one)
+        TW = 1;
         tiles = ceil_div(inner, kWave * VEC * TW);
         const uint64_t base_blocks = static_cast<uint64_t>(tiles) * outer;
         // Few column tiles and a long axis: 16 waves per workgroup fold 16 rows at a time
@@ -768,13 +771,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
 #undef ROWS_LAUNCH
         } else if (kind == COLS) {
 #define COLS_LAUNCH(VV, YY, TT) hipLaunchKernelGGL((reduce_cols_kernel<R, VV, YY, TT>), grid, dim3(kWave, YY), 0, stream, in, out, partial, g, tiles)
-            if (TW == 4) {
-                if (VEC == 4 && WY == 16) COLS_LAUNCH(4, 16, 4); else if (VEC == 4) COLS_LAUNCH(4, 4, 4);
-                else if (WY == 16) COLS_LAUNCH(1, 16, 4); else COLS_LAUNCH(1, 4, 4);
-            } else {
-                if (VEC == 4 && WY == 16) COLS_LAUNCH(4, 16, 1); else if (VEC == 4) COLS_LAUNCH(4, 4, 1);
-                else if (WY == 16) COLS_LAUNCH(1, 16, 1); else COLS_LAUNCH(1, 4, 1);
-            }
+            if (WY == 16) COLS_LAUNCH(4, 16, 1); else COLS_LAUNCH(4, 4, 1);
 #undef COLS_LAUNCH
         } else if (kind == STREAM) {
             const FastDiv cols_div = make_div(inner / VEC);
