@@ -28,9 +28,9 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the plain copy kernel unary_kernel<OpIdentity>
-# of 262 144 KiB (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.000). Source: profiles/*.md.
+# of 262 144 KiB (FETCH_SIZE x 1.9999, WRITE_SIZE x 1.000). Source: profiles/*.md.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg5", "binary_same_kernel<OpTimes>"): int((262155 * (262144 / 131083) + 262144) * 1024),
+    ("cfg5", "binary_same_kernel<OpTimes>"): int((262155 * (262144 / 131077) + 262144) * 1024),
 }
 METRIC = "achieved HBM GB/s (% of MI355X peak) for broadcast binary ops and axis sum"
 
