@@ -466,8 +466,8 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
 // ---------------------------------------------------------------- few rows: axis of 2 ... 7 over wide columns
 
 // With so short an axis a column gives a thread only a handful of loads, so a thread takes four
-// columns (float4-wide with VEC = 4), 256 * VEC apart: 8 loads in flight (two axis positions of
-// its four columns), each a contiguous span across the workgroup. Axis positions in ascending order.
+// columns (float4-wide with VEC = 4; in use: VEC = 1), 256 * VEC apart: 8 loads in flight (two axis positions
+// of its four columns), each a contiguous span across the workgroup. Axis positions in ascending order.
 template <class R, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_few_kernel(const float* __restrict__ in, float* __restrict__ out, Geom g, uint32_t tiles) {
     using Acc = typename R::Acc;
@@ -686,17 +686,17 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     // 3.3-6.1) and for float4 columns below 512; from there on the column kernel's 1 KiB spans win.
     const bool stream_fits = slab >= kStreamMinSlab && (inner < 256 || (inner < 512 && inner % 4 == 0)) &&
                              outer <= 0x7fffffffu / 64;
-    if ((axis <= 7 || (inner % 4 != 0 && axis <= 16)) && inner >= 1024 && !stream_fits && n_out >= 65536) {
+    if (axis <= 7 && inner >= 1024 && !stream_fits && n_out >= 65536) {
         // (slabs of such an axis that fit a tile were taken above)
-        const int vec = inner % 4 == 0 ? 4 : 1;
-        const uint32_t tiles = ceil_div(inner, 4u * kBlock * vec);
+        // one column per lane and load, for any inner size: measured 7-9 % ahead of float4 columns here
+        // (66 against 72 us on [23,2,1456700]), whose 16 accumulators per thread cost more than the wider loads gain
+        const uint32_t tiles = ceil_div(inner, 4u * kBlock);
         const uint64_t few_blocks = static_cast<uint64_t>(tiles) * outer;
         if (few_blocks <= 0x7fffffffull) {
             hipError_t e;
             {
                 LaunchScope scope("reduce_few_kernel", R::name, (static_cast<uint64_t>(outer) * slab + n_out) * 4);
-                if (vec == 4) hipLaunchKernelGGL((reduce_few_kernel<R, 4>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
-                else          hipLaunchKernelGGL((reduce_few_kernel<R, 1>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
+                hipLaunchKernelGGL((reduce_few_kernel<R, 1>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
                 e = hipGetLastError();
             }
             if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
