@@ -408,7 +408,9 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __r
 // inner / VEC threads walk the rows `lanes` apart, so a load instruction of the workgroup covers
 // lanes * inner consecutive floats and every thread stays on its own column(s). The lanes'
 // partials meet in LDS and one thread per column merges them in lane order.
-// VEC = 4 requires inner % 4 == 0 (every row then starts 16-byte aligned).
+// VEC = 4: a thread owns four adjacent columns, loaded as 16 bytes from a dword address, for any inner size of
+// at least 4; when inner is not a multiple of 4 the last group starts at inner - 4 and overlaps its neighbour
+// (both fold the same rows, so the columns they share get the same value twice).
 template <class R, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                               typename R::Acc* __restrict__ partial, Geom g,
@@ -417,24 +419,25 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     __shared__ Acc fold[kBlock * VEC];
     const uint32_t s = blockIdx.x % g.segments;
     const uint32_t o = blockIdx.x / g.segments;
-    const uint32_t cols = g.inner / VEC;
+    const uint32_t cols = (g.inner + VEC - 1) / VEC;
     const uint32_t t = threadIdx.x;
     const uint32_t lane = (__umulhi(t, cols_div.mul) + t) >> cols_div.shift;
     const uint32_t c = t - lane * cols;
+    const uint32_t col = (VEC == 4 && c * 4 + 4 > g.inner) ? g.inner - 4 : c * VEC;      // first column of this thread
     const uint32_t begin = s * g.seg_len;
     const uint32_t end = min(begin + g.seg_len, g.axis);
     Acc acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; v++) acc[v] = R::init();
     if (lane < lanes) {
-        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + c * VEC;
+        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
         constexpr uint32_t kBatch = VEC == 4 ? 4 : 8;
         // every pass issues its (up to) kBatch loads before consuming any; the last pass is predicated
         for (uint32_t r = begin + lane; r < end; r += kBatch * lanes) {
             if (VEC == 4) {
                 float4 w[kBatch];
 #pragma unroll
-                for (uint32_t k = 0; k < kBatch; k++) if (r + k * lanes < end) w[k] = ld4_stream(base + static_cast<size_t>(r + k * lanes) * g.inner);
+                for (uint32_t k = 0; k < kBatch; k++) if (r + k * lanes < end) w[k] = ld4_stream_unaligned(base + static_cast<size_t>(r + k * lanes) * g.inner);
 #pragma unroll
                 for (uint32_t k = 0; k < kBatch; k++) {
                     const uint32_t rr = r + k * lanes;
@@ -452,9 +455,11 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
             }
         }
     }
-    // fold[lane][column]: thread t owns columns c * VEC .. c * VEC + VEC - 1 of lane t / cols
+    // fold[lane][column]: lanes * inner <= kBlock * VEC entries
+    if (lane < lanes) {
 #pragma unroll
-    for (int v = 0; v < VEC; v++) fold[t * VEC + v] = acc[v];
+        for (int v = 0; v < VEC; v++) fold[lane * g.inner + col + v] = acc[v];
+    }
     __syncthreads();
     for (uint32_t i = t; i < g.inner; i += kBlock) {
         Acc a = fold[i];
@@ -682,10 +687,9 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         return KTH_OK;
     }
 
-    // Measured against the column kernel: ahead for every inner size below 256 (5.0-6.5 TB/s against
-    // 3.3-6.1) and for float4 columns below 512; from there on the column kernel's 1 KiB spans win.
-    const bool stream_fits = slab >= kStreamMinSlab && (inner < 256 || (inner < 512 && inner % 4 == 0)) &&
-                             outer <= 0x7fffffffu / 64;
+    // Measured against the column kernel: ahead for every inner size below 512 (5.8-6.4 TB/s against
+    // 3.3-6.1); from there on the column kernel's 1 KiB spans win.
+    const bool stream_fits = slab >= kStreamMinSlab && inner < 512 && outer <= 0x7fffffffu / 64;
     if (axis <= 7 && inner >= 1024 && !stream_fits && n_out >= 65536) {
         // (slabs of such an axis that fit a tile were taken above)
         // one column per lane and load, for any inner size: measured 7-9 % ahead of float4 columns here
@@ -732,8 +736,8 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     } else if (stream_fits) {
         // A long axis over a small inner size: one workgroup streams a whole slab (or a segment of it).
         kind = STREAM;
-        VEC = (inner % 4 == 0) ? 4 : 1;
-        stream_lanes = kBlock / (inner / VEC);
+        VEC = inner >= 4 ? 4 : 1;
+        stream_lanes = kBlock / ((inner + VEC - 1) / VEC);
         plan_segments(&g, outer, target / 2, stream_lanes, stream_lanes * 8);
         blocks = static_cast<uint64_t>(outer) * g.segments;
     } else {
@@ -774,7 +778,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
             if (WY == 16) COLS_LAUNCH(4, 16, 1); else COLS_LAUNCH(4, 4, 1);
 #undef COLS_LAUNCH
         } else if (kind == STREAM) {
-            const FastDiv cols_div = make_div(inner / VEC);
+            const FastDiv cols_div = make_div((inner + VEC - 1) / VEC);
             if (VEC == 4) hipLaunchKernelGGL((reduce_stream_kernel<R, 4>), grid, dim3(kBlock), 0, stream, in, out, partial, g, stream_lanes, cols_div);
             else          hipLaunchKernelGGL((reduce_stream_kernel<R, 1>), grid, dim3(kBlock), 0, stream, in, out, partial, g, stream_lanes, cols_div);
         } else {
