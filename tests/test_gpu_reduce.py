@@ -41,6 +41,10 @@ GEOMETRIES = [
     # a slab (or a segment of it) streamed by one workgroup: scalar and float4 columns, with and without segments
     ([300, 700, 3], 1), ([2, 50000, 12], 1), ([2000, 64, 33], 1), ([1500, 100, 40], 1), ([5, 2049, 1, 63], 1),
     ([3, 40000, 2], 1), ([1, 100000, 7], 1),
+    # groups of four columns when the inner size is not a multiple of 4 (the last group overlaps its neighbour): streamed
+    # slabs with inner 5 ... 511, the column kernel from 513 on, one and several outer indices, with and without segments
+    ([3, 3000, 5], 1), ([2, 2500, 6], 1), ([4, 700, 7], 1), ([3, 900, 257], 1), ([1, 2000, 301], 1), ([2, 300, 479], 1), ([5000, 511], 0),
+    ([2, 600, 513], 1), ([3000, 1001], 0), ([1, 4100, 515], 1), ([40000, 65], 0), ([9, 70, 130], 1),
     # scalar columns in tiles four waves wide, with and without segments
     ([300, 1001], 0), ([3, 500, 257], 1), ([2, 5000, 259], 1), ([7, 300], 0),
     # streamed slabs with wide columns: one group of threads per row, float4 columns up to 511
