@@ -174,6 +174,25 @@ int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t 
 /* sum() / mean() (RAW:121-122; JVM:146-152) of n values into out[0]. op: KTH_SUM, KTH_MEAN. */
 int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
 
+/* kth_reduce_axis for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference.
+ * Same arguments, checks and results (bit for bit: the same kernels and the same plan) as
+ * kth_reduce_axis, but the partials of a two-pass reduction go to a fixed array of
+ * kth_reduce_scratch_bytes() = 4 MiB in the library's device code instead of a pool
+ * workspace, and the call creates nothing: no hipMalloc / hipFree, no pool traffic, no
+ * events (its launches are counted by kth_metrics but left out of a kth_profile recording).
+ * A shape whose plan needs more partial bytes than the array holds (outputs x axis segments
+ * x 8 bytes; only reductions whose outputs alone cannot fill the device are cut into
+ * segments) returns KTH_E_ARGUMENT before anything is launched; single-pass shapes of any
+ * size are accepted. Every call on a device shares that device's array, which keeps the last
+ * call's partials; nothing in it needs clearing because every partial is written before it is
+ * read. The library's mutex and its one in-order stream keep calls of one process apart;
+ * anything that made two such calls overlap on one GPU would race on the array. */
+int kth_reduce_axis_static(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner);
+
+/* Size of that array in bytes. */
+int kth_reduce_scratch_bytes(uint64_t* bytes);
+
 /* ------------------------------------------------------------------ indexed moves along an axis */
 
 /* gather (RAW:164; JVM:334-353). in and index have `dims` dims; out has index's shape:

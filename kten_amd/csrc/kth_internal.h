@@ -95,15 +95,21 @@ int permute_device(const char* what, const float* in, float* out, const int32_t*
 hipError_t sort_pairs_u32(void* temp, size_t* temp_bytes, const uint32_t* keys_in, uint32_t* keys_out,
                           const uint32_t* vals_in, uint32_t* vals_out, uint32_t n, int end_bit, hipStream_t stream);
 
+// Resolves the device address of the static scratch array of kth_reduce_axis_static for
+// `device`, which must be the current device (kth_reduce.hip). Called once from kth_init.
+hipError_t reduce_scratch_init(int device);
+
 // Computes the exp / log tables on the host (extended precision) and copies them into the
 // device symbols of the elementwise kernels. Called once from kth_init.
 hipError_t init_math_tables();
 
 // Brackets the launch of one kernel: counts it for kth_metrics and, while a profile is
-// being recorded, puts a HIP event before and after it on the library's stream.
+// being recorded, puts a HIP event before and after it on the library's stream (the events
+// are created on demand; may_profile = false leaves them out for callers that must not
+// create anything).
 class LaunchScope {
 public:
-    LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes);
+    LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes, bool may_profile = true);
     ~LaunchScope();
     LaunchScope(const LaunchScope&) = delete;
     LaunchScope& operator=(const LaunchScope&) = delete;

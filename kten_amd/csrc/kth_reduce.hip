@@ -585,6 +585,19 @@ __global__ __launch_bounds__(kWave * TY) void reduce_finalize_tile_kernel(const 
     if (ty == 0 && idx < n_out) out[idx] = R::finish(acc, g.axis);
 }
 
+// ---------------------------------------------------------------- static scratch
+
+// Partials of kth_reduce_axis_static, the entry point that allocates nothing: a fixed array in
+// the code object's global segment instead of a pool workspace. Every device the library runs on
+// holds its own copy at its own address until the process ends. Host code never uses the array's
+// name as an address: reduce_scratch_init resolves the device address once per device and the
+// kernels get that pointer as their `partial` argument.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kScratchDevices = 64;
+void* g_scratch_ptr[kScratchDevices] = {nullptr};
+
 // ---------------------------------------------------------------- host planning
 
 uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
@@ -608,10 +621,13 @@ void plan_segments(Geom* g, uint64_t base_blocks, uint64_t target, uint32_t quan
 // per output (6 TB/s against 1-4.5); below that the per-workgroup fold dominates.
 constexpr uint64_t kStreamMinSlab = 2048;
 
+// use_static: partials go to the static scratch array (no pool, no events, nothing allocated);
+// a plan whose partials do not fit is refused before anything is launched.
 template <class R>
-int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
+int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static) {
     using Acc = typename R::Acc;
     State& st = state();
+    const bool may_profile = !use_static;
     hipStream_t stream = st.stream;
     const uint64_t target = static_cast<uint64_t>(st.compute_units) * 8;
     Geom g{outer, axis, inner, 1, axis};
@@ -621,7 +637,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         const uint32_t n = static_cast<uint32_t>(n_out);
         hipError_t e;
         {
-            LaunchScope scope("reduce_unit_axis_kernel", R::name, n_out * 8);
+            LaunchScope scope("reduce_unit_axis_kernel", R::name, n_out * 8, may_profile);
             hipLaunchKernelGGL((reduce_unit_axis_kernel<R>), dim3(static_cast<uint32_t>(ceil_div((n >> 2) + 3, kBlock))), dim3(kBlock), 0, stream, in, out, n);
             e = hipGetLastError();
         }
@@ -639,7 +655,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         const dim3 grid(static_cast<uint32_t>(ceil_div(outer, rows)));
         hipError_t e;
         {
-            LaunchScope scope("reduce_short_rows_kernel", R::name, (static_cast<uint64_t>(outer) * axis + n_out) * 4);
+            LaunchScope scope("reduce_short_rows_kernel", R::name, (static_cast<uint64_t>(outer) * axis + n_out) * 4, may_profile);
 #define SHORT_LAUNCH(GG) hipLaunchKernelGGL((reduce_short_rows_kernel<R, GG>), grid, dim3(kBlock), 0, stream, in, out, pl)
             switch (rows >= kBlock ? 1 : kBlock / rows) {
             case 1: SHORT_LAUNCH(1); break;   case 2: SHORT_LAUNCH(2); break;   case 4: SHORT_LAUNCH(4); break;
@@ -679,7 +695,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         pl.axis_div = make_div(length); pl.inner_div = make_div(inner);
         hipError_t e;
         {
-            LaunchScope scope("reduce_short_slabs_kernel", R::name, (static_cast<uint64_t>(outer) * length + n_out) * 4);
+            LaunchScope scope("reduce_short_slabs_kernel", R::name, (static_cast<uint64_t>(outer) * length + n_out) * 4, may_profile);
             hipLaunchKernelGGL((reduce_short_slabs_kernel<R>), dim3(static_cast<uint32_t>(ceil_div(outer, rows))), dim3(kBlock), 0, stream, in, out, pl);
             e = hipGetLastError();
         }
@@ -699,7 +715,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         if (few_blocks <= 0x7fffffffull) {
             hipError_t e;
             {
-                LaunchScope scope("reduce_few_kernel", R::name, (static_cast<uint64_t>(outer) * slab + n_out) * 4);
+                LaunchScope scope("reduce_few_kernel", R::name, (static_cast<uint64_t>(outer) * slab + n_out) * 4, may_profile);
                 hipLaunchKernelGGL((reduce_few_kernel<R, 1>), dim3(static_cast<uint32_t>(few_blocks)), dim3(kBlock), 0, stream, in, out, g, tiles);
                 e = hipGetLastError();
             }
@@ -750,7 +766,14 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
 
     Acc* partial = nullptr;
     uint64_t cap = 0;
-    if (g.segments > 1) {
+    if (g.segments > 1 && use_static) {
+        const uint64_t need = n_out * g.segments * sizeof(Acc);
+        if (need > kStaticScratchBytes)
+            return fail(KTH_E_ARGUMENT, "kth_reduce_axis_static: [%u,%u,%u] needs %llu bytes of partials (%llu outputs x %u axis segments), "
+                        "the static scratch holds %llu; use kth_reduce_axis", outer, axis, inner, (unsigned long long)need,
+                        (unsigned long long)n_out, g.segments, (unsigned long long)kStaticScratchBytes);
+        partial = reinterpret_cast<Acc*>(g_scratch_ptr[st.device]);
+    } else if (g.segments > 1) {
         partial = reinterpret_cast<Acc*>(workspace_acquire(n_out * g.segments * sizeof(Acc), &cap));
         if (!partial) return fail(KTH_E_MEMORY, "kth_reduce: no workspace for %llu partials",
                                   (unsigned long long)(n_out * g.segments));
@@ -760,7 +783,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     hipError_t e;
     {
         LaunchScope scope(kind == ROWS ? "reduce_rows_kernel" : kind == COLS ? "reduce_cols_kernel" : kind == STREAM ? "reduce_stream_kernel" : "reduce_strided_kernel",
-                          R::name, bytes);
+                          R::name, bytes, may_profile);
         if (kind == ROWS) {
 #define ROWS_LAUNCH(GG, VV) hipLaunchKernelGGL((reduce_rows_kernel<R, GG, VV>), grid, dim3(kBlock), 0, stream, in, out, partial, g)
             if (VEC == 4) {
@@ -787,7 +810,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         e = hipGetLastError();
     }
     if (e == hipSuccess && g.segments > 1) {
-        LaunchScope scope("reduce_finalize_kernel", R::name, 0);
+        LaunchScope scope("reduce_finalize_kernel", R::name, 0, may_profile);
         if (n_out < 64)
             hipLaunchKernelGGL((reduce_finalize_wave_kernel<R>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
                                partial, out, g);
@@ -799,48 +822,82 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
                                partial, out, g);
         e = hipGetLastError();
     }
-    if (partial) workspace_release(reinterpret_cast<float*>(partial), cap);
+    if (partial && !use_static) workspace_release(reinterpret_cast<float*>(partial), cap);
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
     return KTH_OK;
 }
 
-int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
+int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static = false) {
     switch (op) {
-    case KTH_SUM:     return run_reduce<RedSum>(in, out, outer, axis, inner);
-    case KTH_MEAN:    return run_reduce<RedMean>(in, out, outer, axis, inner);
-    case KTH_MAX:     return run_reduce<RedMax>(in, out, outer, axis, inner);
-    case KTH_MIN:     return run_reduce<RedMin>(in, out, outer, axis, inner);
-    case KTH_ARG_MAX: return run_reduce<RedArgMax>(in, out, outer, axis, inner);
-    case KTH_ARG_MIN: return run_reduce<RedArgMin>(in, out, outer, axis, inner);
+    case KTH_SUM:     return run_reduce<RedSum>(in, out, outer, axis, inner, use_static);
+    case KTH_MEAN:    return run_reduce<RedMean>(in, out, outer, axis, inner, use_static);
+    case KTH_MAX:     return run_reduce<RedMax>(in, out, outer, axis, inner, use_static);
+    case KTH_MIN:     return run_reduce<RedMin>(in, out, outer, axis, inner, use_static);
+    case KTH_ARG_MAX: return run_reduce<RedArgMax>(in, out, outer, axis, inner, use_static);
+    case KTH_ARG_MIN: return run_reduce<RedArgMin>(in, out, outer, axis, inner, use_static);
     default:          return fail(KTH_E_ARGUMENT, "kth_reduce: op %d is not an aggregating operation", op);
     }
 }
 
+// The argument checks of both axis entry points, then the launch.
+int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
+    if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "%s: op %d is not an aggregating operation", who, op);
+    Store* si = lookup(in, who);
+    if (!si) return KTH_E_HANDLE;
+    Store* so = lookup(out, who);
+    if (!so) return KTH_E_HANDLE;
+    if (axis == 0) return fail(KTH_E_ARGUMENT, "%s: empty axis", who);
+    if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
+        outer * axis > kMaxElements || outer * axis * inner > kMaxElements)
+        return fail(KTH_E_ARGUMENT, "%s: more than 2^31-1 elements", who);
+    if ((op == KTH_ARG_MAX || op == KTH_ARG_MIN) && axis > (1ull << 24))
+        return fail(KTH_E_ARGUMENT, "%s: axis %llu too long for an index stored as float", who, (unsigned long long)axis);
+    if (outer * axis * inner > si->n_floats || outer * inner > so->n_floats)
+        return fail(KTH_E_ARGUMENT, "%s: [%llu,%llu,%llu] exceeds a store", who, (unsigned long long)outer,
+                    (unsigned long long)axis, (unsigned long long)inner);
+    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", who);
+    if (outer * inner == 0) return KTH_OK;
+    return dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
+                           static_cast<uint32_t>(inner), use_static);
+}
+
 }  // namespace
+
+namespace kth {
+
+// Called by kth_init with `device` current: resolves this device's copy of the scratch array.
+hipError_t reduce_scratch_init(int device) {
+    if (device < 0 || device >= kScratchDevices) return hipErrorInvalidDevice;
+    if (g_scratch_ptr[device]) return hipSuccess;
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = p;
+    return hipSuccess;
+}
+
+}  // namespace kth
 
 extern "C" {
 
 int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: op %d is not an aggregating operation", op);
-    Store* si = lookup(in, "kth_reduce_axis(in)");
-    if (!si) return KTH_E_HANDLE;
-    Store* so = lookup(out, "kth_reduce_axis(out)");
-    if (!so) return KTH_E_HANDLE;
-    if (axis == 0) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: empty axis");
-    if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
-        outer * axis > kMaxElements || outer * axis * inner > kMaxElements)
-        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: more than 2^31-1 elements");
-    if ((op == KTH_ARG_MAX || op == KTH_ARG_MIN) && axis > (1ull << 24))
-        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: axis %llu too long for an index stored as float", (unsigned long long)axis);
-    if (outer * axis * inner > si->n_floats || outer * inner > so->n_floats)
-        return fail(KTH_E_ARGUMENT, "kth_reduce_axis: [%llu,%llu,%llu] exceeds a store", (unsigned long long)outer,
-                    (unsigned long long)axis, (unsigned long long)inner);
-    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "kth_reduce_axis: output aliases the input");
-    if (outer * inner == 0) return KTH_OK;
-    return dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
-                           static_cast<uint32_t>(inner));
+    return reduce_axis_checked("kth_reduce_axis", false, op, in, out, outer, axis, inner);
+}
+
+int kth_reduce_axis_static(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (!g_scratch_ptr[state().device]) return fail(KTH_E_DEVICE, "kth_reduce_axis_static: the scratch array of device %d was not resolved", state().device);
+    return reduce_axis_checked("kth_reduce_axis_static", true, op, in, out, outer, axis, inner);
+}
+
+int kth_reduce_scratch_bytes(uint64_t* bytes) {
+    if (!bytes) return fail(KTH_E_ARGUMENT, "kth_reduce_scratch_bytes: null output");
+    *bytes = kStaticScratchBytes;
+    return KTH_OK;
 }
 
 int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out) {

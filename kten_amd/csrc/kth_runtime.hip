@@ -123,11 +123,11 @@ static hipEvent_t take_event() {
     return e;
 }
 
-LaunchScope::LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes) {
+LaunchScope::LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes, bool may_profile) {
     State& s = state();
     s.launches += 1;
     s.bytes_moved += algorithmic_bytes;
-    if (!s.profiling) return;
+    if (!s.profiling || !may_profile) return;
     LaunchRecord r{family, op, algorithmic_bytes, take_event(), take_event()};
     if (!r.begin || !r.end) return;
     (void)hipEventRecord(r.begin, s.stream);
@@ -173,6 +173,7 @@ int kth_init(int device) {
     KTH_HIP(hipEventCreate(&s.ev_begin));
     KTH_HIP(hipEventCreate(&s.ev_end));
     KTH_HIP(init_math_tables());
+    KTH_HIP(reduce_scratch_init(device));
     s.device = device;
     s.ready = true;
     g_epoch += 1;
