@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../include/kten_hip.h"
+#include "kth_fastdiv.h"
 
 namespace kth {
 
@@ -138,18 +139,5 @@ private:
     } while (0)
 
 constexpr uint64_t kMaxElements = 0x7fffffffull;   // store size is a Kotlin Int
-
-// Division by a launch-constant divisor d for numerators below 2^31:
-// q = (mulhi(n, mul) + n) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
-struct FastDiv { uint32_t mul, shift; };
-
-inline FastDiv make_div(uint32_t d) {
-    FastDiv f;
-    uint32_t shift = 0;
-    while ((1ull << shift) < d) shift++;
-    f.shift = shift;
-    f.mul = static_cast<uint32_t>((((1ull << shift) - d) << 32) / d + 1);
-    return f;
-}
 
 }  // namespace kth

@@ -31,6 +31,21 @@ def test_header_is_plain_c_too(tmp_path):
                     "-I", os.path.join(ROOT, "include"), str(src)], check=True)
 
 
+def test_fast_divider_on_the_host(tmp_path):
+    """make_div(0) (a dim of an empty tensor) must not divide by zero on the host; every other divisor
+    gives exact quotients. Built with the undefined-behaviour sanitizer, host code only."""
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = tmp_path / "fastdiv_test"
+    subprocess.run([gxx, "-std=c++17", "-O1", "-Wall", "-Wextra", "-Werror", "-fsanitize=undefined", "-fno-sanitize-recover=all",
+                    "-I", os.path.join(ROOT, "kten_amd", "csrc"), os.path.join(ROOT, "tests", "cpp", "fastdiv_test.cpp"),
+                    "-o", str(exe)], check=True)
+    done = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "fastdiv ok" in done.stdout
+
+
 @pytest.mark.gpu
 def test_cpp_host_mirror_known_answers():
     assert os.path.exists(BINARY), "tests/cpp/host_mirror_test is not built (python __graft_entry__.py build)"

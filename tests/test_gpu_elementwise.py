@@ -176,6 +176,27 @@ def test_shape_errors_are_raised_before_any_launch(gc):
     assert gc.getMetrics()["launches"] == launches
 
 
+def test_empty_tensors_give_empty_results_without_a_launch(gc):
+    """A dim of 0 (e.g. the result of indexSelect with no index) reaches the plan builders: the JVM returns empty
+    tensors there (JVMRawTensor.kt:75-87 over an empty FloatArray); nothing may be launched or divided by."""
+    a = gc.createRaw([0, 3]); b = gc.createRaw([0, 3]); c = raw(gc, np.ones([3])); d = raw(gc, np.ones([1, 3]))
+    mask = raw(gc, np.ones([3]))
+    launches = gc.getMetrics()["launches"]
+    for res in (a + b, a * c, c - a, a.pow(b), a.maskedFill(mask, 2.0), d.broadcastTo([0, 3]), c.broadcastTo([2, 0, 3]),
+                a + 1.0, a.exp(), a.clamp(0.0, 1.0), a.copy()):
+        assert res.shape[-1] == 3 and res.size == 0 and res.toArray().size == 0
+    a.plusAssign(b); a.timesAssign(2.0)
+    # straight through the ABI with numpy's rule for a dim of 1 against a dim of 0 as well
+    out = gc.createRaw([0, 3])
+    abi.check(gc.lib.kth_binary(abi.Op.DIV, a.storeReference, abi.shape_array([0, 3]), 2, d.storeReference, abi.shape_array([1, 3]), 2,
+                                out.storeReference, abi.shape_array([0, 3]), 2))
+    assert gc.getMetrics()["launches"] == launches
+    with pytest.raises(ValueError):
+        a + raw(gc, np.ones([2]))
+    with pytest.raises(ValueError):
+        a / d           # the common shape of [0, 3] and [1, 3] is the per-dim maximum [1, 3] (AbstractRawTensor.kt:170-192): no broadcast
+
+
 def test_abi_rejects_bad_arguments(hip):
     L = hip.lib
     sh = abi.shape_array([2, 3])
