@@ -5,6 +5,7 @@
 #include "kth_internal.h"
 #include "kth_ops.h"
 #include "kth_tables.h"
+#include "kth_fast.h"
 
 #include <cmath>
 #include <cstring>
@@ -71,75 +72,155 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const float* a, float* ou
 __device__ LogEntry g_log_table[kLogTableEntries];
 __device__ double   g_exp_table[kExpTableEntries];
 __device__ double   g_atan_table[kAtanTableEntries];
+__device__ double   g_sincos_table[2 * kSinCosTableEntries];
+__device__ double   g_asin_table[2 * kAsinTableEntries];
+
+// Copies `count` doubles of a device table into LDS, all threads of the workgroup taking part.
+__device__ __forceinline__ void stage_table(double* lds, const double* table, int count) {
+    for (int i = threadIdx.x; i < count; i += kBlock) lds[i] = table[i];
+}
 
 struct OpLogT {
     static constexpr const char* name = "OpLog";
     static constexpr int kTableDoubles = 2 * kLogTableEntries;
-    static __device__ __forceinline__ const double* table() { return reinterpret_cast<const double*>(g_log_table); }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, reinterpret_cast<const double*>(g_log_table), kTableDoubles); }
     static __device__ __forceinline__ float apply(float x, const double* lds) {
         return table_log(x, reinterpret_cast<const LogEntry*>(lds));
+    }
+    static __device__ __forceinline__ float4 apply4(float4 v, const double* lds) {
+        return make_float4(apply(v.x, lds), apply(v.y, lds), apply(v.z, lds), apply(v.w, lds));
     }
 };
 struct OpExpT {
     static constexpr const char* name = "OpExp";
     static constexpr int kTableDoubles = kExpTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
     static __device__ __forceinline__ float apply(float x, const double* lds) { return table_exp(x, lds); }
+    static __device__ __forceinline__ float4 apply4(float4 v, const double* lds) {
+        return make_float4(apply(v.x, lds), apply(v.y, lds), apply(v.z, lds), apply(v.w, lds));
+    }
 };
 // sigmoid = 1f / (1f + exp(-1f * x)), exp rounded to float first (JVMRawTensor.kt:399).
 struct OpSigmoidT {
     static constexpr const char* name = "OpSigmoid";
     static constexpr int kTableDoubles = kExpTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_exp_table; }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
     static __device__ __forceinline__ float apply(float x, const double* lds) {
         float m = -1.0f * x;
         float e = table_exp(m, lds);
         float d = 1.0f + e;
         return 1.0f / d;
     }
+    static __device__ __forceinline__ float4 apply4(float4 v, const double* lds) {
+        return make_float4(apply(v.x, lds), apply(v.y, lds), apply(v.z, lds), apply(v.w, lds));
+    }
 };
+
+// The maps below take the short evaluation of kth_fast.h and fall back to the long routine of
+// kth_tables.h for the lanes whose rounding the short value does not decide.
+__device__ __forceinline__ float with_sign_of(float magnitude_result, float x) {      // odd maps evaluated at |x|
+    return __uint_as_float(__float_as_uint(magnitude_result) ^ (__float_as_uint(x) & 0x80000000u));
+}
+
+// Four elements through a short routine, then one branch for the lanes of the wave whose rounding it left open:
+// the four evaluations are independent straight-line code, and the long routine is reached about once in
+// several hundred waves.
+#define KTH_SHORT_THEN_LONG(FAST, SIGNED, LONG_CALL)                                                     \
+    static __device__ __forceinline__ float apply(float x, const double* lds) {                          \
+        double y;                                                                                         \
+        const bool ok = FAST(x, lds, y);                                                                 \
+        float r = SIGNED ? with_sign_of(static_cast<float>(y), x) : static_cast<float>(y);               \
+        if (!(ok && rounds_safely(y))) r = LONG_CALL;                                                    \
+        return r;                                                                                         \
+    }                                                                                                     \
+    static __device__ __forceinline__ float4 apply4(float4 v, const double* lds) {                       \
+        const float xs[4] = {v.x, v.y, v.z, v.w};                                                        \
+        float rs[4];                                                                                      \
+        bool open[4];                                                                                     \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                                  \
+            const float x = xs[j];                                                                        \
+            double y;                                                                                     \
+            const bool ok = FAST(x, lds, y);                                                             \
+            rs[j] = SIGNED ? with_sign_of(static_cast<float>(y), x) : static_cast<float>(y);             \
+            open[j] = !(ok && rounds_safely(y));                                                         \
+        }                                                                                                 \
+        if (open[0] | open[1] | open[2] | open[3]) {                                                     \
+            _Pragma("unroll") for (int j = 0; j < 4; j++) {                                              \
+                const float x = xs[j];                                                                    \
+                if (open[j]) rs[j] = LONG_CALL;                                                          \
+            }                                                                                             \
+        }                                                                                                 \
+        return make_float4(rs[0], rs[1], rs[2], rs[3]);                                                  \
+    }
 
 struct OpTanhT {
     static constexpr const char* name = "OpTanh";
     static constexpr int kTableDoubles = kExpTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_exp_table; }
-    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_tanh(x, lds); }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_tanh, true, table_tanh(x, lds))
 };
 struct OpSinhT {
     static constexpr const char* name = "OpSinh";
     static constexpr int kTableDoubles = kExpTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_exp_table; }
-    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_sinh(x, lds); }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_sinh, true, table_sinh(x, lds))
 };
 struct OpCoshT {
     static constexpr const char* name = "OpCosh";
     static constexpr int kTableDoubles = kExpTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_exp_table; }
-    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_cosh(x, lds); }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_cosh, false, table_cosh(x, lds))
 };
 
+// atan keeps the long routine alone: with one reciprocal per lane it is already the cheaper one
+// (100 us per 268 MB map against 111 us for the short routine with its selects).
 struct OpAtanT {
     static constexpr const char* name = "OpAtan";
     static constexpr int kTableDoubles = kAtanTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_atan_table; }
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_atan_table, kTableDoubles); }
     static __device__ __forceinline__ float apply(float x, const double* lds) { return table_atan(x, lds); }
+    static __device__ __forceinline__ float4 apply4(float4 v, const double* lds) {
+        return make_float4(apply(v.x, lds), apply(v.y, lds), apply(v.z, lds), apply(v.w, lds));
+    }
 };
+// asin and acos: the {asin c, sqrt(1 - c^2)} table of the short routine first, then the atan table of the long one.
 struct OpAsinT {
     static constexpr const char* name = "OpAsin";
-    static constexpr int kTableDoubles = kAtanTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_atan_table; }
-    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_asin(x, lds); }
+    static constexpr int kTableDoubles = 2 * kAsinTableEntries + kAtanTableEntries;
+    static __device__ __forceinline__ void stage(double* lds) {
+        stage_table(lds, g_asin_table, 2 * kAsinTableEntries);
+        stage_table(lds + 2 * kAsinTableEntries, g_atan_table, kAtanTableEntries);
+    }
+    KTH_SHORT_THEN_LONG(fast_asin, true, table_asin(x, lds + 2 * kAsinTableEntries))
 };
 struct OpAcosT {
     static constexpr const char* name = "OpAcos";
-    static constexpr int kTableDoubles = kAtanTableEntries;
-    static __device__ __forceinline__ const double* table() { return g_atan_table; }
-    static __device__ __forceinline__ float apply(float x, const double* lds) { return table_acos(x, lds); }
+    static constexpr int kTableDoubles = 2 * kAsinTableEntries + kAtanTableEntries;
+    static __device__ __forceinline__ void stage(double* lds) {
+        stage_table(lds, g_asin_table, 2 * kAsinTableEntries);
+        stage_table(lds + 2 * kAsinTableEntries, g_atan_table, kAtanTableEntries);
+    }
+    KTH_SHORT_THEN_LONG(fast_acos, false, table_acos(x, lds + 2 * kAsinTableEntries))
 };
-// sin, cos, tan need no table: reduction constants and Taylor coefficients are immediates.
-struct OpSinT { static constexpr const char* name = "OpSin"; static __device__ __forceinline__ float apply(float x, float, float) { return table_sin(x); } };
-struct OpCosT { static constexpr const char* name = "OpCos"; static __device__ __forceinline__ float apply(float x, float, float) { return table_cos(x); } };
-struct OpTanT { static constexpr const char* name = "OpTan"; static __device__ __forceinline__ float apply(float x, float, float) { return table_tan(x); } };
+// sin, cos, tan: the short routine reads {sin, cos}(j pi / 32) through LDS; the long one needs no table.
+struct OpSinT {
+    static constexpr const char* name = "OpSin";
+    static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_sin, true, table_sin(x))
+};
+struct OpCosT {
+    static constexpr const char* name = "OpCos";
+    static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_cos, false, table_cos(x))
+};
+struct OpTanT {
+    static constexpr const char* name = "OpTan";
+    static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
+    static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
+    KTH_SHORT_THEN_LONG(fast_tan, true, table_tan(x))
+};
 
 // pow(tensor | Float): the common operands (finite non-zero base, finite exponent) go through
 // the exp / log tables, read from global memory (3 KiB, cache resident); zeros, infinities
@@ -169,17 +250,12 @@ __global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float
         uint32_t i = base + k * kBlock;
         if (i < n4) v[k] = ld4(a, i);
     }
-    for (int i = threadIdx.x; i < Op::kTableDoubles; i += kBlock) tab[i] = Op::table()[i];
+    Op::stage(tab);
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < kLdsUnroll; k++) {
         uint32_t i = base + k * kBlock;
-        if (i < n4) {
-            float4 r;
-            r.x = Op::apply(v[k].x, tab); r.y = Op::apply(v[k].y, tab);
-            r.z = Op::apply(v[k].z, tab); r.w = Op::apply(v[k].w, tab);
-            st4(out, i, r);
-        }
+        if (i < n4) st4(out, i, Op::apply4(v[k], tab));
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
         uint32_t i = (n4 << 2) + threadIdx.x;
@@ -661,8 +737,10 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
     case KTH_SINH: if (n32) launch_unary_lds<OpSinhT>(pa, po, n32); break;
     case KTH_COSH: if (n32) launch_unary_lds<OpCoshT>(pa, po, n32); break;
     case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
-    case KTH_SQRT: U(OpSqrt); break;         case KTH_SIN: U(OpSinT); break;
-    case KTH_COS: U(OpCosT); break;          case KTH_TAN: U(OpTanT); break;
+    case KTH_SQRT: U(OpSqrt); break;
+    case KTH_SIN: if (n32) launch_unary_lds<OpSinT>(pa, po, n32); break;
+    case KTH_COS: if (n32) launch_unary_lds<OpCosT>(pa, po, n32); break;
+    case KTH_TAN: if (n32) launch_unary_lds<OpTanT>(pa, po, n32); break;
     case KTH_ASIN: if (n32) launch_unary_lds<OpAsinT>(pa, po, n32); break;
     case KTH_ACOS: if (n32) launch_unary_lds<OpAcosT>(pa, po, n32); break;
     case KTH_ATAN: if (n32) launch_unary_lds<OpAtanT>(pa, po, n32); break;         case KTH_FLOOR: U(OpFloor); break;
@@ -914,9 +992,27 @@ hipError_t init_math_tables() {
         exp_tab[i] = static_cast<double>(exp2l(static_cast<long double>(i) / kExpTableEntries));
     double atan_tab[kAtanTableEntries];
     for (int i = 0; i < kAtanTableEntries; i++) atan_tab[i] = static_cast<double>(atanl(static_cast<long double>(i) / 64.0L));
+    // {sin, cos}(j pi / 32): exact 0 and +-1 at the multiples of pi / 2, which the long double routines miss by an ulp
+    double sincos_tab[2 * kSinCosTableEntries];
+    const long double pi = 3.14159265358979323846264338327950288419716939937510L;
+    for (int j = 0; j < kSinCosTableEntries; j++) {
+        sincos_tab[2 * j] = j % 32 == 0 ? 0.0 : static_cast<double>(sinl(pi * j / 32.0L));
+        sincos_tab[2 * j + 1] = j % 32 == 16 ? 0.0 : static_cast<double>(cosl(pi * j / 32.0L));
+    }
+    sincos_tab[1] = 1.0; sincos_tab[2 * 32 + 1] = -1.0; sincos_tab[2 * 16] = 1.0; sincos_tab[2 * 48] = -1.0;
+    double asin_tab[2 * kAsinTableEntries];
+    for (int j = 0; j < kAsinTableEntries; j++) {
+        const long double c = static_cast<long double>(j) / 64.0L;
+        asin_tab[2 * j] = static_cast<double>(asinl(c));
+        asin_tab[2 * j + 1] = static_cast<double>(sqrtl((1.0L - c) * (1.0L + c)));
+    }
     hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_log_table), log_tab, sizeof(log_tab));
     if (e != hipSuccess) return e;
     e = hipMemcpyToSymbol(HIP_SYMBOL(g_exp_table), exp_tab, sizeof(exp_tab));
+    if (e != hipSuccess) return e;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_sincos_table), sincos_tab, sizeof(sincos_tab));
+    if (e != hipSuccess) return e;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_asin_table), asin_tab, sizeof(asin_tab));
     if (e != hipSuccess) return e;
     return hipMemcpyToSymbol(HIP_SYMBOL(g_atan_table), atan_tab, sizeof(atan_tab));
 }
