@@ -6,7 +6,7 @@ as hand-written HIP kernels behind a C ABI (libkten_hip.so, include/kten_hip.h).
 PlatformProvider.defaultOps() once a HIP PlatformInitializer has registered itself).
 """
 from .abi import Op, LIB_PATH          # noqa: F401
-from .raw_tensor import AbstractRawTensor, AggregatingOperation   # noqa: F401
+from .host_mirror.raw_tensor import AbstractRawTensor, AggregatingOperation   # noqa: F401
 
 _platform = None
 

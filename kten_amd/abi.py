@@ -76,6 +76,9 @@ SIGNATURES = {
     "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
     "kth_timer_begin": (c_int, []),
     "kth_timer_end": (c_int, [POINTER(c_float)]),
+    "kth_timer_lap": (c_int, []),
+    "kth_timer_laps": (c_int, [POINTER(c_float), c_int, POINTER(c_int), POINTER(c_float)]),
+    "kth_measure_copy": (c_int, [c_uint64, c_int, POINTER(c_float), POINTER(c_float)]),
     "kth_profile_begin": (c_int, []),
     "kth_profile_end": (c_int, []),
     "kth_profile_count": (c_int, [POINTER(c_int)]),

@@ -62,6 +62,8 @@ struct State {
     bool       stage_used[kStageSlots] = {false};
     int        stage_next = 0;
 
+    std::vector<hipEvent_t> laps;           // kth_timer_lap events not yet read by kth_timer_laps
+
     bool profiling = false;
     std::vector<LaunchRecord> records;      // launches of the current / last profile
     std::vector<hipEvent_t>   event_pool;   // idle events, reused across profiles

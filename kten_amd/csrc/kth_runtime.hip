@@ -192,6 +192,7 @@ int kth_shutdown(void) {
     trim_pool();
     for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
     for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
+    for (hipEvent_t e : s.laps) (void)hipEventDestroy(e);
     for (int i = 0; i < State::kStageSlots; i++) {
         if (s.stage[i]) (void)hipHostFree(s.stage[i]);
         if (s.stage_done[i]) (void)hipEventDestroy(s.stage_done[i]);
@@ -456,6 +457,80 @@ int kth_timer_end(float* milliseconds) {
     KTH_HIP(hipEventElapsedTime(milliseconds, s.ev_begin, s.ev_end));
     s.timer_open = false;
     return KTH_OK;
+}
+
+int kth_timer_lap(void) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    hipEvent_t e = take_event();
+    if (!e) return fail(KTH_E_DEVICE, "kth_timer_lap: no event");
+    KTH_HIP(hipEventRecord(e, s.stream));
+    s.laps.push_back(e);
+    return KTH_OK;
+}
+
+int kth_timer_laps(float* milliseconds, int capacity, int* count, float* total_ms) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    if (!count) return fail(KTH_E_ARGUMENT, "kth_timer_laps: null count");
+    const int intervals = s.laps.empty() ? 0 : static_cast<int>(s.laps.size()) - 1;
+    *count = intervals;
+    if (total_ms) *total_ms = 0.0f;
+    int rc = KTH_OK;
+    if (!s.laps.empty()) {
+        hipError_t e = hipEventSynchronize(s.laps.back());
+        if (e != hipSuccess) rc = fail(KTH_E_DEVICE, "kth_timer_laps: %s", hipGetErrorString(e));
+        for (int i = 0; rc == KTH_OK && i < intervals && i < capacity && milliseconds; i++) {
+            e = hipEventElapsedTime(&milliseconds[i], s.laps[i], s.laps[i + 1]);
+            if (e != hipSuccess) rc = fail(KTH_E_DEVICE, "kth_timer_laps: %s", hipGetErrorString(e));
+        }
+        if (rc == KTH_OK && total_ms && intervals > 0) {
+            e = hipEventElapsedTime(total_ms, s.laps.front(), s.laps.back());
+            if (e != hipSuccess) rc = fail(KTH_E_DEVICE, "kth_timer_laps: %s", hipGetErrorString(e));
+        }
+    }
+    for (hipEvent_t ev : s.laps) s.event_pool.push_back(ev);
+    s.laps.clear();
+    return rc;
+}
+
+int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kernel_ms) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    if (n_floats == 0 || n_floats > kMaxElements || n_floats % 4 != 0 || reps < 1)
+        return fail(KTH_E_ARGUMENT, "kth_measure_copy: need a multiple of 4 floats below 2^31 and at least one repetition");
+    State& s = state();
+    uint64_t cap_a = 0, cap_b = 0;
+    float* a = workspace_acquire(n_floats * 4, &cap_a);
+    float* b = a ? workspace_acquire(n_floats * 4, &cap_b) : nullptr;
+    int rc = KTH_OK;
+    if (!a || !b) rc = fail(KTH_E_MEMORY, "kth_measure_copy: no room for two buffers of %llu floats", (unsigned long long)n_floats);
+    auto timed = [&](bool kernel, float* out_ms) -> hipError_t {
+        const uint32_t n = static_cast<uint32_t>(n_floats);
+        const uint32_t blocks = (n / 4 + 255) / 256;
+        for (int i = -1; i < reps; i++) {              // one untimed pass first
+            if (i == 0) { hipError_t e = hipEventRecord(s.ev_begin, s.stream); if (e != hipSuccess) return e; }
+            if (kernel) hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, s.stream, a, b, n);
+            else { hipError_t e = hipMemcpyAsync(b, a, n_floats * 4, hipMemcpyDeviceToDevice, s.stream); if (e != hipSuccess) return e; }
+        }
+        hipError_t e = hipEventRecord(s.ev_end, s.stream);
+        if (e == hipSuccess) e = hipEventSynchronize(s.ev_end);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, s.ev_begin, s.ev_end);
+        if (out_ms) *out_ms = ms / static_cast<float>(reps);
+        return e;
+    };
+    if (rc == KTH_OK) {
+        hipError_t e = hipMemsetAsync(a, 0x3c, n_floats * 4, s.stream);     // finite floats, not zeros
+        if (e == hipSuccess) e = timed(false, memcpy_ms);
+        if (e == hipSuccess) e = timed(true, kernel_ms);
+        if (e != hipSuccess) rc = fail(KTH_E_DEVICE, "kth_measure_copy: %s", hipGetErrorString(e));
+    }
+    if (b) workspace_release(b, cap_b);
+    if (a) workspace_release(a, cap_a);
+    return rc;
 }
 
 int kth_profile_begin(void) {

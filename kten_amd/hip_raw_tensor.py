@@ -15,9 +15,9 @@ from typing import Callable, List, Optional, Sequence
 import numpy as np
 
 from . import abi
-from . import shape_functions as sf
+from .host_mirror import shape_functions as sf
 from .abi import Op, check
-from .raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
+from .host_mirror.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
 
 _BINARY = {"plus": Op.PLUS, "minus": Op.MINUS, "times": Op.TIMES, "div": Op.DIV, "pow": Op.POW,
            "lt": Op.LT, "lte": Op.LTE, "gt": Op.GT, "gte": Op.GTE, "eq": Op.EQ, "neq": Op.NEQ}
@@ -495,12 +495,12 @@ class HipTensorOperations:
 
     # --- Tensor-level factories (BasicTensorOperations.kt:10-12) ----------------------------
     def create(self, shape, requiresGrad: bool = False, init=None):
-        from .autograd import NoGradVariable, Variable
+        from .host_mirror.autograd import NoGradVariable, Variable
         raw = self.createRaw(shape, init) if init is not None else self.createRawFill(shape, 0.0)
         return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
 
     def createFillConst(self, shape, requiresGrad: bool = False, constant: float = 0.0):
-        from .autograd import NoGradVariable, Variable
+        from .host_mirror.autograd import NoGradVariable, Variable
         raw = self.createRawFill(shape, constant)
         return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
 
@@ -536,6 +536,24 @@ class HipTensorOperations:
         ms = ctypes.c_float()
         check(self.lib.kth_timer_end(ctypes.byref(ms)))
         return ms.value
+
+    def timerLap(self):
+        check(self.lib.kth_timer_lap())
+
+    def timerLaps(self):
+        """(milliseconds between consecutive laps, milliseconds from the first lap to the last); forgets the laps."""
+        cap = 1 << 16
+        buf = (ctypes.c_float * cap)()
+        n, total = ctypes.c_int(), ctypes.c_float()
+        check(self.lib.kth_timer_laps(buf, cap, ctypes.byref(n), ctypes.byref(total)))
+        return [buf[i] for i in range(min(n.value, cap))], total.value
+
+    def measureCopy(self, n_floats: int, reps: int = 10):
+        """(GB/s of hipMemcpyAsync device to device, GB/s of the library's copy kernel) for n_floats values,
+        read + written bytes counted."""
+        a, b = ctypes.c_float(), ctypes.c_float()
+        check(self.lib.kth_measure_copy(n_floats, reps, ctypes.byref(a), ctypes.byref(b)))
+        return 8.0 * n_floats / a.value / 1e6, 8.0 * n_floats / b.value / 1e6
 
     def profileBegin(self):
         check(self.lib.kth_profile_begin())

@@ -23,6 +23,9 @@ class Workload:
     make_inputs: Callable[[Dict[str, int]], Dict[str, np.ndarray]]
     run: Callable            # (ops, inputs) -> dict name -> Tensor
     algorithmic_bytes: Callable[[Dict[str, int]], int]
+    # Bytes a single fused kernel would have to move for the same results (inputs once, outputs once): context
+    # for the op-at-a-time figure, which is what the raw-tensor contract makes a backend do.
+    fused_lower_bound_bytes: Callable[[Dict[str, int]], int] = None
 
 
 # ---- 1: broadcast + full reduction ------------------------------------------------------
@@ -433,14 +436,18 @@ WORKLOADS: Dict[str, Workload] = {
                                          "(max, minus, exp, sum, div, clamp, log, gather, mean; scatter, +=, /=)",
                            {"batch": 32768, "classes": 2048}, _in_sce, _run_sce, _bytes_sce),
     "cfg1": Workload("cfg1", "y=(x+b)*x; sum(y): x[2048,1024], b[1024], U(-1,1), seed 0",
-                     {"rows": 2048, "cols": 1024}, _in1, _run1, _bytes1),
+                     {"rows": 2048, "cols": 1024}, _in1, _run1, _bytes1,
+                     lambda d: 4 * (2 * d["rows"] * d["cols"] + d["cols"] + 1)),                  # read x and b, write y and s
     "cfg2": Workload("cfg2", "z=exp(-(x pow 2))+log(abs(x)+1e-3): x[2^26], N(0,1), seed 1",
-                     {"n": 1 << 26}, _in2, _run2, _bytes2),
+                     {"n": 1 << 26}, _in2, _run2, _bytes2, lambda d: 4 * 2 * d["n"]),              # read x, write z
     "cfg3": Workload("cfg3", "sum/mean over axis 0 and 1, max and argmax over axis 1: x[8192,8192], N(0,1), seed 2",
-                     {"rows": 8192, "cols": 8192}, _in3, _run3, _bytes3),
+                     {"rows": 8192, "cols": 8192}, _in3, _run3, _bytes3,
+                     lambda d: 4 * (d["rows"] * d["cols"] + 2 * d["cols"] + 4 * d["rows"])),     # one read of x, the six results
     "cfg4": Workload("cfg4", "act*scale+bias on NCHW [64,128,56,56] with [1,128,1,1] operands, then sum and mean "
                              "over axes (0,2,3); seed 3",
-                     {"n": 64, "c": 128, "h": 56, "w": 56}, _in4, _run4, _bytes4),
+                     {"n": 64, "c": 128, "h": 56, "w": 56}, _in4, _run4, _bytes4,
+                     lambda d: 4 * (2 * d["n"] * d["c"] * d["h"] * d["w"] + 4 * d["c"])),        # read act, write out; scale, bias, sum, mean
     "cfg5": Workload("cfg5", "loss=sum(((x*w)+b) pow 2); backward(): x[16384,4096], w[4096], b[1], seed 4",
-                     {"rows": 16384, "cols": 4096}, _in5, _run5, _bytes5),
+                     {"rows": 16384, "cols": 4096}, _in5, _run5, _bytes5,
+                     lambda d: 4 * (d["rows"] * d["cols"] + 2 * d["cols"] + 3)),                 # one read of x; w, b; loss, grad w, grad b
 }

@@ -14,8 +14,8 @@ from ctypes import POINTER, c_double, c_float, c_int, c_int32, c_int64, c_void_p
 
 import numpy as np
 
-from kten_amd import shape_functions as sf
-from kten_amd.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
+from kten_amd.host_mirror import shape_functions as sf
+from kten_amd.host_mirror.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libkten_jvm_oracle.so")
@@ -515,12 +515,12 @@ class JvmOracleOperations:
         return JvmOracleBatchNorm(axis, momentum, epsilon, training, self)
 
     def create(self, shape, requiresGrad=False, init=None):
-        from kten_amd.autograd import NoGradVariable, Variable
+        from kten_amd.host_mirror.autograd import NoGradVariable, Variable
         raw = self.createRaw(shape, init)
         return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
 
     def createFillConst(self, shape, requiresGrad=False, constant=0.0):
-        from kten_amd.autograd import NoGradVariable, Variable
+        from kten_amd.host_mirror.autograd import NoGradVariable, Variable
         raw = self.createRawFill(shape, constant)
         return Variable(self, raw) if requiresGrad else NoGradVariable(self, raw)
 

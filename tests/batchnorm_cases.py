@@ -8,7 +8,7 @@ noise of a few 1e-6 around 0, and the reference's 1e-6 holds or fails by chance;
 used instead."""
 import numpy as np
 
-from kten_amd.inputs import SplitMix64
+from kten_amd.host_mirror.inputs import SplitMix64
 from known_answer_cases import assertTensorEquals
 
 

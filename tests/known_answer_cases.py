@@ -9,8 +9,8 @@ import os
 
 import numpy as np
 
-from kten_amd.autograd import concat, ones, tensorOf
-from kten_amd.shape_functions import ALL
+from kten_amd.host_mirror.autograd import concat, ones, tensorOf
+from kten_amd.host_mirror.shape_functions import ALL
 
 with open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")) as f:
     K = json.load(f)
@@ -213,7 +213,7 @@ def case_gather_with_grads(ops):
 
 
 def case_scatter(ops):
-    from kten_amd.autograd import zeros
+    from kten_amd.host_mirror.autograd import zeros
     c = K["scatter"]
     t1 = T(ops, c["t1"])
     res1 = zeros(ops, *c["target_shape"]).scatter(c["axis1"], T(ops, c["index1"]), t1)
@@ -223,7 +223,7 @@ def case_scatter(ops):
 
 
 def case_scatter_with_grads(ops):
-    from kten_amd.autograd import zeros
+    from kten_amd.host_mirror.autograd import zeros
     c = K["scatter_with_grads"]
     t1 = T(ops, c["t1"], True)
     target = zeros(ops, *c["target_shape"]).asVariable(requiresGrad=True)
@@ -240,7 +240,7 @@ def case_softmax_cross_entropy_two_formulations(ops):
     gradients, at the reference's 1e-6 tolerance. Inputs are seeded here (the reference
     draws them unseeded); the one-hot targets are built on the host."""
     import numpy as np
-    from kten_amd.inputs import SplitMix64
+    from kten_amd.host_mirror.inputs import SplitMix64
     g = SplitMix64(11)
     n, classes = 64, 200
     logits = g.normal([n, classes])

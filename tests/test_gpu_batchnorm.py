@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import batchnorm_cases as bnc
-from kten_amd.inputs import SplitMix64
+from kten_amd.host_mirror.inputs import SplitMix64
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal, assert_reduction_close
 
@@ -162,7 +162,7 @@ def test_batch_norm_workload_at_benchmark_size(gc):
     """NCHW [64,128,56,56], training forward + backward: statistics against float64, the two
     elementwise halves bit for bit from the device's statistics, and what batch normalisation
     guarantees of its own output (per-channel mean beta, variance gamma^2 var / (var + eps))."""
-    from kten_amd.workloads import WORKLOADS
+    from kten_amd.host_mirror.workloads import WORKLOADS
     wl = WORKLOADS["batch_norm"]
     inp = wl.make_inputs(wl.full_dims)
     out = {k: v.toArray() for k, v in wl.run(gc, inp).items()}

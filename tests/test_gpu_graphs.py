@@ -8,8 +8,8 @@ import numpy as np
 import pytest
 from hypothesis import HealthCheck, given, settings, strategies as st
 
-from kten_amd.autograd import concat
-from kten_amd.shape_functions import ALL
+from kten_amd.host_mirror.autograd import concat
+from kten_amd.host_mirror.shape_functions import ALL
 from oracle import jvm_oracle as jo
 
 pytestmark = pytest.mark.gpu

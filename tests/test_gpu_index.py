@@ -70,7 +70,7 @@ def test_bad_indices_raise_like_the_reference(gc):
 def test_max_backward_at_scale_matches_checker(gc):
     """Max over the last axis with its scatter backward, and a softmax-cross-entropy step,
     on [512, 1000]: device against the checker running the same graph."""
-    from kten_amd.inputs import SplitMix64
+    from kten_amd.host_mirror.inputs import SplitMix64
     g = SplitMix64(5)
     x = g.normal([512, 1000])
     labels = (g.uniform([512], 0.0, 1.0) * 1000).astype(np.int64).clip(0, 999).astype(np.float32)

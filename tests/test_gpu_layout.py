@@ -6,7 +6,7 @@ import itertools
 import numpy as np
 import pytest
 
-from kten_amd.shape_functions import ALL
+from kten_amd.host_mirror.shape_functions import ALL
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal
 
@@ -169,7 +169,7 @@ def test_large_properties(gc):
     """At sizes the CPU checker would take long for: a transpose applied twice, a permute
     followed by its inverse and a narrow / concat round trip return the input bits, and a row
     of a transpose is a column of the input."""
-    from kten_amd import inputs
+    from kten_amd.host_mirror import inputs
     n = 4096
     x = inputs.SplitMix64(5).uniform([n, n], -1.0, 1.0)
     g = gc.createRaw([n, n], x)
@@ -189,7 +189,7 @@ def test_large_properties(gc):
 @pytest.mark.parametrize("name,dims", [("transpose", {"rows": 300, "cols": 520}), ("permute", {"n": 6, "c": 16, "h": 12, "w": 20}),
                                        ("concat_mask", {"rows": 96, "left": 200, "right": 120})])
 def test_layout_workloads_small_against_the_checker(name, dims, gc):
-    from kten_amd.workloads import WORKLOADS
+    from kten_amd.host_mirror.workloads import WORKLOADS
     wl = WORKLOADS[name]
     inputs = wl.make_inputs(dims)
     got = {k: v.toArray() for k, v in wl.run(gc, inputs).items()}
@@ -201,7 +201,7 @@ def test_layout_workloads_small_against_the_checker(name, dims, gc):
 def test_layout_workloads_full_size(gc):
     """The benchmark shapes, against numpy's own movers (independent of both the device code
     and the checker)."""
-    from kten_amd.workloads import WORKLOADS
+    from kten_amd.host_mirror.workloads import WORKLOADS
     wl = WORKLOADS["transpose"]
     inp = wl.make_inputs(wl.full_dims)
     assert_bits_equal(wl.run(gc, inp)["xt"].toArray(), inp["x"].T, "transpose")

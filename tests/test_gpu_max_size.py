@@ -5,7 +5,7 @@ x[i, j] = r[i] + c[j] is built on the device by a doubly broadcast add."""
 import numpy as np
 import pytest
 
-from kten_amd.shape_functions import ALL
+from kten_amd.host_mirror.shape_functions import ALL
 from oracle import jvm_oracle as jo
 
 pytestmark = pytest.mark.gpu

@@ -8,7 +8,7 @@ argmax against numpy on tie-free data."""
 import numpy as np
 import pytest
 
-from kten_amd.workloads import WORKLOADS, layout_shapes_at, reduce_shapes_at
+from kten_amd.host_mirror.workloads import WORKLOADS, layout_shapes_at, reduce_shapes_at
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal, assert_reduction_close, assert_ulp_close, ulp_distance
 
@@ -94,7 +94,7 @@ def test_cfg5_raw_op_sequence_intermediates_bit_exact(gc):
 
 
 def test_cfg5_gradient_accumulates_over_two_backward_passes(gc):
-    from kten_amd.workloads import cfg5_setup, cfg5_step
+    from kten_amd.host_mirror.workloads import cfg5_setup, cfg5_step
     inp = WORKLOADS["cfg5"].make_inputs({"rows": 64, "cols": 128})
     x, w, b = cfg5_setup(gc, inp)
     cfg5_step(x, w, b)

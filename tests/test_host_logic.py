@@ -9,9 +9,10 @@ import re
 import numpy as np
 import pytest
 
-from kten_amd import abi, shape_functions as sf
-from kten_amd.inputs import SplitMix64
-from kten_amd.workloads import WORKLOADS
+from kten_amd import abi
+from kten_amd.host_mirror import shape_functions as sf
+from kten_amd.host_mirror.inputs import SplitMix64
+from kten_amd.host_mirror.workloads import WORKLOADS
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -122,7 +123,7 @@ def test_contract_error_behaviour_on_the_host(oracle_ops):
 
 
 def test_may_unexpand_axis_order(oracle_ops):
-    from kten_amd.autograd import mayUnexpand
+    from kten_amd.host_mirror.autograd import mayUnexpand
     calls = []
     g = oracle_ops.createRaw([2, 3, 4, 5], np.arange(120, dtype=np.float32))
     orig = type(g).sum
@@ -251,3 +252,129 @@ def test_workload_byte_formula_equals_the_ops_it_runs(oracle_ops):
         type(oracle_ops).create = orig_tensor_create
         for name, orig in saved.items():
             setattr(R, name, orig)
+
+
+# ---------------------------------------------------------------- the shared host layer against numpy alone
+
+# The checker and the HIP backend run the same host_mirror code, so a comparison of the two says nothing about it.
+# These cases hold that layer (shape inference, keepDims and negative axes, reduce-to-shape, the shape rules of the
+# indexed moves, autograd's gradients of broadcast operands) against numpy's own statement of the same rules, on
+# random shapes, with values small enough that every float sum is exact.
+
+def _random_shape(rng, dims, hi=5):
+    return [int(rng.integers(1, hi + 1)) for _ in range(dims)]
+
+
+def _ints(rng, shape, lo=-3, hi=4):
+    return rng.integers(lo, hi, size=shape).astype(np.float32)
+
+
+def test_reduce_to_shape_equals_numpy_sum_over_the_broadcast_axes(oracle_ops):
+    from kten_amd.host_mirror.autograd import mayUnexpand
+    rng = np.random.default_rng(101)
+    for _ in range(300):
+        gshape = _random_shape(rng, int(rng.integers(1, 6)))
+        keep = int(rng.integers(1, len(gshape) + 1))                       # the operand's number of dims
+        orig = [d if rng.random() < 0.5 else 1 for d in gshape[len(gshape) - keep:]]
+        g = _ints(rng, gshape)
+        res = mayUnexpand(oracle_ops.createRaw(gshape, g), orig, oracle_ops)
+        lead = tuple(range(len(gshape) - keep))
+        want = g.sum(axis=lead) if lead else g
+        axes = tuple(i for i, (o, d) in enumerate(zip(orig, want.shape)) if o == 1 and d != 1)
+        want = want.sum(axis=axes, keepdims=True) if axes else want
+        assert res.shape == orig
+        np.testing.assert_array_equal(res.toArray().reshape(orig), want.reshape(orig))
+
+
+def test_axis_ops_keepdims_and_negative_axes_equal_numpy(oracle_ops):
+    rng = np.random.default_rng(102)
+    for _ in range(300):
+        shape = _random_shape(rng, int(rng.integers(1, 5)))
+        x = _ints(rng, shape)
+        t = oracle_ops.createRaw(shape, x)
+        axis = int(rng.integers(-len(shape), len(shape)))
+        keep = bool(rng.integers(0, 2))
+        for name, fn in (("sum", np.sum), ("max", np.max), ("min", np.min)):
+            got = getattr(t, name)(axis, keep)
+            want = fn(x, axis=axis, keepdims=keep)
+            want_shape = list(want.shape) if want.ndim else [1]            # never 0-D (AbstractRawTensor.kt:101-105)
+            assert got.shape == want_shape, (name, shape, axis, keep)
+            np.testing.assert_array_equal(got.toArray().reshape(want_shape), np.asarray(want).reshape(want_shape))
+        got = t.argMax(axis, keep)
+        np.testing.assert_array_equal(got.toArray().reshape(-1), np.argmax(x, axis=axis).reshape(-1).astype(np.float32))
+        with pytest.raises(ValueError):
+            t.sum(len(shape))
+        with pytest.raises(ValueError):
+            t.sum(-len(shape) - 1)
+
+
+def test_broadcast_binary_shapes_and_values_equal_numpy(oracle_ops):
+    rng = np.random.default_rng(103)
+    for _ in range(300):
+        out = _random_shape(rng, int(rng.integers(1, 5)))
+        a_shape = [d if rng.random() < 0.6 else 1 for d in out][int(rng.integers(0, len(out))):] or [1]
+        b_shape = [d if rng.random() < 0.6 else 1 for d in out][int(rng.integers(0, len(out))):] or [1]
+        a, b = _ints(rng, a_shape), _ints(rng, b_shape)
+        want = a * b + a
+        ta, tb = oracle_ops.createRaw(a_shape, a), oracle_ops.createRaw(b_shape, b)
+        got = ta.times(tb).plus(ta)
+        assert got.shape == list(want.shape)
+        np.testing.assert_array_equal(got.toArray().reshape(want.shape), want)
+    for a_shape, b_shape in (([3], [4]), ([2, 3], [3, 2]), ([2, 1, 3], [2, 2])):
+        with pytest.raises(ValueError):
+            oracle_ops.createRaw(a_shape, np.zeros(a_shape)).plus(oracle_ops.createRaw(b_shape, np.zeros(b_shape)))
+
+
+def test_gradients_of_broadcast_operands_equal_the_closed_form(oracle_ops):
+    """d/da and d/db of sum(a * b + b) for operands that broadcast against each other: the autograd mirror's
+    backward formulas and its reduce-to-shape against the sums numpy takes over the broadcast axes."""
+    rng = np.random.default_rng(104)
+    for _ in range(100):
+        out = _random_shape(rng, int(rng.integers(1, 5)), hi=4)
+        a_shape = [d if rng.random() < 0.6 else 1 for d in out][int(rng.integers(0, len(out))):] or [1]
+        b_shape = [d if rng.random() < 0.6 else 1 for d in out][int(rng.integers(0, len(out))):] or [1]
+        a, b = _ints(rng, a_shape), _ints(rng, b_shape)
+        ta = oracle_ops.create(a_shape, True, a)
+        tb = oracle_ops.create(b_shape, True, b)
+        (ta * tb + tb).sum().backward()
+        full = np.broadcast_shapes(tuple(a_shape), tuple(b_shape))
+
+        def reduce_to(g, shape):
+            g = g.sum(axis=tuple(range(g.ndim - len(shape)))) if g.ndim > len(shape) else g
+            axes = tuple(i for i, (o, d) in enumerate(zip(shape, g.shape)) if o == 1 and d != 1)
+            return (g.sum(axis=axes, keepdims=True) if axes else g).reshape(shape)
+        want_a = reduce_to(np.broadcast_to(b, full).astype(np.float32), a_shape)
+        want_b = reduce_to(np.broadcast_to(a, full).astype(np.float32) + 1.0, b_shape)
+        np.testing.assert_array_equal(ta.grad().toArray().reshape(a_shape), want_a)
+        np.testing.assert_array_equal(tb.grad().toArray().reshape(b_shape), want_b)
+
+
+def test_indexed_move_shape_rules_equal_numpy(oracle_ops):
+    rng = np.random.default_rng(105)
+    for _ in range(200):
+        shape = _random_shape(rng, int(rng.integers(1, 4)))
+        axis = int(rng.integers(-len(shape), len(shape)))
+        ax = axis % len(shape)
+        x = _ints(rng, shape)
+        t = oracle_ops.createRaw(shape, x)
+        k = int(rng.integers(1, 6))
+        idx = rng.integers(0, shape[ax], size=k)
+        sel = t.indexSelect(axis, oracle_ops.createRaw([k], idx.astype(np.float32)))
+        want = np.take(x, idx, axis=ax)
+        assert sel.shape == list(want.shape)
+        np.testing.assert_array_equal(sel.toArray().reshape(want.shape), want)
+        # gather with an index of the tensor's own shape equals numpy.take_along_axis
+        gi = rng.integers(0, shape[ax], size=shape)
+        got = t.gather(axis, oracle_ops.createRaw(shape, gi.astype(np.float32)))
+        np.testing.assert_array_equal(got.toArray().reshape(shape), np.take_along_axis(x, gi, axis=ax))
+        # indexAdd accumulates repeated rows in index order; the source must have the axis resized to k
+        src_shape = list(shape); src_shape[ax] = k
+        src = _ints(rng, src_shape)
+        target = oracle_ops.createRaw(shape, x.copy())
+        target.indexAdd(axis, oracle_ops.createRaw([k], idx.astype(np.float32)), oracle_ops.createRaw(src_shape, src), 2.0)
+        want = x.copy()
+        np.add.at(want, tuple(idx if d == ax else slice(None) for d in range(len(shape))), 2.0 * src)
+        np.testing.assert_array_equal(target.toArray().reshape(shape), want)
+        bad = list(src_shape); bad[ax] = k + 1
+        with pytest.raises(ValueError):
+            target.indexAdd(axis, oracle_ops.createRaw([k], idx.astype(np.float32)), oracle_ops.createRaw(bad, np.zeros(bad)), 1.0)

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import batchnorm_cases as bnc
-from kten_amd.inputs import SplitMix64
+from kten_amd.host_mirror.inputs import SplitMix64
 from oracle import jvm_oracle as jo
 
 

@@ -8,8 +8,8 @@ import itertools
 import numpy as np
 import pytest
 
-from kten_amd import shape_functions as sf
-from kten_amd.shape_functions import ALL, IntRange
+from kten_amd.host_mirror import shape_functions as sf
+from kten_amd.host_mirror.shape_functions import ALL, IntRange
 from oracle import jvm_oracle as jo
 
 
