@@ -2,6 +2,7 @@
 """Benchmark of the kten-hip hot path on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg5] [--cpu-baseline/--no-cpu-baseline]
+                  [--no-kernel-events] [--no-cold] [--no-copy-ceiling]
 
 A step is one pass of the chosen workload's raw-op sequence over device-resident
 synthetic inputs (kten_amd/workloads.py). The default workload is cfg5: the autograd
@@ -9,10 +10,17 @@ forward + backward of loss = sum(((x*w)+b) pow 2) on x[16384,4096], which exerci
 broadcast binary ops, tensor-scalar ops, the full sum and the reduce-to-shape axis sums.
 Prints ONE JSON line on stdout; everything else goes to stderr.
 
-Timing: HIP events on the library's own stream around the K timed steps (kth_timer_*),
-with a host-side wall clock around the same region as a cross-check. Per-kernel
-durations come from HIP event pairs the library records around every launch inside the
-same timed region (kth_profile_*).
+Timing: a HIP event on the library's own stream before the first and after every one of the K
+timed steps (kth_timer_lap): `value` comes from the time between the first and the last event,
+median and minimum from the steps' own intervals; a host-side wall clock around the same region
+is the cross-check. Per-kernel durations come from HIP event pairs the library records around
+every launch over a second pass of the same K steps (kth_profile_*).
+
+Two context figures are measured in the same run: the device-to-device copy rate of this GPU
+(`roofline.copy_ceiling`, hipMemcpyAsync and the library's copy kernel on 1 GiB), and the
+dominant kernel launched over a rotation of buffer sets that no recent launch has touched
+(`roofline.achieved_cold`), to tell what the memory-side cache contributes to `achieved`, which
+is measured inside the op-at-a-time chain where every kernel reads what the previous one wrote.
 """
 import argparse
 import json
@@ -28,10 +36,12 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
 # scaled by what the same counter reads for the plain copy kernel unary_kernel<OpIdentity>
-# of 262 144 KiB (FETCH_SIZE x 1.9999, WRITE_SIZE x 1.000). Source: profiles/*.md.
+# of 262 144 KiB (FETCH_SIZE x 1.9999, WRITE_SIZE x 1.000). Transcribed from the profile named
+# beside it; this run does not measure it.
 MEASURED_TRAFFIC_BYTES = {
     ("cfg5", "binary_same_kernel<OpTimes>"): int((262155 * (262144 / 131077) + 262144) * 1024),
 }
+TRAFFIC_SOURCE = "profiles/cfg5_autograd_kernels.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of an earlier run; transcribed, not measured by this run)"
 METRIC = "achieved HBM GB/s (% of MI355X peak) for broadcast binary ops and axis sum"
 
 
@@ -41,7 +51,7 @@ def log(*a):
 
 def make_step(name, ops, inputs):
     """Returns a zero-argument callable running one pass of the workload on resident inputs."""
-    from kten_amd.workloads import WORKLOADS, cfg5_setup, cfg5_step
+    from kten_amd.host_mirror.workloads import WORKLOADS, cfg5_setup, cfg5_step
     wl = WORKLOADS[name]
     if name == "cfg5":
         x, w, b = cfg5_setup(ops, inputs)
@@ -73,7 +83,7 @@ def make_step(name, ops, inputs):
         def __getattr__(self, k):
             return getattr(self.ops, k)
         def create(self, shape, requiresGrad, init):
-            from kten_amd.autograd import NoGradVariable
+            from kten_amd.host_mirror.autograd import NoGradVariable
             for key, v in inputs.items():
                 if v is init:
                     return NoGradVariable(self.ops, resident[key])
@@ -87,9 +97,71 @@ def make_step(name, ops, inputs):
     return step
 
 
+def cold_probe(ops, kernel, nbytes_per_launch, dims, sets=8, rounds=3):
+    """Average microseconds of `kernel` when each launch works on a buffer set of its own, `sets` of them in
+    rotation, so that nothing it reads or writes was touched by the launches just before it (the sets together
+    are several times the 256 MB memory-side cache). None for kernels it has no recipe for."""
+    import ctypes
+    import numpy as np
+    from kten_amd import abi
+    from kten_amd.abi import Op, check
+    family, _, op = kernel.partition("<")
+    op = op.rstrip(">")
+    lib = ops.lib
+    binary = {"OpPlus": Op.PLUS, "OpMinus": Op.MINUS, "OpTimes": Op.TIMES, "OpDiv": Op.DIV}
+    unary = {"OpNeg": Op.NEG, "OpAbs": Op.ABS, "OpExp": Op.EXP, "OpLog": Op.LOG, "OpSqrt": Op.SQRT, "OpTanh": Op.TANH,
+             "OpSigmoid": Op.SIGMOID, "OpSinh": Op.SINH, "OpCosh": Op.COSH, "OpSin": Op.SIN, "OpCos": Op.COS, "OpTan": Op.TAN,
+             "OpAsin": Op.ASIN, "OpAcos": Op.ACOS, "OpAtan": Op.ATAN}
+    rng = np.random.default_rng(0)
+
+    def tensor(n):
+        chunk = rng.standard_normal(1 << 20).astype(np.float32)
+        t = ops.createRaw([n])
+        for off in range(0, n, chunk.size):
+            m = min(chunk.size, n - off)
+            check(lib.kth_upload(t.storeReference, off, chunk.ctypes.data_as(ctypes.c_void_p), m))
+        return t
+
+    if family == "binary_same_kernel" and op in binary:
+        n = nbytes_per_launch // 12
+        make = lambda: (tensor(n), tensor(n), ops.createRaw([n]))
+        sh = abi.shape_array([n])
+        run = lambda s: check(lib.kth_binary(binary[op], s[0].storeReference, sh, 1, s[1].storeReference, sh, 1, s[2].storeReference, sh, 1))
+    elif family in ("unary_kernel", "unary_lds_kernel") and (op in unary or op in ("OpSquare", "OpIdentity")):
+        n = nbytes_per_launch // 8
+        make = lambda: (tensor(n), ops.createRaw([n]))
+        if op in unary:
+            run = lambda s: check(lib.kth_unary(unary[op], s[0].storeReference, s[1].storeReference, n))
+        else:
+            run = lambda s: check(lib.kth_scalar(Op.POW, s[0].storeReference, 2.0 if op == "OpSquare" else 1.0, 0, s[1].storeReference, n))
+    elif family == "scalar_kernel" and op in binary:
+        n = nbytes_per_launch // 8
+        make = lambda: (tensor(n), ops.createRaw([n]))
+        run = lambda s: check(lib.kth_scalar(binary[op], s[0].storeReference, 1.25, 0, s[1].storeReference, n))
+    elif family == "reduce_cols_kernel" and op in ("RedSum", "RedMean") and "rows" in dims and "cols" in dims:
+        rows, cols = dims["rows"], dims["cols"]
+        make = lambda: (tensor(rows * cols), ops.createRaw([cols]))
+        code = Op.SUM if op == "RedSum" else Op.MEAN
+        run = lambda s: check(lib.kth_reduce_axis(code, s[0].storeReference, s[1].storeReference, 1, rows, cols))
+    else:
+        return None
+    with ops.garbageCollector():
+        group = [make() for _ in range(sets)]
+        for s in group:
+            run(s)
+        ops.sync()
+        ops.profileBegin()
+        for _ in range(rounds):
+            for s in group:
+                run(s)
+        prof = ops.profileEnd()
+    launches, _, ms = prof.get(kernel, (0, 0, 0.0))
+    return ms / launches * 1e3 if launches else None
+
+
 def cpu_baseline(name, threads):
     """The CPU restatement of kten-jvm on a bounded sample of the same workload."""
-    from kten_amd.workloads import WORKLOADS
+    from kten_amd.host_mirror.workloads import WORKLOADS
     from oracle import jvm_oracle as jo
     wl = WORKLOADS[name]
     sample = {"cfg1": dict(wl.full_dims), "cfg2": dict(wl.full_dims), "cfg3": dict(wl.full_dims),
@@ -106,7 +178,7 @@ def cpu_baseline(name, threads):
     finally:
         jo.set_threads(1)
     nbytes = wl.algorithmic_bytes(sample)
-    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": os.cpu_count() or 1, "threads": threads, "kind": "port",
             "sample": f"{name} at {sample} ({nbytes / 1e6:.0f} MB algorithmic, {dt:.2f} s): C restatement of kten-jvm "
                       "semantics, not kten-jvm itself; copy-producing ops and sum() single-threaded as in the "
                       f"reference, in-place ops and axis reductions on {threads} threads"}
@@ -115,22 +187,26 @@ def cpu_baseline(name, threads):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="cfg5",
                     choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce", "transpose", "permute",
                              "concat_mask", "batch_norm", "reduce_shapes", "indexed_moves", "layout_shapes", "unary_maps"])
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,
-                    help="do not bracket every launch with an event pair inside the timed region")
+                    help="skip the second pass that brackets every launch with an event pair")
+    ap.add_argument("--no-cold", dest="cold", action="store_false", default=True,
+                    help="skip the dominant kernel's run over a rotation of untouched buffer sets")
+    ap.add_argument("--no-copy-ceiling", dest="ceiling", action="store_false", default=True,
+                    help="skip the device-to-device copy measurement")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this backend drives one GPU; the hot path has no cross-GPU step. Run with --gpus 1.")
         sys.exit(2)
 
     import kten_amd
-    from kten_amd.workloads import WORKLOADS
+    from kten_amd.host_mirror.workloads import WORKLOADS
     wl = WORKLOADS[args.config]
     dims = wl.full_dims
     nbytes = wl.algorithmic_bytes(dims)
@@ -149,18 +225,23 @@ def main():
     # Timed region: exactly K steps between two events on the library's stream, with a
     # host wall clock around the same region (stream drained on both sides).
     wall0 = time.perf_counter()
-    ops.timerBegin()
+    ops.timerLap()
     for _ in range(args.steps):
         last = step()
-    total_ms = ops.timerEnd()
+        ops.timerLap()
+    laps, total_ms = ops.timerLaps()
     ops.sync()
     wall_ms = (time.perf_counter() - wall0) * 1e3
+    laps.sort()
+    median_ms = laps[len(laps) // 2] if len(laps) % 2 else 0.5 * (laps[len(laps) // 2 - 1] + laps[len(laps) // 2])
+    min_ms = laps[0]
     m = ops.getMetrics()
     counted = (m["bytesMoved"] - m0["bytesMoved"]) / args.steps
     launches = (m["launches"] - m0["launches"]) / args.steps
     ms_per_step = total_ms / args.steps
     gbps = nbytes / ms_per_step / 1e6
-    log(f"{args.steps} steps: {total_ms:.3f} ms on the stream, {wall_ms:.3f} ms wall; {launches:.0f} launches/step; "
+    log(f"{args.steps} steps: {total_ms:.3f} ms on the stream ({ms_per_step:.4f} ms/step mean, {median_ms:.4f} median, "
+        f"{min_ms:.4f} min), {wall_ms:.3f} ms wall; {launches:.0f} launches/step; "
         f"library counted {counted:.0f} B/step (formula {nbytes})")
 
     # Per-kernel durations: the same K steps again, now with a HIP event pair around
@@ -184,19 +265,40 @@ def main():
             log(f"{k:48s} {n:8d} {ms / n * 1e3:9.2f} {(b / ms / 1e6) if ms else 0:9.1f} {100 * ms / tot:7.1f}")
         dom, (n, b, ms) = max(kernels.items(), key=lambda kv: kv[1][2])
         achieved = b / ms / 1e6
+        traffic = MEASURED_TRAFFIC_BYTES.get((args.config, dom))
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                    "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                     "bytes_per_launch": b // n, "avg_launch_us": round(ms / n * 1e3, 3), "launches": n,
-                    "kernel_time_share": round(ms / tot, 4)}
+                    "kernel_time_share": round(ms / tot, 4),
+                    "achieved_context": "inside the op-at-a-time chain: the kernel reads what the previous launch wrote, part of "
+                                        "which the 256 MB memory-side cache still holds"}
+        if args.cold:
+            cold_us = cold_probe(ops, dom, b // n, dims)
+            if cold_us:
+                roofline["achieved_cold"] = round((b // n) / cold_us / 1e3, 1)
+                roofline["frac_cold"] = round((b // n) / cold_us / 1e3 / HBM_PEAK_GBPS, 4)
+                roofline["cold_launch_us"] = round(cold_us, 3)
+                roofline["cold_context"] = "8 buffer sets in rotation, 3 rounds: no operand was read or written by the 7 launches before"
+                log(f"{dom} on untouched buffers: {cold_us:.2f} us ({roofline['achieved_cold']} GB/s) against {ms / n * 1e3:.2f} us in the chain")
+            else:
+                roofline["achieved_cold"] = None
+    if roofline is not None and args.ceiling:
+        d2d, own = ops.measureCopy(1 << 28, 10)
+        roofline["copy_ceiling"] = {"hipMemcpyDtoD_GBps": round(d2d, 1), "copy_kernel_GBps": round(own, 1), "bytes_each_way": 1 << 30,
+                                    "note": "read + written bytes over time, 10 copies of 1 GiB back to back on this GPU"}
+        log(f"device-to-device copy of 1 GiB: hipMemcpyAsync {d2d:.0f} GB/s, the library's copy kernel {own:.0f} GB/s")
 
     line = {
         "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(median_ms, 4),
+        "ms_per_step_min": round(min_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{wl.name}: {wl.description}", "algorithmic_bytes_per_step": nbytes,
-                   "launches_per_step": launches, "elements_per_s": round(sum(int(v.size) for v in inputs.values())
-                                                                         / (ms_per_step / 1e3)),
+                   "fused_lower_bound_bytes": wl.fused_lower_bound_bytes(dims) if wl.fused_lower_bound_bytes else None,
+                   "launches_per_step": launches,
+                   "fp32_elements_per_s": round(nbytes / 4 / (ms_per_step / 1e3)),
+                   "fp32_elements_per_s_means": "algorithmic bytes / 4 per second: every fp32 value a raw op reads or writes",
                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "wall_ms_per_step": round(wall_ms / args.steps, 4),
                    "per_kernel_durations": "HIP event pair around every launch, over a second pass of the same K steps"
                    if args.events else None},
@@ -204,7 +306,7 @@ def main():
     }
     if args.cpu:
         threads = min(16, os.cpu_count() or 1)
-        log(f"timing the CPU restatement on {threads} threads ...")
+        log(f"timing the CPU restatement on {threads} threads of {os.cpu_count()} host cores ...")
         line["cpu_baseline"] = cpu_baseline(args.config, threads)
         log(f"cpu baseline: {line['cpu_baseline']['value']} GB/s")
     print(json.dumps(line), flush=True)

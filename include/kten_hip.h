@@ -311,6 +311,19 @@ int kth_metrics(uint64_t* live_bytes, uint64_t* pool_bytes, uint64_t* launches, 
 int kth_timer_begin(void);
 int kth_timer_end(float* milliseconds);
 
+/* Lap timing on the internal stream, for benchmarks that report the spread of a repeated step. No
+ * counterpart in the reference. kth_timer_lap records a HIP event (nothing blocks); kth_timer_laps waits for
+ * the last one, writes the time between consecutive laps (count = laps - 1; at most `capacity` values are
+ * written) and the time from the first lap to the last, and forgets the laps. */
+int kth_timer_lap(void);
+int kth_timer_laps(float* milliseconds, int capacity, int* count, float* total_ms);
+
+/* The device-to-device copy rate of this GPU, the practical ceiling a streaming kernel is measured against:
+ * times `reps` copies of n_floats values (a multiple of 4) between two pool buffers, once with hipMemcpyAsync
+ * and once with the library's own copy kernel, and returns the milliseconds per copy of each. Blocking; no
+ * counterpart in the reference. */
+int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kernel_ms);
+
 /* Per-kernel device timing, for benchmarks that must attribute the time of a region to
  * the kernels in it. No counterpart in the reference. Between kth_profile_begin and
  * kth_profile_end every kernel launch is bracketed by a HIP event pair on the internal
