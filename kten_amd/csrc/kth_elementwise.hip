@@ -515,6 +515,94 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float*
     }
 }
 
+// ---------------------------------------------------------------- both operands small: out[i][j][v] = Op(row[i][v], col[j][v])
+
+// The broadcast of two operands that are both smaller than the output, in the shape every such pair coalesces to
+// when it is two- or three-dimensional: [N,1] o [1,M] (V = 1), or the same with an innermost run of V floats that
+// both operands keep ([N,1,V] o [M,V]). The mixed kernel pays a vector-memory instruction per operand element
+// there, and the address unit of a compute unit takes a wave's memory instruction for about 16 cycles whatever it
+// moves: 8 loads and a store per 256 outputs hold it to 2.3-3.8 TB/s. Here a workgroup owns 4096 consecutive
+// outputs, brings the slices of both operands that the span touches into LDS with 16-byte loads (the row operand's
+// rows i_lo..i_hi as one range; the column operand whole when it is no longer than the span, while a longer one
+// is read from memory 16 bytes per thread), and every thread then resolves the position of its four
+// outputs with one division pair and steps through them, reading both operands from LDS: one store and less
+// than one load instruction per 256 outputs reach the address unit.
+constexpr uint32_t kOuterTile = 8192;            // outputs per workgroup
+constexpr uint32_t kOuterMaxRun = 1024;          // longest innermost run V
+
+struct OuterPlan {
+    uint32_t n;                  // outputs
+    uint32_t run;                // V
+    uint32_t span;               // M * V: outputs per row index
+    uint32_t a_is_row;           // operand a is indexed by [i][v], b by [j][v]; or the other way round
+    uint32_t row_lds;            // floats of LDS for the row operand's slice; the column operand's follows
+    FastDiv  span_div, run_div;
+};
+
+// LDS[0 .. count) = src[first .. first + count): 16-byte loads from dword addresses, float stores into LDS
+// at `at` (any offset).
+__device__ __forceinline__ void stage_range(float* lds, uint32_t at, const float* __restrict__ src, uint32_t first, uint32_t count) {
+    for (uint32_t u = threadIdx.x * 4; u < count; u += kBlock * 4) {
+        if (u + 4 <= count) {
+            const v4f_unaligned x = *reinterpret_cast<const v4f_unaligned*>(src + first + u);
+            lds[at + u] = x.x; lds[at + u + 1] = x.y; lds[at + u + 2] = x.z; lds[at + u + 3] = x.w;
+        } else {
+            for (uint32_t j = u; j < count; j++) lds[at + j] = src[first + j];
+        }
+    }
+}
+
+template <class Op>
+__global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                             float* __restrict__ out, float eps, OuterPlan pl) {
+    // sized at launch to what the shape needs (at most 56 KiB), so that short operands leave room for eight workgroups per CU
+    extern __shared__ float outer_lds[];
+    float* row_lds = outer_lds;
+    float* col_lds = outer_lds + pl.row_lds;
+    const float* rowp = pl.a_is_row ? a : b;
+    const float* colp = pl.a_is_row ? b : a;
+    const uint32_t s = blockIdx.x * kOuterTile;
+    const uint32_t len = min(kOuterTile, pl.n - s);
+    const uint32_t i_lo = (__umulhi(s, pl.span_div.mul) + s) >> pl.span_div.shift;
+    const uint32_t last = s + len - 1;
+    const uint32_t i_hi = (__umulhi(last, pl.span_div.mul) + last) >> pl.span_div.shift;
+    stage_range(row_lds, 0, rowp, i_lo * pl.run, (i_hi - i_lo + 1) * pl.run);
+    // the column operand: staged whole when it is no longer than the span; a longer one is read from memory,
+    // 16 bytes per thread (its four outputs are neighbours there too, except where the span passes its end)
+    const bool staged = pl.span <= len;
+    if (staged) stage_range(col_lds, 0, colp, 0, pl.span);
+    __syncthreads();
+    for (uint32_t g = threadIdx.x * 4; g < len; g += kBlock * 4) {
+        const uint32_t e0 = s + g;
+        const uint32_t i = (__umulhi(e0, pl.span_div.mul) + e0) >> pl.span_div.shift;
+        uint32_t c = e0 - i * pl.span;                                     // column operand offset j * V + v
+        uint32_t v = c - ((__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift) * pl.run;
+        uint32_t row_base = (i - i_lo) * pl.run;
+        float y[4];
+        if (!staged) {
+            if (c + 4 <= pl.span) {
+                const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(colp + c);
+                y[0] = t.x; y[1] = t.y; y[2] = t.z; y[3] = t.w;
+            } else {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; j++) y[j] = colp[c + j < pl.span ? c + j : c + j - pl.span];
+            }
+        }
+        float r[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float x = row_lds[row_base + v];
+            const float yy = staged ? col_lds[c] : y[j];
+            r[j] = pl.a_is_row ? Op::apply(x, yy, eps) : Op::apply(yy, x, eps);
+            c++; v++;
+            if (v == pl.run) v = 0;
+            if (c == pl.span) { c = 0; row_base += pl.run; }
+        }
+        if (g + 4 <= len) st4(out, e0 >> 2, make_float4(r[0], r[1], r[2], r[3]));
+        else for (uint32_t j = 0; g + j < len; j++) out[e0 + j] = r[j];
+    }
+}
+
 struct OpFirst { static constexpr const char* name = "OpFirst"; static __device__ __forceinline__ float apply(float a, float, float) { return a; } };
 // maskedFill (JVMRawTensor.kt:537-540): the fill value rides in the third argument.
 struct OpMaskedFill { static constexpr const char* name = "OpMaskedFill"; static __device__ __forceinline__ float apply(float a, float m, float value) { return m == 1.0f ? value : a; } };
@@ -652,6 +740,28 @@ template <class Op>
 void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n, float eps,
                          BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec, uint64_t bytes) {
     hipStream_t st = state().stream;
+    // Both operands smaller than the output, in the two- or three-dimensional outer-product shape, and the
+    // innermost dim not a multiple of 4 (a multiple of 4 has the float4 kernels): the LDS-staged kernel.
+    if (!vec_ok && !plan.a_stream && !plan.b_stream && n >= 4 * kOuterTile && (plan.ndim == 2 || plan.ndim == 3)) {
+        const int d = plan.ndim;
+        const bool with_run = d == 3;
+        const uint32_t run = with_run ? plan.size[0] : 1u;
+        const bool run_ok = !with_run || (plan.astride[0] == 1 && plan.bstride[0] == 1 && run <= kOuterMaxRun);
+        // the dim next to the outermost one is the column index, the outermost the row index
+        const bool a_row = plan.astride[d - 2] == 0 && plan.astride[d - 1] == run && plan.bstride[d - 2] == run && plan.bstride[d - 1] == 0;
+        const bool b_row = plan.bstride[d - 2] == 0 && plan.bstride[d - 1] == run && plan.astride[d - 2] == run && plan.astride[d - 1] == 0;
+        if (run_ok && (a_row || b_row) && plan.size[d - 2] >= 2) {
+            OuterPlan op{};
+            op.n = n; op.run = run; op.span = plan.size[d - 2] * run; op.a_is_row = a_row ? 1u : 0u;
+            op.span_div = make_div(op.span); op.run_div = make_div(run);
+            op.row_lds = (((kOuterTile - 1) / op.span + 2) * run + 3u) & ~3u;
+            const uint32_t col_lds = op.span <= kOuterTile ? op.span : 4u;      // a longer column operand is not staged
+            LaunchScope scope("binary_outer_kernel", Op::name, bytes);
+            hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((n + kOuterTile - 1) / kOuterTile), dim3(kBlock),
+                               (op.row_lds + col_lds) * sizeof(float), st, a, b, out, eps, op);
+            return;
+        }
+    }
     LaunchScope scope(!vec_ok ? "binary_bcast_mixed_kernel" : (a_vec && b_vec) ? "binary_bcast_vec_kernel_vv"
                       : a_vec ? "binary_bcast_vec_kernel_vs" : b_vec ? "binary_bcast_vec_kernel_sv"
                       : "binary_bcast_vec_kernel_ss", Op::name, bytes);

@@ -102,6 +102,32 @@ def test_binary_broadcast_index_map_bit_exact(sa, sb, gc):
             assert_bits_equal(got, f(x, y), f"{op} {list(x.shape)} {list(y.shape)}")
 
 
+# Two operands that are both smaller than the output, innermost dim not a multiple of 4: the outer-product kernel
+# that stages both in LDS. Column counts shorter and longer than a workgroup's span of 4096 outputs (the window of
+# columns wraps, or the whole operand is staged), runs of 1, 2, 3 and 5 floats that both operands keep, outputs that
+# do not end on a group of four, and the two shapes of the measured gap at full size.
+OUTER_PAIRS = [
+    ([3000, 1], [1, 111]), ([70001, 1], [1, 5]), ([300, 1], [1, 5001]), ([40, 1], [1, 4099]), ([9, 1], [1, 100003]),
+    ([20011, 1], [1, 3]), ([56, 1, 2], [3001, 2]), ([700, 1, 3], [37, 3]), ([5, 1, 5], [4001, 5]), ([2, 1, 1023], [17, 1023]),
+    ([33, 1, 7], [1, 1250, 7]), ([302683, 1], [1, 111]), ([56, 1, 2], [277788, 2]),
+]
+
+
+@pytest.mark.parametrize("sa,sb", OUTER_PAIRS, ids=lambda s: "x".join(map(str, s)))
+def test_broadcast_of_two_small_operands_bit_exact(sa, sb, gc):
+    rng = np.random.default_rng(sum(sa) * 7 + sum(sb))
+    a = rng.standard_normal(sa).astype(np.float32); b = rng.standard_normal(sb).astype(np.float32)
+    gc.profileBegin()
+    results = []
+    for op, f in (("minus", np.subtract), ("div", np.divide)):
+        for x, y in ((a, b), (b, a)):
+            results.append((raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}"))
+    kernels = gc.profileEnd()
+    assert any(k.startswith("binary_outer_kernel") for k in kernels), f"expected the outer-product kernel, saw {sorted(kernels)}"
+    for got, want, what in results:
+        assert_bits_equal(got, want, what)
+
+
 def test_binary_matches_checker_on_small_broadcasts(gc):
     rng = np.random.default_rng(5)
     for sa, sb in SHAPE_PAIRS[:12]:
