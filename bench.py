@@ -34,14 +34,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each
-# scaled by what the same counter reads for the plain copy kernel unary_kernel<OpIdentity>
-# of 262 144 KiB (FETCH_SIZE x 1.9999, WRITE_SIZE x 1.000). Transcribed from the profile named
-# beside it; this run does not measure it.
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc request counters: reads as
+# 64 x TCC_EA0_RDREQ_64B + 128 x TCC_EA0_RDREQ_128B (no 32-byte requests), writes as 64 x TCC_EA0_WRREQ_64B.
+# Transcribed from the profile named beside it; this run does not measure it.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg5", "binary_same_kernel<OpTimes>"): int((262155 * (262144 / 131077) + 262144) * 1024),
+    ("cfg5", "binary_same_kernel<OpTimes>"): 147 * 64 + 4194304 * 128 + 4194304 * 64,
 }
-TRAFFIC_SOURCE = "profiles/cfg5_autograd_kernels.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of an earlier run; transcribed, not measured by this run)"
+TRAFFIC_SOURCE = ("profiles/cfg5_autograd_kernels.md (rocprofv3 --pmc TCC_EA0_RDREQ_{32B,64B,128B}_sum, TCC_EA0_WRREQ_{,64B}_sum of an "
+                  "earlier run: requests times their sizes; transcribed, not measured by this run)")
 METRIC = "achieved HBM GB/s (% of MI355X peak) for broadcast binary ops and axis sum"
 
 
