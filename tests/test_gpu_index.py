@@ -93,7 +93,12 @@ ROW_CASES = [([3, 3, 3], 1, 3), ([5, 7], 0, 9), ([5, 7], -1, 4), ([2, 3, 4, 5], 
              # lists of 64 entries or more are sorted on the device: the threshold, long runs of one target row,
              # a flat tensor, a short middle axis, columns that are not a multiple of 4
              ([9, 7], 0, 63), ([9, 7], 0, 64), ([3, 40], 0, 5000), ([2, 5, 3], 1, 1000), ([100000], 0, 300000),
-             ([20, 4100], 1, 9000), ([1, 2, 1], 1, 4097)]
+             ([20, 4100], 1, 9000), ([1, 2, 1], 1, 4097),
+             # the device's own radix sort: one, two and three 8-bit passes (axes of up to 256, 65 536 and more rows),
+             # lists of less than a tile of 4096 pairs, of many tiles, and of more than 65 536 histogram entries
+             # (the scan in three kernels), values whose sums depend on the order of the adds
+             ([200], 0, 100000), ([256, 2], 0, 70001), ([257], 0, 4095), ([60000], 0, 4097), ([65536], 0, 200000),
+             ([65537, 1], 0, 1200000), ([1000003], 0, 1100000), ([3, 70000], 1, 300001)]
 
 
 @pytest.mark.parametrize("shape,axis,k", ROW_CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
@@ -107,6 +112,7 @@ def test_index_select_and_index_add_parity(shape, axis, k, gc):
     assert got.shape == want.shape
     assert_bits_equal(got.toArray(), want.toArray(), "indexSelect")
     src = rng.standard_normal(want.shape).astype(np.float32)
+    src *= np.exp(rng.uniform(-12, 12, src.shape)).astype(np.float32)      # sums that depend on the order of the adds
     gs, cs = both(gc, want.shape, src)
     for alpha in (1.0, -0.3):
         gt, ct = both(gc, shape, x)
