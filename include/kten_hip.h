@@ -195,6 +195,14 @@ int kth_reduce_scratch_bytes(uint64_t* bytes);
 
 /* ------------------------------------------------------------------ indexed moves along an axis */
 
+/* When the indexed moves below report an index value outside its axis. immediate != 0 (the default): every such
+ * call waits for its own kernels and returns KTH_E_ARGUMENT itself, as the reference throws IllegalArgumentException
+ * at the operation (JVM:238-239,345-346,494-496). immediate == 0: the calls do not wait; an out-of-range index sets a
+ * flag on the device and the next blocking call (kth_sync, kth_download, kth_read_scalar) returns KTH_E_ARGUMENT in
+ * its place, once. Either way the kernels skip the offending entry and the in-place target of a scatter or indexAdd has
+ * been updated by the entries before it (the JVM, too, has assigned those when it throws). */
+int kth_set_index_check(int immediate);
+
 /* gather (RAW:164; JVM:334-353). in and index have `dims` dims; out has index's shape:
  * out[p, i] = in[p, (int) index[p, i]] for every position p of index's shape without the
  * axis. index dims other than the axis must not exceed in's. Blocking: an index value

@@ -56,6 +56,7 @@ SIGNATURES = {
     "kth_reduce_all": (c_int, [c_int, c_uint64, c_uint64, c_uint64]),
     "kth_reduce_axis_static": (c_int, [c_int, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
     "kth_reduce_scratch_bytes": (c_int, [POINTER(c_uint64)]),
+    "kth_set_index_check": (c_int, [c_int]),
     "kth_gather": (c_int, [c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_int, c_int, c_uint64]),
     "kth_scatter": (c_int, [c_int, c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32), c_uint64, POINTER(c_int32),
                             c_int, c_int]),

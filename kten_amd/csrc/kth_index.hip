@@ -467,6 +467,13 @@ void strides_without_axis(const int32_t* shape, int dims, int axis, uint32_t* po
 template <class F>
 int with_index_check(const char* what, F launch) {
     State& s = state();
+    if (!s.index_check_immediate) {
+        // deferred: the kernels set the persistent flag, the next blocking call reports it; nothing waits here
+        launch(s.deferred_index_flag);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
+        return KTH_OK;
+    }
     uint64_t cap;
     int* flag = reinterpret_cast<int*>(workspace_acquire(4, &cap));
     if (!flag) return fail(KTH_E_MEMORY, "%s: no workspace", what);

@@ -62,6 +62,11 @@ struct State {
     bool       stage_used[kStageSlots] = {false};
     int        stage_next = 0;
 
+    // Out-of-range index values of the indexed moves: with index_check_immediate every such op waits for its own
+    // flag; otherwise the kernels set this persistent device word and the next blocking call reports it.
+    bool index_check_immediate = true;
+    int* deferred_index_flag = nullptr;
+
     std::vector<hipEvent_t> laps;           // kth_timer_lap events not yet read by kth_timer_laps
 
     bool profiling = false;
@@ -101,6 +106,10 @@ hipError_t sort_pairs_u32(void* temp, size_t* temp_bytes, const uint32_t* keys_i
 // Resolves the device address of the static scratch array of kth_reduce_axis_static for
 // `device`, which must be the current device (kth_reduce.hip). Called once from kth_init.
 hipError_t reduce_scratch_init(int device);
+
+// In deferred index checking: reads and clears the persistent flag (the stream must be drained) and returns
+// KTH_E_ARGUMENT if an indexed move since the last report met an index outside its axis, KTH_OK otherwise.
+int report_deferred_index_error();
 
 // Computes the exp / log tables on the host (extended precision) and copies them into the
 // device symbols of the elementwise kernels. Called once from kth_init.

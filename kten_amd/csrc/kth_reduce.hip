@@ -68,7 +68,11 @@ struct RedSumT {
     static __device__ __forceinline__ Acc init() { return 0.0; }
     static __device__ __forceinline__ void step(Acc& a, float x, uint32_t) { a += static_cast<double>(x); }
     static __device__ __forceinline__ Acc merge(Acc a, Acc b) { return a + b; }
-    // MEAN divides once in f64 and rounds once (FloatArray.average, JVMRawTensor.kt:150-152).
+    // MEAN divides once in f64 and rounds once. That is what the full mean() of the reference does
+    // (FloatArray.average: double accumulator, JVMRawTensor.kt:150-152). Its axis SUM and MEAN are a serial float
+    // accumulation, MEAN followed by a float divide (JVMRawTensor.kt:186-192): there this backend is closer to the
+    // exact result rather than identical, and differs in kind where the float running sum overflows or absorbs
+    // terms: [3e38, 3e38, -3e38] sums to +inf on kten-jvm and to 3e38 here.
     static __device__ __forceinline__ float finish(Acc a, uint32_t n) {
         return MEAN ? static_cast<float>(a / static_cast<double>(n)) : static_cast<float>(a);
     }

@@ -135,6 +135,18 @@ LaunchScope::LaunchScope(const char* family, const char* op, uint64_t algorithmi
     record_ = static_cast<int>(s.records.size()) - 1;
 }
 
+int report_deferred_index_error() {
+    State& s = state();
+    if (s.index_check_immediate || !s.deferred_index_flag) return KTH_OK;
+    int host_flag = 0;
+    KTH_HIP(hipMemcpyAsync(&host_flag, s.deferred_index_flag, 4, hipMemcpyDeviceToHost, s.stream));
+    KTH_HIP(hipStreamSynchronize(s.stream));
+    if (!host_flag) return KTH_OK;
+    KTH_HIP(hipMemsetAsync(s.deferred_index_flag, 0, 4, s.stream));
+    return fail(KTH_E_ARGUMENT, "an indexed move since the last blocking call got an invalid index, an index value is out of "
+                                "bounds at the axis (its target was updated up to that entry)");
+}
+
 LaunchScope::~LaunchScope() {
     if (record_ < 0) return;
     State& s = state();
@@ -174,6 +186,8 @@ int kth_init(int device) {
     KTH_HIP(hipEventCreate(&s.ev_end));
     KTH_HIP(init_math_tables());
     KTH_HIP(reduce_scratch_init(device));
+    KTH_HIP(hipMalloc(reinterpret_cast<void**>(&s.deferred_index_flag), 256));
+    KTH_HIP(hipMemset(s.deferred_index_flag, 0, 256));
     s.device = device;
     s.ready = true;
     g_epoch += 1;
@@ -190,6 +204,7 @@ int kth_shutdown(void) {
     s.table.clear();
     s.free_slots.clear();
     trim_pool();
+    if (s.deferred_index_flag) (void)hipFree(s.deferred_index_flag);
     for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
     for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
     for (hipEvent_t e : s.laps) (void)hipEventDestroy(e);
@@ -337,7 +352,7 @@ int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n) {
     State& s = state();
     KTH_HIP(hipMemcpyAsync(dst, st->ptr + offset, n * 4, hipMemcpyDeviceToHost, s.stream));
     KTH_HIP(hipStreamSynchronize(s.stream));
-    return KTH_OK;
+    return report_deferred_index_error();
 }
 
 int kth_read_scalar(uint64_t handle, uint64_t index, float* out) {
@@ -423,6 +438,18 @@ int kth_sync(void) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     KTH_HIP(hipStreamSynchronize(state().stream));
+    return report_deferred_index_error();
+}
+
+int kth_set_index_check(int immediate) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    State& s = state();
+    if (!s.index_check_immediate && immediate) {        // leaving deferred mode: report what is pending first
+        KTH_HIP(hipStreamSynchronize(s.stream));
+        if (int rc = report_deferred_index_error()) { s.index_check_immediate = true; return rc; }
+    }
+    s.index_check_immediate = immediate != 0;
     return KTH_OK;
 }
 

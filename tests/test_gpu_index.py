@@ -4,6 +4,8 @@ last write wins; add: summed in ascending order) and the error behaviour."""
 import numpy as np
 import pytest
 
+from kten_amd import abi
+
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal
 
@@ -242,3 +244,30 @@ def test_scatter_add_with_hot_elements(shape, ishape, gc):
     gt, ct = both(gc, [shape[1]], x[0]); gr, cr = both(gc, [ishape[1]], rows); ga, ca = both(gc, [ishape[1]], add)
     gt.indexAdd(0, gr, ga, 0.3); ct.indexAdd(0, cr, ca, 0.3)
     assert_bits_equal(gt.toArray(), ct.toArray(), "indexAdd on a vector")
+
+
+def test_deferred_index_check_reports_at_the_next_blocking_call(gc):
+    """kth_set_index_check(0): an indexed move with an index outside its axis does not wait and returns OK; the next
+    blocking call reports it, once; valid entries before the bad one are applied, the bad one is skipped."""
+    lib = gc.lib
+    x = gc.createRaw([2, 3], np.arange(6, dtype=np.float32))
+    good = gc.createRaw([2], [0.0, 2.0]); bad = gc.createRaw([2], [1.0, 3.0])
+    src = gc.createRaw([2, 2], np.ones(4, dtype=np.float32))
+    abi.check(lib.kth_set_index_check(0))
+    try:
+        launches = gc.getMetrics()["launches"]
+        x.indexAdd(1, bad, src)                      # no error here
+        sel = x.indexSelect(1, good)                 # nor here: the flag is reported by a blocking call, not by the next op
+        assert gc.getMetrics()["launches"] > launches
+        with pytest.raises(ValueError, match="invalid index"):
+            gc.sync()
+        gc.sync()                                    # reported once
+        np.testing.assert_array_equal(x.toArray(), np.array([[0, 2, 2], [3, 5, 5]], dtype=np.float32))
+        np.testing.assert_array_equal(sel.toArray(), np.array([[0, 2], [3, 5]], dtype=np.float32))
+        x.indexAdd(1, bad, src)
+        with pytest.raises(ValueError, match="invalid index"):
+            x.toArray()                              # a download reports it too
+    finally:
+        abi.check(lib.kth_set_index_check(1))
+    with pytest.raises(ValueError):
+        x.indexAdd(1, bad, src)                      # immediate again

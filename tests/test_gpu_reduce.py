@@ -154,3 +154,22 @@ def test_reduce_to_shape_matches_numpy(gc):
         assert res.shape == oshape
         ref = g.astype(np.float64).sum(axes, keepdims=True).reshape(oshape)
         np.testing.assert_allclose(res.toArray(), ref, rtol=1e-5, atol=1e-5)
+
+
+def test_sums_whose_float_running_sum_overflows_or_absorbs(gc):
+    """Where kten-jvm's serial float accumulation (JVMRawTensor.kt:146-148,186-192) overflows or absorbs terms, this
+    backend (f64 accumulation, one rounding) returns the correctly rounded sum instead: a divergence in kind, inside
+    the reduction bar (its error is the smaller one), and not pinned by any test of the reference."""
+    rows = np.array([[3e38, 3e38, -3e38, 1.0], [1e8, 1.0, -1e8, 0.0], [-3e38, -3e38, 3e38, 5.0], [16777216.0, 1.0, 1.0, 1.0]], dtype=np.float32)
+    exact = rows.astype(np.float64).sum(1)
+    for x, axis in ((rows, 1), (np.ascontiguousarray(rows.T), 0)):
+        t = raw(gc, x)
+        with np.errstate(all="ignore"):
+            jvm_sum = jo.aggregate("sum", x, axis).reshape(-1)
+            jvm_mean = jo.aggregate("mean", x, axis).reshape(-1)
+        got_sum = t.sum(axis).toArray().reshape(-1)
+        got_mean = t.mean(axis).toArray().reshape(-1)
+        assert np.isposinf(jvm_sum[0]) and np.isneginf(jvm_sum[2]) and jvm_sum[1] == 0.0 and jvm_sum[3] == 16777216.0
+        assert_bits_equal(got_sum, exact.astype(np.float32), "sum: the correctly rounded value")
+        assert_bits_equal(got_mean, (exact / 4.0).astype(np.float32), "mean: the correctly rounded value")
+        assert np.isinf(jvm_mean[0]) and np.isfinite(got_mean[0])
