@@ -74,6 +74,7 @@ __device__ double   g_exp_table[kExpTableEntries];
 __device__ double   g_atan_table[kAtanTableEntries];
 __device__ double   g_sincos_table[2 * kSinCosTableEntries];
 __device__ double   g_asin_table[2 * kAsinTableEntries];
+__device__ Log2Entry g_log2_table[kLogTableEntries];
 
 // Copies `count` doubles of a device table into LDS, all threads of the workgroup taking part.
 __device__ __forceinline__ void stage_table(double* lds, const double* table, int count) {
@@ -230,9 +231,18 @@ __device__ __forceinline__ float pow_with_tables(float a, float b, const LogEntr
     if (common) return table_pow_finite(a, b, log_tab, exp_tab);
     return jpow(a, b);
 }
+// The short base-2 evaluation first (a finite base above zero, a finite exponent other than zero), the routine above for
+// the lanes whose rounding it leaves open and for every other operand.
+__device__ __forceinline__ float pow_short_then_long(float a, float b, const Log2Entry* log2_tab, const LogEntry* log_tab, const double* exp_tab) {
+    double y;
+    const bool ok = fast_pow(a, b, log2_tab, exp_tab, y);
+    float r = static_cast<float>(y);
+    if (!(ok && rounds_safely(y))) r = pow_with_tables(a, b, log_tab, exp_tab);
+    return r;
+}
 struct OpPowT {
     static constexpr const char* name = "OpPow";
-    static __device__ __forceinline__ float apply(float a, float b, float) { return pow_with_tables(a, b, g_log_table, g_exp_table); }
+    static __device__ __forceinline__ float apply(float a, float b, float) { return pow_short_then_long(a, b, g_log2_table, g_log_table, g_exp_table); }
 };
 
 // Unary map whose op reads a small f64 table through LDS. The data loads of the tile are
@@ -269,7 +279,7 @@ __global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const float* b, float* out, uint32_t n, float c) {
     constexpr int kLogDoubles = 2 * kLogTableEntries;
-    __shared__ double tab[kLogDoubles + kExpTableEntries];
+    __shared__ double tab[2 * kLogDoubles + kExpTableEntries];       // {1/c, ln c}, 2^(i/128), {1/c, log2 c}
     const uint32_t n4 = n >> 2;
     const uint32_t base = blockIdx.x * (kBlock * kLdsUnroll) + threadIdx.x;
     float4 v[kLdsUnroll], w[kLdsUnroll];
@@ -278,23 +288,45 @@ __global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const f
         uint32_t i = base + k * kBlock;
         if (i < n4) { v[k] = ld4(a, i); if (MODE == 2) w[k] = ld4(b, i); }
     }
-    for (int i = threadIdx.x; i < kLogDoubles + kExpTableEntries; i += kBlock)
-        tab[i] = i < kLogDoubles ? reinterpret_cast<const double*>(g_log_table)[i] : g_exp_table[i - kLogDoubles];
+    stage_table(tab, reinterpret_cast<const double*>(g_log_table), kLogDoubles);
+    stage_table(tab + kLogDoubles, g_exp_table, kExpTableEntries);
+    stage_table(tab + kLogDoubles + kExpTableEntries, reinterpret_cast<const double*>(g_log2_table), kLogDoubles);
     __syncthreads();
     const LogEntry* log_tab = reinterpret_cast<const LogEntry*>(tab);
     const double* exp_tab = tab + kLogDoubles;
+    const Log2Entry* log2_tab = reinterpret_cast<const Log2Entry*>(tab + kLogDoubles + kExpTableEntries);
     auto one = [&](float x, float y) {
-        return MODE == 1 ? pow_with_tables(c, x, log_tab, exp_tab) : pow_with_tables(x, MODE == 2 ? y : c, log_tab, exp_tab);
+        return MODE == 1 ? pow_short_then_long(c, x, log2_tab, log_tab, exp_tab)
+                         : pow_short_then_long(x, MODE == 2 ? y : c, log2_tab, log_tab, exp_tab);
+    };
+    // four elements through the short routine, then one branch for the lanes of the wave it leaves open
+    auto four = [&](float4 x, float4 y) {
+        const float xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
+        float rs[4];
+        bool open[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float base_ = MODE == 1 ? c : xs[j];
+            const float expo = MODE == 1 ? xs[j] : MODE == 2 ? ys[j] : c;
+            double val;
+            const bool ok = fast_pow(base_, expo, log2_tab, exp_tab, val);
+            rs[j] = static_cast<float>(val);
+            open[j] = !(ok && rounds_safely(val));
+        }
+        if (open[0] | open[1] | open[2] | open[3]) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float base_ = MODE == 1 ? c : xs[j];
+                const float expo = MODE == 1 ? xs[j] : MODE == 2 ? ys[j] : c;
+                if (open[j]) rs[j] = pow_with_tables(base_, expo, log_tab, exp_tab);
+            }
+        }
+        return make_float4(rs[0], rs[1], rs[2], rs[3]);
     };
 #pragma unroll
     for (int k = 0; k < kLdsUnroll; k++) {
         uint32_t i = base + k * kBlock;
-        if (i < n4) {
-            float4 r;
-            r.x = one(v[k].x, MODE == 2 ? w[k].x : 0.0f); r.y = one(v[k].y, MODE == 2 ? w[k].y : 0.0f);
-            r.z = one(v[k].z, MODE == 2 ? w[k].z : 0.0f); r.w = one(v[k].w, MODE == 2 ? w[k].w : 0.0f);
-            st4(out, i, r);
-        }
+        if (i < n4) st4(out, i, four(v[k], MODE == 2 ? w[k] : v[k]));
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3u)) {
         uint32_t i = (n4 << 2) + threadIdx.x;
@@ -1098,6 +1130,11 @@ hipError_t init_math_tables() {
         log_tab[i].invc = invc;
         log_tab[i].logc = static_cast<double>(-logl(static_cast<long double>(invc)));
     }
+    Log2Entry log2_tab[kLogTableEntries];
+    for (int i = 0; i < kLogTableEntries; i++) {
+        log2_tab[i].invc = log_tab[i].invc;
+        log2_tab[i].log2c = log_tab[i].invc == 1.0 ? 0.0 : static_cast<double>(-log2l(static_cast<long double>(log_tab[i].invc)));
+    }
     for (int i = 0; i < kExpTableEntries; i++)
         exp_tab[i] = static_cast<double>(exp2l(static_cast<long double>(i) / kExpTableEntries));
     double atan_tab[kAtanTableEntries];
@@ -1119,6 +1156,8 @@ hipError_t init_math_tables() {
     hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_log_table), log_tab, sizeof(log_tab));
     if (e != hipSuccess) return e;
     e = hipMemcpyToSymbol(HIP_SYMBOL(g_exp_table), exp_tab, sizeof(exp_tab));
+    if (e != hipSuccess) return e;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_log2_table), log2_tab, sizeof(log2_tab));
     if (e != hipSuccess) return e;
     e = hipMemcpyToSymbol(HIP_SYMBOL(g_sincos_table), sincos_tab, sizeof(sincos_tab));
     if (e != hipSuccess) return e;

@@ -185,4 +185,47 @@ __device__ __forceinline__ bool fast_acos(float x, const double* tab, double& y)
     return a32 < 1.0f;
 }
 
+// ---------------------------------------------------------------- pow
+
+// a^b = 2^(b log2 a) for a finite base above zero and a finite exponent other than zero, in base 2 so that the
+// reduction of the exponent function is exact: log2 a = k + log2 c + log2(1 + r) with the decomposition of
+// table_log_d (z = a 2^-k in [0.6875, 1.375), c the centre of z's interval, r = z / c - 1 by one fma, |r| < 2^-7)
+// and the table's {1 / c, log2 c}; log2(1 + r) by its series to r^7 (next term below 2^-56 of the value), good to
+// 2^-51 also next to a = 1, where the table's interval has c = 1 and the series is all there is.
+// w = b log2 a is then off by at most 1100 x 2^-51 absolute; 2^w = 2^m T[j] 2^q with 128 w = 128 m + j + 128 q
+// exactly (q = w - round(128 w) / 128 is an exact difference), 2^q - 1 by its series to q^5 (|q| <= 2^-8: the
+// next term is below 2^-55). The result is good to 2^-44 for |w| up to 128, beyond which it is 0 or inf anyway.
+struct Log2Entry { double invc, log2c; };
+
+__device__ __forceinline__ bool fast_pow(float a, float b, const Log2Entry* log2_tab, const double* exp_tab, double& y) {
+    const double d = static_cast<double>(a);
+    const uint64_t ix = static_cast<uint64_t>(__double_as_longlong(d));
+    const uint64_t tmp = ix - kLogOff;
+    const int i = static_cast<int>(tmp >> 45) & (kLogTableEntries - 1);
+    const int k = static_cast<int>(static_cast<int64_t>(tmp) >> 52);
+    const double z = __longlong_as_double(static_cast<long long>(ix - (tmp & 0xfff0000000000000ull)));
+    const Log2Entry e = log2_tab[i];
+    const double r = fma(z, e.invc, -1.0);
+    // log2(1 + r) = r (c1 + r (c2 + ...)), c_n = (-1)^(n+1) / (n ln 2)
+    double p = fma(r, 0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3);        // 1/(7 ln2), -1/(6 ln2)
+    p = fma(r, p, 0x1.2776c50ef9bfep-2);                                     // 1/(5 ln2)
+    p = fma(r, p, -0x1.71547652b82fep-2);                                    // -1/(4 ln2)
+    p = fma(r, p, 0x1.ec709dc3a03fdp-2);                                     // 1/(3 ln2)
+    p = fma(r, p, -0x1.71547652b82fep-1);                                    // -1/(2 ln2)
+    p = fma(r, p, 0x1.71547652b82fep+0);                                     // 1/ln2
+    const double t = fma(r, p, static_cast<double>(k) + e.log2c);
+    const double w = fmin(fmax(static_cast<double>(b) * t, -1100.0), 1100.0);
+    const double kd = rint(w * 128.0);
+    const int j = static_cast<int>(kd);
+    const double q = fma(kd, -0.0078125, w);
+    // 2^q - 1 = q (l1 + q (l2 + ...)), l_n = ln2^n / n!
+    double g = fma(q, 0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7);        // ln2^5/120, ln2^4/24
+    g = fma(q, g, 0x1.c6b08d704a0c0p-5);                                     // ln2^3/6
+    g = fma(q, g, 0x1.ebfbdff82c58fp-3);                                     // ln2^2/2
+    g = fma(q, g, 0x1.62e42fefa39efp-1);                                     // ln2
+    const double s = exp_tab[j & (kExpTableEntries - 1)];
+    y = ldexp(fma(s, q * g, s), j >> 7);
+    return a > 0.0f && a < INFINITY && fabsf(b) < INFINITY && b != 0.0f;
+}
+
 }  // namespace kth
