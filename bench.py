@@ -299,7 +299,16 @@ def main():
                    "launches_per_step": launches,
                    "fp32_elements_per_s": round(nbytes / 4 / (ms_per_step / 1e3)),
                    "fp32_elements_per_s_means": "algorithmic bytes / 4 per second: every fp32 value a raw op reads or writes",
-                   "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "wall_ms_per_step": round(wall_ms / args.steps, 4),
+                   "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                   "moved_bytes_per_step": round(counted),
+                   "GBps_on_moved_bytes": round(counted / ms_per_step / 1e6, 1),
+                   "frac_of_hbm_peak_on_moved_bytes": round(counted / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4),
+                   "moved_bytes_means": "what the library's launches of one step read and wrote, summed from their own byte counts; "
+                                        "`value` uses the op-at-a-time byte total of the reference's op list instead. The two differ "
+                                        "where the library does not write out a tensor that is one constant (a fresh zerosLike, the "
+                                        "broadcast seed gradient) and hands the constant to the consumer's kernel, and where it moves "
+                                        "more than the op list names (transposed copies of a scatter along an outer axis)",
+                   "wall_ms_per_step": round(wall_ms / args.steps, 4),
                    "per_kernel_durations": "HIP event pair around every launch, over a second pass of the same K steps"
                    if args.events else None},
         "roofline": roofline,

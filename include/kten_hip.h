@@ -121,7 +121,15 @@ int kth_read_scalar(uint64_t handle, uint64_t index, float* out);
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n);
 
 /* inplaceFill (RAW:244), zerosLike / zeroOut (OPS:24-26), createRawFill (OPS:18-20),
- * set(range, Float) on a contiguous range (RAW:35-37). */
+ * set(range, Float) on a contiguous range (RAW:35-37).
+ * A fill that starts at offset 0 (and the upload of a single value at offset 0) is noted on the
+ * store and launched only when some call reads the store as memory; every entry point sees the
+ * filled values. Calls that can use the constant directly do so and produce the bits of the plain
+ * sequence: kth_binary / kth_binary_inplace with + - x / take it as the scalar operand,
+ * kth_scalar of such a store with + - x / yields another noted constant, kth_broadcast_to and a
+ * whole-range kth_copy pass it on, kth_scatter / kth_scatter_fill (row form) and kth_index_add
+ * (sorted form) start the target's rows from it, a result that overwrites the store drops it,
+ * kth_release forgets it. */
 int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value);
 
 /* containsNan (RAW:240, JVM:520-522). Blocking. */

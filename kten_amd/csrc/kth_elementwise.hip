@@ -836,24 +836,75 @@ bool is_binary_op(int op) {
     return (op >= KTH_PLUS && op <= KTH_POW) || (op >= KTH_LT && op <= KTH_NEQ);
 }
 
+// The four single-rounding operations: a tensor operand that is one constant everywhere may be
+// taken as the scalar operand of the same functor, with the same bits in the result.
+bool folds_a_constant(int op) { return op >= KTH_PLUS && op <= KTH_DIV; }
+
+// op(x, y) of two constants on the host, for the result of a scalar operation on a store that is one
+// owed constant: the store of the result is then owed the outcome and nothing is launched. Done only
+// where the host's arithmetic cannot differ from the kernel's: finite-or-infinite operands that are not
+// subnormal, a result that is neither NaN nor subnormal. The value is formed in double and rounded once
+// more to float; for + - x / of floats that second rounding changes nothing (53 >= 2 * 24 + 2).
+bool fold_constants(int op, float x, float y, float* out) {
+    auto plain = [](float v) {
+        uint32_t b; memcpy(&b, &v, 4);
+        const uint32_t e = (b >> 23) & 0xffu;
+        return (e != 0u || (b & 0x7fffffu) == 0u) && !(e == 0xffu && (b & 0x7fffffu) != 0u);   // not subnormal, not NaN
+    };
+    if (!plain(x) || !plain(y)) return false;
+    const double dx = x, dy = y;
+    double r;
+    switch (op) {
+    case KTH_PLUS:  r = dx + dy; break;
+    case KTH_MINUS: r = dx - dy; break;
+    case KTH_TIMES: r = dx * dy; break;
+    case KTH_DIV:   r = dx / dy; break;
+    default: return false;
+    }
+    if (r != r) return false;
+    if (r != 0.0 && (r < 0 ? -r : r) < 1.17549435082228750797e-38) return false;
+    *out = static_cast<float>(r);
+    return true;
+}
+
+// out = op(a, c), or op(c, a) with rev, through the scalar kernels.
+void launch_scalar_op(int op, bool rev, const float* pa, float* po, uint32_t n32, float c, float eps) {
+#define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
+    KTH_BINARY_DISPATCH(op, S)
+#undef S
+}
+
 }  // namespace
+
+namespace kth {
+void launch_fill(float* p, uint64_t n, float value) {
+    if (n == 0) return;
+    const uint32_t n32 = static_cast<uint32_t>(n);
+    LaunchScope scope("fill_kernel", "", n * 4);
+    hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(n32 >> 2)), dim3(kBlock), 0, state().stream, p, n32, value);
+}
+}  // namespace kth
 
 extern "C" {
 
 int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup(handle, "kth_fill");
+    Store* st = lookup_unsettled(handle, "kth_fill");
     if (!st) return KTH_E_HANDLE;
     if (offset > st->n_floats || n > st->n_floats - offset)
         return fail(KTH_E_ARGUMENT, "kth_fill: range [%llu, +%llu) outside a store of %llu floats",
                     (unsigned long long)offset, (unsigned long long)n, (unsigned long long)st->n_floats);
     if (n == 0) return KTH_OK;
-    uint32_t n32 = static_cast<uint32_t>(n);
-    {
-        LaunchScope scope("fill_kernel", "", n * 4);
-        hipLaunchKernelGGL(fill_kernel, dim3(blocks_for(n32 >> 2)), dim3(kBlock), 0, state().stream, st->ptr + offset, n32, value);
+    if (offset == 0) {
+        // A fill of the store's head is only noted: whoever reads the store next either folds the
+        // constant into its own kernel or has the fill launched first (kth_internal.h, Store::fill_n).
+        settle_for_overwrite(st, n);
+        st->fill_n = n; st->fill_value = value;
+        return KTH_OK;
     }
+    settle(st);
+    launch_fill(st->ptr + offset, n, value);
     KTH_LAUNCH_CHECK("fill");
     return KTH_OK;
 }
@@ -915,13 +966,24 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_scalar: op %d is not a binary op", op);
-    Store* sa = lookup(a, "kth_scalar(a)");
+    Store* sa = lookup_unsettled(a, "kth_scalar(a)");
     if (!sa) return KTH_E_HANDLE;
-    Store* so = lookup(out, "kth_scalar(out)");
+    Store* so = lookup_unsettled(out, "kth_scalar(out)");
     if (!so) return KTH_E_HANDLE;
     if (n > sa->n_floats || n > so->n_floats)
         return fail(KTH_E_ARGUMENT, "kth_scalar: n=%llu exceeds a store", (unsigned long long)n);
     if (n == 0) return KTH_OK;
+    // A constant times (plus, ...) a constant: the broadcast seed gradient times an exponent, a fresh
+    // zerosLike plus a bias. The result is owed the folded constant; nothing is read or written now.
+    float folded;
+    if (folds_a_constant(op) && sa->fill_n >= n && (so != sa || sa->fill_n == n) &&
+        fold_constants(op, reverse ? c : sa->fill_value, reverse ? sa->fill_value : c, &folded)) {
+        if (so != sa) settle_for_overwrite(so, n);
+        so->fill_n = n; so->fill_value = folded;
+        return KTH_OK;
+    }
+    settle(sa);
+    if (so != sa) settle_for_overwrite(so, n);
     const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
     const float eps = state().epsilon;
     const bool rev = reverse != 0;
@@ -936,11 +998,7 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     else if (op == KTH_POW && !rev && c == 0.5f)  launch_unary<OpPowHalf>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW && !rev && c == -2.0f) launch_unary<OpPowInverseSquare>(pa, po, n32, 0.0f, 0.0f);
     else if (op == KTH_POW) launch_pow(rev ? 1 : 0, pa, nullptr, po, n32, c);
-    else {
-#define S(OP) launch_scalar<OP>(rev, pa, po, n32, c, eps)
-        KTH_BINARY_DISPATCH(op, S)
-#undef S
-    }
+    else launch_scalar_op(op, rev, pa, po, n32, c, eps);
     KTH_LAUNCH_CHECK("scalar");
     return KTH_OK;
 }
@@ -949,9 +1007,9 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_binary_inplace: op %d is not a binary op", op);
-    Store* sa = lookup(a, "kth_binary_inplace(a)");
+    Store* sa = lookup_unsettled(a, "kth_binary_inplace(a)");
     if (!sa) return KTH_E_HANDLE;
-    Store* sb = lookup(b, "kth_binary_inplace(b)");
+    Store* sb = lookup_unsettled(b, "kth_binary_inplace(b)");
     if (!sb) return KTH_E_HANDLE;
     if (n > sa->n_floats || n > sb->n_floats)
         return fail(KTH_E_SHAPE, "kth_binary_inplace: n=%llu exceeds a store (%llu, %llu)", (unsigned long long)n,
@@ -959,6 +1017,23 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
     if (n == 0) return KTH_OK;
     float* pa = sa->ptr; const float* pb = sb->ptr; uint32_t n32 = static_cast<uint32_t>(n);
     const float eps = state().epsilon;
+    // An operand that is still an owed constant (a gradient buffer fresh from zerosLike, a broadcast
+    // seed) rides as the scalar operand: one stream less to read, the same bits.
+    if (folds_a_constant(op) && sa != sb && sb->fill_n >= n) {
+        settle(sa);
+        launch_scalar_op(op, false, pa, pa, n32, sb->fill_value, eps);
+        KTH_LAUNCH_CHECK("binary_inplace");
+        return KTH_OK;
+    }
+    if (folds_a_constant(op) && sa != sb && sa->fill_n == n) {
+        const float c = sa->fill_value;
+        sa->fill_n = 0;
+        settle(sb);
+        launch_scalar_op(op, true, pb, pa, n32, c, eps);
+        KTH_LAUNCH_CHECK("binary_inplace");
+        return KTH_OK;
+    }
+    settle(sa); settle(sb);
     if (op == KTH_POW) launch_pow(2, pa, pb, pa, n32, 0.0f);
     else {
 #define B(OP) launch_binary_same<OP>(pa, pb, pa, n32, eps)
@@ -980,11 +1055,11 @@ int kth_binary(int op,
     if (int rc = check_shape(ashape, adims, "kth_binary(a)", &an)) return rc;
     if (int rc = check_shape(bshape, bdims, "kth_binary(b)", &bn)) return rc;
     if (int rc = check_shape(oshape, odims, "kth_binary(out)", &on)) return rc;
-    Store* sa = lookup(a, "kth_binary(a)");
+    Store* sa = lookup_unsettled(a, "kth_binary(a)");
     if (!sa) return KTH_E_HANDLE;
-    Store* sb = lookup(b, "kth_binary(b)");
+    Store* sb = lookup_unsettled(b, "kth_binary(b)");
     if (!sb) return KTH_E_HANDLE;
-    Store* so = lookup(out, "kth_binary(out)");
+    Store* so = lookup_unsettled(out, "kth_binary(out)");
     if (!so) return KTH_E_HANDLE;
     if (an > sa->n_floats || bn > sb->n_floats || on > so->n_floats)
         return fail(KTH_E_ARGUMENT, "kth_binary: a shape needs more elements than its store holds");
@@ -998,10 +1073,20 @@ int kth_binary(int op,
     if (!all_same && (so->ptr == sa->ptr || so->ptr == sb->ptr))
         return fail(KTH_E_ARGUMENT, "kth_binary: output aliases a broadcast operand");
     if (on == 0) return KTH_OK;
+    // An operand that is one owed constant over its whole shape, whatever that shape, is the scalar
+    // operand of the same functor when the other operand has the output's shape.
+    const bool fold_b = folds_a_constant(op) && sb->fill_n >= bn && bn > 0 && an == on && so != sb && sa != sb;
+    const bool fold_a = !fold_b && folds_a_constant(op) && sa->fill_n >= an && an > 0 && bn == on && so != sa && sa != sb;
+    if (!fold_a) settle(sa);
+    if (!fold_b) settle(sb);
+    if (so != sa && so != sb) settle_for_overwrite(so, on); else settle(so);
     const float* pa = sa->ptr; const float* pb = sb->ptr; float* po = so->ptr;
     const uint32_t n32 = static_cast<uint32_t>(on);
     const float eps = state().epsilon;
-    if (all_same && op == KTH_POW) {
+    if (fold_a || fold_b) {
+        if (fold_b) launch_scalar_op(op, false, pa, po, n32, sb->fill_value, eps);
+        else        launch_scalar_op(op, true, pb, po, n32, sa->fill_value, eps);
+    } else if (all_same && op == KTH_POW) {
         launch_pow(2, pa, pb, po, n32, 0.0f);
     } else if (all_same) {
 #define B(OP) launch_binary_same<OP>(pa, pb, po, n32, eps)
@@ -1053,9 +1138,9 @@ int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
     uint64_t sn, dn;
     if (int rc = check_shape(sshape, sdims, "kth_broadcast_to(src)", &sn)) return rc;
     if (int rc = check_shape(dshape, ddims, "kth_broadcast_to(dst)", &dn)) return rc;
-    Store* ss = lookup(src, "kth_broadcast_to(src)");
+    Store* ss = lookup_unsettled(src, "kth_broadcast_to(src)");
     if (!ss) return KTH_E_HANDLE;
-    Store* sd = lookup(dst, "kth_broadcast_to(dst)");
+    Store* sd = lookup_unsettled(dst, "kth_broadcast_to(dst)");
     if (!sd) return KTH_E_HANDLE;
     if (sn > ss->n_floats || dn > sd->n_floats)
         return fail(KTH_E_ARGUMENT, "kth_broadcast_to: a shape needs more elements than its store holds");
@@ -1067,6 +1152,14 @@ int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
     if (ss->ptr == sd->ptr) return fail(KTH_E_ARGUMENT, "kth_broadcast_to: source and target are the same store");
     plan.a_stream = plan.b_stream = false;
     if (dn == 0) return KTH_OK;
+    const bool constant_source = ss != sd && sn > 0 && ss->fill_n >= sn;
+    if (!constant_source) settle(ss);
+    if (ss != sd) settle_for_overwrite(sd, dn); else settle(sd);
+    if (constant_source) {
+        // every element of the result is the source's one constant: the result is owed the same fill
+        sd->fill_n = dn; sd->fill_value = ss->fill_value;
+        return KTH_OK;
+    }
     if (sn == dn) {
         LaunchScope scope("memcpy_d2d", "", dn * 8);
         KTH_HIP(hipMemcpyAsync(sd->ptr, ss->ptr, dn * 4, hipMemcpyDeviceToDevice, state().stream));

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 template <int MODE, int THREADS>
 __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __restrict__ target, const float* __restrict__ index,
                                                                  const float* __restrict__ src, float value, IndexPlan pl, int* bad,
-                                                                 uint32_t band_len) {
+                                                                 uint32_t band_len, uint32_t from_constant, float constant) {
     extern __shared__ __attribute__((aligned(16))) float row_lds[];
     constexpr uint32_t kFirstEpoch = 0x3ffffeu;               // 22 bits above the 10 bits of a thread id
     static_assert(THREADS <= 1024, "a bid keeps the thread id in 10 bits");
@@ -183,7 +183,9 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         const uint32_t band = min(band_len, pl.a_axis_len - band0);
         float* trow = target + ao + band0;
         if (band0 > 0) __syncthreads();                       // the previous band has left the tile
-        row_to_lds<THREADS>(trow, tile, band);
+        // from_constant: the target is owed a fill with `constant` that was never launched; the rows start from it
+        if (from_constant) { for (uint32_t j = tid; j < band; j += THREADS) tile[j] = constant; }
+        else row_to_lds<THREADS>(trow, tile, band);
         if (MODE == 1) for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
         if (MODE == 1 && tid < 3) any_pending[tid] = 0u;
         uint32_t epoch = kFirstEpoch;                         // MODE 1: the round counter, uniform over the workgroup
@@ -348,6 +350,69 @@ __global__ __launch_bounds__(kBlock) void index_heads_kernel(const uint32_t* __r
     if (i >= k) return;
     const uint32_t key = keys[i];
     flags[i] = (key < axis_len && (i == 0 || keys[i - 1] != key)) ? 1 : 0;
+}
+
+// row_first[r] = where target row r's run starts in the sorted list, ~0u for a row no entry names.
+__global__ __launch_bounds__(kBlock) void index_row_first_clear_kernel(uint32_t* __restrict__ row_first, uint32_t axis_len) {
+    const uint32_t r = blockIdx.x * kBlock + threadIdx.x;
+    if (r < axis_len) row_first[r] = 0xffffffffu;
+}
+__global__ __launch_bounds__(kBlock) void index_row_first_kernel(const uint32_t* __restrict__ keys, uint32_t k, uint32_t axis_len,
+                                                                uint32_t* __restrict__ row_first) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= k) return;
+    const uint32_t key = keys[i];
+    if (key < axis_len && (i == 0 || keys[i - 1] != key)) row_first[key] = i;
+}
+
+// indexAdd into a target that is owed one constant everywhere and holds nothing yet (fresh from
+// zerosLike): one thread per unit (float or float4) of the whole target [outer, axis, inner]. A row that
+// the list names starts from the constant and takes its run's source rows in order, as below; any
+// other row is the constant. Every element is written once and none is read.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                 const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                                                                 const uint32_t* __restrict__ row_first, float alpha, float constant,
+                                                                 uint32_t units, RowsPlan pl, FastDiv axis_div) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= units) return;
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * axis_len + r
+    const uint32_t col = e - row * pl.inner;
+    const uint32_t o = (__umulhi(row, axis_div.mul) + row) >> axis_div.shift;
+    const uint32_t key = row - o * pl.axis_len;
+    uint32_t r = row_first[key];
+    const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
+    if (VEC) {
+        float4 acc = make_float4(constant, constant, constant, constant);
+        if (r != 0xffffffffu) {
+            const float4* s = reinterpret_cast<const float4*>(src) + s_base;
+            float4 v = s[static_cast<size_t>(vals[r]) * pl.inner];
+            while (true) {
+                const bool more = r + 1 < pl.k && keys[r + 1] == key;
+                float4 next = v;
+                if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];     // in flight during the adds
+                acc.x = acc.x + v.x * alpha; acc.y = acc.y + v.y * alpha; acc.z = acc.z + v.z * alpha; acc.w = acc.w + v.w * alpha;
+                if (!more) break;
+                v = next; r++;
+            }
+        }
+        reinterpret_cast<float4*>(target)[e] = acc;
+    } else {
+        float acc = constant;
+        if (r != 0xffffffffu) {
+            const float* s = src + s_base;
+            float v = s[static_cast<size_t>(vals[r]) * pl.inner];
+            while (true) {
+                const bool more = r + 1 < pl.k && keys[r + 1] == key;
+                float next = v;
+                if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];
+                acc = acc + v * alpha;
+                if (!more) break;
+                v = next; r++;
+            }
+        }
+        target[e] = acc;
+    }
 }
 
 // The runs of equal keys are the touched target rows; their first positions (`heads`, *head_count
@@ -588,9 +653,20 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
     });
 }
 
-// Plans and launches on device pointers; shapes are validated by the caller.
+// Whether the scatter takes the row kernel, which rewrites every target row an index position names.
+static bool scatter_takes_rows(int mode, const int32_t* target_shape, const int32_t* index_shape, int dims, int axis) {
+    uint64_t positions = 1;
+    for (int d = 0; d < dims; d++) if (d != axis) positions *= static_cast<uint64_t>(index_shape[d]);
+    return axis == dims - 1 && positions <= 0x7fffffffull &&
+           scatter_rows_fit_lds(mode, static_cast<uint32_t>(target_shape[axis]), static_cast<uint32_t>(index_shape[axis]));
+}
+
+// Plans and launches on device pointers; shapes are validated by the caller. With `constant` the target is
+// taken to hold *constant everywhere without being read (only where scatter_takes_rows holds and the index
+// covers the target off the axis, so that every row is rewritten).
 static int scatter_launch(int mode, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
-                          const float* psrc, const int32_t* src_shape, int dims, int axis, float value, uint64_t idx_n) {
+                          const float* psrc, const int32_t* src_shape, int dims, int axis, float value, uint64_t idx_n,
+                          const float* constant = nullptr) {
     IndexPlan pl{};
     pl.ndim = dims - 1;
     uint64_t positions = 1;
@@ -615,18 +691,21 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
         if (static_cast<uint64_t>(band_len) * per_element > rows_lds_limit()) band_len = (rows_lds_limit() / per_element) & ~3u;
         const uint32_t lds_bytes = band_len * per_element;
         const uint64_t bands = (pl.a_axis_len + band_len - 1) / band_len;
-        const uint64_t row_bytes = (2ull * pl.a_axis_len * positions + bands * (mode == 2 ? 1 : 2) * idx_n) * 4;
+        const uint64_t row_bytes = ((constant ? 1ull : 2ull) * pl.a_axis_len * positions + bands * (mode == 2 ? 1 : 2) * idx_n) * 4;
+        const uint32_t from_constant = constant ? 1u : 0u;
+        const float start = constant ? *constant : 0.0f;
         return with_index_check("Scatter", [&](int* flag) {
             LaunchScope scope("scatter_rows_lds_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", row_bytes);
             const dim3 grid(static_cast<uint32_t>(positions));
             hipStream_t stream = state().stream;
             const float factor = mode == 1 ? 1.0f : value;
-#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag, band_len)
+#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag, band_len, from_constant, start)
             if (lds_bytes > 32768u) { if (mode == 0) ROWS_LAUNCH(0, 1024); else if (mode == 1) ROWS_LAUNCH(1, 1024); else ROWS_LAUNCH(2, 1024); }
             else                    { if (mode == 0) ROWS_LAUNCH(0, 256);  else if (mode == 1) ROWS_LAUNCH(1, 256);  else ROWS_LAUNCH(2, 256); }
 #undef ROWS_LAUNCH
         });
     }
+    if (constant) return fail(KTH_E_ARGUMENT, "kth_scatter: internal: the serial form cannot start from a constant");
     return with_index_check("Scatter", [&](int* flag) {
         LaunchScope scope("scatter_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
         const dim3 grid(blocks), block(kBlock);
@@ -656,7 +735,7 @@ static bool scatter_pays_transposing(int mode, const int32_t* target_shape, cons
 
 static int scatter_transposed(int mode, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
                               const float* psrc, const int32_t* src_shape, int dims, int axis, float value,
-                              uint64_t t_n, uint64_t idx_n, uint64_t src_n) {
+                              uint64_t t_n, uint64_t idx_n, uint64_t src_n, const float* constant) {
     int32_t to_last[KTH_MAX_DIMS], from_last[KTH_MAX_DIMS];          // axis -> innermost, and back
     int32_t t_shape[KTH_MAX_DIMS], i_shape[KTH_MAX_DIMS], s_shape[KTH_MAX_DIMS];
     for (int d = 0, k = 0; d < dims; d++) if (d != axis) to_last[k++] = d;
@@ -673,11 +752,12 @@ static int scatter_transposed(int mode, float* target, const int32_t* target_sha
     float* s_moved = (i_moved && mode != 2) ? workspace_acquire(src_n * 4, &s_cap) : nullptr;
     int rc = KTH_E_MEMORY;
     if (t_moved && i_moved && (mode == 2 || s_moved)) {
-        rc = permute_device("kth_scatter", target, t_moved, target_shape, dims, to_last);
+        // a target that is one owed constant has nothing to bring along: its rows start from the constant
+        rc = constant ? KTH_OK : permute_device("kth_scatter", target, t_moved, target_shape, dims, to_last);
         if (rc == KTH_OK) rc = permute_device("kth_scatter", index, i_moved, index_shape, dims, to_last);
         if (rc == KTH_OK && mode != 2) rc = permute_device("kth_scatter", psrc, s_moved, src_shape, dims, to_last);
         if (rc == KTH_OK) {
-            rc = scatter_launch(mode, t_moved, t_shape, i_moved, i_shape, s_moved, s_shape, dims, dims - 1, value, idx_n);
+            rc = scatter_launch(mode, t_moved, t_shape, i_moved, i_shape, s_moved, s_shape, dims, dims - 1, value, idx_n, constant);
             // also after a reported index: the valid entries have been applied, as in the serial form
             if (rc == KTH_OK || rc == KTH_E_ARGUMENT) {
                 const int back = permute_device("kth_scatter", t_moved, target, t_shape, dims, from_last);
@@ -707,7 +787,7 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
         if (d != axis && index_shape[d] > target_shape[d])
             return fail(KTH_E_SHAPE, "Scatter requires that index.shape[a] <= target.shape[a] for all axis 'a' except the specified axis");
     }
-    Store* st = lookup(target, "kth_scatter(target)");
+    Store* st = lookup_unsettled(target, "kth_scatter(target)");
     if (!st) return KTH_E_HANDLE;
     Store* sx = lookup(index, "kth_scatter(index)");
     if (!sx) return KTH_E_HANDLE;
@@ -718,11 +798,22 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
     if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
     if (idx_n == 0) return KTH_OK;
     const float* psrc = ss ? ss->ptr : nullptr;
-    if (scatter_pays_transposing(mode, target_shape, index_shape, dims, axis, t_n, idx_n, src_n))
-        if (int rc = scatter_transposed(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value,
-                                        t_n, idx_n, src_n); rc != KTH_E_MEMORY)
-            return rc;                                   // no room for the transposed copies: the serial form below
-    return scatter_launch(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value, idx_n);
+    // A target that is still an owed constant (fresh from zerosLike) need not be filled and read back
+    // when the row kernel rewrites all of it: the index covers every position off the axis.
+    const bool transposing = scatter_pays_transposing(mode, target_shape, index_shape, dims, axis, t_n, idx_n, src_n);
+    bool from_constant = st->fill_n == t_n && (transposing || scatter_takes_rows(mode, target_shape, index_shape, dims, axis));
+    for (int d = 0; d < dims; d++) if (d != axis && index_shape[d] != target_shape[d]) from_constant = false;
+    const float constant = st->fill_value;
+    if (!from_constant) settle(st);
+    if (transposing) {
+        const int rc = scatter_transposed(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value,
+                                          t_n, idx_n, src_n, from_constant ? &constant : nullptr);
+        if (rc != KTH_E_MEMORY) { if (from_constant) st->fill_n = 0; return rc; }
+        if (from_constant) { settle(st); from_constant = false; }      // no room for the transposed copies: the serial form below
+    }
+    if (from_constant) st->fill_n = 0;
+    return scatter_launch(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value, idx_n,
+                          from_constant ? &constant : nullptr);
 }
 
 int kth_scatter(int add, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
@@ -818,7 +909,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (int rc = rows_geometry("kth_index_add", shape, dims, axis, &outer, &inner, &total)) return rc;
     const uint64_t n_src = outer * k * inner;
     if (n_src > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_add: more than 2^31-1 source elements");
-    Store* st = lookup(target, "kth_index_add(target)");
+    Store* st = lookup_unsettled(target, "kth_index_add(target)");
     if (!st) return KTH_E_HANDLE;
     Store* sx = lookup(index, "kth_index_add(index)");
     if (!sx) return KTH_E_HANDLE;
@@ -829,6 +920,12 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (st->ptr == sx->ptr || st->ptr == ss->ptr) return fail(KTH_E_ARGUMENT, "kth_index_add: target aliases an input");
     const uint64_t positions = outer * inner;
     if (positions == 0 || k == 0) return KTH_OK;
+    // A target that is one owed constant (fresh from zerosLike) and a list long enough to be sorted: the
+    // rows are written from the constant, nothing of the target is read. Every other case has the fill launched.
+    const bool vec_inner = inner % 4 == 0;
+    const bool from_constant = st->fill_n == total && k >= 64 && total / (vec_inner ? 4 : 1) <= kMaxElements;
+    const float constant = st->fill_value;
+    if (!from_constant) settle(st);
     RowsPlan pl{};
     pl.axis_len = static_cast<uint32_t>(shape[axis]); pl.k = static_cast<uint32_t>(k); pl.inner = static_cast<uint32_t>(inner);
     pl.inner_div = make_div(pl.inner); pl.k_div = make_div(pl.k);
@@ -839,6 +936,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     // list of 1.1 million takes 43 ms here and a few hundred microseconds sorted)
     const bool rows_pay = outer >= static_cast<uint64_t>(state().compute_units) || k < 4096;
     if (inner == 1 && rows_pay && scatter_rows_fit_lds(1, pl.axis_len, pl.k)) {
+        if (from_constant) st->fill_n = 0;                   // every row of the target is rewritten from the constant
         // columns added into contiguous rows: the scatter row kernel in its add form, one index row for
         // every position and alpha as the factor on the source
         IndexPlan rp{};
@@ -854,9 +952,9 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
             LaunchScope scope("scatter_rows_lds_kernel", "indexAdd", (2 * total + n_src + k) * 4);
             const dim3 grid(static_cast<uint32_t>(outer));
             if (lds_bytes > 32768u)
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant);
             else
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant);
         });
     }
 
@@ -876,11 +974,14 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
         select_flagged_positions(nullptr, &select_bytes, nullptr, nullptr, nullptr, pl.k, stream) == hipSuccess) {
         if (select_bytes > temp_bytes) temp_bytes = select_bytes;           // the two passes share their scratch
         temp_bytes = (temp_bytes + 255) & ~static_cast<size_t>(255);
-        // keys, vals, sorted keys, sorted vals, heads: k_pad each; count: 64; flags: k_pad bytes
-        keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 64 * 4 + k_pad + temp_bytes, &cap));
+        // keys, vals, sorted keys, sorted vals, heads: k_pad each; count: 64; flags: k_pad bytes; then, for a target
+        // written from a constant, the first list position of every target row
+        keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 64 * 4 + k_pad + temp_bytes +
+                                                             (from_constant ? (static_cast<uint64_t>(pl.axis_len) + 64) * 4 : 0), &cap));
     }
     if (!keys) {
         (void)hipGetLastError();
+        if (from_constant) settle(st);
         const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
         return with_index_check("Index Add", [&](int* flag) {
             LaunchScope scope("index_add_kernel", "", 3 * n_src * 4 + k * 4);
@@ -895,6 +996,33 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     uint32_t* head_count = heads + k_pad;
     void* temp = head_count + 64;
     uint8_t* flags = reinterpret_cast<uint8_t*>(temp) + temp_bytes;
+    if (from_constant) {
+        uint32_t* row_first = reinterpret_cast<uint32_t*>(flags + k_pad);
+        if (vec_inner) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }
+        const uint32_t units = static_cast<uint32_t>(total / (vec_inner ? 4 : 1));
+        hipError_t sort_status = hipSuccess;
+        int rc = with_index_check("Index Add", [&](int* flag) {
+            {
+                LaunchScope scope("index_sort", "", k * 4 * 7);
+                hipLaunchKernelGGL(index_keys_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, sx->ptr, pl.k,
+                                   pl.axis_len, keys, vals, flag);
+                size_t scratch = temp_bytes;
+                sort_status = sort_pairs_u32(temp, &scratch, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
+                if (sort_status != hipSuccess) return;
+                hipLaunchKernelGGL(index_row_first_clear_kernel, dim3((pl.axis_len + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, row_first, pl.axis_len);
+                hipLaunchKernelGGL(index_row_first_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, row_first);
+            }
+            LaunchScope scope("index_add_filled_kernel", vec_inner ? "float4" : "float", (total + n_src) * 4 + k * 4);
+            const dim3 grid((units + kBlock - 1) / kBlock);
+            const FastDiv axis_div = make_div(pl.axis_len);
+            if (vec_inner) hipLaunchKernelGGL((index_add_filled_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, row_first, alpha, constant, units, pl, axis_div);
+            else           hipLaunchKernelGGL((index_add_filled_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, row_first, alpha, constant, units, pl, axis_div);
+        });
+        workspace_release(reinterpret_cast<float*>(keys), cap);
+        if (sort_status != hipSuccess) { return fail(KTH_E_DEVICE, "kth_index_add: sorting the index list failed: %s", hipGetErrorString(sort_status)); }
+        st->fill_n = 0;
+        return rc;
+    }
     const bool vec = inner % 4 == 0;
     const bool ragged = !vec && inner > 4 && outer * k * ((inner + 3) / 4) <= kMaxElements;
     if (vec) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }

@@ -22,6 +22,13 @@ struct Store {
     uint64_t cap_bytes = 0;
     uint32_t refs = 0;
     uint32_t generation = 0;   // bumped on release so stale handles are detected
+    // A fill that has not been launched yet: floats [0, fill_n) are to hold fill_value (0 = nothing owed).
+    // kth_fill over a store's head and the upload of one value leave this note instead of a kernel;
+    // `settle` launches the fill, `lookup` settles before it returns, and the few callers that can fold the
+    // constant into their own kernel (a binary op takes it as a scalar operand, a scatter starts its rows from it,
+    // a broadcast passes it on) take the store with `lookup_unsettled` and clear or keep the note themselves.
+    uint64_t fill_n = 0;
+    float    fill_value = 0.0f;
 };
 
 // One profiled launch: which kernel, the algorithmic bytes it moved, its event pair.
@@ -80,8 +87,17 @@ std::mutex& lock();
 // Records the message for kth_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);
 
-// Handle -> store, or nullptr (with the error recorded).
+// Handle -> store, or nullptr (with the error recorded). A fill the store is owed is launched first.
 Store* lookup(uint64_t handle, const char* what);
+// The same without launching an owed fill: for callers that fold, overwrite or drop it.
+Store* lookup_unsettled(uint64_t handle, const char* what);
+// Launches the fill the store is owed, if any, on the library's stream.
+void settle(Store* st);
+// The store is about to be written over floats [0, n) by a kernel that reads none of them: an owed
+// fill that this covers is dropped, a longer one is launched first.
+void settle_for_overwrite(Store* st, uint64_t n);
+// fill_kernel over p[0, n) on the library's stream (kth_elementwise.hip).
+void launch_fill(float* p, uint64_t n, float value);
 
 // Pool-backed raw device memory for kernels' own workspaces (partials of two-pass
 // reductions). Stream-ordered: a workspace returned to the pool may be reused by a

@@ -846,9 +846,9 @@ int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_
 // The argument checks of both axis entry points, then the launch.
 int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
     if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "%s: op %d is not an aggregating operation", who, op);
-    Store* si = lookup(in, who);
+    Store* si = lookup_unsettled(in, who);
     if (!si) return KTH_E_HANDLE;
-    Store* so = lookup(out, who);
+    Store* so = lookup_unsettled(out, who);
     if (!so) return KTH_E_HANDLE;
     if (axis == 0) return fail(KTH_E_ARGUMENT, "%s: empty axis", who);
     if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
@@ -861,8 +861,23 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
                     (unsigned long long)axis, (unsigned long long)inner);
     if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", who);
     if (outer * inner == 0) return KTH_OK;
-    return dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
-                           static_cast<uint32_t>(inner), use_static);
+    const uint64_t owed_n = so->fill_n;
+    const float owed_value = so->fill_value;
+    {
+        // A fill the input is still owed is launched here, one the output is owed is dropped if the result
+        // covers it; for the entry point that creates nothing, without the event pair of a running profile.
+        State& s = state();
+        const bool profiling = s.profiling;
+        if (use_static) s.profiling = false;
+        settle(si);
+        settle_for_overwrite(so, outer * inner);
+        s.profiling = profiling;
+    }
+    const int rc = dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
+                                   static_cast<uint32_t>(inner), use_static);
+    // a refused plan has written nothing: the output is still owed what it was owed
+    if (rc != KTH_OK && owed_n != 0 && so->fill_n == 0) { so->fill_n = owed_n; so->fill_value = owed_value; }
+    return rc;
 }
 
 }  // namespace

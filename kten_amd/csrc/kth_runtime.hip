@@ -27,7 +27,7 @@ static inline uint64_t make_handle(uint32_t index, uint32_t generation) {
     return (static_cast<uint64_t>(generation) << 32) | static_cast<uint64_t>(index + 1);
 }
 
-Store* lookup(uint64_t handle, const char* what) {
+Store* lookup_unsettled(uint64_t handle, const char* what) {
     State& s = state();
     uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
     uint32_t gen = static_cast<uint32_t>(handle >> 32);
@@ -41,6 +41,24 @@ Store* lookup(uint64_t handle, const char* what) {
         return nullptr;
     }
     return &st;
+}
+
+void settle(Store* st) {
+    if (st->fill_n == 0) return;
+    const uint64_t n = st->fill_n;
+    st->fill_n = 0;
+    launch_fill(st->ptr, n, st->fill_value);
+}
+
+void settle_for_overwrite(Store* st, uint64_t n) {
+    if (st->fill_n <= n) st->fill_n = 0;
+    else settle(st);
+}
+
+Store* lookup(uint64_t handle, const char* what) {
+    Store* st = lookup_unsettled(handle, what);
+    if (st) settle(st);
+    return st;
 }
 
 // Size classes: 512-byte granules up to 1 MiB, then 1/8-octave steps (at most 12.5 %
@@ -262,7 +280,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
     if (!s.free_slots.empty()) { idx = s.free_slots.back(); s.free_slots.pop_back(); }
     else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); s.table.back().generation = g_epoch << 20; }
     Store& st = s.table[idx];
-    st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1;
+    st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1; st.fill_n = 0;
     s.live_bytes += cap;
     *handle = make_handle(idx, st.generation);
     return KTH_OK;
@@ -271,7 +289,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
 int kth_retain(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup(handle, "kth_retain");
+    Store* st = lookup_unsettled(handle, "kth_retain");
     if (!st) return KTH_E_HANDLE;
     st->refs += 1;
     return KTH_OK;
@@ -280,7 +298,7 @@ int kth_retain(uint64_t handle) {
 int kth_release(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup(handle, "kth_release");
+    Store* st = lookup_unsettled(handle, "kth_release");      // a fill nobody read is never launched
     if (!st) return KTH_E_HANDLE;
     st->refs -= 1;
     if (st->refs == 0) {
@@ -289,6 +307,7 @@ int kth_release(uint64_t handle) {
         s.live_bytes -= st->cap_bytes;
         s.pool_bytes += st->cap_bytes;
         st->ptr = nullptr;
+        st->fill_n = 0;
         st->generation += 1;
         s.free_slots.push_back(static_cast<uint32_t>((handle & 0xffffffffu) - 1));
     }
@@ -305,12 +324,19 @@ static int check_range(const Store* st, uint64_t off, uint64_t n, const char* wh
 int kth_upload(uint64_t handle, uint64_t offset, const float* src, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup(handle, "kth_upload");
+    Store* st = lookup_unsettled(handle, "kth_upload");
     if (!st) return KTH_E_HANDLE;
     if (int rc = check_range(st, offset, n, "kth_upload")) return rc;
     if (n == 0) return KTH_OK;
     if (!src) return fail(KTH_E_ARGUMENT, "kth_upload: null source");
     State& s = state();
+    if (offset == 0) settle_for_overwrite(st, n); else settle(st);
+    if (n == 1 && offset == 0) {
+        // One value (a [1]-shaped seed gradient, a scalar operand) is a fill of one float: noted, and
+        // launched only if somebody reads the store as memory.
+        st->fill_n = 1; st->fill_value = src[0];
+        return KTH_OK;
+    }
     if (n <= kConstFloats) {
         // A few values (a [1]-shaped seed gradient, a scalar operand): they ride in the
         // kernel arguments, so nothing blocks and no staging memory is involved.
@@ -398,13 +424,21 @@ __global__ __launch_bounds__(256) void copy_any_kernel(const float* __restrict__
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* d = lookup(dst, "kth_copy(dst)");
+    Store* d = lookup_unsettled(dst, "kth_copy(dst)");
     if (!d) return KTH_E_HANDLE;
-    Store* sst = lookup(src, "kth_copy(src)");
+    Store* sst = lookup_unsettled(src, "kth_copy(src)");
     if (!sst) return KTH_E_HANDLE;
     if (int rc = check_range(d, dst_offset, n, "kth_copy(dst)")) return rc;
     if (int rc = check_range(sst, src_offset, n, "kth_copy(src)")) return rc;
     if (n == 0) return KTH_OK;
+    if (d != sst && dst_offset == 0 && sst->fill_n >= src_offset + n) {
+        // a copy of floats that are all one owed constant: the head of the destination is owed it too
+        settle_for_overwrite(d, n);
+        d->fill_n = n; d->fill_value = sst->fill_value;
+        return KTH_OK;
+    }
+    settle(sst);
+    if (d != sst && dst_offset == 0) settle_for_overwrite(d, n); else settle(d);
     if (d->ptr == sst->ptr) {
         uint64_t lo = dst_offset < src_offset ? dst_offset : src_offset;
         uint64_t hi = dst_offset < src_offset ? src_offset : dst_offset;

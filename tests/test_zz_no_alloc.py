@@ -92,6 +92,7 @@ def test_static_reduction_refuses_what_does_not_fit(gc):
     shape = [128, 200000]
     t = gc.createRawFill(shape, 1.0)
     out = gc.createRawFill([1, 200000], -7.0)
+    assert t.getSingleValue([0, 0]) == 1.0                    # the input is in memory, not a fill still to be launched
     launches = gc.getMetrics()["launches"]
     rc = gc.lib.kth_reduce_axis_static(Op.SUM, t.storeReference, out.storeReference, 1, 128, 200000)
     assert rc == -3, "a plan beyond the scratch array must return KTH_E_ARGUMENT"
