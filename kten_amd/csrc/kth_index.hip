@@ -503,7 +503,6 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_ragged_kernel(float* 
     else for (uint32_t j = 0; j < cnt; j++) t[j] = acc[j];
 }
 
-__global__ void clear_int_kernel(int* p) { *p = 0; }
 
 int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
     if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
@@ -539,16 +538,13 @@ int with_index_check(const char* what, F launch) {
         if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
         return KTH_OK;
     }
-    uint64_t cap;
-    int* flag = reinterpret_cast<int*>(workspace_acquire(4, &cap));
-    if (!flag) return fail(KTH_E_MEMORY, "%s: no workspace", what);
-    hipLaunchKernelGGL(clear_int_kernel, dim3(1), dim3(1), 0, s.stream, flag);
-    launch(flag);
+    // immediate: the kernels write a word of pinned host memory, read here once the stream has drained (the
+    // word is zero whenever no indexed move is in flight: only this function lets kernels at it, and it waits)
+    launch(s.host_index_flag_device);
     hipError_t e = hipGetLastError();
-    int host_flag = 0;
-    if (e == hipSuccess) e = hipMemcpyAsync(&host_flag, flag, 4, hipMemcpyDeviceToHost, s.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
-    workspace_release(reinterpret_cast<float*>(flag), cap);
+    const int host_flag = *s.host_index_flag;
+    *s.host_index_flag = 0;
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
     if (host_flag) return fail(KTH_E_ARGUMENT, "%s got invalid index, an index value is out of bounds at the axis", what);
     return KTH_OK;

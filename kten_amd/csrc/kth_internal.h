@@ -73,6 +73,10 @@ struct State {
     // flag; otherwise the kernels set this persistent device word and the next blocking call reports it.
     bool index_check_immediate = true;
     int* deferred_index_flag = nullptr;
+    // immediate checking: a word of pinned host memory that the kernels write directly (and its device address),
+    // so that the check costs one wait for the stream and neither a clearing kernel nor a copy back
+    volatile int* host_index_flag = nullptr;
+    int*          host_index_flag_device = nullptr;
 
     std::vector<hipEvent_t> laps;           // kth_timer_lap events not yet read by kth_timer_laps
 

@@ -206,6 +206,14 @@ int kth_init(int device) {
     KTH_HIP(reduce_scratch_init(device));
     KTH_HIP(hipMalloc(reinterpret_cast<void**>(&s.deferred_index_flag), 256));
     KTH_HIP(hipMemset(s.deferred_index_flag, 0, 256));
+    {
+        void* host = nullptr; void* dev = nullptr;
+        KTH_HIP(hipHostMalloc(&host, 256, hipHostMallocDefault));
+        KTH_HIP(hipHostGetDevicePointer(&dev, host, 0));
+        s.host_index_flag = static_cast<volatile int*>(host);
+        s.host_index_flag_device = static_cast<int*>(dev);
+        *s.host_index_flag = 0;
+    }
     s.device = device;
     s.ready = true;
     g_epoch += 1;
@@ -223,6 +231,8 @@ int kth_shutdown(void) {
     s.free_slots.clear();
     trim_pool();
     if (s.deferred_index_flag) (void)hipFree(s.deferred_index_flag);
+    if (s.host_index_flag) (void)hipHostFree(const_cast<int*>(s.host_index_flag));
+    s.host_index_flag = nullptr; s.host_index_flag_device = nullptr;
     for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
     for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
     for (hipEvent_t e : s.laps) (void)hipEventDestroy(e);
