@@ -5,10 +5,17 @@
                   [--no-kernel-events] [--no-cold] [--no-copy-ceiling]
 
 A step is one pass of the chosen workload's raw-op sequence over device-resident
-synthetic inputs (kten_amd/workloads.py). The default workload is cfg5: the autograd
+synthetic inputs (kten_amd/host_mirror/workloads.py). The default workload is cfg5: the autograd
 forward + backward of loss = sum(((x*w)+b) pow 2) on x[16384,4096], which exercises
 broadcast binary ops, tensor-scalar ops, the full sum and the reduce-to-shape axis sums.
 Prints ONE JSON line on stdout; everything else goes to stderr.
+
+`value` = bytes per step / time per step, with the bytes taken as the smaller of two totals: the
+op-at-a-time total of the reference's op list (operands at their un-broadcast size, every result
+once) and what the library's launches of that step really read and wrote. The second is smaller
+where a tensor that is one constant (a fresh zerosLike, the broadcast seed gradient) is never
+written out and read back; bytes that did not cross the memory bus are not counted as bandwidth.
+`config` carries both totals and both rates.
 
 Timing: a HIP event on the library's own stream before the first and after every one of the K
 timed steps (kth_timer_lap): `value` comes from the time between the first and the last event,
@@ -39,6 +46,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 # Transcribed from the profile named beside it; this run does not measure it.
 MEASURED_TRAFFIC_BYTES = {
     ("cfg5", "binary_same_kernel<OpTimes>"): 147 * 64 + 4194304 * 128 + 4194304 * 64,
+    ("cfg5", "binary_bcast_vec_kernel_vv<OpTimes>"): 315 * 64 + 2097830 * 128 + 4194304 * 64,
 }
 TRAFFIC_SOURCE = ("profiles/cfg5_autograd_kernels.md (rocprofv3 --pmc TCC_EA0_RDREQ_{32B,64B,128B}_sum, TCC_EA0_WRREQ_{,64B}_sum of an "
                   "earlier run: requests times their sizes; transcribed, not measured by this run)")
@@ -127,6 +135,11 @@ def cold_probe(ops, kernel, nbytes_per_launch, dims, sets=8, rounds=3):
         make = lambda: (tensor(n), tensor(n), ops.createRaw([n]))
         sh = abi.shape_array([n])
         run = lambda s: check(lib.kth_binary(binary[op], s[0].storeReference, sh, 1, s[1].storeReference, sh, 1, s[2].storeReference, sh, 1))
+    elif family == "binary_bcast_vec_kernel_vv" and op in binary and "rows" in dims and "cols" in dims:
+        rows, cols = dims["rows"], dims["cols"]                      # [rows, cols] (op) [cols]
+        make = lambda: (tensor(rows * cols), tensor(cols), ops.createRaw([rows * cols]))
+        sa, sb = abi.shape_array([rows, cols]), abi.shape_array([cols])
+        run = lambda s: check(lib.kth_binary(binary[op], s[0].storeReference, sa, 2, s[1].storeReference, sb, 1, s[2].storeReference, sa, 2))
     elif family in ("unary_kernel", "unary_lds_kernel") and (op in unary or op in ("OpSquare", "OpIdentity")):
         n = nbytes_per_launch // 8
         make = lambda: (tensor(n), ops.createRaw([n]))
@@ -239,7 +252,11 @@ def main():
     counted = (m["bytesMoved"] - m0["bytesMoved"]) / args.steps
     launches = (m["launches"] - m0["launches"]) / args.steps
     ms_per_step = total_ms / args.steps
-    gbps = nbytes / ms_per_step / 1e6
+    # `value` never counts bytes that were not moved: where the library folds a constant tensor into its
+    # consumer (no fill written, no operand read) its launches move less than the reference's op list names,
+    # and the rate is taken on what they moved. Where they move more (transposed copies), the op list stands.
+    algorithmic_gbps = nbytes / ms_per_step / 1e6
+    gbps = min(nbytes, counted) / ms_per_step / 1e6
     log(f"{args.steps} steps: {total_ms:.3f} ms on the stream ({ms_per_step:.4f} ms/step mean, {median_ms:.4f} median, "
         f"{min_ms:.4f} min), {wall_ms:.3f} ms wall; {launches:.0f} launches/step; "
         f"library counted {counted:.0f} B/step (formula {nbytes})")
@@ -297,17 +314,20 @@ def main():
         "config": {"workload": f"{wl.name}: {wl.description}", "algorithmic_bytes_per_step": nbytes,
                    "fused_lower_bound_bytes": wl.fused_lower_bound_bytes(dims) if wl.fused_lower_bound_bytes else None,
                    "launches_per_step": launches,
-                   "fp32_elements_per_s": round(nbytes / 4 / (ms_per_step / 1e3)),
-                   "fp32_elements_per_s_means": "algorithmic bytes / 4 per second: every fp32 value a raw op reads or writes",
+                   "fp32_elements_per_s": round(min(nbytes, counted) / 4 / (ms_per_step / 1e3)),
+                   "fp32_elements_per_s_means": "the bytes of `value` / 4 per second: every fp32 value a launch reads or writes",
                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
                    "moved_bytes_per_step": round(counted),
                    "GBps_on_moved_bytes": round(counted / ms_per_step / 1e6, 1),
-                   "frac_of_hbm_peak_on_moved_bytes": round(counted / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4),
-                   "moved_bytes_means": "what the library's launches of one step read and wrote, summed from their own byte counts; "
-                                        "`value` uses the op-at-a-time byte total of the reference's op list instead. The two differ "
-                                        "where the library does not write out a tensor that is one constant (a fresh zerosLike, the "
-                                        "broadcast seed gradient) and hands the constant to the consumer's kernel, and where it moves "
-                                        "more than the op list names (transposed copies of a scatter along an outer axis)",
+                   "GBps_on_the_op_list": round(algorithmic_gbps, 1),
+                   "value_means": "min(algorithmic_bytes_per_step, moved_bytes_per_step) / ms_per_step. moved_bytes_per_step is what "
+                                  "the library's launches of one step read and wrote, summed from their own byte counts; "
+                                  "algorithmic_bytes_per_step is the op-at-a-time total of the reference's op list. The two differ "
+                                  "where the library does not write out a tensor that is one constant (a fresh zerosLike, the "
+                                  "broadcast seed gradient) and hands the constant to the consumer's kernel (fewer bytes moved: "
+                                  "GBps_on_the_op_list would count bytes that never crossed the memory bus, ms_per_step shows the "
+                                  "gain), and where it moves more than the op list names (transposed copies of a scatter along an "
+                                  "outer axis)",
                    "wall_ms_per_step": round(wall_ms / args.steps, 4),
                    "per_kernel_durations": "HIP event pair around every launch, over a second pass of the same K steps"
                    if args.events else None},
