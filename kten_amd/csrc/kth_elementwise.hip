@@ -603,23 +603,39 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
     // 16 bytes per thread (its four outputs are neighbours there too, except where the span passes its end)
     const bool staged = pl.span <= len;
     if (staged) stage_range(col_lds, 0, colp, 0, pl.span);
+    // a column operand read from memory: all of a thread's loads are issued before the first is used
+    constexpr uint32_t kGroups = kOuterTile / (kBlock * 4);
+    v4f_unaligned ahead[kGroups];
+    if (!staged) {
+#pragma unroll
+        for (uint32_t k = 0; k < kGroups; k++) {
+            const uint32_t g = threadIdx.x * 4 + k * kBlock * 4;
+            if (g < len) {
+                const uint32_t e0 = s + g;
+                const uint32_t i = (__umulhi(e0, pl.span_div.mul) + e0) >> pl.span_div.shift;
+                const uint32_t c = e0 - i * pl.span;
+                if (c + 4 <= pl.span) ahead[k] = *reinterpret_cast<const v4f_unaligned*>(colp + c);
+                else {
+                    float t[4];
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; j++) t[j] = colp[c + j < pl.span ? c + j : c + j - pl.span];
+                    ahead[k] = v4f_unaligned{t[0], t[1], t[2], t[3]};
+                }
+            }
+        }
+    }
     __syncthreads();
-    for (uint32_t g = threadIdx.x * 4; g < len; g += kBlock * 4) {
+#pragma unroll
+    for (uint32_t k = 0; k < kGroups; k++) {
+        const uint32_t g = threadIdx.x * 4 + k * kBlock * 4;
+        if (g >= len) break;
         const uint32_t e0 = s + g;
         const uint32_t i = (__umulhi(e0, pl.span_div.mul) + e0) >> pl.span_div.shift;
         uint32_t c = e0 - i * pl.span;                                     // column operand offset j * V + v
         uint32_t v = c - ((__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift) * pl.run;
         uint32_t row_base = (i - i_lo) * pl.run;
-        float y[4];
-        if (!staged) {
-            if (c + 4 <= pl.span) {
-                const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(colp + c);
-                y[0] = t.x; y[1] = t.y; y[2] = t.z; y[3] = t.w;
-            } else {
-#pragma unroll
-                for (uint32_t j = 0; j < 4; j++) y[j] = colp[c + j < pl.span ? c + j : c + j - pl.span];
-            }
-        }
+        float y[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (!staged) { y[0] = ahead[k].x; y[1] = ahead[k].y; y[2] = ahead[k].z; y[3] = ahead[k].w; }
         float r[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -632,6 +648,50 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
         }
         if (g + 4 <= len) st4(out, e0 >> 2, make_float4(r[0], r[1], r[2], r[3]));
         else for (uint32_t j = 0; g + j < len; j++) out[e0 + j] = r[j];
+    }
+}
+
+// The same operands when the column operand is longer than a tile (span > kOuterTile): a workgroup takes a
+// block of kOuterRows row indexes by kOuterCols column offsets, so that a thread's 16 bytes of the column operand
+// are loaded once and serve kOuterRows output rows, and nothing but the row index changes between its stores.
+// The rows' slice of the row operand (kOuterRows * run floats) is staged in LDS. Grid: (column blocks, row blocks).
+constexpr uint32_t kOuterRows = 8;
+constexpr uint32_t kOuterCols = kOuterTile / kOuterRows;      // 1024 column offsets: four per thread
+template <class Op>
+__global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                  float* __restrict__ out, float eps, OuterPlan pl, uint32_t rows) {
+    extern __shared__ float outer_rows_lds[];
+    const float* rowp = pl.a_is_row ? a : b;
+    const float* colp = pl.a_is_row ? b : a;
+    const uint32_t i0 = blockIdx.y * kOuterRows;
+    const uint32_t nrows = min(kOuterRows, rows - i0);
+    const uint32_t c0 = blockIdx.x * kOuterCols + threadIdx.x * 4;
+    float y[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t count = 0;                                        // column offsets of this thread inside the span
+    if (c0 < pl.span) {
+        count = min(4u, pl.span - c0);
+        if (count == 4) {
+            const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(colp + c0);
+            y[0] = t.x; y[1] = t.y; y[2] = t.z; y[3] = t.w;
+        } else {
+            for (uint32_t j = 0; j < count; j++) y[j] = colp[c0 + j];
+        }
+    }
+    stage_range(outer_rows_lds, 0, rowp, i0 * pl.run, nrows * pl.run);
+    __syncthreads();
+    if (count == 0) return;
+    uint32_t v[4];
+    v[0] = c0 - ((__umulhi(c0, pl.run_div.mul) + c0) >> pl.run_div.shift) * pl.run;
+#pragma unroll
+    for (int j = 1; j < 4; j++) { v[j] = v[j - 1] + 1; if (v[j] == pl.run) v[j] = 0; }
+    for (uint32_t r = 0; r < nrows; r++) {
+        const float* xs = outer_rows_lds + r * pl.run;
+        float res[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) res[j] = pl.a_is_row ? Op::apply(xs[v[j]], y[j], eps) : Op::apply(y[j], xs[v[j]], eps);
+        float* to = out + static_cast<size_t>(i0 + r) * pl.span + c0;
+        if (count == 4) *reinterpret_cast<v4f_unaligned*>(to) = v4f_unaligned{res[0], res[1], res[2], res[3]};
+        else for (uint32_t j = 0; j < count; j++) to[j] = res[j];
     }
 }
 
@@ -787,6 +847,13 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
             op.n = n; op.run = run; op.span = plan.size[d - 2] * run; op.a_is_row = a_row ? 1u : 0u;
             op.span_div = make_div(op.span); op.run_div = make_div(run);
             op.row_lds = (((kOuterTile - 1) / op.span + 2) * run + 3u) & ~3u;
+            const uint32_t rows = plan.size[d - 1];
+            if (op.span >= 2048u && rows <= 65535u * kOuterRows) {
+                LaunchScope scope("binary_outer_rows_kernel", Op::name, bytes);
+                const dim3 grid((op.span + kOuterCols - 1) / kOuterCols, (rows + kOuterRows - 1) / kOuterRows);
+                hipLaunchKernelGGL((binary_outer_rows_kernel<Op>), grid, dim3(kBlock), kOuterRows * run * sizeof(float), st, a, b, out, eps, op, rows);
+                return;
+            }
             const uint32_t col_lds = op.span <= kOuterTile ? op.span : 4u;      // a longer column operand is not staged
             LaunchScope scope("binary_outer_kernel", Op::name, bytes);
             hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((n + kOuterTile - 1) / kOuterTile), dim3(kBlock),
