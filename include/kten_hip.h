@@ -191,8 +191,9 @@ int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
  * events (its launches are counted by kth_metrics but left out of a kth_profile recording).
  * A shape whose plan needs more partial bytes than the array holds (outputs x axis segments
  * x 8 bytes; only reductions whose outputs alone cannot fill the device are cut into
- * segments) returns KTH_E_ARGUMENT before anything is launched; single-pass shapes of any
- * size are accepted. Every call on a device shares that device's array, which keeps the last
+ * segments) returns KTH_E_ARGUMENT before any reduction kernel is launched; single-pass shapes of any
+ * size are accepted. An input that is a noted constant (see kth_fill) has its fill launched first:
+ * a kernel launch into the store's own memory, nothing is allocated for it. Every call on a device shares that device's array, which keeps the last
  * call's partials; nothing in it needs clearing because every partial is written before it is
  * read. The library's mutex and its one in-order stream keep calls of one process apart;
  * anything that made two such calls overlap on one GPU would race on the array. */
