@@ -163,7 +163,8 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
 template <int MODE, int THREADS>
 __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __restrict__ target, const float* __restrict__ index,
                                                                  const float* __restrict__ src, float value, IndexPlan pl, int* bad,
-                                                                 uint32_t band_len, uint32_t from_constant, float constant) {
+                                                                 uint32_t band_len, uint32_t from_constant, float constant,
+                                                                 uint32_t tag_slots, FastDiv tag_div) {
     extern __shared__ __attribute__((aligned(16))) float row_lds[];
     constexpr uint32_t kFirstEpoch = 0x3ffffeu;               // 22 bits above the 10 bits of a thread id
     static_assert(THREADS <= 1024, "a bid keeps the thread id in 10 bits");
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         // from_constant: the target is owed a fill with `constant` that was never launched; the rows start from it
         if (from_constant) { for (uint32_t j = tid; j < band; j += THREADS) tile[j] = constant; }
         else row_to_lds<THREADS>(trow, tile, band);
-        if (MODE == 1) for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
+        if (MODE == 1) for (uint32_t j = tid; j < tag_slots; j += THREADS) tag[j] = 0xffffffffu;
         if (MODE == 1 && tid < 3) any_pending[tid] = 0u;
         uint32_t epoch = kFirstEpoch;                         // MODE 1: the round counter, uniform over the workgroup
         // the first chunk's entries are fetched while the row arrives
@@ -223,16 +224,20 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                 // (same round, lower tid): the order is kept.
                 if (epoch < 2u * THREADS + 4u) {              // (only after millions of rounds on one band)
                     __syncthreads();
-                    for (uint32_t j = tid; j < band; j += THREADS) tag[j] = 0xffffffffu;
+                    for (uint32_t j = tid; j < tag_slots; j += THREADS) tag[j] = 0xffffffffu;
                     if (tid < 3) any_pending[tid] = 0u;
                     epoch = kFirstEpoch;
                     __syncthreads();
                 }
                 bool pending = have;
+                // fewer tags than elements (tag_slots < band_len): elements share a tag by their remainder. Entries
+                // for one element still meet at one tag; entries for different elements that meet there only wait
+                // a round for each other.
+                const uint32_t at = tag_slots >= band_len ? sel : sel - ((__umulhi(sel, tag_div.mul) + sel) >> tag_div.shift) * tag_slots;
                 for (uint32_t rounds = 0;; rounds++) {
                     const uint32_t bid = (epoch << 10) | tid;
                     const uint32_t slot = epoch % 3u;
-                    if (pending) { atomicMin(&tag[sel], bid); any_pending[slot] = 1u; }
+                    if (pending) { atomicMin(&tag[at], bid); any_pending[slot] = 1u; }
                     // three flags in turn: this round's is read after the barrier; the next round's, last
                     // read two rounds ago (before the previous barrier), is cleared now. The last round's may
                     // still be being read by a slow thread and is left alone. Every round, the last one of a
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                     const bool more = any_pending[slot] != 0u;
                     epoch--;
                     if (!more) break;
-                    if (pending && tag[sel] == bid) {      // one lane per element gets here
+                    if (pending && tag[at] == bid) {       // one lane per tag gets here
                         tile[sel] = tile[sel] + v;
                         pending = false;
                     }
@@ -572,6 +577,32 @@ static uint32_t rows_lds_limit() {
     return limit;
 }
 
+// How a target row of a_axis_len floats sits in LDS: band_len floats of the row at a time (all of it when it
+// fits) and, for the add form, tag_slots tags behind them. A row of up to 8192 floats has a tag per element
+// (64 KiB together: two workgroups on a CU). A longer one is taken up to 16384 floats at a time with
+// kSharedTags tags that its elements share by remainder: 80 KiB less a little, so that two workgroups still fit
+// the CU's 160 KiB and one's rounds of LDS traffic fill the other's waits.
+constexpr uint32_t kSharedTags = 3968;
+static void rows_lds_plan(int mode, uint32_t a_axis_len, uint32_t* band_len, uint32_t* tag_slots, uint32_t* lds_bytes) {
+    const uint32_t limit = rows_lds_limit();
+    if (mode != 1) {
+        *band_len = a_axis_len;
+        if (static_cast<uint64_t>(a_axis_len) * 4u > limit) *band_len = (limit / 4u) & ~3u;
+        *tag_slots = 0;
+        *lds_bytes = *band_len * 4u;
+        return;
+    }
+    if (static_cast<uint64_t>(a_axis_len) * 8u <= 65536u || limit < 131072u) {
+        *band_len = a_axis_len;
+        if (static_cast<uint64_t>(a_axis_len) * 8u > limit) *band_len = (limit / 8u) & ~3u;
+        *tag_slots = *band_len;
+    } else {
+        *band_len = a_axis_len < 16384u ? a_axis_len : 16384u;
+        *tag_slots = kSharedTags;
+    }
+    *lds_bytes = (*band_len + *tag_slots) * 4u;
+}
+
 static bool gather_rows_fit_lds(uint32_t a_axis_len, uint32_t i_axis_len) {
     return static_cast<uint64_t>(a_axis_len) * 4u <= rows_lds_limit() && i_axis_len >= 64 && i_axis_len >= a_axis_len / 8;
 }
@@ -682,10 +713,9 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
     const uint32_t blocks = static_cast<uint32_t>((positions + kBlock - 1) / kBlock);
     const uint64_t bytes = (mode == 2 ? 2 : mode == 1 ? 4 : 3) * idx_n * 4;
     if (axis == dims - 1 && scatter_rows_fit_lds(mode, pl.a_axis_len, pl.i_axis_len) && positions <= 0x7fffffffull) {
-        const uint32_t per_element = mode == 1 ? 8u : 4u;
-        uint32_t band_len = pl.a_axis_len;
-        if (static_cast<uint64_t>(band_len) * per_element > rows_lds_limit()) band_len = (rows_lds_limit() / per_element) & ~3u;
-        const uint32_t lds_bytes = band_len * per_element;
+        uint32_t band_len, tag_slots, lds_bytes;
+        rows_lds_plan(mode, pl.a_axis_len, &band_len, &tag_slots, &lds_bytes);
+        const FastDiv tag_div = make_div(tag_slots ? tag_slots : 1u);
         const uint64_t bands = (pl.a_axis_len + band_len - 1) / band_len;
         const uint64_t row_bytes = ((constant ? 1ull : 2ull) * pl.a_axis_len * positions + bands * (mode == 2 ? 1 : 2) * idx_n) * 4;
         const uint32_t from_constant = constant ? 1u : 0u;
@@ -695,7 +725,7 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
             const dim3 grid(static_cast<uint32_t>(positions));
             hipStream_t stream = state().stream;
             const float factor = mode == 1 ? 1.0f : value;
-#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag, band_len, from_constant, start)
+#define ROWS_LAUNCH(MM, TT) hipLaunchKernelGGL((scatter_rows_lds_kernel<MM, TT>), grid, dim3(TT), lds_bytes, stream, target, index, psrc, factor, pl, flag, band_len, from_constant, start, tag_slots, tag_div)
             if (lds_bytes > 32768u) { if (mode == 0) ROWS_LAUNCH(0, 1024); else if (mode == 1) ROWS_LAUNCH(1, 1024); else ROWS_LAUNCH(2, 1024); }
             else                    { if (mode == 0) ROWS_LAUNCH(0, 256);  else if (mode == 1) ROWS_LAUNCH(1, 256);  else ROWS_LAUNCH(2, 256); }
 #undef ROWS_LAUNCH
@@ -941,16 +971,16 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
         rp.i_stride[0] = 0; rp.a_stride[0] = pl.axis_len; rp.b_stride[0] = pl.k;
         rp.i_axis_stride = rp.a_axis_stride = rp.b_axis_stride = 1;
         rp.i_axis_len = pl.k; rp.a_axis_len = pl.axis_len;
-        uint32_t band_len = rp.a_axis_len;
-        if (static_cast<uint64_t>(band_len) * 8u > rows_lds_limit()) band_len = (rows_lds_limit() / 8u) & ~3u;
-        const uint32_t lds_bytes = band_len * 8u;
+        uint32_t band_len, tag_slots, lds_bytes;
+        rows_lds_plan(1, rp.a_axis_len, &band_len, &tag_slots, &lds_bytes);
+        const FastDiv tag_div = make_div(tag_slots);
         return with_index_check("Index Add", [&](int* flag) {
             LaunchScope scope("scatter_rows_lds_kernel", "indexAdd", (2 * total + n_src + k) * 4);
             const dim3 grid(static_cast<uint32_t>(outer));
             if (lds_bytes > 32768u)
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 1024>), grid, dim3(1024), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant, tag_slots, tag_div);
             else
-                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant);
+                hipLaunchKernelGGL((scatter_rows_lds_kernel<1, 256>), grid, dim3(256), lds_bytes, stream, st->ptr, sx->ptr, ss->ptr, alpha, rp, flag, band_len, from_constant ? 1u : 0u, constant, tag_slots, tag_div);
         });
     }
 
