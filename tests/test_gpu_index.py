@@ -23,7 +23,9 @@ CASES = [([4, 5], [4, 3], 1), ([4, 5], [2, 5], 0), ([3, 4, 5], [3, 2, 5], 1), ([
          ([2, 32768], [2, 5000], 1), ([2, 32769], [2, 5000], 1), ([3, 100001], [3, 40000], 1), ([70001, 6], [30000, 5], 0),
          ([10, 6, 300], [7, 4, 100], 2), ([5, 1], [5, 700], 1), ([1, 4096], [1, 4096], 1),
          # a long axis that is not the innermost: scattered as rows between two permutes
-         ([4096, 96], [4096, 96], 0), ([2, 3000, 40], [2, 2500, 33], 1), ([8192, 3, 5], [8000, 2, 5], 0), ([5000, 7], [700, 7], 0)]
+         ([4096, 96], [4096, 96], 0), ([2, 3000, 40], [2, 2500, 33], 1), ([8192, 3, 5], [8000, 2, 5], 0), ([5000, 7], [700, 7], 0),
+         # gathered as rows between permutes too: a long outer or middle axis and an index about as large as the input
+         ([3, 3000, 40], [3, 2600, 37], 1), ([9000, 33], [8000, 33], 0), ([2, 300, 5, 101], [2, 300, 5, 101], 1)]
 
 
 def both(gc, shape, array):
@@ -48,6 +50,20 @@ def test_gather_scatter_parity(shape, ishape, axis, gc):
     assert_bits_equal(gt.toArray(), ct.toArray(), "inplaceScatter(Float)")
     assert_bits_equal(gx.scatter(axis, gi, gs).toArray(), cx.scatter(axis, ci, cs).toArray(), "scatter (copy)")
     assert_bits_equal(gx.toArray(), x, "scatter must not touch its receiver")
+
+
+def test_gather_along_an_outer_axis_goes_through_rows(gc):
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal([5000, 70]).astype(np.float32)
+    idx = rng.integers(0, 5000, size=[4500, 70]).astype(np.float32)
+    gc.profileBegin()
+    got = gc.createRaw([5000, 70], x).gather(0, gc.createRaw([4500, 70], idx)).toArray()
+    kernels = gc.profileEnd()
+    assert any(k.startswith("gather_rows_lds_kernel") for k in kernels) and any(k.startswith("permute") for k in kernels), sorted(kernels)
+    assert_bits_equal(got, np.take_along_axis(x, idx.astype(np.int64), axis=0), "gather along axis 0")
+    bad = idx.copy(); bad[17, 3] = 5000.0
+    with pytest.raises(ValueError):
+        gc.createRaw([5000, 70], x).gather(0, gc.createRaw([4500, 70], bad))
 
 
 def test_bad_indices_raise_like_the_reference(gc):
