@@ -46,6 +46,21 @@ def test_fast_divider_on_the_host(tmp_path):
     assert "fastdiv ok" in done.stdout
 
 
+def test_constant_folding_on_the_host(tmp_path):
+    """constant (op) constant computed by the library on the host (kth_fold.h) must be the bits of the float
+    operation wherever it is accepted, and must be declined for subnormal or NaN operands and results."""
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = tmp_path / "fold_test"
+    subprocess.run([gxx, "-std=c++17", "-O1", "-Wall", "-Wextra", "-Werror", "-fsanitize=undefined", "-fno-sanitize-recover=all",
+                    "-I", os.path.join(ROOT, "kten_amd", "csrc"), os.path.join(ROOT, "tests", "cpp", "fold_test.cpp"),
+                    "-o", str(exe)], check=True)
+    done = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "fold ok" in done.stdout
+
+
 @pytest.mark.gpu
 def test_cpp_host_mirror_known_answers():
     assert os.path.exists(BINARY), "tests/cpp/host_mirror_test is not built (python __graft_entry__.py build)"
