@@ -63,7 +63,7 @@ template <int THREADS>
 __device__ __forceinline__ void row_to_lds(const float* __restrict__ row, float* tile, uint32_t len) {
     const uint32_t body = len & ~3u;
     for (uint32_t j = threadIdx.x * 4; j < body; j += THREADS * 4) {
-        const v4f_unaligned v = *reinterpret_cast<const v4f_unaligned*>(row + j);
+        const v4f_unaligned v = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(row + j));
         *reinterpret_cast<v4f_lds*>(tile + j) = v4f_lds{v.x, v.y, v.z, v.w};
     }
     if (threadIdx.x < len - body) tile[body + threadIdx.x] = row[body + threadIdx.x];
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(THREADS) void gather_rows_lds_kernel(const float* _
     for (uint32_t r0 = tid; r0 < pl.i_axis_len; r0 += kBatch * THREADS) {
         float fi[kBatch];
 #pragma unroll
-        for (uint32_t k = 0; k < kBatch; k++) if (r0 + k * THREADS < pl.i_axis_len) fi[k] = irow[r0 + k * THREADS];
+        for (uint32_t k = 0; k < kBatch; k++) if (r0 + k * THREADS < pl.i_axis_len) fi[k] = __builtin_nontemporal_load(irow + r0 + k * THREADS);
 #pragma unroll
         for (uint32_t k = 0; k < kBatch; k++) {
             if (r0 + k * THREADS < pl.i_axis_len) {
@@ -192,14 +192,14 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
         uint32_t epoch = kFirstEpoch;                         // MODE 1: the round counter, uniform over the workgroup
         // the first chunk's entries are fetched while the row arrives
         float next_i = 0.0f, next_v = value;
-        if (tid < pl.i_axis_len) { next_i = irow[tid]; if (MODE != 2) next_v = srow[tid]; }
+        if (tid < pl.i_axis_len) { next_i = __builtin_nontemporal_load(irow + tid); if (MODE != 2) next_v = __builtin_nontemporal_load(srow + tid); }
         __syncthreads();
         for (uint32_t r0 = 0; r0 < pl.i_axis_len; r0 += THREADS) {
             const uint32_t r = r0 + tid;
             bool have = r < pl.i_axis_len;
             const int sel_raw = static_cast<int>(next_i);
             const float v = MODE == 1 ? next_v * value : next_v;  // add form: value is the factor on the source (1 for scatterAdd)
-            if (r + THREADS < pl.i_axis_len) { next_i = irow[r + THREADS]; if (MODE != 2) next_v = srow[r + THREADS]; }
+            if (r + THREADS < pl.i_axis_len) { next_i = __builtin_nontemporal_load(irow + r + THREADS); if (MODE != 2) next_v = __builtin_nontemporal_load(srow + r + THREADS); }
             if (have && (sel_raw < 0 || static_cast<uint32_t>(sel_raw) >= pl.a_axis_len)) { *bad = 1; have = false; }
             if (have && (static_cast<uint32_t>(sel_raw) < band0 || static_cast<uint32_t>(sel_raw) >= band0 + band)) have = false;
             const uint32_t sel = have ? static_cast<uint32_t>(sel_raw) - band0 : 0u;
