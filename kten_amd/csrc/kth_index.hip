@@ -282,8 +282,10 @@ __global__ __launch_bounds__(kBlock) void index_select_kernel(const float* __res
     const int sel = static_cast<int>(index[row - o * pl.k]);
     if (sel < 0 || static_cast<uint32_t>(sel) >= pl.axis_len) { *bad = 1; return; }
     const uint32_t from = (o * pl.axis_len + static_cast<uint32_t>(sel)) * pl.inner + col;
-    if (VEC) reinterpret_cast<float4*>(out)[e] = reinterpret_cast<const float4*>(in)[from];
-    else out[e] = in[from];
+    if (VEC) {
+        const v4f_lds v = __builtin_nontemporal_load(reinterpret_cast<const v4f_lds*>(in) + from);
+        reinterpret_cast<v4f_lds*>(out)[e] = v;
+    } else out[e] = __builtin_nontemporal_load(in + from);
 }
 
 // The same for rows whose length is not a multiple of 4 (but at least 4): a row is covered by
@@ -390,12 +392,12 @@ __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restr
     if (VEC) {
         float4 acc = make_float4(constant, constant, constant, constant);
         if (r != 0xffffffffu) {
-            const float4* s = reinterpret_cast<const float4*>(src) + s_base;
-            float4 v = s[static_cast<size_t>(vals[r]) * pl.inner];
+            const v4f_lds* s = reinterpret_cast<const v4f_lds*>(src) + s_base;
+            v4f_lds v = __builtin_nontemporal_load(s + static_cast<size_t>(vals[r]) * pl.inner);
             while (true) {
                 const bool more = r + 1 < pl.k && keys[r + 1] == key;
-                float4 next = v;
-                if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];     // in flight during the adds
+                v4f_lds next = v;
+                if (more) next = __builtin_nontemporal_load(s + static_cast<size_t>(vals[r + 1]) * pl.inner);     // in flight during the adds
                 acc.x = acc.x + v.x * alpha; acc.y = acc.y + v.y * alpha; acc.z = acc.z + v.z * alpha; acc.w = acc.w + v.w * alpha;
                 if (!more) break;
                 v = next; r++;
