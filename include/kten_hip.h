@@ -209,7 +209,11 @@ int kth_reduce_scratch_bytes(uint64_t* bytes);
  * at the operation (JVM:238-239,345-346,494-496). immediate == 0: the calls do not wait; an out-of-range index sets a
  * flag on the device and the next blocking call (kth_sync, kth_download, kth_read_scalar) returns KTH_E_ARGUMENT in
  * its place, once. Either way the kernels skip the offending entry and the in-place target of a scatter or indexAdd has
- * been updated by the entries before it (the JVM, too, has assigned those when it throws). */
+ * been updated by the entries before it (the JVM, too, has assigned those when it throws).
+ * In immediate mode a call does not wait when its index store is known to hold only valid values: an earlier indexed
+ * move checked it against an axis no longer than this one (or kth_reduce_axis wrote it as ARG_MAX / ARG_MIN positions
+ * of such an axis) and no call has taken the store since. Any call that takes the store other than as the index of
+ * an indexed move forgets that, so a changed index is checked again and reported at its next use. */
 int kth_set_index_check(int immediate);
 
 /* gather (RAW:164; JVM:334-353). in and index have `dims` dims; out has index's shape:

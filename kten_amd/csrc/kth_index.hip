@@ -540,20 +540,32 @@ int with_index_check(const char* what, F launch) {
     State& s = state();
     if (!s.index_check_immediate) {
         // deferred: the kernels set the persistent flag, the next blocking call reports it; nothing waits here
+        s.index_use = IndexUse{};
         launch(s.deferred_index_flag);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
         return KTH_OK;
     }
     // immediate: the kernels write a word of pinned host memory, read here once the stream has drained (the
-    // word is zero whenever no indexed move is in flight: only this function lets kernels at it, and it waits)
+    // word is zero whenever no indexed move is in flight: only this function lets kernels at it, and it waits).
+    // An index store that an earlier move (or ARG_MAX / ARG_MIN) has left marked as holding only values below
+    // this axis length, and that nothing has touched since, cannot raise the flag: nothing waits for it.
+    const IndexUse use = s.index_use;
+    s.index_use = IndexUse{};
+    const bool known = use.store && use.store->index_valid_below != 0 && use.store->index_valid_below <= use.axis_len &&
+                       use.store->index_valid_n >= use.n;
     launch(s.host_index_flag_device);
     hipError_t e = hipGetLastError();
+    if (known) {
+        if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
+        return KTH_OK;
+    }
     if (e == hipSuccess) e = hipStreamSynchronize(s.stream);
     const int host_flag = *s.host_index_flag;
     *s.host_index_flag = 0;
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
     if (host_flag) return fail(KTH_E_ARGUMENT, "%s got invalid index, an index value is out of bounds at the axis", what);
+    if (use.store) { use.store->index_valid_below = use.axis_len; use.store->index_valid_n = use.n; }
     return KTH_OK;
 }
 
@@ -717,7 +729,7 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
             return fail(KTH_E_SHAPE, "kth_gather: index dim %d (%d) exceeds the input's (%d)", d, index_shape[d], in_shape[d]);
     Store* si = lookup(in, "kth_gather(in)");
     if (!si) return KTH_E_HANDLE;
-    Store* sx = lookup(index, "kth_gather(index)");
+    Store* sx = lookup_index(index, "kth_gather(index)");
     if (!sx) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_gather(out)");
     if (!so) return KTH_E_HANDLE;
@@ -725,6 +737,7 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
         return fail(KTH_E_ARGUMENT, "kth_gather: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_gather: output aliases an input");
     if (idx_n == 0) return KTH_OK;
+    state().index_use = IndexUse{sx, static_cast<uint32_t>(in_shape[axis]), idx_n};
     if (gather_pays_transposing(in_shape, index_shape, dims, axis, in_n, idx_n))
         if (int rc = gather_transposed(si->ptr, in_shape, sx->ptr, index_shape, so->ptr, dims, axis, in_n, idx_n); rc != KTH_E_MEMORY)
             return rc;                                   // no room for the transposed copies: the element form below
@@ -866,7 +879,7 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
     }
     Store* st = lookup_unsettled(target, "kth_scatter(target)");
     if (!st) return KTH_E_HANDLE;
-    Store* sx = lookup(index, "kth_scatter(index)");
+    Store* sx = lookup_index(index, "kth_scatter(index)");
     if (!sx) return KTH_E_HANDLE;
     Store* ss = nullptr;
     if (mode != 2) { ss = lookup(src, "kth_scatter(src)"); if (!ss) return KTH_E_HANDLE; }
@@ -874,6 +887,7 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
         return fail(KTH_E_ARGUMENT, "kth_scatter: a shape needs more elements than its store holds");
     if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
     if (idx_n == 0) return KTH_OK;
+    state().index_use = IndexUse{sx, static_cast<uint32_t>(target_shape[axis]), idx_n};
     const float* psrc = ss ? ss->ptr : nullptr;
     // A target that is still an owed constant (fresh from zerosLike) need not be filled and read back
     // when the row kernel rewrites all of it: the index covers every position off the axis.
@@ -924,7 +938,7 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
     if (n_out > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_select: more than 2^31-1 result elements");
     Store* si = lookup(in, "kth_index_select(in)");
     if (!si) return KTH_E_HANDLE;
-    Store* sx = lookup(index, "kth_index_select(index)");
+    Store* sx = lookup_index(index, "kth_index_select(index)");
     if (!sx) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_index_select(out)");
     if (!so) return KTH_E_HANDLE;
@@ -932,6 +946,7 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
         return fail(KTH_E_ARGUMENT, "kth_index_select: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_index_select: output aliases an input");
     if (n_out == 0) return KTH_OK;
+    state().index_use = IndexUse{sx, static_cast<uint32_t>(shape[axis]), k};
     if (inner == 1 && gather_rows_fit_lds(static_cast<uint32_t>(shape[axis]), static_cast<uint32_t>(k))) {
         // columns picked from contiguous rows: the gather row kernel with one index row for every position
         IndexPlan rp{};
@@ -988,7 +1003,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (n_src > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_add: more than 2^31-1 source elements");
     Store* st = lookup_unsettled(target, "kth_index_add(target)");
     if (!st) return KTH_E_HANDLE;
-    Store* sx = lookup(index, "kth_index_add(index)");
+    Store* sx = lookup_index(index, "kth_index_add(index)");
     if (!sx) return KTH_E_HANDLE;
     Store* ss = lookup(src, "kth_index_add(src)");
     if (!ss) return KTH_E_HANDLE;
@@ -997,6 +1012,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (st->ptr == sx->ptr || st->ptr == ss->ptr) return fail(KTH_E_ARGUMENT, "kth_index_add: target aliases an input");
     const uint64_t positions = outer * inner;
     if (positions == 0 || k == 0) return KTH_OK;
+    state().index_use = IndexUse{sx, static_cast<uint32_t>(shape[axis]), k};
     // A target that is one owed constant (fresh from zerosLike) and a list long enough to be sorted: the
     // rows are written from the constant, nothing of the target is read. Every other case has the fill launched.
     const bool vec_inner = inner % 4 == 0;

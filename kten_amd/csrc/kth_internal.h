@@ -29,6 +29,19 @@ struct Store {
     // a broadcast passes it on) take the store with `lookup_unsettled` and clear or keep the note themselves.
     uint64_t fill_n = 0;
     float    fill_value = 0.0f;
+    // Set when an indexed move has checked floats [0, index_valid_n) of this store as index values and found every
+    // one inside [0, index_valid_below), or when ARG_MAX / ARG_MIN wrote them: the next indexed move with an axis at
+    // least that long skips the check and its wait for the stream. Every lookup other than `lookup_index` clears
+    // it, so anything that could have changed the store's contents makes the next use check again.
+    uint32_t index_valid_below = 0;
+    uint64_t index_valid_n = 0;
+};
+
+// The index operand of the indexed move that is about to be launched (set by its entry point, taken by the check).
+struct IndexUse {
+    Store*   store = nullptr;
+    uint32_t axis_len = 0;
+    uint64_t n = 0;
 };
 
 // One profiled launch: which kernel, the algorithmic bytes it moved, its event pair.
@@ -77,6 +90,7 @@ struct State {
     // so that the check costs one wait for the stream and neither a clearing kernel nor a copy back
     volatile int* host_index_flag = nullptr;
     int*          host_index_flag_device = nullptr;
+    IndexUse      index_use;
 
     std::vector<hipEvent_t> laps;           // kth_timer_lap events not yet read by kth_timer_laps
 
@@ -95,6 +109,8 @@ int fail(int code, const char* fmt, ...);
 Store* lookup(uint64_t handle, const char* what);
 // The same without launching an owed fill: for callers that fold, overwrite or drop it.
 Store* lookup_unsettled(uint64_t handle, const char* what);
+// `lookup` for the index operand of an indexed move: keeps the store's record of having been checked as an index.
+Store* lookup_index(uint64_t handle, const char* what);
 // Launches the fill the store is owed, if any, on the library's stream.
 void settle(Store* st);
 // The store is about to be written over floats [0, n) by a kernel that reads none of them: an owed

@@ -877,6 +877,12 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
                                    static_cast<uint32_t>(inner), use_static);
     // a refused plan has written nothing: the output is still owed what it was owed
     if (rc != KTH_OK && owed_n != 0 && so->fill_n == 0) { so->fill_n = owed_n; so->fill_value = owed_value; }
+    // the positions ARG_MAX / ARG_MIN wrote are index values below the axis length: an indexed move that takes
+    // them next (the scatter of a Max / Min backward) need not check them
+    if (rc == KTH_OK && (op == KTH_ARG_MAX || op == KTH_ARG_MIN)) {
+        so->index_valid_below = static_cast<uint32_t>(axis);
+        so->index_valid_n = outer * inner;
+    }
     return rc;
 }
 

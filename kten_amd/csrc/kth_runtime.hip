@@ -40,6 +40,8 @@ Store* lookup_unsettled(uint64_t handle, const char* what) {
         fail(KTH_E_HANDLE, "%s: handle 0x%llx was released", what, (unsigned long long)handle);
         return nullptr;
     }
+    st.index_valid_below = 0;          // whoever takes the store may write it: its values are unknown again
+    st.index_valid_n = 0;
     return &st;
 }
 
@@ -58,6 +60,16 @@ void settle_for_overwrite(Store* st, uint64_t n) {
 Store* lookup(uint64_t handle, const char* what) {
     Store* st = lookup_unsettled(handle, what);
     if (st) settle(st);
+    return st;
+}
+
+Store* lookup_index(uint64_t handle, const char* what) {
+    State& s = state();
+    const uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
+    uint32_t below = 0; uint64_t n = 0;
+    if (low != 0 && low <= s.table.size()) { below = s.table[low - 1].index_valid_below; n = s.table[low - 1].index_valid_n; }
+    Store* st = lookup(handle, what);
+    if (st) { st->index_valid_below = below; st->index_valid_n = n; }
     return st;
 }
 
@@ -290,7 +302,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
     if (!s.free_slots.empty()) { idx = s.free_slots.back(); s.free_slots.pop_back(); }
     else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); s.table.back().generation = g_epoch << 20; }
     Store& st = s.table[idx];
-    st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1; st.fill_n = 0;
+    st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1; st.fill_n = 0; st.index_valid_below = 0; st.index_valid_n = 0;
     s.live_bytes += cap;
     *handle = make_handle(idx, st.generation);
     return KTH_OK;

@@ -66,6 +66,67 @@ def test_gather_along_an_outer_axis_goes_through_rows(gc):
         gc.createRaw([5000, 70], x).gather(0, gc.createRaw([4500, 70], bad))
 
 
+def test_an_index_checked_once_is_checked_again_after_any_change(gc):
+    """An index tensor that an indexed move found valid is not checked again while nothing touches it; every
+    way of changing it (a range fill, an upload, an in-place op, a copy into it, a kernel writing it as its result)
+    and a shorter axis must bring the check back."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal([50, 40]).astype(np.float32)
+    gx = gc.createRaw([50, 40], x)
+    idx = rng.integers(0, 40, size=[50, 12]).astype(np.float32)
+    want = np.take_along_axis(x, idx.astype(np.int64), axis=1)
+
+    def fresh():
+        gi = gc.createRaw([50, 12], idx)
+        assert_bits_equal(gx.gather(1, gi).toArray(), want, "gather")          # checked here
+        assert_bits_equal(gx.gather(1, gi).toArray(), want, "gather again")    # known to be valid
+        return gi
+
+    gi = fresh(); gi._set_store_range(7, 1, 40.0)
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    gi = fresh(); gi._set_ranges([3, 2], [3, 2], -1.0)
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    gi = fresh(); gi._scalar_assign("plus", 30.0)
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    gi = fresh(); gi._binary_assign("times", gc.createRawFill([50, 12], 2.0))
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    gi = fresh(); gi._set_store_range(0, 600, gc.createRawFill([600], 41.0))     # a copy into it
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    gi = fresh(); gi.inplaceScatter(1, gc.createRaw([50, 1], np.zeros([50, 1], np.float32)), 99.0)   # written as a target
+    with pytest.raises(ValueError):
+        gx.gather(1, gi)
+    # valid for an axis of 40, not for one of 30
+    gi = fresh()
+    with pytest.raises(ValueError):
+        gc.createRaw([50, 30], x[:, :30].copy()).gather(1, gi)
+    # and valid again for a longer one, for every kind of indexed move
+    wide = gc.createRaw([50, 64], np.zeros([50, 64], np.float32))
+    wide.inplaceScatterAdd(1, gi, gc.createRawFill([50, 12], 1.0))
+    assert wide.toArray().sum() == 600.0
+    # the positions ARG_MAX wrote are valid for the axis they came from; changed afterwards, they are checked again
+    am = gx.argMax(1, True)
+    t = gc.createRawFill([50, 40], 0.0)
+    t.inplaceScatter(1, am, 1.0)
+    assert_bits_equal(t.toArray().sum(1), np.ones([50], np.float32), "one-hot of the row maxima")
+    am._scalar_assign("plus", 40.0)
+    with pytest.raises(ValueError):
+        t.inplaceScatter(1, am, 1.0)
+    rows = gc.createRaw([20], rng.integers(0, 50, size=[20]).astype(np.float32))
+    sel = gx.indexSelect(0, rows)
+    acc = gc.createRawFill([50, 40], 0.0)
+    acc.indexAdd(0, rows, sel, 1.0)                                           # the list was checked by indexSelect
+    rows._set_store_range(19, 1, 50.0)
+    with pytest.raises(ValueError):
+        acc.indexAdd(0, rows, sel, 1.0)
+    with pytest.raises(ValueError):
+        gx.indexSelect(0, rows)
+
+
 def test_bad_indices_raise_like_the_reference(gc):
     x = gc.createRaw([2, 3], np.arange(6, dtype=np.float32))
     for bad in (3.0, -1.0, 1e10):
