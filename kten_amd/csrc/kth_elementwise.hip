@@ -127,7 +127,7 @@ __device__ __forceinline__ float with_sign_of(float magnitude_result, float x) {
 // Four elements through a short routine, then one branch for the lanes of the wave whose rounding it left open:
 // the four evaluations are independent straight-line code, and the long routine is reached about once in
 // several hundred waves.
-#define KTH_SHORT_THEN_LONG(FAST, SIGNED, LONG_CALL)                                                     \
+#define KTH_SHORT_THEN_LONG(FAST, SIGNED, ROLLED, LONG_CALL)                                                     \
     static __device__ __forceinline__ float apply(float x, const double* lds) {                          \
         double y;                                                                                         \
         const bool ok = FAST(x, lds, y);                                                                 \
@@ -146,7 +146,18 @@ __device__ __forceinline__ float with_sign_of(float magnitude_result, float x) {
             rs[j] = SIGNED ? with_sign_of(static_cast<float>(y), x) : static_cast<float>(y);             \
             open[j] = !(ok && rounds_safely(y));                                                         \
         }                                                                                                 \
-        if (open[0] | open[1] | open[2] | open[3]) {                                                     \
+        if (ROLLED && (open[0] | open[1] | open[2] | open[3])) {                                         \
+            /* one copy of the long routine for the four elements: the loop stays rolled, j is uniform */ \
+            _Pragma("unroll 1") for (int j = 0; j < 4; j++) {                                            \
+                const bool o = j == 0 ? open[0] : j == 1 ? open[1] : j == 2 ? open[2] : open[3];         \
+                if (o) {                                                                                  \
+                    const float x = j == 0 ? xs[0] : j == 1 ? xs[1] : j == 2 ? xs[2] : xs[3];            \
+                    const float y = LONG_CALL;                                                           \
+                    if (j == 0) rs[0] = y; else if (j == 1) rs[1] = y; else if (j == 2) rs[2] = y; else rs[3] = y; \
+                }                                                                                         \
+            }                                                                                             \
+        }                                                                                                 \
+        if (!ROLLED && (open[0] | open[1] | open[2] | open[3])) {                                        \
             _Pragma("unroll") for (int j = 0; j < 4; j++) {                                              \
                 const float x = xs[j];                                                                    \
                 if (open[j]) rs[j] = LONG_CALL;                                                          \
@@ -159,19 +170,19 @@ struct OpTanhT {
     static constexpr const char* name = "OpTanh";
     static constexpr int kTableDoubles = kExpTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_tanh, true, table_tanh(x, lds))
+    KTH_SHORT_THEN_LONG(fast_tanh, true, true, table_tanh(x, lds))
 };
 struct OpSinhT {
     static constexpr const char* name = "OpSinh";
     static constexpr int kTableDoubles = kExpTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_sinh, true, table_sinh(x, lds))
+    KTH_SHORT_THEN_LONG(fast_sinh, true, true, table_sinh(x, lds))
 };
 struct OpCoshT {
     static constexpr const char* name = "OpCosh";
     static constexpr int kTableDoubles = kExpTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_exp_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_cosh, false, table_cosh(x, lds))
+    KTH_SHORT_THEN_LONG(fast_cosh, false, true, table_cosh(x, lds))
 };
 
 // atan keeps the long routine alone: with one reciprocal per lane it is already the cheaper one
@@ -193,7 +204,7 @@ struct OpAsinT {
         stage_table(lds, g_asin_table, 2 * kAsinTableEntries);
         stage_table(lds + 2 * kAsinTableEntries, g_atan_table, kAtanTableEntries);
     }
-    KTH_SHORT_THEN_LONG(fast_asin, true, table_asin(x, lds + 2 * kAsinTableEntries))
+    KTH_SHORT_THEN_LONG(fast_asin, true, true, table_asin(x, lds + 2 * kAsinTableEntries))
 };
 struct OpAcosT {
     static constexpr const char* name = "OpAcos";
@@ -202,26 +213,26 @@ struct OpAcosT {
         stage_table(lds, g_asin_table, 2 * kAsinTableEntries);
         stage_table(lds + 2 * kAsinTableEntries, g_atan_table, kAtanTableEntries);
     }
-    KTH_SHORT_THEN_LONG(fast_acos, false, table_acos(x, lds + 2 * kAsinTableEntries))
+    KTH_SHORT_THEN_LONG(fast_acos, false, true, table_acos(x, lds + 2 * kAsinTableEntries))
 };
 // sin, cos, tan: the short routine reads {sin, cos}(j pi / 32) through LDS; the long one needs no table.
 struct OpSinT {
     static constexpr const char* name = "OpSin";
     static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_sin, true, table_sin(x))
+    KTH_SHORT_THEN_LONG(fast_sin, true, false, table_sin(x))
 };
 struct OpCosT {
     static constexpr const char* name = "OpCos";
     static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_cos, false, table_cos(x))
+    KTH_SHORT_THEN_LONG(fast_cos, false, false, table_cos(x))
 };
 struct OpTanT {
     static constexpr const char* name = "OpTan";
     static constexpr int kTableDoubles = 2 * kSinCosTableEntries;
     static __device__ __forceinline__ void stage(double* lds) { stage_table(lds, g_sincos_table, kTableDoubles); }
-    KTH_SHORT_THEN_LONG(fast_tan, true, table_tan(x))
+    KTH_SHORT_THEN_LONG(fast_tan, true, false, table_tan(x))
 };
 
 // pow(tensor | Float): the common operands (finite non-zero base, finite exponent) go through
