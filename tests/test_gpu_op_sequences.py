@@ -289,6 +289,8 @@ class Program:
         x = self.rows_for(sa, sa.shape[axis])
         sx = self.slots[x]
         shape = list(sa.shape); shape[axis] = sx.shape[0]
+        if int(np.prod(shape)) > 8 * int(np.prod(self.dims)):
+            return False
         src = self.maybe(lambda s: not shares(s, sa) and s.shape == shape)
         if src is None or self.rng.random() < 0.5:
             if self.rng.random() < 0.3:
