@@ -534,6 +534,15 @@ void strides_without_axis(const int32_t* shape, int dims, int axis, uint32_t* po
     }
 }
 
+// Names the index operand of the move its entry point is about to launch, until that entry point returns
+// (whichever way: a plan that fails before the check must not leave the store's address behind).
+struct IndexUseScope {
+    explicit IndexUseScope(const IndexUse& use) { state().index_use = use; }
+    ~IndexUseScope() { state().index_use = IndexUse{}; }
+    IndexUseScope(const IndexUseScope&) = delete;
+    IndexUseScope& operator=(const IndexUseScope&) = delete;
+};
+
 // Runs `launch(flag)` with a cleared device flag and reports a set flag as an argument error.
 template <class F>
 int with_index_check(const char* what, F launch) {
@@ -737,7 +746,7 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
         return fail(KTH_E_ARGUMENT, "kth_gather: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_gather: output aliases an input");
     if (idx_n == 0) return KTH_OK;
-    state().index_use = IndexUse{sx, static_cast<uint32_t>(in_shape[axis]), idx_n};
+    const IndexUseScope index_use(IndexUse{sx, static_cast<uint32_t>(in_shape[axis]), idx_n});
     if (gather_pays_transposing(in_shape, index_shape, dims, axis, in_n, idx_n))
         if (int rc = gather_transposed(si->ptr, in_shape, sx->ptr, index_shape, so->ptr, dims, axis, in_n, idx_n); rc != KTH_E_MEMORY)
             return rc;                                   // no room for the transposed copies: the element form below
@@ -887,7 +896,7 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
         return fail(KTH_E_ARGUMENT, "kth_scatter: a shape needs more elements than its store holds");
     if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
     if (idx_n == 0) return KTH_OK;
-    state().index_use = IndexUse{sx, static_cast<uint32_t>(target_shape[axis]), idx_n};
+    const IndexUseScope index_use(IndexUse{sx, static_cast<uint32_t>(target_shape[axis]), idx_n});
     const float* psrc = ss ? ss->ptr : nullptr;
     // A target that is still an owed constant (fresh from zerosLike) need not be filled and read back
     // when the row kernel rewrites all of it: the index covers every position off the axis.
@@ -946,7 +955,7 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
         return fail(KTH_E_ARGUMENT, "kth_index_select: a shape needs more elements than its store holds");
     if (so->ptr == si->ptr || so->ptr == sx->ptr) return fail(KTH_E_ARGUMENT, "kth_index_select: output aliases an input");
     if (n_out == 0) return KTH_OK;
-    state().index_use = IndexUse{sx, static_cast<uint32_t>(shape[axis]), k};
+    const IndexUseScope index_use(IndexUse{sx, static_cast<uint32_t>(shape[axis]), k});
     if (inner == 1 && gather_rows_fit_lds(static_cast<uint32_t>(shape[axis]), static_cast<uint32_t>(k))) {
         // columns picked from contiguous rows: the gather row kernel with one index row for every position
         IndexPlan rp{};
@@ -1012,7 +1021,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (st->ptr == sx->ptr || st->ptr == ss->ptr) return fail(KTH_E_ARGUMENT, "kth_index_add: target aliases an input");
     const uint64_t positions = outer * inner;
     if (positions == 0 || k == 0) return KTH_OK;
-    state().index_use = IndexUse{sx, static_cast<uint32_t>(shape[axis]), k};
+    const IndexUseScope index_use(IndexUse{sx, static_cast<uint32_t>(shape[axis]), k});
     // A target that is one owed constant (fresh from zerosLike) and a list long enough to be sorted: the
     // rows are written from the constant, nothing of the target is read. Every other case has the fill launched.
     const bool vec_inner = inner % 4 == 0;
