@@ -268,6 +268,9 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
 struct RowsPlan {
     uint32_t axis_len, k, inner;       // inner in the kernel's units (float4s for the vector form)
     FastDiv  inner_div, k_div;
+    uint32_t heads;                    // indexAdd through the sorted list: no more runs than this (min(k, axis_len + 1))
+    FastDiv  heads_div;
+    uint32_t long_from;                // ... and runs of this many entries or more are left to the long-run kernel
 };
 
 // One thread per unit of the result [outer, k, inner]: out[o, i, :] = in[o, index[i], :].
@@ -341,8 +344,10 @@ __global__ __launch_bounds__(kBlock) void index_add_kernel(float* __restrict__ t
 // reported); vals[i] = i. After a stable sort by key, the source rows that add into one target
 // row stand next to each other in their original order.
 __global__ __launch_bounds__(kBlock) void index_keys_kernel(const float* __restrict__ index, uint32_t k, uint32_t axis_len,
-                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, int* bad) {
+                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, int* bad,
+                                                           uint32_t* __restrict__ long_count) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i == 0) *long_count = 0;
     if (i >= k) return;
     const int sel = static_cast<int>(index[i]);
     const bool ok = sel >= 0 && static_cast<uint32_t>(sel) < axis_len;
@@ -351,12 +356,51 @@ __global__ __launch_bounds__(kBlock) void index_keys_kernel(const float* __restr
     vals[i] = i;
 }
 
-// flags[i] = 1 where a run of equal, valid keys starts in the sorted list.
-__global__ __launch_bounds__(kBlock) void index_heads_kernel(const uint32_t* __restrict__ keys, uint32_t k, uint32_t axis_len, uint8_t* __restrict__ flags) {
+// flags[i] = 1 where a run of equal keys starts in the sorted list. The invalid entries (key axis_len) stand at
+// the end as a run of their own, so that every run ends where the next one starts (or at k).
+__global__ __launch_bounds__(kBlock) void index_heads_kernel(const uint32_t* __restrict__ keys, uint32_t k, uint8_t* __restrict__ flags) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= k) return;
+    flags[i] = (i == 0 || keys[i - 1] != keys[i]) ? 1 : 0;
+}
+
+// A long run is not walked by one thread per element (a batch of the walk costs a memory latency, and one hot row
+// holds up the whole launch): it goes on a list for index_add_long_runs_kernel. The walk streams the source at the
+// memory's rate as long as there are threads enough and no thread walks for longer than the whole source takes to
+// read, so "long" is a 2^18-th of the source's elements, no less than kLongRunMin and no more than kLongRunMax.
+constexpr uint32_t kLongRunMin = 256, kLongRunMax = 4096;
+constexpr uint32_t kLongWaves = 16, kLongEntries = 32;
+struct LongRuns {
+    uint32_t* start;        // where the run starts in the sorted list
+    uint32_t* len;
+    uint32_t* key;          // its target row
+    uint32_t* count;
+};
+// One thread per run of the compacted heads.
+__global__ __launch_bounds__(kBlock) void index_long_runs_of_heads_kernel(const uint32_t* __restrict__ keys, const uint32_t* __restrict__ heads,
+                                                                         const uint32_t* __restrict__ head_count, uint32_t k, uint32_t axis_len,
+                                                                         uint32_t long_from, LongRuns runs) {
+    const uint32_t h = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t n = *head_count;
+    if (h >= n) return;
+    const uint32_t i = heads[h];
+    const uint32_t len = (h + 1 < n ? heads[h + 1] : k) - i;
     const uint32_t key = keys[i];
-    flags[i] = (key < axis_len && (i == 0 || keys[i - 1] != key)) ? 1 : 0;
+    if (len < long_from || key >= axis_len) return;
+    const uint32_t slot = atomicAdd(runs.count, 1u);
+    runs.start[slot] = i; runs.len[slot] = len; runs.key[slot] = key;
+}
+// One thread per target row, for the form that knows every row's first and one-past-last list position.
+__global__ __launch_bounds__(kBlock) void index_long_runs_of_rows_kernel(const uint32_t* __restrict__ row_first, const uint32_t* __restrict__ row_end,
+                                                                        uint32_t axis_len, uint32_t long_from, LongRuns runs) {
+    const uint32_t key = blockIdx.x * kBlock + threadIdx.x;
+    if (key >= axis_len) return;
+    const uint32_t i = row_first[key];
+    if (i == 0xffffffffu) return;
+    const uint32_t len = row_end[key] - i;
+    if (len < long_from) return;
+    const uint32_t slot = atomicAdd(runs.count, 1u);
+    runs.start[slot] = i; runs.len[slot] = len; runs.key[slot] = key;
 }
 
 // row_first[r] = where target row r's run starts in the sorted list, ~0u for a row no entry names.
@@ -364,22 +408,47 @@ __global__ __launch_bounds__(kBlock) void index_row_first_clear_kernel(uint32_t*
     const uint32_t r = blockIdx.x * kBlock + threadIdx.x;
     if (r < axis_len) row_first[r] = 0xffffffffu;
 }
+// ... and row_end[r] = one past where it ends (only read for rows that have a first position).
 __global__ __launch_bounds__(kBlock) void index_row_first_kernel(const uint32_t* __restrict__ keys, uint32_t k, uint32_t axis_len,
-                                                                uint32_t* __restrict__ row_first) {
+                                                                uint32_t* __restrict__ row_first, uint32_t* __restrict__ row_end) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= k) return;
     const uint32_t key = keys[i];
-    if (key < axis_len && (i == 0 || keys[i - 1] != key)) row_first[key] = i;
+    if (key >= axis_len) return;
+    if (i == 0 || keys[i - 1] != key) row_first[key] = i;
+    if (i + 1 == k || keys[i + 1] != key) row_end[key] = i + 1;
+}
+
+// acc + rows[vals[first]] * alpha + rows[vals[first + 1]] * alpha + ... up to `end`, one rounding per product and per
+// sum, in list order. The run's length is known, so up to kWalkBatch row numbers and then as many source loads are in
+// flight before the adds that wait for them: a thread that walks a run pays the memory latency once per batch.
+constexpr uint32_t kWalkBatch = 8;
+template <class T>
+__device__ __forceinline__ T walk_run(T acc, const T* __restrict__ s, size_t row_stride, const uint32_t* __restrict__ vals,
+                                      uint32_t first, uint32_t end, float alpha) {
+    for (uint32_t r = first; r < end; r += kWalkBatch) {
+        const uint32_t m = min(kWalkBatch, end - r);
+        uint32_t rows[kWalkBatch];
+        T v[kWalkBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) rows[j] = vals[r + j];
+#pragma unroll
+        for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) v[j] = __builtin_nontemporal_load(s + static_cast<size_t>(rows[j]) * row_stride);
+#pragma unroll
+        for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) acc = acc + v[j] * alpha;
+    }
+    return acc;
 }
 
 // indexAdd into a target that is owed one constant everywhere and holds nothing yet (fresh from
 // zerosLike): one thread per unit (float or float4) of the whole target [outer, axis, inner]. A row that
 // the list names starts from the constant and takes its run's source rows in order, as below; any
-// other row is the constant. Every element is written once and none is read.
+// other row is the constant. Every element is written once and none is read. Rows with a long run are left
+// to index_add_long_runs_kernel.
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restrict__ target, const float* __restrict__ src,
-                                                                 const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
-                                                                 const uint32_t* __restrict__ row_first, float alpha, float constant,
+                                                                 const uint32_t* __restrict__ vals, const uint32_t* __restrict__ row_first,
+                                                                 const uint32_t* __restrict__ row_end, float alpha, float constant,
                                                                  uint32_t units, RowsPlan pl, FastDiv axis_div) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
@@ -387,37 +456,17 @@ __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restr
     const uint32_t col = e - row * pl.inner;
     const uint32_t o = (__umulhi(row, axis_div.mul) + row) >> axis_div.shift;
     const uint32_t key = row - o * pl.axis_len;
-    uint32_t r = row_first[key];
+    const uint32_t first = row_first[key];
+    const uint32_t end = first != 0xffffffffu ? row_end[key] : 0u;
+    if (first != 0xffffffffu && end - first >= pl.long_from) return;
     const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
     if (VEC) {
-        float4 acc = make_float4(constant, constant, constant, constant);
-        if (r != 0xffffffffu) {
-            const v4f_lds* s = reinterpret_cast<const v4f_lds*>(src) + s_base;
-            v4f_lds v = __builtin_nontemporal_load(s + static_cast<size_t>(vals[r]) * pl.inner);
-            while (true) {
-                const bool more = r + 1 < pl.k && keys[r + 1] == key;
-                v4f_lds next = v;
-                if (more) next = __builtin_nontemporal_load(s + static_cast<size_t>(vals[r + 1]) * pl.inner);     // in flight during the adds
-                acc.x = acc.x + v.x * alpha; acc.y = acc.y + v.y * alpha; acc.z = acc.z + v.z * alpha; acc.w = acc.w + v.w * alpha;
-                if (!more) break;
-                v = next; r++;
-            }
-        }
-        reinterpret_cast<float4*>(target)[e] = acc;
+        v4f_lds acc = {constant, constant, constant, constant};
+        if (first != 0xffffffffu) acc = walk_run(acc, reinterpret_cast<const v4f_lds*>(src) + s_base, pl.inner, vals, first, end, alpha);
+        reinterpret_cast<v4f_lds*>(target)[e] = acc;
     } else {
         float acc = constant;
-        if (r != 0xffffffffu) {
-            const float* s = src + s_base;
-            float v = s[static_cast<size_t>(vals[r]) * pl.inner];
-            while (true) {
-                const bool more = r + 1 < pl.k && keys[r + 1] == key;
-                float next = v;
-                if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];
-                acc = acc + v * alpha;
-                if (!more) break;
-                v = next; r++;
-            }
-        }
+        if (first != 0xffffffffu) acc = walk_run(acc, src + s_base, pl.inner, vals, first, end, alpha);
         target[e] = acc;
     }
 }
@@ -425,8 +474,9 @@ __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restr
 // The runs of equal keys are the touched target rows; their first positions (`heads`, *head_count
 // of them) come from a compaction of the sorted list. One thread per unit (float or float4) of
 // [outer, touched row, inner]: it adds the run's source rows in order, target = target + src * alpha
-// each time (two roundings, as JVMRawTensor.kt:515). The grid covers k rows per outer index; threads
-// past the number of touched rows leave at once. No two threads write the same element.
+// each time (two roundings, as JVMRawTensor.kt:515). The grid covers min(k, axis_len + 1) rows per outer index (there
+// cannot be more runs); threads past the number of touched rows leave at once, and so do those of a long run (index_add_long_runs_kernel
+// takes it) and of the run of invalid entries. No two threads write the same element.
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                  const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
@@ -434,45 +484,24 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restr
                                                                  float alpha, uint32_t units, RowsPlan pl) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
-    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * heads + h
     const uint32_t col = e - row * pl.inner;
-    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
-    const uint32_t h = row - o * pl.k;                     // the h-th touched target row
-    if (h >= *head_count) return;
-    const uint32_t i = heads[h];
-    const uint32_t key = keys[i];
+    const uint32_t o = (__umulhi(row, pl.heads_div.mul) + row) >> pl.heads_div.shift;
+    const uint32_t h = row - o * pl.heads;                 // the h-th touched target row
+    const uint32_t n_heads = *head_count;
+    if (h >= n_heads) return;
+    const uint32_t first = heads[h];
+    const uint32_t end = h + 1 < n_heads ? heads[h + 1] : pl.k;
+    const uint32_t key = keys[first];
+    if (key >= pl.axis_len || end - first >= pl.long_from) return;
     const size_t t_at = (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
     const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
     if (VEC) {
-        float4* t = reinterpret_cast<float4*>(target) + t_at;
-        const float4* s = reinterpret_cast<const float4*>(src) + s_base;
-        float4 acc = *t;
-        uint32_t r = i;
-        float4 v = s[static_cast<size_t>(vals[r]) * pl.inner];
-        while (true) {
-            const bool more = r + 1 < pl.k && keys[r + 1] == key;
-            float4 next = v;
-            if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];     // in flight during the adds
-            acc.x = acc.x + v.x * alpha; acc.y = acc.y + v.y * alpha; acc.z = acc.z + v.z * alpha; acc.w = acc.w + v.w * alpha;
-            if (!more) break;
-            v = next; r++;
-        }
-        *t = acc;
+        v4f_lds* t = reinterpret_cast<v4f_lds*>(target) + t_at;
+        *t = walk_run(*t, reinterpret_cast<const v4f_lds*>(src) + s_base, pl.inner, vals, first, end, alpha);
     } else {
         float* t = target + t_at;
-        const float* s = src + s_base;
-        float acc = *t;
-        uint32_t r = i;
-        float v = s[static_cast<size_t>(vals[r]) * pl.inner];
-        while (true) {
-            const bool more = r + 1 < pl.k && keys[r + 1] == key;
-            float next = v;
-            if (more) next = s[static_cast<size_t>(vals[r + 1]) * pl.inner];
-            acc = acc + v * alpha;
-            if (!more) break;
-            v = next; r++;
-        }
-        *t = acc;
+        *t = walk_run(*t, src + s_base, pl.inner, vals, first, end, alpha);
     }
 }
 
@@ -485,29 +514,131 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_ragged_kernel(float* 
                                                                         float alpha, uint32_t units, uint32_t row_floats, RowsPlan pl) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
-    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * k + i
+    const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * heads + h
     const uint32_t off = (e - row * pl.inner) * 4u;
-    const uint32_t o = (__umulhi(row, pl.k_div.mul) + row) >> pl.k_div.shift;
-    const uint32_t h = row - o * pl.k;                     // the h-th touched target row
-    if (h >= *head_count) return;
-    const uint32_t i = heads[h];
-    const uint32_t key = keys[i];
+    const uint32_t o = (__umulhi(row, pl.heads_div.mul) + row) >> pl.heads_div.shift;
+    const uint32_t h = row - o * pl.heads;                 // the h-th touched target row
+    const uint32_t n_heads = *head_count;
+    if (h >= n_heads) return;
+    const uint32_t first = heads[h];
+    const uint32_t end = h + 1 < n_heads ? heads[h + 1] : pl.k;
+    const uint32_t key = keys[first];
+    if (key >= pl.axis_len || end - first >= pl.long_from) return;
     float* t = target + (static_cast<size_t>(o) * pl.axis_len + key) * row_floats + off;
     const float* s = src + static_cast<size_t>(o) * pl.k * row_floats + off;
     const uint32_t cnt = min(4u, row_floats - off);
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (cnt == 4) { const v4f_unaligned v = *reinterpret_cast<const v4f_unaligned*>(t); acc[0] = v.x; acc[1] = v.y; acc[2] = v.z; acc[3] = v.w; }
-    else for (uint32_t j = 0; j < cnt; j++) acc[j] = t[j];
-    for (uint32_t r = i; r < pl.k && keys[r] == key; r++) {
-        const float* p = s + static_cast<size_t>(vals[r]) * row_floats;
-        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (cnt == 4) { const v4f_unaligned w = *reinterpret_cast<const v4f_unaligned*>(p); v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w; }
-        else for (uint32_t j = 0; j < cnt; j++) v[j] = p[j];
+    if (cnt == 4) {
+        v4f_unaligned* t4 = reinterpret_cast<v4f_unaligned*>(t);
+        // the row stride is counted in floats here: units of one float, read as four at a dword address
+        v4f_unaligned acc = *t4;
+        for (uint32_t r = first; r < end; r += kWalkBatch) {
+            const uint32_t m = min(kWalkBatch, end - r);
+            uint32_t rows[kWalkBatch];
+            v4f_unaligned v[kWalkBatch];
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[j] = acc[j] + v[j] * alpha;
+            for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) rows[j] = vals[r + j];
+#pragma unroll
+            for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) v[j] = *reinterpret_cast<const v4f_unaligned*>(s + static_cast<size_t>(rows[j]) * row_floats);
+#pragma unroll
+            for (uint32_t j = 0; j < kWalkBatch; j++) if (j < m) acc = acc + v[j] * alpha;
+        }
+        *t4 = acc;
+    } else {
+        for (uint32_t j = 0; j < cnt; j++) t[j] = walk_run(t[j], s + j, row_floats, vals, first, end, alpha);
     }
-    if (cnt == 4) *reinterpret_cast<v4f_unaligned*>(t) = v4f_unaligned{acc[0], acc[1], acc[2], acc[3]};
-    else for (uint32_t j = 0; j < cnt; j++) t[j] = acc[j];
+}
+
+// A long run (RowsPlan::long_from entries or more into one target row), by a workgroup of WAVES waves per 64 positions
+// (outer index and column) of that row. The adds into one element are a chain that nothing can shorten (4 cycles
+// each), but the loads they wait for need not stand in it. A round is WAVES x E entries: every wave holds its E
+// source values in registers (a lane per position, so a round has WAVES x E x 256 bytes in flight), and then the
+// waves take turns, in list order, adding their values to the 64 sums, which stand in LDS between turns. The
+// values of the next round and the row numbers of the one after it are requested before the turns begin (a wave
+// reads its E row numbers as one word per lane and hands them out with v_readlane), so a round costs its
+// turns and the memory latency is paid once per run. Workgroups take (run, 64 positions) items in a strided loop
+// until the list is done.
+constexpr uint32_t kWave = 64;
+template <uint32_t WAVES, uint32_t E>
+__global__ __launch_bounds__(WAVES * kWave) void index_add_long_runs_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                           const uint32_t* __restrict__ vals, LongRuns runs, float alpha,
+                                                                           uint32_t from_constant, float constant, uint32_t positions,
+                                                                           RowsPlan pl) {
+    static_assert(E <= kWave, "a wave reads its row numbers one per lane");
+    constexpr uint32_t kRound = WAVES * E;
+    __shared__ float carry[kWave];
+    const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    const uint32_t mine = w * E;                               // where this wave's entries start in a round
+    const uint32_t chunks = (positions + kWave - 1) / kWave;
+    const uint64_t n_items = static_cast<uint64_t>(*runs.count) * chunks;
+    for (uint64_t item = blockIdx.x; item < n_items; item += gridDim.x) {
+        const uint32_t slot = static_cast<uint32_t>(item / chunks);
+        const uint32_t p = static_cast<uint32_t>(item - static_cast<uint64_t>(slot) * chunks) * kWave + lane;     // o * inner + column
+        const bool active = p < positions;
+        const uint32_t o = active ? (__umulhi(p, pl.inner_div.mul) + p) >> pl.inner_div.shift : 0u;
+        const uint32_t col = active ? p - o * pl.inner : 0u;
+        const uint32_t first = runs.start[slot], len = runs.len[slot], key = runs.key[slot];
+        float* t = target + (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
+        const float* s = src + static_cast<size_t>(o) * pl.k * pl.inner + col;
+        if (w == 0) carry[lane] = (active && !from_constant) ? *t : constant;
+        // the wave's row numbers of the round that starts at `base`: lane j holds entry j's (0 past the run's end)
+        auto rows_of = [&](uint32_t base) -> uint32_t {
+            const uint32_t at = base + mine + lane;
+            return (lane < E && at < len) ? vals[first + at] : 0u;
+        };
+        auto count_of = [&](uint32_t base) -> uint32_t {
+            const uint32_t at = base + mine;
+            return at < len ? min(E, len - at) : 0u;
+        };
+        float v[E], v_next[E];
+        uint32_t rows_next = rows_of(0);
+#pragma unroll
+        for (uint32_t j = 0; j < E; j++) v_next[j] = 0.0f;
+        {
+            const uint32_t cnt = count_of(0);
+#pragma unroll
+            for (uint32_t j = 0; j < E; j++) {
+                const uint32_t row = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(rows_next), static_cast<int>(j)));
+                if (j < cnt && active) v_next[j] = __builtin_nontemporal_load(s + static_cast<size_t>(row) * pl.inner);
+            }
+        }
+        rows_next = rows_of(kRound);
+        for (uint32_t base = 0; base < len; base += kRound) {
+#pragma unroll
+            for (uint32_t j = 0; j < E; j++) v[j] = v_next[j];
+            const uint32_t cnt = count_of(base);
+            // what the later rounds need goes out before this one's turns: the next round's values first (their row
+            // numbers arrived a round ago), then the row numbers of the round after it
+            {
+                const uint32_t cnt_next = count_of(base + kRound);
+#pragma unroll
+                for (uint32_t j = 0; j < E; j++) {
+                    const uint32_t row = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(rows_next), static_cast<int>(j)));
+                    v_next[j] = 0.0f;
+                    if (j < cnt_next && active) v_next[j] = __builtin_nontemporal_load(s + static_cast<size_t>(row) * pl.inner);
+                }
+            }
+            rows_next = rows_of(base + 2 * kRound);
+#pragma unroll
+            for (uint32_t j = 0; j < E; j++) v[j] = v[j] * alpha;
+            const uint32_t in_round = min(kRound, len - base);
+            const uint32_t turns = (in_round + E - 1) / E;
+            for (uint32_t turn = 0; turn < turns; turn++) {
+                if (w == turn) {
+                    float acc = carry[lane];
+                    if (cnt == E) {                             // a full batch: nothing but the chain of adds
+#pragma unroll
+                        for (uint32_t j = 0; j < E; j++) acc = acc + v[j];
+                    } else {
+#pragma unroll
+                        for (uint32_t j = 0; j < E; j++) if (j < cnt) acc = acc + v[j];
+                    }
+                    carry[lane] = acc;
+                }
+                __syncthreads();
+            }
+        }
+        if (w == 0 && active) *t = carry[lane];
+    }
 }
 
 
@@ -1070,16 +1201,23 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     int end_bit = 1;
     while (end_bit < 32 && (1ull << end_bit) <= pl.axis_len) end_bit++;      // keys run up to axis_len inclusive
     const uint64_t k_pad = (k + 63) & ~63ull;                                // keeps the four arrays 256-byte aligned
+    // (the walk needs a couple of waves on every SIMD to keep the memory busy, and rows whose length is not a multiple
+    // of 4 walk at a quarter of the rate: with fewer than 100 000 threads, or such rows, the smallest threshold)
+    const uint64_t walk_threads = outer * std::min<uint64_t>(k, pl.axis_len) * ((inner + 3) / 4);
+    pl.long_from = static_cast<uint32_t>(std::min<uint64_t>(std::max<uint64_t>(n_src >> 18, kLongRunMin), kLongRunMax));
+    if (walk_threads < 100000 || (inner % 4 != 0 && inner > 4)) pl.long_from = kLongRunMin;
+    const uint64_t long_pad = (k / pl.long_from + 64) & ~63ull;              // no more runs than that can be long
     size_t select_bytes = 0;
     if (k >= kSortedFrom &&
         sort_pairs_u32(nullptr, &temp_bytes, nullptr, nullptr, nullptr, nullptr, pl.k, end_bit, stream) == hipSuccess &&
         select_flagged_positions(nullptr, &select_bytes, nullptr, nullptr, nullptr, pl.k, stream) == hipSuccess) {
         if (select_bytes > temp_bytes) temp_bytes = select_bytes;           // the two passes share their scratch
         temp_bytes = (temp_bytes + 255) & ~static_cast<size_t>(255);
-        // keys, vals, sorted keys, sorted vals, heads: k_pad each; count: 64; flags: k_pad bytes; then, for a target
-        // written from a constant, the first list position of every target row
-        keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 64 * 4 + k_pad + temp_bytes +
-                                                             (from_constant ? (static_cast<uint64_t>(pl.axis_len) + 64) * 4 : 0), &cap));
+        // keys, vals, sorted keys, sorted vals, heads: k_pad each; two counts: 64 each; start, length and target row of
+        // the long runs: long_pad each; the passes' scratch; flags: k_pad bytes; then, for a target written from a
+        // constant, the first and the one-past-last list position of every target row
+        keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 2 * 64 * 4 + 3 * long_pad * 4 + k_pad + temp_bytes +
+                                                             (from_constant ? 2 * (static_cast<uint64_t>(pl.axis_len) + 64) * 4 : 0), &cap));
     }
     if (!keys) {
         (void)hipGetLastError();
@@ -1096,10 +1234,19 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     uint32_t* vals_sorted = keys_sorted + k_pad;
     uint32_t* heads = vals_sorted + k_pad;
     uint32_t* head_count = heads + k_pad;
-    void* temp = head_count + 64;
+    LongRuns runs{};
+    runs.count = head_count + 64;
+    runs.start = runs.count + 64; runs.len = runs.start + long_pad; runs.key = runs.len + long_pad;
+    void* temp = runs.key + long_pad;
     uint8_t* flags = reinterpret_cast<uint8_t*>(temp) + temp_bytes;
+    // the long runs: a lane per float position of the row, whatever unit the walking kernel takes
+    RowsPlan long_pl = pl;
+    const uint32_t long_chunks = static_cast<uint32_t>((positions + kWave - 1) / kWave);
+    const uint64_t long_items = (k / pl.long_from) * long_chunks;           // at most
+    const dim3 long_grid(static_cast<uint32_t>(std::min<uint64_t>(long_items, 8ull * static_cast<uint64_t>(state().compute_units))));
     if (from_constant) {
         uint32_t* row_first = reinterpret_cast<uint32_t*>(flags + k_pad);
+        uint32_t* row_end = row_first + pl.axis_len + 64;
         if (vec_inner) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }
         const uint32_t units = static_cast<uint32_t>(total / (vec_inner ? 4 : 1));
         hipError_t sort_status = hipSuccess;
@@ -1107,18 +1254,27 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
             {
                 LaunchScope scope("index_sort", "", k * 4 * 7);
                 hipLaunchKernelGGL(index_keys_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, sx->ptr, pl.k,
-                                   pl.axis_len, keys, vals, flag);
+                                   pl.axis_len, keys, vals, flag, runs.count);
                 size_t scratch = temp_bytes;
                 sort_status = sort_pairs_u32(temp, &scratch, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
                 if (sort_status != hipSuccess) return;
                 hipLaunchKernelGGL(index_row_first_clear_kernel, dim3((pl.axis_len + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, row_first, pl.axis_len);
-                hipLaunchKernelGGL(index_row_first_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, row_first);
+                hipLaunchKernelGGL(index_row_first_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, row_first, row_end);
+                if (long_items > 0)
+                    hipLaunchKernelGGL(index_long_runs_of_rows_kernel, dim3((pl.axis_len + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, row_first, row_end, pl.axis_len, pl.long_from, runs);
             }
-            LaunchScope scope("index_add_filled_kernel", vec_inner ? "float4" : "float", (total + n_src) * 4 + k * 4);
-            const dim3 grid((units + kBlock - 1) / kBlock);
-            const FastDiv axis_div = make_div(pl.axis_len);
-            if (vec_inner) hipLaunchKernelGGL((index_add_filled_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, row_first, alpha, constant, units, pl, axis_div);
-            else           hipLaunchKernelGGL((index_add_filled_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, row_first, alpha, constant, units, pl, axis_div);
+            {
+                LaunchScope scope("index_add_filled_kernel", vec_inner ? "float4" : "float", (total + n_src) * 4 + k * 4);
+                const dim3 grid((units + kBlock - 1) / kBlock);
+                const FastDiv axis_div = make_div(pl.axis_len);
+                if (vec_inner) hipLaunchKernelGGL((index_add_filled_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div);
+                else           hipLaunchKernelGGL((index_add_filled_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div);
+            }
+            if (long_items > 0) {
+                LaunchScope scope("index_add_long_runs_kernel", "from a constant", 0);
+                hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 1u, constant,
+                                   static_cast<uint32_t>(positions), long_pl);
+            }
         });
         workspace_release(reinterpret_cast<float*>(keys), cap);
         if (sort_status != hipSuccess) { return fail(KTH_E_DEVICE, "kth_index_add: sorting the index list failed: %s", hipGetErrorString(sort_status)); }
@@ -1129,28 +1285,40 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     const bool ragged = !vec && inner > 4 && outer * k * ((inner + 3) / 4) <= kMaxElements;
     if (vec) { pl.inner = static_cast<uint32_t>(inner / 4); pl.inner_div = make_div(pl.inner); }
     if (ragged) { pl.inner = static_cast<uint32_t>((inner + 3) / 4); pl.inner_div = make_div(pl.inner); }
-    const uint32_t units = static_cast<uint32_t>(vec ? n_src / 4 : ragged ? outer * k * pl.inner : n_src);
+    pl.heads = static_cast<uint32_t>(std::min<uint64_t>(k, static_cast<uint64_t>(pl.axis_len) + 1));
+    pl.heads_div = make_div(pl.heads);
+    const uint32_t units = static_cast<uint32_t>(outer * pl.heads * pl.inner);
     hipError_t sort_status = hipSuccess;
     int rc = with_index_check("Index Add", [&](int* flag) {
         {
             LaunchScope scope("index_sort", "", k * 4 * 7);
             hipLaunchKernelGGL(index_keys_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, sx->ptr, pl.k,
-                               pl.axis_len, keys, vals, flag);
+                               pl.axis_len, keys, vals, flag, runs.count);
             size_t scratch = temp_bytes;
             sort_status = sort_pairs_u32(temp, &scratch, keys, keys_sorted, vals, vals_sorted, pl.k, end_bit, stream);
             if (sort_status == hipSuccess) {
-                hipLaunchKernelGGL(index_heads_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, flags);
+                hipLaunchKernelGGL(index_heads_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, flags);
                 scratch = temp_bytes;
                 sort_status = select_flagged_positions(temp, &scratch, flags, heads, head_count, pl.k, stream);
             }
+            if (sort_status == hipSuccess && long_items > 0)
+                hipLaunchKernelGGL(index_long_runs_of_heads_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, heads, head_count, pl.k,
+                                   pl.axis_len, pl.long_from, runs);
         }
         if (sort_status != hipSuccess) return;
-        LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : ragged ? "float4 at dword addresses" : "float", 3 * n_src * 4 + k * 4);
-        const dim3 grid((units + kBlock - 1) / kBlock);
-        if (ragged) hipLaunchKernelGGL(index_add_sorted_ragged_kernel, grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units,
-                                       static_cast<uint32_t>(inner), pl);
-        else if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
-        else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
+        {
+            LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : ragged ? "float4 at dword addresses" : "float", 3 * n_src * 4 + k * 4);
+            const dim3 grid((units + kBlock - 1) / kBlock);
+            if (ragged) hipLaunchKernelGGL(index_add_sorted_ragged_kernel, grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units,
+                                           static_cast<uint32_t>(inner), pl);
+            else if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
+            else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
+        }
+        if (long_items > 0) {
+            LaunchScope scope("index_add_long_runs_kernel", "", 0);
+            hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 0u, 0.0f,
+                               static_cast<uint32_t>(positions), long_pl);
+        }
     });
     workspace_release(reinterpret_cast<float*>(keys), cap);
     if (sort_status != hipSuccess) return fail(KTH_E_DEVICE, "kth_index_add: sorting the index list failed: %s", hipGetErrorString(sort_status));

@@ -199,6 +199,58 @@ def test_index_select_and_index_add_parity(shape, axis, k, gc):
         assert_bits_equal(gt.toArray(), ct.toArray(), f"indexAdd alpha {alpha} (repeated indices accumulate in index order)")
 
 
+def skewed_rows(rng, n_rows, k, hot):
+    """k row numbers below n_rows of which the share `hot` names row 3 % n_rows, the others uniform."""
+    idx = rng.integers(0, n_rows, [k])
+    idx[rng.random(k) < hot] = 3 % n_rows
+    return idx.astype(np.float32)
+
+
+# target shape, axis, list length, share of the list that names one hot row. Runs of 256 entries or more of one target row are
+# added by a workgroup whose sixteen waves take turns over 32 entries each (512 a round): run lengths around the
+# threshold, around one round and several, rows of 1, 3, 64, 65, 256 and 1023 floats, an outer index, rows that
+# only the hot run touches, and lists in which every run is long.
+LONG_RUN_CASES = [([7], 0, 300, 0.9), ([40], 0, 20000, 0.5), ([5, 64], 0, 2000, 0.3), ([5, 65], 0, 2600, 0.6), ([300, 256], 0, 9000, 0.2),
+                  ([3, 1023], 0, 1500, 0.0), ([2, 6, 3], 1, 4000, 0.4), ([3, 50, 8], 1, 30000, 0.7), ([64, 1], 0, 100000, 0.25),
+                  ([1, 100], 0, 255, 0.0), ([1, 100], 0, 256, 0.0), ([1, 100], 0, 257, 0.0), ([1, 100], 0, 511, 0.0), ([1, 100], 0, 512, 0.0),
+                  ([1, 100], 0, 513, 0.0), ([1, 100], 0, 1024, 0.0), ([1, 100], 0, 1025, 0.0), ([1, 100], 0, 1056, 0.0), ([2, 4], 0, 1537, 0.0),
+                  ([1000, 128], 0, 60000, 0.5), ([12, 2048], 0, 12000, 0.1)]
+
+
+@pytest.mark.parametrize("shape,axis,k,hot", LONG_RUN_CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_index_add_with_long_runs(shape, axis, k, hot, gc):
+    rng = np.random.default_rng(sum(shape) * 7 + k)
+    cpu = jo.JvmOracleOperations()
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = skewed_rows(rng, shape[axis], k, hot)
+    sshape = list(shape); sshape[axis] = k
+    src = rng.standard_normal(sshape).astype(np.float32)
+    src *= np.exp(rng.uniform(-12, 12, src.shape)).astype(np.float32)      # sums that depend on the order of the adds
+    src[rng.random(src.shape) < 0.01] = -0.0
+    gi, ci = gc.createRaw([k], idx), cpu.createRaw([k], idx)
+    gs, cs = gc.createRaw(sshape, src), cpu.createRaw(sshape, src)
+    for alpha in (1.0, -0.3):
+        gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
+        gt.indexAdd(axis, gi, gs, alpha); ct.indexAdd(axis, ci, cs, alpha)
+        assert_bits_equal(gt.toArray(), ct.toArray(), f"indexAdd alpha {alpha}")
+        # into a target that is a constant nobody has written out (-0.0: 0 + s would lose the sign of a -0 sum)
+        for constant in (0.0, -0.0, 1.5):
+            gz, cz = gc.createRawFill(shape, constant), cpu.createRawFill(shape, constant)
+            gz.indexAdd(axis, gi, gs, alpha); cz.indexAdd(axis, ci, cs, alpha)
+            assert_bits_equal(gz.toArray(), cz.toArray(), f"indexAdd into a fill of {constant}, alpha {alpha}")
+
+
+def test_index_add_long_run_with_a_bad_entry(gc):
+    """A list whose runs are long and that holds values out of range: the call is refused, and the valid entries that
+    were added before the refusal leave a tensor that still works."""
+    idx = np.zeros(5000, dtype=np.float32); idx[1000:3000] = 1.0; idx[4000] = 9.0; idx[4500] = -2.0
+    t = gc.createRaw([2, 16], np.zeros(32, dtype=np.float32))
+    with pytest.raises(ValueError):
+        t.indexAdd(0, gc.createRaw([5000], idx), gc.createRaw([5000, 16], np.ones(80000, dtype=np.float32)))
+    t.inplaceFill(1.0)
+    assert t.toList() == [1.0] * 32
+
+
 def test_index_select_errors(gc):
     x = gc.createRaw([2, 3], np.arange(6, dtype=np.float32))
     for bad in (3.0, -1.0):
