@@ -132,6 +132,29 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
                 if (MODE != 2) fv[k] = src[bo + (i0 + k) * pl.b_axis_stride];
             }
         }
+        if (MODE == 1 && i0 + kScatterBatch <= pl.i_axis_len) {
+            // a full batch of adds whose eight entries are valid and name eight different elements: the elements
+            // are read together and written together. (A repeated element needs its adds one after the other,
+            // through memory: the loop below.)
+            uint32_t sel[kScatterBatch];
+            bool apart = true;
+#pragma unroll
+            for (uint32_t k = 0; k < kScatterBatch; k++) {
+                const int v = static_cast<int>(fi[k]);
+                sel[k] = static_cast<uint32_t>(v);
+                apart = apart && v >= 0 && sel[k] < pl.a_axis_len;
+#pragma unroll
+                for (uint32_t j = 0; j < k; j++) apart = apart && sel[j] != sel[k];
+            }
+            if (apart) {
+                float cur[kScatterBatch];
+#pragma unroll
+                for (uint32_t k = 0; k < kScatterBatch; k++) cur[k] = target[ao + sel[k] * pl.a_axis_stride];
+#pragma unroll
+                for (uint32_t k = 0; k < kScatterBatch; k++) target[ao + sel[k] * pl.a_axis_stride] = cur[k] + fv[k];
+                continue;
+            }
+        }
 #pragma unroll
         for (uint32_t k = 0; k < kScatterBatch; k++) {
             if (i0 + k < pl.i_axis_len) {
@@ -143,6 +166,62 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(float* __restrict__ tar
                 else *to = fv[k];
             }
         }
+    }
+}
+
+// Scatter along the innermost axis, a wave per position: its lanes take 64 consecutive entries of the index row at
+// a time (coalesced reads of index and source, 64 elements of the target in flight), where scatter_kernel has one
+// thread walk the row. Entries of one step that name the same element find each other by a ballot per bit of the
+// element number. An assignment is then made by the highest lane of each such group (the last entry wins). For an add
+// the group's first lane reads the element, the sum goes from lane to lane in lane order (one shuffle per round, as
+// many rounds as the step's most frequent element occurs: nearly always none) and the last lane writes it. Steps
+// follow each other in the order of the row, a step's writes made visible to the wave before the next one's reads;
+// the next step's index and source values are requested before that wait.
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void scatter_wave_kernel(float* __restrict__ target, const float* __restrict__ index,
+                                                             const float* __restrict__ src, float value, uint32_t positions,
+                                                             IndexPlan pl, int* bad, int element_bits) {
+    const uint32_t pos = blockIdx.x * (kBlock / 64) + threadIdx.x / 64;
+    const uint32_t lane = threadIdx.x & 63u;
+    if (pos >= positions) return;                              // the whole wave
+    uint32_t io, ao, bo;
+    locate(pl, pos, io, ao, bo);
+    float fi_next = lane < pl.i_axis_len ? __builtin_nontemporal_load(index + io + lane) : 0.0f;
+    float fv_next = (MODE != 2 && lane < pl.i_axis_len) ? __builtin_nontemporal_load(src + bo + lane * pl.b_axis_stride) : 0.0f;
+    for (uint32_t i0 = 0; i0 < pl.i_axis_len; i0 += 64) {
+        const bool have = i0 + lane < pl.i_axis_len;
+        const float fi = fi_next, fv = fv_next;
+        const uint32_t ahead = i0 + 64 + lane;
+        if (ahead < pl.i_axis_len) {
+            fi_next = __builtin_nontemporal_load(index + io + ahead);
+            if (MODE != 2) fv_next = __builtin_nontemporal_load(src + bo + ahead * pl.b_axis_stride);
+        }
+        const int sel = static_cast<int>(fi);
+        const bool ok = have && sel >= 0 && static_cast<uint32_t>(sel) < pl.a_axis_len;
+        if (have && !ok) *bad = 1;
+        unsigned long long same = __ballot(ok);
+        for (int bit = 0; bit < element_bits; bit++) {
+            const bool set = (sel >> bit) & 1;
+            const unsigned long long with = __ballot(ok && set);
+            same &= set ? with : ~with;
+        }
+        float* to = target + ao + static_cast<uint32_t>(ok ? sel : 0);
+        const bool last = ok && ((same >> lane) >> 1) == 0;    // no later entry of the step names the element
+        if (MODE != 1) {
+            if (last) *to = MODE == 2 ? value : fv;
+        } else {
+            const unsigned long long before = same & ((1ull << lane) - 1ull);
+            const uint32_t rank = ok ? __popcll(before) : 0u;
+            const int from = before ? 63 - __clzll(static_cast<long long>(before)) : static_cast<int>(lane);
+            float sum = 0.0f;
+            if (ok && rank == 0) sum = *to + fv;
+            for (uint32_t round = 1; __ballot(ok && rank >= round) != 0; round++) {
+                const float carried = __shfl(sum, from);
+                if (ok && rank == round) sum = carried + fv;
+            }
+            if (last) *to = sum;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
     }
 }
 
@@ -936,6 +1015,20 @@ static int scatter_launch(int mode, float* target, const int32_t* target_shape, 
         });
     }
     if (constant) return fail(KTH_E_ARGUMENT, "kth_scatter: internal: the serial form cannot start from a constant");
+    // along the innermost axis, with index rows of half a wave or more: a wave per position
+    if (axis == dims - 1 && pl.i_axis_len >= 32 && positions <= 0x3fffffffull) {
+        int element_bits = 1;
+        while (element_bits < 31 && (1u << element_bits) < pl.a_axis_len) element_bits++;
+        return with_index_check("Scatter", [&](int* flag) {
+            LaunchScope scope("scatter_wave_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
+            const uint32_t p32 = static_cast<uint32_t>(positions);
+            const dim3 grid((p32 + kBlock / 64 - 1) / (kBlock / 64)), block(kBlock);
+            hipStream_t stream = state().stream;
+            if (mode == 0)      hipLaunchKernelGGL((scatter_wave_kernel<0>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag, element_bits);
+            else if (mode == 1) hipLaunchKernelGGL((scatter_wave_kernel<1>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag, element_bits);
+            else                hipLaunchKernelGGL((scatter_wave_kernel<2>), grid, block, 0, stream, target, index, psrc, value, p32, pl, flag, element_bits);
+        });
+    }
     return with_index_check("Scatter", [&](int* flag) {
         LaunchScope scope("scatter_kernel", mode == 0 ? "set" : mode == 1 ? "add" : "fill", bytes);
         const dim3 grid(blocks), block(kBlock);

@@ -199,6 +199,32 @@ def test_index_select_and_index_add_parity(shape, axis, k, gc):
         assert_bits_equal(gt.toArray(), ct.toArray(), f"indexAdd alpha {alpha} (repeated indices accumulate in index order)")
 
 
+@pytest.mark.parametrize("shape,i_len,spread", [([300, 5000], 200, 5000), ([300, 5000], 200, 8), ([300, 5000], 200, 1), ([40, 70000], 100, 70000),
+                                                ([40, 70000], 333, 3), ([7, 3, 900], 65, 40), ([1000, 600], 32, 600), ([5, 100000], 1000, 2)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_scatter_by_a_wave_per_row_with_repeated_elements(shape, i_len, spread, gc):
+    """Index rows of 32 entries or more along the innermost axis that are too short (or whose target rows are too long)
+    for the rows-through-LDS kernel: a wave per row, 64 entries a step. `spread` is how many different elements a row's
+    entries name: with few, most lanes of a step share their element and the order of the adds and the last entry
+    of an assignment are decided inside the wave."""
+    rng = np.random.default_rng(sum(shape) + i_len + spread)
+    cpu = jo.JvmOracleOperations()
+    ishape = list(shape); ishape[-1] = i_len
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = (rng.integers(0, spread, ishape) * (shape[-1] // spread)).astype(np.float32)
+    src = rng.standard_normal(ishape).astype(np.float32)
+    src *= np.exp(rng.uniform(-12, 12, src.shape)).astype(np.float32)      # sums that depend on the order of the adds
+    gi, ci = gc.createRaw(ishape, idx), cpu.createRaw(ishape, idx)
+    gs, cs = gc.createRaw(ishape, src), cpu.createRaw(ishape, src)
+    gc.profileBegin()
+    for name, source in (("inplaceScatter", (gs, cs)), ("inplaceScatterAdd", (gs, cs)), ("inplaceScatter", (2.5, 2.5))):
+        gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
+        getattr(gt, name)(-1, gi, source[0]); getattr(ct, name)(-1, ci, source[1])
+        assert_bits_equal(gt.toArray(), ct.toArray(), f"{name} {'constant' if source[0] == 2.5 else 'tensor'}")
+    names = set(gc.profileEnd())
+    assert {"scatter_wave_kernel<set>", "scatter_wave_kernel<add>", "scatter_wave_kernel<fill>"} <= names, names
+
+
 def skewed_rows(rng, n_rows, k, hot):
     """k row numbers below n_rows of which the share `hot` names row 3 % n_rows, the others uniform."""
     idx = rng.integers(0, n_rows, [k])
