@@ -1336,7 +1336,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     RowsPlan long_pl = pl;
     const uint32_t long_chunks = static_cast<uint32_t>((positions + kWave - 1) / kWave);
     const uint64_t long_items = (k / pl.long_from) * long_chunks;           // at most
-    const dim3 long_grid(static_cast<uint32_t>(std::min<uint64_t>(long_items, 8ull * static_cast<uint64_t>(state().compute_units))));
+    const dim3 long_grid(static_cast<uint32_t>(std::min<uint64_t>(long_items, 2ull * static_cast<uint64_t>(state().compute_units))));
     if (from_constant) {
         uint32_t* row_first = reinterpret_cast<uint32_t*>(flags + k_pad);
         uint32_t* row_end = row_first + pl.axis_len + 64;
