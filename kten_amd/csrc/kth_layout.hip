@@ -170,6 +170,8 @@ struct TilePlan {
     uint32_t x_out_stride, y_in_stride;
     uint32_t x_tiles, y_tiles;
     FastDiv  x_tiles_div, y_tiles_div;
+    uint32_t tiles;                          // permute_tile_kernel: the grid holds this many rounded up to a multiple of 8
+    uint32_t by_xcd;                         // ... and an XCD takes a contiguous eighth of them (rows that do not start on a cache line)
     int      nbatch;
     uint32_t bsize[KTH_MAX_DIMS];
     FastDiv  bdiv[KTH_MAX_DIMS];
@@ -189,7 +191,13 @@ template <int TX, int TY, class V>
 __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restrict__ in, V* __restrict__ out, TilePlan pl) {
     static_assert(TX * TY * sizeof(V) == kTileElems * sizeof(float), "a tile holds 16 KiB");
     __shared__ V tile[TY * (TX + 1)];
-    uint32_t t = blockIdx.x;
+    // Workgroups go to the eight XCDs in turn. When the rows of the output or of the input do not start on a cache
+    // line, each XCD takes one contiguous eighth of the tiles, so that the two tiles that share a line write it into
+    // one L2, where the halves meet, and not into two, each of which would send a partial line to memory. With
+    // aligned rows the tiles go round the XCDs one by one, which spreads the memory channels better (6.2 TB/s on
+    // 8192 x 8192 against 3.8 by eighths).
+    uint32_t t = pl.by_xcd ? (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    if (t >= pl.tiles) return;
     uint32_t q = (__umulhi(t, pl.x_tiles_div.mul) + t) >> pl.x_tiles_div.shift;
     const uint32_t x0 = (t - q * pl.x_tiles) * TX;
     t = q;
@@ -656,8 +664,12 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     pl.nbatch = nb;
     for (int d = 0; d < nb; d++) { pl.bsize[d] = bsize[d]; pl.bdiv[d] = make_div(bsize[d]); pl.b_in[d] = b_in[d]; pl.b_out[d] = b_out[d]; }
     const uint64_t blocks = static_cast<uint64_t>(pl.x_tiles) * pl.y_tiles * batch;
-    if (blocks > kMaxElements) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
-    const dim3 grid(static_cast<uint32_t>(blocks));
+    if (blocks > kMaxElements - 8) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
+    pl.tiles = static_cast<uint32_t>(blocks);
+    const uint32_t line = 128 / (4 * static_cast<uint32_t>(elem));                  // elements per cache line
+    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0) ? 1u : 0u;
+    for (int d = 0; d < nb; d++) if (b_in[d] % line != 0 || b_out[d] % line != 0) pl.by_xcd = 1u;
+    const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
     LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
     if (elem == 4) {
         hipLaunchKernelGGL((permute_tile_kernel<32, 32, v4f>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const v4f*>(in),
