@@ -13,17 +13,19 @@
 namespace kth {
 
 // java.lang.Math.max(float,float): NaN wins, -0 < +0. (JVMRawTensor.kt:159)
+// v_max_f32 / v_min_f32 order the zeros that way themselves (max(+0, -0) = +0 whichever operand holds which) and
+// return the other operand when one is a NaN, so the instruction and one unordered compare make the Java rule.
 __device__ __forceinline__ float jmax(float a, float b) {
-    if (a != a) return a;
-    if (a == 0.0f && b == 0.0f && __float_as_uint(a) == 0x80000000u) return b;
-    return (a >= b) ? a : b;
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return (a != a || b != b) ? (a != a ? a : b) : r;
 }
 
 // java.lang.Math.min(float,float). (JVMRawTensor.kt:160)
 __device__ __forceinline__ float jmin(float a, float b) {
-    if (a != a) return a;
-    if (a == 0.0f && b == 0.0f && __float_as_uint(b) == 0x80000000u) return b;
-    return (a <= b) ? a : b;
+    float r;
+    asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return (a != a || b != b) ? (a != a ? a : b) : r;
 }
 
 // Float.pow(Float) = Math.pow(double,double).toFloat() (JVMRawTensor.kt:138-140).

@@ -553,8 +553,15 @@ __global__ __launch_bounds__(kBlock) void reduce_finalize_wave_kernel(const type
     if (idx < n_out) {
         const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
         const Acc* p = partial + (static_cast<size_t>(o) * g.segments) * g.inner + i;
-#pragma unroll 8
-        for (uint32_t s = lane; s < g.segments; s += kWave) acc = R::merge(acc, p[static_cast<size_t>(s) * g.inner]);
+        // eight partials are requested before the first is merged (a merge with branches in it would otherwise
+        // wait for every load in turn)
+        for (uint32_t s = lane; s < g.segments; s += 8 * kWave) {
+            Acc v[8];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) if (s + k * kWave < g.segments) v[k] = p[static_cast<size_t>(s + k * kWave) * g.inner];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) if (s + k * kWave < g.segments) acc = R::merge(acc, v[k]);
+        }
     }
 #pragma unroll
     for (int m = kWave / 2; m >= 1; m >>= 1) acc = R::merge(acc, shfl_xor_acc(acc, m));
@@ -574,8 +581,13 @@ __global__ __launch_bounds__(kWave * TY) void reduce_finalize_tile_kernel(const 
     if (idx < n_out) {
         const uint32_t o = static_cast<uint32_t>(idx / g.inner), i = static_cast<uint32_t>(idx % g.inner);
         const Acc* p = partial + (static_cast<size_t>(o) * g.segments) * g.inner + i;
-#pragma unroll 8
-        for (uint32_t s = ty; s < g.segments; s += TY) acc = R::merge(acc, p[static_cast<size_t>(s) * g.inner]);
+        for (uint32_t s = ty; s < g.segments; s += 8 * TY) {
+            Acc v[8];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) if (s + k * TY < g.segments) v[k] = p[static_cast<size_t>(s + k * TY) * g.inner];
+#pragma unroll
+            for (uint32_t k = 0; k < 8; k++) if (s + k * TY < g.segments) acc = R::merge(acc, v[k]);
+        }
     }
     if (TY > 1) {
         __shared__ Acc lds[TY][kWave];
@@ -817,6 +829,9 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         LaunchScope scope("reduce_finalize_kernel", R::name, 0, may_profile);
         if (n_out < 64)
             hipLaunchKernelGGL((reduce_finalize_wave_kernel<R>), dim3(ceil_div(n_out * kWave, kBlock)), dim3(kBlock), 0, stream,
+                               partial, out, g);
+        else if (g.segments >= 128 && n_out <= 16384)       // few workgroups: sixteen waves each
+            hipLaunchKernelGGL((reduce_finalize_tile_kernel<R, 16>), dim3(ceil_div(n_out, kWave)), dim3(kWave, 16), 0, stream,
                                partial, out, g);
         else if (g.segments >= 8)
             hipLaunchKernelGGL((reduce_finalize_tile_kernel<R, 4>), dim3(ceil_div(n_out, kWave)), dim3(kWave, 4), 0, stream,
