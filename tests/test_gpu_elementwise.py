@@ -130,6 +130,26 @@ def test_broadcast_of_two_small_operands_bit_exact(sa, sb, gc):
         assert_bits_equal(got, want, what)
 
 
+# Two operands that are both smaller than the output in the arrangements the outer-product kernels do not take: an
+# operand that keeps the outermost and the innermost dim but not the one between, a batch dim both keep, four to six
+# dims, an operand of one value per batch, innermost dims that are no multiple of 4.
+MANY_DIM_PAIRS = [
+    ([4225, 1, 5], [1, 158, 1]), ([1, 5833, 1], [115, 1, 5]), ([111, 549, 1], [111, 1, 55]), ([248, 4, 1, 21], [1, 4, 161, 1]),
+    ([3, 1, 7, 1, 9, 1], [1, 11, 1, 5, 1, 13]), ([2, 90001, 1], [2, 1, 3]), ([7, 1, 1, 3], [7, 6000, 1, 1]), ([50, 1, 3], [50, 401, 1]),
+    ([2, 3, 1, 5, 1], [2, 1, 300, 1, 7]), ([1, 3, 1, 3], [40001, 1, 1, 1]), ([9, 1, 1201], [1, 5, 1]), ([1201, 1, 9], [1, 5, 1]),
+    ([33000, 1, 3], [1, 2, 1]),
+]
+
+
+@pytest.mark.parametrize("sa,sb", MANY_DIM_PAIRS, ids=lambda s: "x".join(map(str, s)))
+def test_broadcast_of_two_small_operands_in_many_dims_bit_exact(sa, sb, gc):
+    rng = np.random.default_rng(sum(sa) * 11 + sum(sb))
+    a = rng.standard_normal(sa).astype(np.float32); b = rng.standard_normal(sb).astype(np.float32)
+    for op, f in (("minus", np.subtract), ("div", np.divide)):
+        for x, y in ((a, b), (b, a)):
+            assert_bits_equal(raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}")
+
+
 def test_binary_matches_checker_on_small_broadcasts(gc):
     rng = np.random.default_rng(5)
     for sa, sb in SHAPE_PAIRS[:12]:
