@@ -721,6 +721,55 @@ __global__ __launch_bounds__(WAVES * kWave) void index_add_long_runs_kernel(floa
 }
 
 
+// ---- scatter through a sorted list of its entries -----------------------------------------
+// A scatter with few positions and long index rows (a flat tensor, a long axis next to a handful of columns) gives
+// the kernels above one row walker per position and nothing else to do: a flat tensor of 16 million elements with as
+// many entries took seconds. Every entry of the index tensor becomes a pair (target element, source element) instead,
+// in the index tensor's memory order, which lists the entries of one position in the order of the axis. After the
+// stable sort by target element, the entries that fall on one element stand together in that order: an assignment
+// takes the last one of each run, an add takes them all in order (the sorted indexAdd kernels, with rows of one float).
+struct EntryPlan {
+    int      ndim;                         // the dims of the index shape, innermost first
+    uint32_t size[KTH_MAX_DIMS];
+    FastDiv  div[KTH_MAX_DIMS];
+    uint32_t t_stride[KTH_MAX_DIMS];       // target elements per step of the dim (0 at the axis)
+    uint32_t s_stride[KTH_MAX_DIMS];       // source elements per step of the dim
+    uint32_t t_axis_stride, a_axis_len;
+};
+__global__ __launch_bounds__(kBlock) void scatter_keys_kernel(const float* __restrict__ index, uint32_t n, EntryPlan pl, uint32_t invalid,
+                                                             uint32_t* __restrict__ keys, uint32_t* __restrict__ vals, int* bad,
+                                                             uint32_t* __restrict__ long_count) {
+    const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e == 0) *long_count = 0;
+    if (e >= n) return;
+    uint32_t rest = e, t = 0, sc = 0;
+    for (int d = 0; d < pl.ndim; d++) {
+        const uint32_t q = (__umulhi(rest, pl.div[d].mul) + rest) >> pl.div[d].shift;
+        const uint32_t c = rest - q * pl.size[d];
+        t += c * pl.t_stride[d]; sc += c * pl.s_stride[d];
+        rest = q;
+    }
+    const int sel = static_cast<int>(__builtin_nontemporal_load(index + e));
+    const bool ok = sel >= 0 && static_cast<uint32_t>(sel) < pl.a_axis_len;
+    if (!ok) *bad = 1;
+    keys[e] = ok ? t + static_cast<uint32_t>(sel) * pl.t_axis_stride : invalid;
+    vals[e] = sc;
+}
+// One thread per run: the element takes the run's last entry (or the constant).
+__global__ __launch_bounds__(kBlock) void scatter_sorted_assign_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                      const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                                                                      const uint32_t* __restrict__ heads, const uint32_t* __restrict__ head_count,
+                                                                      uint32_t k, uint32_t invalid, float value, uint32_t fill) {
+    const uint32_t h = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t n = *head_count;
+    if (h >= n) return;
+    const uint32_t first = heads[h];
+    const uint32_t end = h + 1 < n ? heads[h + 1] : k;
+    const uint32_t key = keys[first];
+    if (key >= invalid) return;
+    target[key] = fill ? value : __builtin_nontemporal_load(src + vals[end - 1]);
+}
+
 int shape_count(const int32_t* shape, int dims, const char* what, uint64_t* count) {
     if (!shape) return fail(KTH_E_ARGUMENT, "%s: null shape", what);
     uint64_t n = 1;
@@ -1094,6 +1143,118 @@ static int scatter_transposed(int mode, float* target, const int32_t* target_sha
     return rc;
 }
 
+// What the walk of the index rows costs on the path the scatter would take, against what sorting its entries costs.
+// The walkers run side by side, so the time is one row's: per chunk of 1024 entries and band of the target row in the
+// rows-through-LDS kernel (measured 0.35 us for an assignment, 0.8 us for an add, 0.23 us for a constant), per step of
+// 64 entries for a wave (1.4 us), per entry for a thread (30 to 85 ns with neighbouring positions sharing cache lines);
+// times the rounds it takes to seat all positions. The sort and what follows it cost about a tenth of a nanosecond
+// per entry (16.7 million entries: 1.2 ms sorted, 1.5 ms in all) and some 100 us of launches.
+static bool scatter_pays_sorting(int mode, const int32_t* target_shape, const int32_t* index_shape, int dims, int axis,
+                                 uint64_t t_n, uint64_t idx_n, bool transposing) {
+    const uint64_t i_len = static_cast<uint64_t>(index_shape[axis]), a_len = static_cast<uint64_t>(target_shape[axis]);
+    if (i_len < 4096 || idx_n > 0x7fffffffull || t_n > 0x7ffffffeull) return false;
+    const double positions = static_cast<double>(idx_n) / static_cast<double>(i_len);
+    double walk_us;
+    if (transposing || scatter_takes_rows(mode, target_shape, index_shape, dims, axis)) {
+        const double bands = static_cast<double>((a_len + 16383) / 16384);
+        const double unit_us = mode == 1 ? 0.8 : mode == 0 ? 0.35 : 0.23;
+        walk_us = bands * static_cast<double>((i_len + 1023) / 1024) * unit_us * std::ceil(positions / 256.0);
+    } else if (axis == dims - 1) {
+        walk_us = static_cast<double>((i_len + 63) / 64) * 1.4 * std::ceil(positions / 8192.0);
+    } else {
+        walk_us = static_cast<double>(i_len) * (mode == 1 ? 0.085 : 0.04) * std::ceil(positions / 524288.0);
+    }
+    const double sort_us = 100.0 + static_cast<double>(idx_n) * 0.0001;
+    return walk_us > 1.5 * sort_us;
+}
+
+static int scatter_sorted(int mode, float* target, const int32_t* target_shape, const float* index, const int32_t* index_shape,
+                          const float* psrc, const int32_t* src_shape, int dims, int axis, float value, uint64_t t_n, uint64_t idx_n) {
+    EntryPlan ep{};
+    ep.ndim = dims;
+    uint64_t t_run = 1, s_run = 1;
+    for (int d = dims - 1, k = 0; d >= 0; d--, k++) {
+        ep.size[k] = static_cast<uint32_t>(index_shape[d]);
+        ep.div[k] = make_div(ep.size[k]);
+        ep.t_stride[k] = d == axis ? 0u : static_cast<uint32_t>(t_run);
+        ep.s_stride[k] = mode == 2 ? 0u : static_cast<uint32_t>(s_run);
+        if (d == axis) ep.t_axis_stride = static_cast<uint32_t>(t_run);
+        t_run *= static_cast<uint64_t>(target_shape[d]);
+        if (mode != 2) s_run *= static_cast<uint64_t>(src_shape[d]);
+    }
+    ep.a_axis_len = static_cast<uint32_t>(target_shape[axis]);
+    const uint32_t k = static_cast<uint32_t>(idx_n), invalid = static_cast<uint32_t>(t_n);
+    int end_bit = 1;
+    while (end_bit < 32 && (1ull << end_bit) <= t_n) end_bit++;              // keys run up to t_n inclusive
+    RowsPlan pl{};
+    pl.axis_len = invalid; pl.k = k; pl.inner = 1;
+    pl.inner_div = make_div(1); pl.k_div = make_div(k);
+    pl.heads = static_cast<uint32_t>(std::min<uint64_t>(idx_n, t_n + 1)); pl.heads_div = make_div(pl.heads);
+    pl.long_from = kLongRunMin;                                              // rows of one float: a thread per run walks alone
+    const uint64_t k_pad = (idx_n + 63) & ~63ull;
+    const uint64_t long_pad = (idx_n / pl.long_from + 64) & ~63ull;
+    hipStream_t stream = state().stream;
+    size_t temp_bytes = 0, select_bytes = 0;
+    if (sort_pairs_u32(nullptr, &temp_bytes, nullptr, nullptr, nullptr, nullptr, k, end_bit, stream) != hipSuccess ||
+        select_flagged_positions(nullptr, &select_bytes, nullptr, nullptr, nullptr, k, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return KTH_E_MEMORY;
+    }
+    if (select_bytes > temp_bytes) temp_bytes = select_bytes;
+    temp_bytes = (temp_bytes + 255) & ~static_cast<size_t>(255);
+    uint64_t cap = 0;
+    uint32_t* keys = reinterpret_cast<uint32_t*>(workspace_acquire(5 * k_pad * 4 + 2 * 64 * 4 + 3 * long_pad * 4 + k_pad + temp_bytes, &cap));
+    if (!keys) { (void)hipGetLastError(); return KTH_E_MEMORY; }
+    uint32_t* vals = keys + k_pad;
+    uint32_t* keys_sorted = vals + k_pad;
+    uint32_t* vals_sorted = keys_sorted + k_pad;
+    uint32_t* heads = vals_sorted + k_pad;
+    uint32_t* head_count = heads + k_pad;
+    LongRuns runs{};
+    runs.count = head_count + 64;
+    runs.start = runs.count + 64; runs.len = runs.start + long_pad; runs.key = runs.len + long_pad;
+    void* temp = runs.key + long_pad;
+    uint8_t* flags = reinterpret_cast<uint8_t*>(temp) + temp_bytes;
+    const uint64_t long_items = idx_n / pl.long_from;                        // at most; one position: one chunk of lanes per run
+    const dim3 long_grid(static_cast<uint32_t>(std::min<uint64_t>(long_items, 2ull * static_cast<uint64_t>(state().compute_units))));
+    const dim3 per_entry((k + kBlock - 1) / kBlock), per_head((pl.heads + kBlock - 1) / kBlock);
+    hipError_t sort_status = hipSuccess;
+    const int rc = with_index_check("Scatter", [&](int* flag) {
+        {
+            LaunchScope scope("scatter_sort", "", idx_n * 4 * 7);
+            hipLaunchKernelGGL(scatter_keys_kernel, per_entry, dim3(kBlock), 0, stream, index, k, ep, invalid, keys, vals, flag, runs.count);
+            size_t scratch = temp_bytes;
+            sort_status = sort_pairs_u32(temp, &scratch, keys, keys_sorted, vals, vals_sorted, k, end_bit, stream);
+            if (sort_status != hipSuccess) return;
+            hipLaunchKernelGGL(index_heads_kernel, per_entry, dim3(kBlock), 0, stream, keys_sorted, k, flags);
+            scratch = temp_bytes;
+            sort_status = select_flagged_positions(temp, &scratch, flags, heads, head_count, k, stream);
+            if (sort_status != hipSuccess) return;
+            if (mode == 1 && long_items > 0)
+                hipLaunchKernelGGL(index_long_runs_of_heads_kernel, per_entry, dim3(kBlock), 0, stream, keys_sorted, heads, head_count, k, invalid, pl.long_from, runs);
+        }
+        if (mode != 1) {
+            LaunchScope scope("scatter_sorted_assign_kernel", mode == 0 ? "set" : "fill", idx_n * (mode == 0 ? 8 : 4));
+            hipLaunchKernelGGL(scatter_sorted_assign_kernel, per_head, dim3(kBlock), 0, stream, target, psrc, keys_sorted, vals_sorted, heads, head_count, k, invalid,
+                               value, mode == 2 ? 1u : 0u);
+            return;
+        }
+        {
+            LaunchScope scope("index_add_sorted_kernel", "scatter", idx_n * 12);
+            hipLaunchKernelGGL((index_add_sorted_kernel<false>), per_head, dim3(kBlock), 0, stream, target, psrc, keys_sorted, vals_sorted, heads, head_count, 1.0f,
+                               pl.heads, pl);
+        }
+        if (long_items > 0) {
+            LaunchScope scope("index_add_long_runs_kernel", "scatter", 0);
+            hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, target, psrc, vals_sorted, runs, 1.0f,
+                               0u, 0.0f, 1u, pl);
+        }
+    });
+    workspace_release(reinterpret_cast<float*>(keys), cap);
+    if (sort_status != hipSuccess) return fail(KTH_E_DEVICE, "kth_scatter: sorting the entries failed: %s", hipGetErrorString(sort_status));
+    return rc;
+}
+
 static int scatter_common(int mode, uint64_t target, const int32_t* target_shape, uint64_t index, const int32_t* index_shape,
                           uint64_t src, const int32_t* src_shape, int dims, int axis, float value) {
     KTH_REQUIRE_INIT();
@@ -1125,6 +1286,11 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
     // A target that is still an owed constant (fresh from zerosLike) need not be filled and read back
     // when the row kernel rewrites all of it: the index covers every position off the axis.
     const bool transposing = scatter_pays_transposing(mode, target_shape, index_shape, dims, axis, t_n, idx_n, src_n);
+    if (scatter_pays_sorting(mode, target_shape, index_shape, dims, axis, t_n, idx_n, transposing)) {
+        settle(st);
+        const int rc = scatter_sorted(mode, st->ptr, target_shape, sx->ptr, index_shape, psrc, src_shape, dims, axis, value, t_n, idx_n);
+        if (rc != KTH_E_MEMORY) return rc;                       // no room for the sorted lists: the walk below
+    }
     bool from_constant = st->fill_n == t_n && (transposing || scatter_takes_rows(mode, target_shape, index_shape, dims, axis));
     for (int d = 0; d < dims; d++) if (d != axis && index_shape[d] != target_shape[d]) from_constant = false;
     const float constant = st->fill_value;

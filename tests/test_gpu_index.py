@@ -225,6 +225,45 @@ def test_scatter_by_a_wave_per_row_with_repeated_elements(shape, i_len, spread, 
     assert {"scatter_wave_kernel<set>", "scatter_wave_kernel<add>", "scatter_wave_kernel<fill>"} <= names, names
 
 
+@pytest.mark.parametrize("shape,axis,i_len,spread,sorted_form", [
+    ([100000], 0, 300000, 100000, True), ([100000], 0, 300000, 3, True), ([1 << 20], 0, 70001, 1 << 20, True),
+    ([50000, 7], 0, 400000, 50000, None), ([6, 1, 90000], 2, 300000, 17, None), ([3, 40000, 2], 1, 100000, 40000, None),
+    ([2, 300000], 1, 500000, 300000, True), ([400], 0, 100000, 400, False)],
+    ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_scatter_of_long_rows_at_few_positions_goes_through_a_sort(shape, axis, i_len, spread, sorted_form, gc):
+    """A handful of positions with index rows of 70 000 to 500 000 entries: the entries are sorted by the element they
+    fall on, an assignment takes the last entry of each run, an add all of them in order. `spread` different elements
+    are named per row: with few, the runs are long (hundreds of thousands of entries on one element)."""
+    rng = np.random.default_rng(sum(shape) + i_len + spread)
+    cpu = jo.JvmOracleOperations()
+    ishape = list(shape); ishape[axis] = i_len
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = (rng.integers(0, spread, ishape) * (shape[axis] // spread)).astype(np.float32)
+    src = rng.standard_normal(ishape).astype(np.float32)
+    src *= np.exp(rng.uniform(-12, 12, src.shape)).astype(np.float32)      # sums that depend on the order of the adds
+    gi, ci = gc.createRaw(ishape, idx), cpu.createRaw(ishape, idx)
+    gs, cs = gc.createRaw(ishape, src), cpu.createRaw(ishape, src)
+    gc.profileBegin()
+    for name, source in (("inplaceScatter", (gs, cs)), ("inplaceScatterAdd", (gs, cs)), ("inplaceScatter", (2.5, 2.5))):
+        gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
+        getattr(gt, name)(axis, gi, source[0]); getattr(ct, name)(axis, ci, source[1])
+        assert_bits_equal(gt.toArray(), ct.toArray(), f"{name} {'constant' if source[0] == 2.5 else 'tensor'}")
+        # a target that is a constant not yet written out
+        gz, cz = gc.createRawFill(shape, -0.0), cpu.createRawFill(shape, -0.0)
+        getattr(gz, name)(axis, gi, source[0]); getattr(cz, name)(axis, ci, source[1])
+        assert_bits_equal(gz.toArray(), cz.toArray(), f"{name} into a fill")
+    names = set(gc.profileEnd())
+    if sorted_form is not None:           # (None: whichever the cost estimate picks; a short target row is cheaper walked)
+        assert ("scatter_sort" in names) == sorted_form, names
+    # a value out of range is refused, the tensor stays usable
+    bad = idx.copy(); bad.reshape(-1)[i_len // 2] = float(shape[axis])
+    t = gc.createRaw(shape, x)
+    with pytest.raises(ValueError):
+        t.inplaceScatterAdd(axis, gc.createRaw(ishape, bad), gs)
+    t.inplaceFill(1.0)
+    assert t.getSingleValue([0] * len(shape)) == 1.0
+
+
 def skewed_rows(rng, n_rows, k, hot):
     """k row numbers below n_rows of which the share `hot` names row 3 % n_rows, the others uniform."""
     idx = rng.integers(0, n_rows, [k])
