@@ -246,6 +246,7 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                                                                  uint32_t tag_slots, FastDiv tag_div) {
     extern __shared__ __attribute__((aligned(16))) float row_lds[];
     constexpr uint32_t kFirstEpoch = 0x3ffffeu;               // 22 bits above the 10 bits of a thread id
+    constexpr uint32_t kTailFrom = 8;                         // MODE 1: rounds of a chunk before the waves take turns
     static_assert(THREADS <= 1024, "a bid keeps the thread id in 10 bits");
     __shared__ uint32_t any_pending[3];
     float* tile = row_lds;
@@ -330,10 +331,41 @@ __global__ __launch_bounds__(THREADS) void scatter_rows_lds_kernel(float* __rest
                         tile[sel] = tile[sel] + v;
                         pending = false;
                     }
-                    // A chunk of THREADS entries needs at most THREADS rounds unless winners keep missing their
-                    // tags; from there on a second barrier keeps the next round's bids behind the winners' reads,
-                    // and every round retires an entry of every element that still has one.
-                    if (rounds >= THREADS) __syncthreads();
+                    // Entries are still pending after kTailFrom rounds: some element is named many times (a round
+                    // retires one entry of it, at a barrier each). The rounds have retired the first entries of every
+                    // element, in order; the waves now take turns, in the order of the row, over what is left: a
+                    // wave's pending entries find the others for their element by a ballot per bit of the element
+                    // number, the first lane of such a group reads the element, the sum goes from lane to lane by a
+                    // shuffle per further entry, and the last lane writes it.
+                    if (rounds + 1 >= kTailFrom) {
+                        __syncthreads();                    // the winners' adds above have landed
+                        const uint32_t lane = tid & 63u;
+                        const int element_bits = 32 - __clz(static_cast<int>(band_len - 1u) | 1);
+                        for (uint32_t w = 0; w < THREADS / 64; w++) {
+                            if (tid / 64 == w && __ballot(pending) != 0) {
+                                unsigned long long same = __ballot(pending);
+                                for (int bit = 0; bit < element_bits; bit++) {
+                                    const bool set = (sel >> bit) & 1u;
+                                    const unsigned long long with = __ballot(pending && set);
+                                    same &= set ? with : ~with;
+                                }
+                                const unsigned long long before = same & ((1ull << lane) - 1ull);
+                                const uint32_t rank = pending ? __popcll(before) : 0u;
+                                const int from = before ? 63 - __clzll(static_cast<long long>(before)) : static_cast<int>(lane);
+                                const bool last = pending && ((same >> lane) >> 1) == 0;
+                                float sum = 0.0f;
+                                if (pending && rank == 0) sum = tile[sel] + v;
+                                for (uint32_t step = 1; __ballot(pending && rank >= step) != 0; step++) {
+                                    const float carried = __shfl(sum, from);
+                                    if (pending && rank == step) sum = carried + v;
+                                }
+                                if (last) tile[sel] = sum;
+                                pending = false;
+                            }
+                            __syncthreads();
+                        }
+                        break;
+                    }
                 }
             }
         }

@@ -264,6 +264,42 @@ def test_scatter_of_long_rows_at_few_positions_goes_through_a_sort(shape, axis, 
     assert t.getSingleValue([0] * len(shape)) == 1.0
 
 
+@pytest.mark.parametrize("shape,i_len,hot", [([40, 3000], 3000, 0.3), ([40, 3000], 9000, 0.9), ([300, 8192], 4096, 0.25), ([12, 16384], 20000, 0.5),
+                                             ([6, 40000], 30000, 0.2), ([3, 5, 9000], 5000, 1.0), ([50, 700], 700, 0.05)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_scatter_add_through_lds_rows_with_a_hot_element(shape, i_len, hot, gc):
+    """The add form of the rows-through-LDS scatter retires one entry per element and round; with an element that a
+    large share of a row's entries name (a histogram with a full bin) it hands over, after a few rounds, to the waves
+    taking turns over what is left. `hot` is the share of the entries that name element 7 (the rest are uniform);
+    rows of 256-thread and of 1024-thread workgroups, one band and several, indexAdd along the innermost axis too."""
+    rng = np.random.default_rng(sum(shape) + i_len)
+    cpu = jo.JvmOracleOperations()
+    ishape = list(shape); ishape[-1] = i_len
+    x = rng.standard_normal(shape).astype(np.float32)
+    idx = rng.integers(0, shape[-1], ishape)
+    idx[rng.random(ishape) < hot] = 7
+    idx = idx.astype(np.float32)
+    src = rng.standard_normal(ishape).astype(np.float32)
+    src *= np.exp(rng.uniform(-12, 12, src.shape)).astype(np.float32)      # sums that depend on the order of the adds
+    gi, ci = gc.createRaw(ishape, idx), cpu.createRaw(ishape, idx)
+    gs, cs = gc.createRaw(ishape, src), cpu.createRaw(ishape, src)
+    gc.profileBegin()
+    gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
+    gt.inplaceScatterAdd(-1, gi, gs); ct.inplaceScatterAdd(-1, ci, cs)
+    assert_bits_equal(gt.toArray(), ct.toArray(), "scatterAdd")
+    gz, cz = gc.createRawFill(shape, -0.0), cpu.createRawFill(shape, -0.0)
+    gz.inplaceScatterAdd(-1, gi, gs); cz.inplaceScatterAdd(-1, ci, cs)
+    assert_bits_equal(gz.toArray(), cz.toArray(), "scatterAdd into a fill")
+    assert "scatter_rows_lds_kernel<add>" in set(gc.profileEnd())
+    # indexAdd along the innermost axis: one list for every row
+    rows = idx.reshape(-1, i_len)[0]
+    sshape = list(shape); sshape[-1] = i_len
+    gr, cr = gc.createRaw([i_len], rows), cpu.createRaw([i_len], rows)
+    gt, ct = gc.createRaw(shape, x), cpu.createRaw(shape, x)
+    gt.indexAdd(-1, gr, gs, 0.7); ct.indexAdd(-1, cr, cs, 0.7)
+    assert_bits_equal(gt.toArray(), ct.toArray(), "indexAdd along the innermost axis")
+
+
 def skewed_rows(rng, n_rows, k, hot):
     """k row numbers below n_rows of which the share `hot` names row 3 % n_rows, the others uniform."""
     idx = rng.integers(0, n_rows, [k])
