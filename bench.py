@@ -180,7 +180,8 @@ def cpu_baseline(name, threads):
     sample = {"cfg1": dict(wl.full_dims), "cfg2": dict(wl.full_dims), "cfg3": dict(wl.full_dims),
               "cfg4": dict(wl.full_dims), "cfg5": dict(wl.full_dims),
               "max_backward": dict(wl.full_dims), "softmax_ce": {"batch": 8192, "classes": 2048},
-              "reduce_shapes": {"scale": 4}, "indexed_moves": {"rows": 4096, "cols": 4096}, "layout_shapes": {"scale": 8}, "unary_maps": {"n": 1 << 25}}.get(name, dict(wl.full_dims))
+              "reduce_shapes": {"scale": 4}, "indexed_moves": {"rows": 4096, "cols": 4096},
+              "indexed_skew": {"table": 50000, "width": 64, "k": 65536, "flat": 1 << 20, "rows": 1024, "cols": 8192, "short": 256}, "layout_shapes": {"scale": 8}, "unary_maps": {"n": 1 << 25}}.get(name, dict(wl.full_dims))
     inputs = wl.make_inputs(sample)
     jo.set_threads(threads)
     try:
@@ -204,7 +205,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="cfg5",
                     choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce", "transpose", "permute",
-                             "concat_mask", "batch_norm", "reduce_shapes", "indexed_moves", "layout_shapes", "unary_maps"])
+                             "concat_mask", "batch_norm", "reduce_shapes", "indexed_moves", "indexed_skew", "layout_shapes", "unary_maps"])
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,

@@ -487,31 +487,10 @@ struct LongRuns {
     uint32_t* key;          // its target row
     uint32_t* count;
 };
-// One thread per run of the compacted heads.
-__global__ __launch_bounds__(kBlock) void index_long_runs_of_heads_kernel(const uint32_t* __restrict__ keys, const uint32_t* __restrict__ heads,
-                                                                         const uint32_t* __restrict__ head_count, uint32_t k, uint32_t axis_len,
-                                                                         uint32_t long_from, LongRuns runs) {
-    const uint32_t h = blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t n = *head_count;
-    if (h >= n) return;
-    const uint32_t i = heads[h];
-    const uint32_t len = (h + 1 < n ? heads[h + 1] : k) - i;
-    const uint32_t key = keys[i];
-    if (len < long_from || key >= axis_len) return;
+// Called by the one thread of a walking kernel that meets the run's first element: the run goes on the list.
+__device__ __forceinline__ void list_long_run(const LongRuns& runs, uint32_t start, uint32_t len, uint32_t key) {
     const uint32_t slot = atomicAdd(runs.count, 1u);
-    runs.start[slot] = i; runs.len[slot] = len; runs.key[slot] = key;
-}
-// One thread per target row, for the form that knows every row's first and one-past-last list position.
-__global__ __launch_bounds__(kBlock) void index_long_runs_of_rows_kernel(const uint32_t* __restrict__ row_first, const uint32_t* __restrict__ row_end,
-                                                                        uint32_t axis_len, uint32_t long_from, LongRuns runs) {
-    const uint32_t key = blockIdx.x * kBlock + threadIdx.x;
-    if (key >= axis_len) return;
-    const uint32_t i = row_first[key];
-    if (i == 0xffffffffu) return;
-    const uint32_t len = row_end[key] - i;
-    if (len < long_from) return;
-    const uint32_t slot = atomicAdd(runs.count, 1u);
-    runs.start[slot] = i; runs.len[slot] = len; runs.key[slot] = key;
+    runs.start[slot] = start; runs.len[slot] = len; runs.key[slot] = key;
 }
 
 // row_first[r] = where target row r's run starts in the sorted list, ~0u for a row no entry names.
@@ -560,7 +539,7 @@ template <bool VEC>
 __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                  const uint32_t* __restrict__ vals, const uint32_t* __restrict__ row_first,
                                                                  const uint32_t* __restrict__ row_end, float alpha, float constant,
-                                                                 uint32_t units, RowsPlan pl, FastDiv axis_div) {
+                                                                 uint32_t units, RowsPlan pl, FastDiv axis_div, LongRuns runs) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
     const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * axis_len + r
@@ -569,7 +548,10 @@ __global__ __launch_bounds__(kBlock) void index_add_filled_kernel(float* __restr
     const uint32_t key = row - o * pl.axis_len;
     const uint32_t first = row_first[key];
     const uint32_t end = first != 0xffffffffu ? row_end[key] : 0u;
-    if (first != 0xffffffffu && end - first >= pl.long_from) return;
+    if (first != 0xffffffffu && end - first >= pl.long_from) {
+        if (o == 0 && col == 0) list_long_run(runs, first, end - first, key);
+        return;
+    }
     const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
     if (VEC) {
         v4f_lds acc = {constant, constant, constant, constant};
@@ -592,7 +574,7 @@ template <bool VEC>
 __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                  const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
                                                                  const uint32_t* __restrict__ heads, const uint32_t* __restrict__ head_count,
-                                                                 float alpha, uint32_t units, RowsPlan pl) {
+                                                                 float alpha, uint32_t units, RowsPlan pl, LongRuns runs) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
     const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * heads + h
@@ -604,7 +586,11 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restr
     const uint32_t first = heads[h];
     const uint32_t end = h + 1 < n_heads ? heads[h + 1] : pl.k;
     const uint32_t key = keys[first];
-    if (key >= pl.axis_len || end - first >= pl.long_from) return;
+    if (key >= pl.axis_len) return;
+    if (end - first >= pl.long_from) {
+        if (o == 0 && col == 0) list_long_run(runs, first, end - first, key);
+        return;
+    }
     const size_t t_at = (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
     const size_t s_base = static_cast<size_t>(o) * pl.k * pl.inner + col;
     if (VEC) {
@@ -622,7 +608,7 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_kernel(float* __restr
 __global__ __launch_bounds__(kBlock) void index_add_sorted_ragged_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                         const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
                                                                         const uint32_t* __restrict__ heads, const uint32_t* __restrict__ head_count,
-                                                                        float alpha, uint32_t units, uint32_t row_floats, RowsPlan pl) {
+                                                                        float alpha, uint32_t units, uint32_t row_floats, RowsPlan pl, LongRuns runs) {
     const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= units) return;
     const uint32_t row = (__umulhi(e, pl.inner_div.mul) + e) >> pl.inner_div.shift;       // o * heads + h
@@ -634,7 +620,11 @@ __global__ __launch_bounds__(kBlock) void index_add_sorted_ragged_kernel(float* 
     const uint32_t first = heads[h];
     const uint32_t end = h + 1 < n_heads ? heads[h + 1] : pl.k;
     const uint32_t key = keys[first];
-    if (key >= pl.axis_len || end - first >= pl.long_from) return;
+    if (key >= pl.axis_len) return;
+    if (end - first >= pl.long_from) {
+        if (o == 0 && off == 0) list_long_run(runs, first, end - first, key);
+        return;
+    }
     float* t = target + (static_cast<size_t>(o) * pl.axis_len + key) * row_floats + off;
     const float* s = src + static_cast<size_t>(o) * pl.k * row_floats + off;
     const uint32_t cnt = min(4u, row_floats - off);
@@ -1262,8 +1252,6 @@ static int scatter_sorted(int mode, float* target, const int32_t* target_shape, 
             scratch = temp_bytes;
             sort_status = select_flagged_positions(temp, &scratch, flags, heads, head_count, k, stream);
             if (sort_status != hipSuccess) return;
-            if (mode == 1 && long_items > 0)
-                hipLaunchKernelGGL(index_long_runs_of_heads_kernel, per_entry, dim3(kBlock), 0, stream, keys_sorted, heads, head_count, k, invalid, pl.long_from, runs);
         }
         if (mode != 1) {
             LaunchScope scope("scatter_sorted_assign_kernel", mode == 0 ? "set" : "fill", idx_n * (mode == 0 ? 8 : 4));
@@ -1274,7 +1262,7 @@ static int scatter_sorted(int mode, float* target, const int32_t* target_shape, 
         {
             LaunchScope scope("index_add_sorted_kernel", "scatter", idx_n * 12);
             hipLaunchKernelGGL((index_add_sorted_kernel<false>), per_head, dim3(kBlock), 0, stream, target, psrc, keys_sorted, vals_sorted, heads, head_count, 1.0f,
-                               pl.heads, pl);
+                               pl.heads, pl, runs);
         }
         if (long_items > 0) {
             LaunchScope scope("index_add_long_runs_kernel", "scatter", 0);
@@ -1551,15 +1539,13 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
                 if (sort_status != hipSuccess) return;
                 hipLaunchKernelGGL(index_row_first_clear_kernel, dim3((pl.axis_len + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, row_first, pl.axis_len);
                 hipLaunchKernelGGL(index_row_first_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, pl.k, pl.axis_len, row_first, row_end);
-                if (long_items > 0)
-                    hipLaunchKernelGGL(index_long_runs_of_rows_kernel, dim3((pl.axis_len + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, row_first, row_end, pl.axis_len, pl.long_from, runs);
             }
             {
                 LaunchScope scope("index_add_filled_kernel", vec_inner ? "float4" : "float", (total + n_src) * 4 + k * 4);
                 const dim3 grid((units + kBlock - 1) / kBlock);
                 const FastDiv axis_div = make_div(pl.axis_len);
-                if (vec_inner) hipLaunchKernelGGL((index_add_filled_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div);
-                else           hipLaunchKernelGGL((index_add_filled_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div);
+                if (vec_inner) hipLaunchKernelGGL((index_add_filled_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div, runs);
+                else           hipLaunchKernelGGL((index_add_filled_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, vals_sorted, row_first, row_end, alpha, constant, units, pl, axis_div, runs);
             }
             if (long_items > 0) {
                 LaunchScope scope("index_add_long_runs_kernel", "from a constant", 0);
@@ -1592,18 +1578,15 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
                 scratch = temp_bytes;
                 sort_status = select_flagged_positions(temp, &scratch, flags, heads, head_count, pl.k, stream);
             }
-            if (sort_status == hipSuccess && long_items > 0)
-                hipLaunchKernelGGL(index_long_runs_of_heads_kernel, dim3((pl.k + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, keys_sorted, heads, head_count, pl.k,
-                                   pl.axis_len, pl.long_from, runs);
         }
         if (sort_status != hipSuccess) return;
         {
             LaunchScope scope("index_add_sorted_kernel", vec ? "float4" : ragged ? "float4 at dword addresses" : "float", 3 * n_src * 4 + k * 4);
             const dim3 grid((units + kBlock - 1) / kBlock);
             if (ragged) hipLaunchKernelGGL(index_add_sorted_ragged_kernel, grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units,
-                                           static_cast<uint32_t>(inner), pl);
-            else if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
-            else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl);
+                                           static_cast<uint32_t>(inner), pl, runs);
+            else if (vec) hipLaunchKernelGGL((index_add_sorted_kernel<true>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl, runs);
+            else     hipLaunchKernelGGL((index_add_sorted_kernel<false>), grid, dim3(kBlock), 0, stream, st->ptr, ss->ptr, keys_sorted, vals_sorted, heads, head_count, alpha, units, pl, runs);
         }
         if (long_items > 0) {
             LaunchScope scope("index_add_long_runs_kernel", "", 0);

@@ -337,6 +337,48 @@ def _bytes_idx(d):
 
 
 
+# ---- indexed moves with skewed positions, flat tensors and short index rows ------------------------
+# What an embedding gradient, a histogram and a top-k scatter ask of the indexed moves: positions drawn from a power law
+# (floor(n u^4): element 0 takes n^(-1/4) of the draws), a flat tensor with twice as many entries as elements, index rows
+# a thirty-second of the target's.
+
+def _in_skew(d):
+    g = SplitMix64(15)
+    table, width, k, flat, rows, cols, short = d["table"], d["width"], d["k"], d["flat"], d["rows"], d["cols"], d["short"]
+    def skewed(shape, limit):
+        u = g.uniform(shape, 0.0, 1.0).astype(np.float64)
+        return np.minimum(np.floor(limit * u ** 4), limit - 1).astype(np.float32)
+    def ints(shape, limit):
+        return np.minimum(np.floor(g.uniform(shape, 0.0, float(limit))), np.float32(limit - 1)).astype(np.float32)
+    return {"grad_rows": g.normal([k, width]), "tokens": skewed([k], table), "weights": g.normal([2 * flat]), "bins": ints([2 * flat], flat),
+            "x": g.normal([rows, cols]), "hot_cols": skewed([rows, cols], cols), "few_cols": ints([rows, short], cols),
+            "picked": g.normal([rows, short]), "table": np.zeros([table, width], np.float32), "flat": np.zeros([flat], np.float32)}
+
+
+def _run_skew(ops, inp):
+    from .autograd import NoGradVariable
+    raw = {k: ops.create(list(v.shape), False, v).getRawValue() for k, v in inp.items()}
+    table_grad = ops.zerosLike(raw["table"])
+    table_grad.indexAdd(0, raw["tokens"], raw["grad_rows"], 1.0)                   # an embedding's gradient
+    histogram = ops.zerosLike(raw["flat"])
+    histogram.inplaceScatterAdd(0, raw["bins"], raw["weights"])                    # weighted counts on a flat tensor
+    latest = ops.zerosLike(raw["flat"])
+    latest.inplaceScatter(0, raw["bins"], raw["weights"])                          # the last entry of every bin
+    row_sums = ops.zerosLike(raw["x"])
+    row_sums.inplaceScatterAdd(1, raw["hot_cols"], raw["x"])                       # rows with a full bin
+    placed = ops.zerosLike(raw["x"])
+    placed.inplaceScatterAdd(1, raw["few_cols"], raw["picked"])                    # a few entries per row
+    res = {"table_grad": table_grad, "histogram": histogram, "latest": latest, "row_sums": row_sums, "placed": placed}
+    return {k: NoGradVariable(ops, v) for k, v in res.items()}
+
+
+def _bytes_skew(d):
+    table, width, k, flat, rows, cols, short = d["table"], d["width"], d["k"], d["flat"], d["rows"], d["cols"], d["short"]
+    # zerosLike 4 N each; indexAdd 12 N_src + list; scatterAdd 16 N_index; scatter 12 N_index
+    return (4 * (table * width + 2 * flat + 2 * rows * cols) + 12 * k * width + 4 * k + (16 + 12) * 2 * flat
+            + 16 * rows * cols + 16 * rows * short)
+
+
 # ---- layout moves on shapes that are not multiples of anything convenient --------------------------
 
 # (shape at scale 1, permutation): a run of 8 floats kept innermost, a run of 3, a run of 33, a long
@@ -414,6 +456,12 @@ WORKLOADS: Dict[str, Workload] = {
                                                "[65536,16,64] sum, [6710,1000,10] sum, [23,2,1456699] max, [32752,2049] argMax, "
                                                "[262144,255] mean; N(0,1), seed 11",
                               {"scale": 1}, _in_red, _run_red, _bytes_red),
+    "indexed_skew": Workload("indexed_skew", "indexAdd of 262144 rows of 256 floats into zerosLike([50000,256]) at power-law rows; "
+                                             "inplaceScatterAdd and inplaceScatter of 2^23 entries into a flat zerosLike([2^22]); "
+                                             "inplaceScatterAdd along axis 1 of [8192,8192] at power-law columns and of [8192,256] "
+                                             "entries at uniform ones; seed 15",
+                             {"table": 50000, "width": 256, "k": 262144, "flat": 1 << 22, "rows": 8192, "cols": 8192, "short": 256},
+                             _in_skew, _run_skew, _bytes_skew),
     "indexed_moves": Workload("indexed_moves", "x[16384,4096] with index tensors of its own size: gather along axis 1, inplaceScatter "
                                                "along axis 1, inplaceScatterAdd along axis 0 (each into zerosLike(x)), indexSelect and "
                                                "indexAdd of 16384 rows; seed 12",

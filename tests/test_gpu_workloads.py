@@ -255,6 +255,27 @@ def test_indexed_moves(dims, gc):
     assert_bits_equal(got["selected"], inp["x"][inp["row_list"].astype(np.int64)], "indexSelect vs numpy")
 
 
+@pytest.mark.parametrize("dims", [{"table": 300, "width": 20, "k": 5000, "flat": 4096, "rows": 64, "cols": 9000, "short": 40},
+                                  {"table": 50000, "width": 256, "k": 262144, "flat": 1 << 22, "rows": 8192, "cols": 8192, "short": 256}],
+                         ids=["small", "full"])
+def test_indexed_skew(dims, gc):
+    """Bit-exact against the checker, full size included: rows and elements that a large share of the entries name (the adds
+    into them in index order), a flat tensor with twice as many entries as elements, index rows far shorter than the target's."""
+    wl = WORKLOADS["indexed_skew"]
+    inp = wl.make_inputs(dims)
+    got = {k: v.toArray() for k, v in wl.run(gc, inp).items()}
+    jo.set_threads(16)
+    try:
+        want = {k: v.toArray() for k, v in wl.run(jo.JvmOracleOperations(), inp).items()}
+    finally:
+        jo.set_threads(1)
+    for k in ("table_grad", "histogram", "latest", "row_sums", "placed"):
+        assert_bits_equal(got[k], want[k], k)
+    last = np.zeros(dims["flat"], np.float32)
+    last[inp["bins"].astype(np.int64)] = inp["weights"]                  # numpy assigns in order: the last entry stays
+    assert_bits_equal(got["latest"], last, "scatter on a flat tensor vs numpy")
+
+
 @pytest.mark.parametrize("scale", [64, 1], ids=["small", "full"])
 def test_layout_shapes(scale, gc):
     """Permutes and the range get against numpy (which the checker is pinned to for these moves), bit for bit."""
