@@ -170,6 +170,9 @@ struct TilePlan {
     uint32_t x_out_stride, y_in_stride;
     uint32_t x_tiles, y_tiles;
     FastDiv  x_tiles_div, y_tiles_div;
+    uint32_t x_split;                        // permute_tile_kernel: X is two dims that the input holds as one run: index x is
+    FastDiv  x_split_div;                    //   (x % x_split) of the inner one and (x / x_split) of the outer one, which has its
+    uint32_t x_hi_out_stride;                //   own place in the output (0: X is one dim)
     uint32_t tiles;                          // permute_tile_kernel: the grid holds this many rounded up to a multiple of 8
     uint32_t by_xcd;                         // ... and an XCD takes a contiguous eighth of them (rows that do not start on a cache line)
     int      nbatch;
@@ -231,7 +234,14 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
         const uint32_t e = k * kBlock + threadIdx.x;
         const uint32_t lx = e / TY, ly = e % TY;
         const uint32_t x = x0 + lx, y = y0 + ly;
-        if (x < pl.x_len && y < pl.y_len) out[out_off + x * pl.x_out_stride + y] = tile[ly * (TX + 1) + lx];
+        if (x < pl.x_len && y < pl.y_len) {
+            uint32_t to = x * pl.x_out_stride;
+            if (pl.x_split) {
+                const uint32_t hi = (__umulhi(x, pl.x_split_div.mul) + x) >> pl.x_split_div.shift;
+                to = (x - hi * pl.x_split) * pl.x_out_stride + hi * pl.x_hi_out_stride;
+            }
+            out[out_off + to + y] = tile[ly * (TX + 1) + lx];
+        }
     }
 }
 
@@ -625,6 +635,20 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     TilePlan pl{};
     pl.x_len = x_len; pl.y_len = y_len; pl.y_in_stride = y_in_stride;
     pl.x_out_stride = static_cast<uint32_t>(x_out_stride);
+    // A short contiguous dim of the input whose neighbour in the input goes elsewhere in the output ([N,206,3] reversed:
+    // rows of 618 floats of which a tile would take 3): the two are one X of 618 for the loads, and the store works
+    // out the two output places from the index.
+    if (elem == 1 && x_len < 64) {
+        for (int d = 0; d < nb; d++) {
+            if (b_in[d] != x_len || static_cast<uint64_t>(x_len) * bsize[d] > 0x7fffffffull) continue;
+            pl.x_split = x_len; pl.x_split_div = make_div(x_len); pl.x_hi_out_stride = b_out[d];
+            pl.x_len = x_len * bsize[d];
+            for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
+            nb--;
+            batch /= (pl.x_len / x_len);
+            break;
+        }
+    }
     if (elem == 3 || elem > 4) {
         RunsPlan rp{};
         const bool vec = elem % 4 == 0;
@@ -667,7 +691,7 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     if (blocks > kMaxElements - 8) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
     pl.tiles = static_cast<uint32_t>(blocks);
     const uint32_t line = 128 / (4 * static_cast<uint32_t>(elem));                  // elements per cache line
-    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0) ? 1u : 0u;
+    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0 || pl.x_hi_out_stride % line != 0) ? 1u : 0u;
     for (int d = 0; d < nb; d++) if (b_in[d] % line != 0 || b_out[d] % line != 0) pl.by_xcd = 1u;
     const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
     LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
