@@ -173,6 +173,9 @@ struct TilePlan {
     uint32_t x_split;                        // permute_tile_kernel: X is two dims that the input holds as one run: index x is
     FastDiv  x_split_div;                    //   (x % x_split) of the inner one and (x / x_split) of the outer one, which has its
     uint32_t x_hi_out_stride;                //   own place in the output (0: X is one dim)
+    uint32_t y_split;                        // ... and the same for Y, two dims that the output holds as one run: the load works
+    FastDiv  y_split_div;                    //   out the two input places
+    uint32_t y_hi_in_stride;
     uint32_t tiles;                          // permute_tile_kernel: the grid holds this many rounded up to a multiple of 8
     uint32_t by_xcd;                         // ... and an XCD takes a contiguous eighth of them (rows that do not start on a cache line)
     int      nbatch;
@@ -221,7 +224,14 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
     for (int k = 0; k < kPasses; k++) {
         const uint32_t e = k * kBlock + threadIdx.x;
         const uint32_t x = x0 + e % TX, y = y0 + e / TX;
-        if (x < pl.x_len && y < pl.y_len) v[k] = __builtin_nontemporal_load(in + in_off + y * pl.y_in_stride + x);
+        if (x < pl.x_len && y < pl.y_len) {
+            uint32_t from = y * pl.y_in_stride;
+            if (pl.y_split) {
+                const uint32_t hi = (__umulhi(y, pl.y_split_div.mul) + y) >> pl.y_split_div.shift;
+                from = (y - hi * pl.y_split) * pl.y_in_stride + hi * pl.y_hi_in_stride;
+            }
+            v[k] = __builtin_nontemporal_load(in + in_off + from + x);
+        }
     }
 #pragma unroll
     for (int k = 0; k < kPasses; k++) {
@@ -649,6 +659,18 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
             break;
         }
     }
+    // ... and a short contiguous dim of the output whose neighbour in the output comes from elsewhere in the input.
+    if (elem == 1 && y_len < 64) {
+        for (int d = 0; d < nb; d++) {
+            if (b_out[d] != y_len || static_cast<uint64_t>(y_len) * bsize[d] > 0x7fffffffull) continue;
+            pl.y_split = y_len; pl.y_split_div = make_div(y_len); pl.y_hi_in_stride = b_in[d];
+            pl.y_len = y_len * bsize[d];
+            for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
+            nb--;
+            batch /= (pl.y_len / y_len);
+            break;
+        }
+    }
     if (elem == 3 || elem > 4) {
         RunsPlan rp{};
         const bool vec = elem % 4 == 0;
@@ -691,7 +713,7 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     if (blocks > kMaxElements - 8) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
     pl.tiles = static_cast<uint32_t>(blocks);
     const uint32_t line = 128 / (4 * static_cast<uint32_t>(elem));                  // elements per cache line
-    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0 || pl.x_hi_out_stride % line != 0) ? 1u : 0u;
+    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0 || pl.x_hi_out_stride % line != 0 || pl.y_hi_in_stride % line != 0) ? 1u : 0u;
     for (int d = 0; d < nb; d++) if (b_in[d] % line != 0 || b_out[d] % line != 0) pl.by_xcd = 1u;
     const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
     LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
