@@ -592,7 +592,9 @@ int box_of(const char* what, const int32_t* shape, int dims, const int32_t* firs
 }
 
 // Permutes through LDS tiles. `v`: the output's dims innermost first with the input's strides,
-// in units of `elem` floats (1, 2, 4, or a run of 3 ... 63), stride[0] != 1. Returns KTH_OK after launching.
+// in units of `elem` floats (1, 2, 4, or a run of 3 ... 63), stride[0] != 1. Returns KTH_OK after launching,
+// kTilesDeclined (nothing launched) when float tiles would be mostly empty.
+constexpr int kTilesDeclined = 1;
 int launch_tiles(const char* what, const StridedDims& v, int elem, const float* in, float* out, uint64_t n) {
     int px = -1;
     for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) px = d;
@@ -703,6 +705,14 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     else if (elem == 2) { tx = 64; ty = 32; }
     else if (pl.x_len < 64 && pl.x_len <= pl.y_len) { tx = 2; while (tx < pl.x_len) tx <<= 1; ty = kTileElems / tx; }
     else if (pl.y_len < 64) { ty = 2; while (ty < pl.y_len) ty <<= 1; tx = kTileElems / ty; }
+    // A tile is 4096 elements, as narrow along a short dim as a power of two allows; when the input's contiguous dim
+    // and the output's are both short (and have no neighbour to join), most of it hangs over: a [2,5] block transposed
+    // inside 3 million batch items filled 10 of 4096 places and ran at 58 GB/s. Below an eighth full the caller's
+    // element gather is the faster one (its reads stay inside the few cache lines of such a block).
+    if (elem == 1) {
+        const double filled = static_cast<double>(std::min(pl.x_len, tx)) / tx * static_cast<double>(std::min(pl.y_len, ty)) / ty;
+        if (filled < 0.12) return kTilesDeclined;
+    }
     pl.x_tiles = (pl.x_len + tx - 1) / tx;
     pl.y_tiles = (pl.y_len + ty - 1) / ty;
     pl.x_tiles_div = make_div(pl.x_tiles);
@@ -807,26 +817,14 @@ int permute_device(const char* what, const float* in, float* out, const int32_t*
         KTH_LAUNCH_CHECK("move_kernel");
         return KTH_OK;
     }
-    // A tile is 4096 elements, as narrow along a short dim as a power of two allows; when the input's contiguous dim
-    // and the output's are both short, most of it hangs over (a [2,5] block transposed inside 3 million batch items
-    // filled 10 of 4096 places and ran at 58 GB/s). Below an eighth full, the element gather of the range moves does
-    // the permutation: its reads stay inside the few cache lines of such a block.
-    {
-        uint64_t x_len = 1;
-        for (int d = 1; d < v.n; d++) if (v.stride[d] == 1) x_len = v.size[d];
-        const uint64_t y_len = v.size[0];
-        uint64_t tx = 64, ty = 64;
-        if (x_len < 64 && x_len <= y_len) { tx = 2; while (tx < x_len) tx <<= 1; ty = kTileElems / tx; }
-        else if (y_len < 64) { ty = 2; while (ty < y_len) ty <<= 1; tx = kTileElems / ty; }
-        const double filled = static_cast<double>(std::min(x_len, tx)) / static_cast<double>(tx) *
-                              static_cast<double>(std::min(y_len, ty)) / static_cast<double>(ty);
-        if (filled < 0.12) {
-            launch_move<0>("move_kernel_permute", in, out, n, 0.0f, v, 0, n * 8);
-            KTH_LAUNCH_CHECK("move_kernel");
-            return KTH_OK;
-        }
+    // (launch_tiles declines shapes whose tiles would be mostly empty: the element gather of the range moves then)
+    const int rc = launch_tiles(what, v, 1, in, out, n);
+    if (rc == kTilesDeclined) {
+        launch_move<0>("move_kernel_permute", in, out, n, 0.0f, v, 0, n * 8);
+        KTH_LAUNCH_CHECK("move_kernel");
+        return KTH_OK;
     }
-    if (int rc = launch_tiles(what, v, 1, in, out, n)) return rc;
+    if (rc) return rc;
     KTH_LAUNCH_CHECK("permute_tile_kernel");
     return KTH_OK;
 }

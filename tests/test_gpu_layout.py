@@ -117,7 +117,10 @@ PERMUTE_SHAPES = [[2, 3, 2], [5, 6, 7], [8, 64, 68], [2, 3, 4, 5], [3, 4, 64, 65
                   # a run of 5 ... 63 floats kept innermost: tiles of runs (float4 and scalar), ragged tile edges, exact tiles,
                   # a batch dim outside, a merged run ([.., 3, 4] -> 12), dims too short for a tile (the strided move instead)
                   [40, 50, 8], [33, 47, 12], [20, 35, 7], [18, 70, 33], [3, 17, 19, 5], [16, 16, 31], [19, 23, 3, 4], [100, 9, 6],
-                  [9, 10, 63], [16, 48, 28], [40, 70, 3], [33, 35, 3], [2, 32, 32, 3]]
+                  [9, 10, 63], [16, 48, 28], [40, 70, 3], [33, 35, 3], [2, 32, 32, 3],
+                  # a short contiguous dim of the input (or of the output) whose neighbour there goes elsewhere: the two as one
+                  # tile dim; both contiguous dims short with no neighbour to join: the element gather instead of mostly empty tiles
+                  [300, 26, 3], [30, 8, 19, 8], [40, 7, 11, 23], [322, 14, 2, 5], [26, 17, 19, 4], [5, 5, 66, 23], [70, 3, 2, 90]]
 
 
 @pytest.mark.parametrize("shape", PERMUTE_SHAPES, ids=lambda s: "x".join(map(str, s)))
