@@ -226,23 +226,27 @@ struct BackwardParams { float mean, stdev, gamma, dot_std_sq, grad_mean, pad0, p
 // One wave folds the partials of channel c, always in the same order: lane l takes the items
 // l, l + 64, ... (item t of a by-columns layout is segment t / inner, column c * inner + t % inner),
 // then the lanes are folded by xor-shuffles. Every lane returns the totals.
+// With very many channels of a few items each a wave per channel is 63 idle lanes: `alone` has one thread fold
+// all items of its channel in ascending order instead.
 __device__ __forceinline__ void fold_partials(const double* partial, uint32_t c, uint32_t segments, bool by_cols,
-                                              uint32_t width, uint32_t inner, double& s1, double& s2) {
+                                              uint32_t width, uint32_t inner, bool alone, double& s1, double& s2) {
     s1 = 0.0; s2 = 0.0;
-    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t lane = alone ? 0u : threadIdx.x & 63;
+    const uint32_t lanes = alone ? 1u : 64u;
     if (by_cols) {
         const uint32_t items = segments * inner;
-        for (uint32_t t = lane; t < items; t += 64) {
+        for (uint32_t t = lane; t < items; t += lanes) {
             const uint32_t seg = t / inner, i = t - seg * inner;
             const uint64_t at = (static_cast<uint64_t>(seg) * width + static_cast<uint64_t>(c) * inner + i) * 2;
             s1 += partial[at]; s2 += partial[at + 1];
         }
     } else {
-        for (uint32_t t = lane; t < segments; t += 64) {
+        for (uint32_t t = lane; t < segments; t += lanes) {
             const uint64_t at = (static_cast<uint64_t>(c) * segments + t) * 2;
             s1 += partial[at]; s2 += partial[at + 1];
         }
     }
+    if (alone) return;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         s1 += __shfl_xor(s1, off);
@@ -255,13 +259,15 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
                                                                     float momentum, float epsilon, float* running_mean, float* running_var,
                                                                     const float* __restrict__ gamma, const float* __restrict__ beta,
                                                                     float* __restrict__ current_mean, float* __restrict__ current_std,
-                                                                    ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch) {
-    const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
+                                                                    ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch,
+                                                                    int alone) {
+    // one wave per channel, or one thread
+    const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (c >= g.channels) return;
     float mean, stdev = 0.0f;
     double s1 = 0.0, s2 = 0.0;
-    if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
-    if ((threadIdx.x & 63) != 0) return;
+    if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    if (!alone && (threadIdx.x & 63) != 0) return;
     if (training) {
         const double n = static_cast<double>(g.per_channel);
         const double k = static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]);
@@ -300,12 +306,12 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
                                                                      const float* __restrict__ current_mean, const float* __restrict__ current_std,
                                                                      const float* __restrict__ gamma, float* __restrict__ grad_gamma,
                                                                      float* __restrict__ grad_beta, BackwardParams* __restrict__ params,
-                                                                     float* __restrict__ soa, uint32_t pitch) {
-    const uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);       // one wave per channel
+                                                                     float* __restrict__ soa, uint32_t pitch, int alone) {
+    const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (c >= g.channels) return;
     double s1 = 0.0, s2 = 0.0;
-    if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, s1, s2);
-    if ((threadIdx.x & 63) != 0) return;
+    if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    if (!alone && (threadIdx.x & 63) != 0) return;
     float mean, stdev;
     if (training) { mean = current_mean[c]; stdev = current_std[c]; }           // JVMBatchNorm.kt:131-133
     else {                                                                      // :134-137
@@ -469,6 +475,12 @@ struct StatsLaunch {
     bool     vec;
 };
 
+// A thread per channel folds the partials when there are very many channels of a few items each.
+static bool finalize_alone(const Geometry& g, const StatsLaunch& st) {
+    const uint64_t items = st.by_cols ? static_cast<uint64_t>(st.segments) * g.inner : st.segments;
+    return g.channels >= 16384 && items <= 32;
+}
+
 StatsLaunch plan_stats(const Geometry& g) {
     StatsLaunch st{};
     const uint32_t target = static_cast<uint32_t>(state().compute_units > 0 ? state().compute_units : 256) * 8;
@@ -594,8 +606,10 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     if (training) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
     {
         LaunchScope scope("bn_finalize_forward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
-                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params, soa, pitch);
+        const int alone = finalize_alone(g, st) ? 1 : 0;
+        const uint32_t per_block = alone ? kBlock : kBlock / 64;
+        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
+                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params, soa, pitch, alone);
     }
     launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr, soa, pitch);
     workspace_release(reinterpret_cast<float*>(ws), cap);
@@ -647,8 +661,10 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     if (need_sums) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
     {
         LaunchScope scope("bn_finalize_backward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, state().stream,
-                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch);
+        const int alone = finalize_alone(g, st) ? 1 : 0;
+        const uint32_t per_block = alone ? kBlock : kBlock / 64;
+        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
+                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch, alone);
     }
     if (sgi) {
         if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
