@@ -147,6 +147,10 @@ struct ColPlan {
     Geometry g;
     uint32_t width, col_blocks, segments, rows_per_seg;
     FastDiv  col_div, inner_div;
+    // a matrix narrower than a wave's 64 column groups: `groups` threads side by side and kBlock / groups rows at a
+    // time, so that a wave still reads consecutive memory (16 columns of a million rows kept 4 lanes of 64 busy)
+    uint32_t groups, row_lanes;
+    FastDiv  groups_div;
 };
 
 template <bool BACKWARD, int W>
@@ -155,8 +159,9 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
     __shared__ double lds[kBlock * 2 * W];
     const uint32_t b = blockIdx.x;
     const uint32_t seg = (__umulhi(b, pl.col_div.mul) + b) >> pl.col_div.shift;
-    const uint32_t col = ((b - seg * pl.col_blocks) * 64 + (threadIdx.x & 63)) * W;   // first of this thread's W columns
-    const uint32_t lane_row = threadIdx.x >> 6;
+    const uint32_t lane_row = (__umulhi(threadIdx.x, pl.groups_div.mul) + threadIdx.x) >> pl.groups_div.shift;
+    const uint32_t group = threadIdx.x - lane_row * pl.groups;
+    const uint32_t col = lane_row < pl.row_lanes ? ((b - seg * pl.col_blocks) * pl.groups + group) * W : pl.width;   // first of this thread's W columns
     double s1[W], s2[W];
 #pragma unroll
     for (int e = 0; e < W; e++) { s1[e] = 0.0; s2[e] = 0.0; }
@@ -171,11 +176,11 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
         const uint32_t first = seg * pl.rows_per_seg;
         uint32_t last = first + pl.rows_per_seg;
         if (last > pl.g.outer) last = pl.g.outer;
-        for (uint32_t r0 = first + lane_row; r0 < last; r0 += 4 * kBatch) {
+        for (uint32_t r0 = first + lane_row; r0 < last; r0 += pl.row_lanes * kBatch) {
             v4f vx[kBatch], vg[kBatch];
 #pragma unroll
             for (int k = 0; k < kBatch; k++) {
-                const uint32_t r = r0 + 4 * k;
+                const uint32_t r = r0 + pl.row_lanes * k;
                 if (r < last) {
                     const uint64_t at = static_cast<uint64_t>(r) * pl.width + col;
                     if (W == 4) {
@@ -189,7 +194,7 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
             }
 #pragma unroll
             for (int k = 0; k < kBatch; k++) {
-                if (r0 + 4 * k < last) {
+                if (r0 + pl.row_lanes * k < last) {
 #pragma unroll
                     for (int e = 0; e < W; e++) {
                         const double d = static_cast<double>(vx[k][e]) - shift[e];
@@ -210,7 +215,9 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
 #pragma unroll
         for (int e = 0; e < W; e++) {
             double a = s1[e], c = s2[e];
-            for (int w = 1; w < 4; w++) { a += lds[((threadIdx.x + 64 * w) * W + e) * 2]; c += lds[((threadIdx.x + 64 * w) * W + e) * 2 + 1]; }
+            for (uint32_t w = 1; w < pl.row_lanes; w++) {
+                a += lds[((threadIdx.x + pl.groups * w) * W + e) * 2]; c += lds[((threadIdx.x + pl.groups * w) * W + e) * 2 + 1];
+            }
             partial[(static_cast<uint64_t>(seg) * pl.width + col + e) * 2] = a;
             partial[(static_cast<uint64_t>(seg) * pl.width + col + e) * 2 + 1] = c;
         }
@@ -508,10 +515,14 @@ StatsLaunch plan_stats(const Geometry& g) {
         p.g = g;
         p.width = g.channels * g.inner;
         st.vec = p.width % 4 == 0;                     // every row then starts 16-byte aligned
-        const uint32_t cols_per_block = st.vec ? 256 : 64;
+        const uint32_t w = st.vec ? 4 : 1;
+        p.groups = std::min<uint32_t>(64, (p.width + w - 1) / w);
+        p.row_lanes = kBlock / p.groups;
+        p.groups_div = make_div(p.groups);
+        const uint32_t cols_per_block = p.groups * w;
         p.col_blocks = (p.width + cols_per_block - 1) / cols_per_block;
         uint32_t segments = (target + p.col_blocks - 1) / p.col_blocks;
-        const uint32_t max_segments = (g.outer + 4 * kBatch - 1) / (4 * kBatch);
+        const uint32_t max_segments = (g.outer + p.row_lanes * kBatch - 1) / (p.row_lanes * kBatch);
         if (segments > max_segments) segments = max_segments;
         if (segments < 1) segments = 1;
         p.rows_per_seg = (g.outer + segments - 1) / segments;
