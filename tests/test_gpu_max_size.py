@@ -235,6 +235,73 @@ def test_scatter_along_a_long_axis_near_the_limit(gc):
         assert index.getSingleValue([i, W - 1]) == float(perm[i])
 
 
+def test_sorted_and_wave_scatter_near_the_limit(gc):
+    """The scatter forms for one long index row and for many short ones, at offsets and keys at the top of the
+    32-bit range. A flat target of 2^31 - 2 elements with one index row of 2^24 entries is sorted by element
+    (keys up to 2^31 - 128, the last element a float32 index can name; the key for a bad entry is 2^31 - 2); a
+    [1 048 575, 2047] target with index rows of 40 entries takes a wave per row. Sampled elements are checked against the entries that name them, in row order."""
+    T, K = 2 ** 31 - 2, 2 ** 24
+    TOP = 2 ** 31 - 128                                                  # the last element a float32 index can name
+    rng = np.random.default_rng(6)
+    idx_f = rng.integers(0, T, K).astype(np.float32)                     # the device sees the rounded values
+    idx_f[idx_f > TOP] = TOP
+    idx_f[0], idx_f[1], idx_f[-1], idx_f[-2] = TOP, 0, TOP, 0            # both ends, each named at least twice
+    idx_f[1000:1400] = idx_f[500]                                        # a run of equal keys
+    idx = idx_f.astype(np.int64)
+    src = (rng.integers(-512, 512, K) / 8.0).astype(np.float32)
+    order = np.argsort(idx, kind="stable")
+    sorted_idx = idx[order]
+    def entries_of(element):                                             # in the order of the index row
+        lo, hi = np.searchsorted(sorted_idx, element, "left"), np.searchsorted(sorted_idx, element, "right")
+        return order[lo:hi]
+    sampled = [TOP, 0, int(idx[500])] + [int(v) for v in idx[rng.integers(0, K, 40)]]
+    untouched = [int(v) for v in rng.integers(0, T, 20)] + [T - 1]
+    untouched = [v for v in untouched if entries_of(v).size == 0]
+    g_idx, g_src = gc.createRaw([K], idx_f), gc.createRaw([K], src)
+    for mode in ("set", "add", "fill"):
+        x = gc.createRawFill([T], -5.0)
+        gc.profileBegin()
+        if mode == "set": x.inplaceScatter(0, g_idx, g_src)
+        elif mode == "add": x.inplaceScatterAdd(0, g_idx, g_src)
+        else: x.inplaceScatter(0, g_idx, 3.5)
+        launched = " ".join(gc.profileEnd().keys())
+        assert "scatter_sort" in launched, launched
+        for element in sampled:
+            e = entries_of(element)
+            assert e.size > 0
+            if mode == "set": want = src[e[-1]]
+            elif mode == "fill": want = np.float32(3.5)
+            else:
+                want = np.float32(-5.0)
+                for i in e: want = np.float32(want + src[i])
+            assert x.getSingleValue([element]) == want, (mode, element)
+        for element in untouched:
+            assert x.getSingleValue([element]) == -5.0
+        gc.release(x)
+    gc.release(g_idx, g_src)
+
+    R, W, L = 1048575, 2047, 40
+    pos = rng.integers(0, W, (R, L))
+    pos[:, 7] = pos[:, 3]                                                # every row names one element twice
+    val = (rng.integers(-512, 512, (R, L)) / 8.0).astype(np.float32)
+    g_pos, g_val = gc.createRaw([R, L], pos.astype(np.float32)), gc.createRaw([R, L], val)
+    rows = [0, R - 1, R - 2] + [int(v) for v in rng.integers(0, R, 40)]
+    for mode in ("set", "add"):
+        y = gc.createRawFill([R, W], 0.25)
+        gc.profileBegin()
+        if mode == "set": y.inplaceScatter(1, g_pos, g_val)
+        else: y.inplaceScatterAdd(1, g_pos, g_val)
+        launched = " ".join(gc.profileEnd().keys())
+        assert "scatter_wave_kernel" in launched, launched
+        for row in rows:
+            want = np.full(W, 0.25, np.float32)
+            for j in range(L):
+                want[pos[row, j]] = val[row, j] if mode == "set" else np.float32(want[pos[row, j]] + val[row, j])
+            got = y.get([(row, row), ALL]).toArray().reshape(-1)
+            assert np.array_equal(got, want), (mode, row)
+        gc.release(y)
+
+
 def test_odd_shaped_tensor_near_the_limit(gc):
     """x[i, j] = r[i] + c[j] on [46339, 46337] (2 147 210 243 elements, rows that start off 16-byte boundaries):
     the forms the kernels take when nothing is a multiple of four -- element gathers in the broadcast, rows read
