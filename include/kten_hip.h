@@ -258,14 +258,23 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
  * the host uses kth_copy for it. */
 int kth_get_range(uint64_t in, const int32_t* shape, int dims, const int32_t* first, const int32_t* last, uint64_t out);
 
-/* set(Array<IntRange>, tensor) (RAW:33; JVM:291-304) and, called once per input, concat
- * (kten-api/.../tensor/operations/TensorOperations.kt:41;
- * backend/kten-jvm/.../operations/AbstractJVMTensorOperations.kt:106-120): the first value_n
+/* set(Array<IntRange>, tensor) (RAW:33; JVM:291-304): the first value_n
  * floats of `value` fill the box in row-major order. As in the reference only the element
  * count is compared (JVM:295-296): a different count returns KTH_E_SHAPE. set(IntArray,
  * tensor) (RAW:31; JVM:282-289) is one contiguous range: the host uses kth_copy. */
 int kth_set_range(uint64_t target, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
                   uint64_t value, uint64_t value_n);
+
+/* TensorOperations.concat(axis, inputs) (kten-api/.../tensor/operations/TensorOperations.kt:41), which every
+ * backend of the reference builds from one range set per input at its offset along the axis
+ * (backend/kten-jvm/.../operations/AbstractJVMTensorOperations.kt:106-120;
+ * backend/kten-opencl/.../operations/OCLTensorOperations.kt:138-152). Here it is one launch that writes every
+ * element of `out` once: out has `out_shape`; input i has the same shape except axis_lens[i] along `axis`
+ * (already normalised), the lengths adding up to out_shape[axis] (else KTH_E_SHAPE; the host has checked the
+ * other dims as ShapeFunctions.kt:85-104 does). Inputs of length 0 are allowed. `out` must not be one of the
+ * inputs. */
+int kth_concat(const uint64_t* inputs, const int32_t* axis_lens, int n_inputs, const int32_t* out_shape, int dims, int axis,
+               uint64_t out);
 
 /* set(Array<IntRange>, Float) (RAW:37; JVM:311-315). set(IntArray, Float) (RAW:35;
  * JVM:306-309) is one contiguous range: the host uses kth_fill. */

@@ -637,20 +637,17 @@ inline Raw HipTensorOperations::createRawFill(const Shape& shape, float constant
 inline Raw HipTensorOperations::zerosLike(const Raw& t) { return createRawFill(t->shape, 0.0f); }
 inline void HipTensorOperations::zeroOut(const Raw& t) { t->inplaceFill(0.0f); }
 inline Raw HipTensorOperations::pow(float constant, const Raw& t) { return t->scalar(KTH_POW, constant, true); }
-inline Raw HipTensorOperations::concat(int axis, const std::vector<Raw>& inputs) {   // AbstractJVMTensorOperations.kt:106-120
+inline Raw HipTensorOperations::concat(int axis, const std::vector<Raw>& inputs) {   // TensorOperations.kt:41
     std::vector<Shape> shapes;
     for (const Raw& t : inputs) shapes.push_back(t->shape);
     const Shape resShape = concatShapes(shapes, axis);
     const int a = normalizeAxis(shapes[0], axis);
-    std::vector<IntRange> target;
-    for (int d : resShape) target.push_back(IntRange{0, d - 1});
     Raw res = createRaw(resShape);
-    int last = 0;
-    for (const Raw& t : inputs) {
-        target[a] = IntRange{last, last + t->shape[a] - 1};
-        res->set(target, t);
-        last += t->shape[a];
-    }
+    std::vector<uint64_t> handles;
+    std::vector<int32_t> lens;
+    for (const Raw& t : inputs) { handles.push_back(t->storeReference); lens.push_back(t->shape[a]); }
+    check(kth_concat(handles.data(), lens.data(), static_cast<int>(inputs.size()), resShape.data(), static_cast<int>(resShape.size()), a,
+                     res->storeReference));
     return res;
 }
 inline HipTensorOperations::BatchNormOutputs HipTensorOperations::BatchNorm::calculateOutput(

@@ -65,6 +65,7 @@ SIGNATURES = {
     "kth_index_add": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_uint64, c_uint64, c_uint64, c_float]),
     "kth_get_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_uint64]),
     "kth_set_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_uint64, c_uint64]),
+    "kth_concat": (c_int, [POINTER(c_uint64), POINTER(c_int32), c_int, POINTER(c_int32), c_int, c_int, c_uint64]),
     "kth_fill_range": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), POINTER(c_int32), c_float]),
     "kth_transpose": (c_int, [c_uint64, POINTER(c_int32), c_int, c_int, c_int, c_uint64]),
     "kth_permute": (c_int, [c_uint64, POINTER(c_int32), c_int, POINTER(c_int32), c_uint64]),

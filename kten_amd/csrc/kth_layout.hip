@@ -566,6 +566,116 @@ void launch_move(const char* family, const float* src, float* dst, uint64_t coun
                                 static_cast<uint32_t>(units), value, pl);
 }
 
+// concat: the output seen as rows of `row` floats, each made of one run per input (the run of input i: its axis
+// length times the dims inside the axis). A thread makes 16 bytes of the output: it finds the row and the place in
+// the row, picks the input whose run holds the place and loads from there -- so every line of the output is written
+// once, whole, however short the runs are, where a range set per input would write each line in pieces. FORM 2: every
+// run is a multiple of four floats, a unit never straddles two runs and loads as 16 aligned bytes. FORM 0: the four
+// floats load one by one, each from where it lies. FORM 1, for long runs: four floats of one run load as 16 bytes
+// from a dword address, the others as in FORM 0 (per 268 MB: one row of 16 777 217 floats 80 us against 96 us float
+// by float, rows of 33 and 31 floats 115 us against 95 us; both forms in one kernel, chosen per unit, measured
+// slower than either).
+constexpr int kConcatMax = 8;
+constexpr int kConcatUnroll = 2;
+constexpr uint64_t kConcatLongRun = 64;      // floats of the longest run from which FORM 1 is taken
+
+struct ConcatPlan {
+    const float* in[kConcatMax];
+    uint32_t from[kConcatMax];               // place in the output row where the run of input i starts
+    uint32_t run[kConcatMax];
+    uint32_t row;
+    FastDiv  row_div;
+};
+
+// The plan's per-input values as wave-uniform registers, so that picking an input is a chain of selects between
+// registers (left as indexed arrays, the compiler fetches the picked entry from the argument block per lane: two
+// dependent loads before every load of data). `org` is the input's address less its place in the row, so that the
+// element at place c of row r is org + 4 (r run + c).
+typedef const float __attribute__((address_space(1)))* global_floats;       // an address made from integers: known to be device memory
+typedef const v4f __attribute__((address_space(1)))* global_v4f;
+typedef const v4f_unaligned __attribute__((address_space(1)))* global_v4f_unaligned;
+
+template <int NI>
+struct ConcatInputs {
+    uint32_t from[NI], run[NI], org_lo[NI], org_hi[NI];
+};
+
+template <int NI>
+__device__ __forceinline__ ConcatInputs<NI> concat_inputs(const ConcatPlan& pl) {
+    ConcatInputs<NI> in;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        const uint64_t org = reinterpret_cast<uint64_t>(pl.in[i]) - 4ull * pl.from[i];
+        in.from[i] = __builtin_amdgcn_readfirstlane(pl.from[i]);
+        in.run[i] = __builtin_amdgcn_readfirstlane(pl.run[i]);
+        in.org_lo[i] = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(org));
+        in.org_hi[i] = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(org >> 32));
+    }
+    return in;
+}
+
+template <int NI>
+__device__ __forceinline__ global_floats concat_source(const ConcatPlan& pl, const ConcatInputs<NI>& in, uint32_t e, uint32_t& left) {
+    const uint32_t r = (__umulhi(e, pl.row_div.mul) + e) >> pl.row_div.shift;
+    const uint32_t c = e - r * pl.row;
+    uint32_t from = 0, run = in.run[0], lo = in.org_lo[0], hi = in.org_hi[0];
+#pragma unroll
+    for (int i = 1; i < NI; i++) {
+        const bool here = c >= in.from[i];
+        from = here ? in.from[i] : from;
+        run = here ? in.run[i] : run;
+        lo = here ? in.org_lo[i] : lo;
+        hi = here ? in.org_hi[i] : hi;
+    }
+    left = from + run - c;                   // floats from here to the end of the run
+    const uint64_t org = (static_cast<uint64_t>(hi) << 32) | lo;
+    return reinterpret_cast<global_floats>(org + 4ull * (r * run + c));
+}
+
+template <int NI, int FORM>
+__global__ __launch_bounds__(kBlock) void concat_kernel(float* __restrict__ out, uint32_t n, ConcatPlan pl) {
+    const uint32_t base = blockIdx.x * (kBlock * kConcatUnroll) + threadIdx.x;
+    const ConcatInputs<NI> in = concat_inputs<NI>(pl);
+    v4f v[kConcatUnroll];
+#pragma unroll
+    for (int k = 0; k < kConcatUnroll; k++) {
+        const uint32_t e = (base + k * kBlock) * 4u;
+        if (e >= n) continue;
+        uint32_t left;
+        const global_floats at = concat_source<NI>(pl, in, e, left);
+        if (FORM == 2) {
+            v[k] = __builtin_nontemporal_load(reinterpret_cast<global_v4f>(at));
+        } else if (FORM == 1 && left >= 4 && e + 4 <= n) {
+            const v4f_unaligned t = __builtin_nontemporal_load(reinterpret_cast<global_v4f_unaligned>(at));
+            v[k] = v4f{t.x, t.y, t.z, t.w};
+        } else {
+            float w[4];
+            w[0] = *at;
+#pragma unroll
+            for (uint32_t j = 1; j < 4; j++) {
+                w[j] = 0.0f;
+                if (e + j < n) {
+                    uint32_t unused;
+                    w[j] = j < left ? at[j] : *concat_source<NI>(pl, in, e + j, unused);
+                }
+            }
+            v[k] = v4f{w[0], w[1], w[2], w[3]};
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kConcatUnroll; k++) {
+        const uint32_t e = (base + k * kBlock) * 4u;
+        if (e >= n) continue;
+        if (e + 4 <= n) {
+            *reinterpret_cast<v4f*>(out + e) = v[k];
+        } else {
+            out[e] = v[k].x;
+            if (e + 1 < n) out[e + 1] = v[k].y;
+            if (e + 2 < n) out[e + 2] = v[k].z;
+        }
+    }
+}
+
 // Validates normalised inclusive ranges and describes the selected box as the strided side
 // of a move (dense side: the box in row-major order).
 int box_of(const char* what, const int32_t* shape, int dims, const int32_t* first, const int32_t* last,
@@ -868,6 +978,85 @@ int kth_set_range(uint64_t target, const int32_t* shape, int dims, const int32_t
     if (st->ptr == sv->ptr) return fail(KTH_E_ARGUMENT, "kth_set_range: value aliases the target");
     launch_move<1>("move_kernel_set", sv->ptr, st->ptr, count, 0.0f, box, base, count * 8);
     KTH_LAUNCH_CHECK("move_kernel");
+    return KTH_OK;
+}
+
+int kth_concat(const uint64_t* inputs, const int32_t* axis_lens, int n_inputs, const int32_t* out_shape, int dims, int axis,
+               uint64_t out) {
+    std::lock_guard<std::mutex> g(lock());
+    KTH_REQUIRE_INIT();
+    uint64_t total;
+    if (int rc = shape_count(out_shape, dims, "kth_concat", &total)) return rc;
+    if (!inputs || !axis_lens || n_inputs < 1) return fail(KTH_E_ARGUMENT, "kth_concat: no inputs");
+    if (axis < 0 || axis >= dims) return fail(KTH_E_ARGUMENT, "kth_concat: axis %d of %d dims", axis, dims);
+    uint64_t inner = 1, outer = 1, along = 0;
+    for (int d = axis + 1; d < dims; d++) inner *= static_cast<uint64_t>(out_shape[d]);
+    for (int d = 0; d < axis; d++) outer *= static_cast<uint64_t>(out_shape[d]);
+    for (int i = 0; i < n_inputs; i++) {
+        if (axis_lens[i] < 0) return fail(KTH_E_ARGUMENT, "kth_concat: negative length %d of input %d", axis_lens[i], i);
+        along += static_cast<uint64_t>(axis_lens[i]);
+    }
+    if (along != static_cast<uint64_t>(out_shape[axis]))
+        return fail(KTH_E_SHAPE, "kth_concat: the inputs hold %llu along axis %d, the result %d",
+                    static_cast<unsigned long long>(along), axis, out_shape[axis]);
+    Store* so = lookup_unsettled(out, "kth_concat(out)");
+    if (!so) return KTH_E_HANDLE;
+    if (total > so->n_floats) return fail(KTH_E_ARGUMENT, "kth_concat: the result needs more elements than its store holds");
+    std::vector<const float*> ptrs;
+    std::vector<uint64_t> runs;
+    for (int i = 0; i < n_inputs; i++) {
+        Store* si = lookup(inputs[i], "kth_concat(input)");
+        if (!si) return KTH_E_HANDLE;
+        const uint64_t run = static_cast<uint64_t>(axis_lens[i]) * inner;
+        if (outer * run > si->n_floats) return fail(KTH_E_ARGUMENT, "kth_concat: input %d needs more elements than its store holds", i);
+        if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "kth_concat: the result aliases input %d", i);
+        if (run == 0) continue;
+        ptrs.push_back(si->ptr);
+        runs.push_back(run);
+    }
+    settle_for_overwrite(so, total);
+    if (total == 0) return KTH_OK;
+    const uint64_t row = along * inner;
+    hipStream_t stream = state().stream;
+    if (ptrs.size() > static_cast<size_t>(kConcatMax)) {                // a range set per input
+        uint64_t from = 0;
+        for (size_t i = 0; i < ptrs.size(); i++) {
+            StridedDims raw{};
+            raw.n = 2;
+            raw.size[0] = runs[i]; raw.stride[0] = 1;
+            raw.size[1] = outer;   raw.stride[1] = row;
+            launch_move<1>("move_kernel_set", ptrs[i], so->ptr, outer * runs[i], 0.0f, coalesce(raw), from, outer * runs[i] * 8);
+            from += runs[i];
+        }
+        KTH_LAUNCH_CHECK("move_kernel");
+        return KTH_OK;
+    }
+    ConcatPlan pl{};
+    bool vec = true;
+    uint64_t from = 0, longest = 0;
+    for (int i = 0; i < kConcatMax; i++) {
+        const bool have = static_cast<size_t>(i) < ptrs.size();
+        pl.in[i] = have ? ptrs[i] : ptrs[0];
+        pl.from[i] = have ? static_cast<uint32_t>(from) : 0xffffffffu;
+        pl.run[i] = have ? static_cast<uint32_t>(runs[i]) : 0u;
+        if (have) { vec = vec && runs[i] % 4 == 0; from += runs[i]; longest = std::max(longest, runs[i]); }
+    }
+    pl.row = static_cast<uint32_t>(row);
+    pl.row_div = make_div(pl.row);
+    const uint32_t n = static_cast<uint32_t>(total);
+    const uint32_t per_block = kBlock * kConcatUnroll * 4;
+    const dim3 grid(static_cast<uint32_t>((total + per_block - 1) / per_block)), block(kBlock);
+    const int ni = ptrs.size() <= 2 ? 2 : ptrs.size() <= 4 ? 4 : 8;
+    {
+        const int form = vec ? 2 : longest >= kConcatLongRun ? 1 : 0;
+        LaunchScope scope("concat_kernel", form == 2 ? "float4" : form == 1 ? "float4 result side, long runs" : "float4 result side", total * 8);
+#define CONCAT_LAUNCH(NI) do { if (form == 2)      hipLaunchKernelGGL((concat_kernel<NI, 2>), grid, block, 0, stream, so->ptr, n, pl); \
+                               else if (form == 1) hipLaunchKernelGGL((concat_kernel<NI, 1>), grid, block, 0, stream, so->ptr, n, pl); \
+                               else                hipLaunchKernelGGL((concat_kernel<NI, 0>), grid, block, 0, stream, so->ptr, n, pl); } while (0)
+        if (ni == 2) CONCAT_LAUNCH(2); else if (ni == 4) CONCAT_LAUNCH(4); else CONCAT_LAUNCH(8);
+#undef CONCAT_LAUNCH
+    }
+    KTH_LAUNCH_CHECK("concat_kernel");
     return KTH_OK;
 }
 

@@ -17,7 +17,7 @@ import numpy as np
 from . import abi
 from .host_mirror import shape_functions as sf
 from .abi import Op, check
-from .host_mirror.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number, concat as raw_concat
+from .host_mirror.raw_tensor import AbstractRawTensor, AggregatingOperation, _is_number
 
 _BINARY = {"plus": Op.PLUS, "minus": Op.MINUS, "times": Op.TIMES, "div": Op.DIV, "pow": Op.POW,
            "lt": Op.LT, "lte": Op.LTE, "gt": Op.GT, "gte": Op.GTE, "eq": Op.EQ, "neq": Op.NEQ}
@@ -486,8 +486,18 @@ class HipTensorOperations:
         return rawTensor._scalar("pow", float(constant), reverse=True)
 
     def concat(self, axis: int, inputs) -> HipRawTensor:
-        """TensorOperations.kt:41."""
-        return raw_concat(self, axis, inputs)
+        """TensorOperations.kt:41. The reference's backends set one range of a new tensor per input
+        (AbstractJVMTensorOperations.kt:106-120, OCLTensorOperations.kt:138-152); here one launch writes every
+        element of the result once. Shape errors as ShapeFunctions.kt:85-104 raises them."""
+        inputs = list(inputs)
+        shapes = [t.shape for t in inputs]
+        res_shape = sf.concat_shapes(shapes, axis)
+        a = sf.normalize_axis(shapes[0], axis)
+        res = self.createRaw(res_shape)
+        handles = (ctypes.c_uint64 * len(inputs))(*[t.storeReference for t in inputs])
+        lens = (ctypes.c_int32 * len(inputs))(*[t.shape[a] for t in inputs])
+        check(self.lib.kth_concat(handles, lens, len(inputs), abi.shape_array(res_shape), len(res_shape), a, res.storeReference))
+        return res
 
     def batchNorm(self, axis: int, momentum: float, epsilon: float, training: bool) -> "HipBatchNorm":
         """TensorOperations.kt:129."""

@@ -1,11 +1,13 @@
 """Layout movers on the device against the CPU checker, bit-exact: get / set / fill by
 index and by ranges, narrow, concat, transpose, permute, maskedFill; float4 and scalar
 forms, tile edges, error behaviour, and size-independent properties at large sizes."""
+import ctypes
 import itertools
 
 import numpy as np
 import pytest
 
+from kten_amd import abi
 from kten_amd.host_mirror.shape_functions import ALL
 from oracle import jvm_oracle as jo
 from parity import assert_bits_equal
@@ -147,6 +149,68 @@ def test_masked_fill_parity(gc):
         for value in (0.0, -2.5, float("inf")):
             assert_bits_equal(g.maskedFill(gm, value).toArray(), c.maskedFill(cm, value).toArray(), f"maskedFill {shape} {mshape}")
         assert_bits_equal(g.toArray(), x, "maskedFill must not touch its receiver")
+
+
+CONCAT_CASES = [
+    # shape (the axis entry is replaced), axis, lengths along the axis
+    ([70001, 0], 1, [7, 3]),                      # rows of ten floats: most 16-byte units straddle both inputs
+    ([300007, 0], 1, [1, 1]),                     # a unit holds two rows
+    ([65536, 0], 1, [64, 64]),                    # aligned runs
+    ([4099, 0], 1, [100, 28, 5]),                 # three inputs, the last unaligned
+    ([0, 1021], 0, [300, 1, 212]),                # along the outermost axis: one row, runs at odd offsets
+    ([33, 0, 517], 1, [2, 9, 1, 4, 3]),           # five inputs, a middle axis
+    ([129, 0, 8], 1, [1, 2, 3, 4, 5, 6, 7, 8]),   # eight inputs: all the plan holds
+    ([129, 0, 8], 1, [1, 2, 3, 4, 5, 6, 7, 8, 9]),# nine: a range set per input
+    ([50, 0, 3], 1, [4, 0, 2]),                   # an empty input between two others
+    ([50, 0, 3], 1, [0, 0, 6, 0]),
+    ([1, 0], 1, [3, 2]),                          # fewer than four floats in all ... and a ragged last unit below
+    ([3, 0], 1, [1, 2]),
+    ([2, 3, 0, 5, 7], 2, [6, 1]),
+]
+
+
+def test_concat_in_one_launch(gc):
+    """concat writes every element of the result once, from whichever input holds it (TensorOperations.kt:41;
+    the reference sets one range per input, AbstractJVMTensorOperations.kt:106-120): against numpy's concatenate."""
+    rng = np.random.default_rng(40)
+    for shape, axis, sizes in CONCAT_CASES:
+        parts = []
+        for length in sizes:
+            sh = list(shape); sh[axis] = length
+            parts.append(rng.standard_normal(sh).astype(np.float32))
+        gc.profileBegin()
+        got = gc.concat(axis, [gc.createRaw(list(p.shape), p) for p in parts])
+        launched = " ".join(gc.profileEnd().keys())
+        want = np.concatenate(parts, axis=axis)
+        assert got.shape == list(want.shape)
+        assert_bits_equal(got.toArray(), want, f"concat {shape} axis {axis} of {sizes}")
+        if want.size:
+            family = "move_kernel_set" if sum(1 for length in sizes if length) > 8 else "concat_kernel"
+            assert family in launched, (shape, sizes, launched)
+    # the result of an earlier operation that is still owed its fill, and a result tensor concatenated with itself
+    z = gc.createRawFill([1000, 5], 2.5)
+    x = gc.createRaw([1000, 3], np.arange(3000, dtype=np.float32))
+    assert_bits_equal(gc.concat(1, [z, x, z]).toArray(),
+                      np.concatenate([np.full((1000, 5), 2.5, np.float32), np.arange(3000, dtype=np.float32).reshape(1000, 3),
+                                      np.full((1000, 5), 2.5, np.float32)], axis=1), "concat of an owed fill")
+    with pytest.raises(ValueError):
+        gc.concat(1, [x, gc.createRaw([999, 3], np.zeros(2997, np.float32))])
+    # the entry point's own checks: lengths that do not add up, a result that is one of the inputs, a store too small
+    L = gc.lib
+    out = gc.createRaw([1000, 8])
+    handles = (ctypes.c_uint64 * 2)(z.storeReference, x.storeReference)
+    u64 = lambda *v: (ctypes.c_uint64 * len(v))(*v)
+    i32 = lambda *v: (ctypes.c_int32 * len(v))(*v)
+    assert L.kth_concat(handles, i32(5, 2), 2, abi.shape_array([1000, 8]), 2, 1, out.storeReference) == abi.KTH_E_SHAPE
+    assert L.kth_concat(handles, i32(5, 3), 2, abi.shape_array([1000, 8]), 2, 2, out.storeReference) == abi.KTH_E_ARGUMENT
+    assert L.kth_concat(u64(z.storeReference, out.storeReference), i32(5, 3), 2, abi.shape_array([1000, 8]), 2, 1,
+                        out.storeReference) == abi.KTH_E_ARGUMENT
+    assert "aliases" in abi.last_error()
+    assert L.kth_concat(handles, i32(5, 3), 2, abi.shape_array([1001, 8]), 2, 1, out.storeReference) == abi.KTH_E_ARGUMENT
+    assert L.kth_concat(u64(z.storeReference, 0xdeadbeef), i32(5, 3), 2, abi.shape_array([1000, 8]), 2, 1,
+                        out.storeReference) == abi.KTH_E_HANDLE
+    assert L.kth_concat(handles, i32(5, 3), 2, abi.shape_array([1000, 8]), 2, 1, out.storeReference) == abi.KTH_OK
+    assert_bits_equal(out.toArray()[:, 5:], np.arange(3000, dtype=np.float32).reshape(1000, 3), "kth_concat")
 
 
 def test_concat_and_narrow_parity(gc):
