@@ -150,6 +150,31 @@ def test_broadcast_of_two_small_operands_in_many_dims_bit_exact(sa, sb, gc):
             assert_bits_equal(raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}")
 
 
+# An operand that repeats along a dim and holds megabytes inside it: the tiles of the output are taken chunk by chunk
+# across the repeats so that the operand's chunk stays in L2. Slices that end inside a tile and inside a chunk, repeats
+# over two dims, both operands repeating, a scalar innermost dim of the repeating operand.
+CHUNKED_PAIRS = [
+    ([3, 511, 1020], [1, 511, 1020]), ([2, 3, 130001, 4], [1, 1, 130001, 4]), ([1, 3, 4, 56860], [5, 1, 4, 56860]),
+    ([2, 1, 3, 131076], [1, 2, 3, 131076]), ([3, 400003, 4], [400003, 1]), ([2, 5, 1, 50021, 8], [1, 1, 3, 50021, 8]),
+    ([2, 4194304], [4194304]), ([2, 2, 3145728], [1, 2, 3145728]),
+]
+
+
+@pytest.mark.parametrize("sa,sb", CHUNKED_PAIRS, ids=lambda s: "x".join(map(str, s)))
+def test_broadcast_with_tiles_ordered_for_reuse_bit_exact(sa, sb, gc):
+    rng = np.random.default_rng(sum(sa) * 13 + sum(sb))
+    a = rng.standard_normal(sa).astype(np.float32); b = rng.standard_normal(sb).astype(np.float32)
+    gc.profileBegin()
+    results = []
+    for op, f in (("minus", np.subtract), ("div", np.divide)):
+        for x, y in ((a, b), (b, a)):
+            results.append((raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}"))
+    kernels = gc.profileEnd()
+    assert any("_chunked" in k for k in kernels), f"expected the chunked tile order, saw {sorted(kernels)}"
+    for got, want, what in results:
+        assert_bits_equal(got, want, what)
+
+
 def test_binary_matches_checker_on_small_broadcasts(gc):
     rng = np.random.default_rng(5)
     for sa, sb in SHAPE_PAIRS[:12]:
