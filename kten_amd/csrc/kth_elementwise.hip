@@ -600,6 +600,8 @@ struct OuterPlan {
     uint32_t span;               // M * V: outputs per row index
     uint32_t a_is_row;           // operand a is indexed by [i][v], b by [j][v]; or the other way round
     uint32_t row_lds;            // floats of LDS for the row operand's slice; the column operand's follows
+    uint32_t col_flat;           // the column operand holds one value per column index j, not a run: [N,1,V] o [1,M,1]
+    uint32_t cols;               // M
     FastDiv  span_div, run_div;
 };
 
@@ -633,8 +635,15 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
     stage_range(row_lds, 0, rowp, i_lo * pl.run, (i_hi - i_lo + 1) * pl.run);
     // the column operand: staged whole when it is no longer than the span; a longer one is read from memory,
     // 16 bytes per thread (its four outputs are neighbours there too, except where the span passes its end)
-    const bool staged = pl.span <= len;
-    if (staged) stage_range(col_lds, 0, colp, 0, pl.span);
+    const bool staged = pl.col_flat || pl.span <= len;
+    // one value per column index: the indexes the tile meets are consecutive (past the last one the first follows)
+    uint32_t j_lo = 0;
+    if (pl.col_flat) {
+        const uint32_t c_lo = s - i_lo * pl.span;
+        const uint32_t window = min(pl.cols, len / pl.run + 2u);
+        if (window < pl.cols) j_lo = (__umulhi(c_lo, pl.run_div.mul) + c_lo) >> pl.run_div.shift;
+        for (uint32_t t = threadIdx.x; t < window; t += kBlock) col_lds[t] = colp[j_lo + t < pl.cols ? j_lo + t : j_lo + t - pl.cols];
+    } else if (staged) stage_range(col_lds, 0, colp, 0, pl.span);
     // a column operand read from memory: all of a thread's loads are issued before the first is used
     constexpr uint32_t kGroups = kOuterTile / (kBlock * 4);
     v4f_unaligned ahead[kGroups];
@@ -664,7 +673,8 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
         const uint32_t e0 = s + g;
         const uint32_t i = (__umulhi(e0, pl.span_div.mul) + e0) >> pl.span_div.shift;
         uint32_t c = e0 - i * pl.span;                                     // column operand offset j * V + v
-        uint32_t v = c - ((__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift) * pl.run;
+        uint32_t col = (__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift;   // column index j
+        uint32_t v = c - col * pl.run;
         uint32_t row_base = (i - i_lo) * pl.run;
         float y[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (!staged) { y[0] = ahead[k].x; y[1] = ahead[k].y; y[2] = ahead[k].z; y[3] = ahead[k].w; }
@@ -672,11 +682,11 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const float x = row_lds[row_base + v];
-            const float yy = staged ? col_lds[c] : y[j];
+            const float yy = pl.col_flat ? col_lds[col >= j_lo ? col - j_lo : col + pl.cols - j_lo] : staged ? col_lds[c] : y[j];
             r[j] = pl.a_is_row ? Op::apply(x, yy, eps) : Op::apply(yy, x, eps);
             c++; v++;
-            if (v == pl.run) v = 0;
-            if (c == pl.span) { c = 0; row_base += pl.run; }
+            if (v == pl.run) { v = 0; col++; }
+            if (c == pl.span) { c = 0; col = 0; row_base += pl.run; }
         }
         if (g + 4 <= len) st4(out, e0 >> 2, make_float4(r[0], r[1], r[2], r[3]));
         else for (uint32_t j = 0; g + j < len; j++) out[e0 + j] = r[j];
@@ -702,7 +712,9 @@ __global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* 
     uint32_t count = 0;                                        // column offsets of this thread inside the span
     if (c0 < pl.span) {
         count = min(4u, pl.span - c0);
-        if (count == 4) {
+        if (pl.col_flat) {
+            for (uint32_t j = 0; j < count; j++) y[j] = colp[(__umulhi(c0 + j, pl.run_div.mul) + c0 + j) >> pl.run_div.shift];
+        } else if (count == 4) {
             const v4f_unaligned t = *reinterpret_cast<const v4f_unaligned*>(colp + c0);
             y[0] = t.x; y[1] = t.y; y[2] = t.z; y[3] = t.w;
         } else {
@@ -915,13 +927,24 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
         const int d = plan.ndim;
         const bool with_run = d == 3;
         const uint32_t run = with_run ? plan.size[0] : 1u;
-        const bool run_ok = !with_run || (plan.astride[0] == 1 && plan.bstride[0] == 1 && run <= kOuterMaxRun);
         // the dim next to the outermost one is the column index, the outermost the row index
-        const bool a_row = plan.astride[d - 2] == 0 && plan.astride[d - 1] == run && plan.bstride[d - 2] == run && plan.bstride[d - 1] == 0;
-        const bool b_row = plan.bstride[d - 2] == 0 && plan.bstride[d - 1] == run && plan.astride[d - 2] == run && plan.astride[d - 1] == 0;
+        bool run_ok = !with_run || (plan.astride[0] == 1 && plan.bstride[0] == 1 && run <= kOuterMaxRun);
+        bool a_row = plan.astride[d - 2] == 0 && plan.astride[d - 1] == run && plan.bstride[d - 2] == run && plan.bstride[d - 1] == 0;
+        bool b_row = plan.bstride[d - 2] == 0 && plan.bstride[d - 1] == run && plan.astride[d - 2] == run && plan.astride[d - 1] == 0;
+        // or the row operand alone keeps the innermost run and the column operand holds one value per column index
+        bool flat = false;
+        if (with_run && !run_ok && run <= kOuterMaxRun) {
+            const bool a_flat_row = plan.astride[0] == 1 && plan.astride[1] == 0 && plan.astride[2] == run &&
+                                    plan.bstride[0] == 0 && plan.bstride[1] == 1 && plan.bstride[2] == 0;
+            const bool b_flat_row = plan.bstride[0] == 1 && plan.bstride[1] == 0 && plan.bstride[2] == run &&
+                                    plan.astride[0] == 0 && plan.astride[1] == 1 && plan.astride[2] == 0;
+            flat = run_ok = a_flat_row || b_flat_row;
+            a_row = a_flat_row; b_row = b_flat_row;
+        }
         if (run_ok && (a_row || b_row) && plan.size[d - 2] >= 2) {
             OuterPlan op{};
             op.n = n; op.run = run; op.span = plan.size[d - 2] * run; op.a_is_row = a_row ? 1u : 0u;
+            op.col_flat = flat ? 1u : 0u; op.cols = plan.size[d - 2];
             op.span_div = make_div(op.span); op.run_div = make_div(run);
             op.row_lds = (((kOuterTile - 1) / op.span + 2) * run + 3u) & ~3u;
             const uint32_t rows = plan.size[d - 1];
@@ -931,7 +954,8 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
                 hipLaunchKernelGGL((binary_outer_rows_kernel<Op>), grid, dim3(kBlock), kOuterRows * run * sizeof(float), st, a, b, out, eps, op, rows);
                 return;
             }
-            const uint32_t col_lds = op.span <= kOuterTile ? op.span : 4u;      // a longer column operand is not staged
+            const uint32_t col_lds = flat ? std::min(op.cols, kOuterTile / run + 2u)
+                                          : op.span <= kOuterTile ? op.span : 4u;  // a longer column operand is not staged
             LaunchScope scope("binary_outer_kernel", Op::name, bytes);
             hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((n + kOuterTile - 1) / kOuterTile), dim3(kBlock),
                                (op.row_lds + col_lds) * sizeof(float), st, a, b, out, eps, op);

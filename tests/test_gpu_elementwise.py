@@ -112,6 +112,11 @@ OUTER_PAIRS = [
     ([33, 1, 7], [1, 1250, 7]), ([302683, 1], [1, 111]), ([56, 1, 2], [277788, 2]),
     # a column operand longer than a workgroup's tile: blocks of 8 row indexes by 1024 column offsets, ragged on both sides
     ([13, 1, 3], [100001, 3]), ([17, 1], [1, 8193]), ([8, 1], [1, 8192 + 1025]), ([1000, 1, 2], [4097, 2]),
+    # the column operand without the innermost run, [N,1,V] o [1,M,1]: windows of column indexes that wrap, whole operands,
+    # two columns, column operands longer than a tile
+    ([4225, 1, 5], [1, 158, 1]), ([197, 1, 2], [1, 57497, 1]), ([48, 1, 1, 111], [1, 6259, 1, 1]), ([219, 1, 1, 70], [1, 1, 2188, 1]),
+    ([3, 1, 78], [1, 143395, 1]), ([33000, 1, 3], [1, 2, 1]), ([8, 1, 2, 3], [1, 69905, 1, 1]), ([15497, 1, 3, 3], [1, 189, 1, 1]),
+    ([7, 1, 1023], [1, 9, 1]), ([600, 1, 7], [1, 1171, 1]), ([2, 1, 5], [1, 4099, 1]),
 ]
 
 
@@ -154,9 +159,9 @@ def test_broadcast_of_two_small_operands_in_many_dims_bit_exact(sa, sb, gc):
 # across the repeats so that the operand's chunk stays in L2. Slices that end inside a tile and inside a chunk, repeats
 # over two dims, both operands repeating, a scalar innermost dim of the repeating operand.
 CHUNKED_PAIRS = [
-    ([3, 511, 1020], [1, 511, 1020]), ([2, 3, 130001, 4], [1, 1, 130001, 4]), ([1, 3, 4, 56860], [5, 1, 4, 56860]),
-    ([2, 1, 3, 131076], [1, 2, 3, 131076]), ([3, 400003, 4], [400003, 1]), ([2, 5, 1, 50021, 8], [1, 1, 3, 50021, 8]),
-    ([2, 4194304], [4194304]), ([2, 2, 3145728], [1, 2, 3145728]),
+    ([6, 511, 1020], [1, 511, 1020]), ([2, 3, 130001, 4], [1, 1, 130001, 4]), ([1, 3, 4, 56860], [5, 1, 4, 56860]),
+    ([3, 1, 3, 131076], [1, 2, 3, 131076]), ([6, 400003, 4], [400003, 1]), ([2, 5, 1, 50021, 8], [1, 1, 3, 50021, 8]),
+    ([6, 4194304], [4194304]), ([6, 2, 1572864], [1, 2, 1572864]),
 ]
 
 
