@@ -583,7 +583,8 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float*
 
 // The broadcast of two operands that are both smaller than the output, in the shape every such pair coalesces to
 // when it is two- or three-dimensional: [N,1] o [1,M] (V = 1), or the same with an innermost run of V floats that
-// both operands keep ([N,1,V] o [M,V]). The mixed kernel pays a vector-memory instruction per operand element
+// both operands keep ([N,1,V] o [M,V]) or that the row operand alone keeps ([N,1,V] o [1,M,1]: the column operand then holds
+// one value per column index, and the tile's window of them goes into LDS). The mixed kernel pays a vector-memory instruction per operand element
 // there, and the address unit of a compute unit takes a wave's memory instruction for about 16 cycles whatever it
 // moves: 8 loads and a store per 256 outputs hold it to 2.3-3.8 TB/s. Here a workgroup owns 4096 consecutive
 // outputs, brings the slices of both operands that the span touches into LDS with 16-byte loads (the row operand's

@@ -165,17 +165,32 @@ __global__ __launch_bounds__(kBlock) void move_mixed_kernel(const float* __restr
 // A permutation that moves the input's contiguous dim X away from the innermost place:
 // the output's innermost dim is Y (input stride y_in_stride), X lands at output stride
 // x_out_stride, and every other dim is a batch dim with its own pair of strides.
+// Two or three dims that lie in memory as one dim on one side of a permutation and apart on the other: index i of the
+// joined dim is (i % len0) of the innermost, ((i / len0) % len1) of the middle and (i / len0 / len1) of the outermost one.
+struct JoinedDims {
+    uint32_t len0;                           // 0: the dim is not a joined one
+    FastDiv  div0;
+    uint32_t len1;                           // 0: two dims
+    FastDiv  div1;
+    uint32_t stride1, stride2;               // the middle and the outermost dim's strides on the other side
+};
+
+__device__ __forceinline__ uint32_t joined_offset(const JoinedDims& j, uint32_t i, uint32_t stride0) {
+    if (!j.len0) return i * stride0;
+    const uint32_t t = (__umulhi(i, j.div0.mul) + i) >> j.div0.shift;
+    const uint32_t lo = i - t * j.len0;
+    if (!j.len1) return lo * stride0 + t * j.stride1;
+    const uint32_t hi = (__umulhi(t, j.div1.mul) + t) >> j.div1.shift;
+    return lo * stride0 + (t - hi * j.len1) * j.stride1 + hi * j.stride2;
+}
+
 struct TilePlan {
     uint32_t x_len, y_len;
     uint32_t x_out_stride, y_in_stride;
     uint32_t x_tiles, y_tiles;
     FastDiv  x_tiles_div, y_tiles_div;
-    uint32_t x_split;                        // permute_tile_kernel: X is two dims that the input holds as one run: index x is
-    FastDiv  x_split_div;                    //   (x % x_split) of the inner one and (x / x_split) of the outer one, which has its
-    uint32_t x_hi_out_stride;                //   own place in the output (0: X is one dim)
-    uint32_t y_split;                        // ... and the same for Y, two dims that the output holds as one run: the load works
-    FastDiv  y_split_div;                    //   out the two input places
-    uint32_t y_hi_in_stride;
+    JoinedDims xs;                           // X is two or three dims that the input holds as one run, each with its own place in the output
+    JoinedDims ys;                           // ... and Y two or three dims that the output holds as one run, each with its own place in the input
     uint32_t tiles;                          // permute_tile_kernel: the grid holds this many rounded up to a multiple of 8
     uint32_t by_xcd;                         // ... and an XCD takes a contiguous eighth of them (rows that do not start on a cache line)
     int      nbatch;
@@ -225,12 +240,7 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
         const uint32_t e = k * kBlock + threadIdx.x;
         const uint32_t x = x0 + e % TX, y = y0 + e / TX;
         if (x < pl.x_len && y < pl.y_len) {
-            uint32_t from = y * pl.y_in_stride;
-            if (pl.y_split) {
-                const uint32_t hi = (__umulhi(y, pl.y_split_div.mul) + y) >> pl.y_split_div.shift;
-                from = (y - hi * pl.y_split) * pl.y_in_stride + hi * pl.y_hi_in_stride;
-            }
-            v[k] = __builtin_nontemporal_load(in + in_off + from + x);
+            v[k] = __builtin_nontemporal_load(in + in_off + joined_offset(pl.ys, y, pl.y_in_stride) + x);
         }
     }
 #pragma unroll
@@ -245,12 +255,7 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
         const uint32_t lx = e / TY, ly = e % TY;
         const uint32_t x = x0 + lx, y = y0 + ly;
         if (x < pl.x_len && y < pl.y_len) {
-            uint32_t to = x * pl.x_out_stride;
-            if (pl.x_split) {
-                const uint32_t hi = (__umulhi(x, pl.x_split_div.mul) + x) >> pl.x_split_div.shift;
-                to = (x - hi * pl.x_split) * pl.x_out_stride + hi * pl.x_hi_out_stride;
-            }
-            out[out_off + to + y] = tile[ly * (TX + 1) + lx];
+            out[out_off + joined_offset(pl.xs, x, pl.x_out_stride) + y] = tile[ly * (TX + 1) + lx];
         }
     }
 }
@@ -313,7 +318,7 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
                 const uint32_t y = (__umulhi(u, rp.unit_row_div.mul) + u) >> rp.unit_row_div.shift;
                 const uint32_t p = (u - y * upr) * 4u;
                 if (y0 + y < pl.y_len && p < x_floats) {
-                    const float* g = src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p;
+                    const float* g = src + static_cast<size_t>(joined_offset(pl.ys, y0 + y, pl.y_in_stride)) * rp.run + p;
                     if (p + 4 <= x_floats) {
                         const v4f_unaligned t4 = __builtin_nontemporal_load(reinterpret_cast<const v4f_unaligned*>(g));
                         v[k] = v4f{t4.x, t4.y, t4.z, t4.w};
@@ -350,7 +355,7 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
                 const uint32_t p = (u - x * upr) * 4u;
                 if (x0 + x < pl.x_len && p < y_floats) {
                     const float* l = tile + x * rp.pitch + p;
-                    float* g = dst + static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p;
+                    float* g = dst + static_cast<size_t>(joined_offset(pl.xs, x0 + x, pl.x_out_stride)) * rp.run + p;
                     if (p + 4 <= y_floats) {
                         *reinterpret_cast<v4f_unaligned*>(g) = v4f_unaligned{l[0], l[1], l[2], l[3]};
                     } else {
@@ -372,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
                 const uint32_t y = (__umulhi(f, rp.in_row_div.mul) + f) >> rp.in_row_div.shift;
                 const uint32_t p = f - y * row;
                 if (y0 + y < pl.y_len && p < x_floats)
-                    v[k] = __builtin_nontemporal_load(src + static_cast<size_t>(y0 + y) * pl.y_in_stride * rp.run + p);
+                    v[k] = __builtin_nontemporal_load(src + static_cast<size_t>(joined_offset(pl.ys, y0 + y, pl.y_in_stride)) * rp.run + p);
             }
         }
 #pragma unroll
@@ -393,7 +398,7 @@ __global__ __launch_bounds__(kBlock) void permute_runs_kernel(const V* __restric
                 const uint32_t x = (__umulhi(f, rp.out_row_div.mul) + f) >> rp.out_row_div.shift;
                 const uint32_t p = f - x * row;
                 if (x0 + x < pl.x_len && p < y_floats)
-                    dst[static_cast<size_t>(x0 + x) * pl.x_out_stride * rp.run + p] = tile[x * rp.pitch + p];
+                    dst[static_cast<size_t>(joined_offset(pl.xs, x0 + x, pl.x_out_stride)) * rp.run + p] = tile[x * rp.pitch + p];
             }
         }
     }
@@ -703,7 +708,7 @@ int box_of(const char* what, const int32_t* shape, int dims, const int32_t* firs
 
 // Permutes through LDS tiles. `v`: the output's dims innermost first with the input's strides,
 // in units of `elem` floats (1, 2, 4, or a run of 3 ... 63), stride[0] != 1. Returns KTH_OK after launching,
-// kTilesDeclined (nothing launched) when float tiles would be mostly empty.
+// kTilesDeclined (nothing launched) when the tiles would be mostly empty.
 constexpr int kTilesDeclined = 1;
 int launch_tiles(const char* what, const StridedDims& v, int elem, const float* in, float* out, uint64_t n) {
     int px = -1;
@@ -759,35 +764,37 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     pl.x_out_stride = static_cast<uint32_t>(x_out_stride);
     // A short contiguous dim of the input whose neighbour in the input goes elsewhere in the output ([N,206,3] reversed:
     // rows of 618 floats of which a tile would take 3): the two are one X of 618 for the loads, and the store works
-    // out the two output places from the index.
-    if (elem == 1 && x_len < 64) {
-        for (int d = 0; d < nb; d++) {
-            if (b_in[d] != x_len || static_cast<uint64_t>(x_len) * bsize[d] > 0x7fffffffull) continue;
-            pl.x_split = x_len; pl.x_split_div = make_div(x_len); pl.x_hi_out_stride = b_out[d];
-            pl.x_len = x_len * bsize[d];
-            for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
-            nb--;
-            batch /= (pl.x_len / x_len);
-            break;
-        }
+    // out the two output places from the index. A third dim joins when the two are still short ([N,189,3,3] by
+    // [1,3,2,0]: X is the whole row of 1701 floats).
+    for (int level = 0; level < 2 && pl.x_len < 64; level++) {
+        int d = 0;
+        while (d < nb && (b_in[d] != pl.x_len || static_cast<uint64_t>(pl.x_len) * bsize[d] > 0x7fffffffull)) d++;
+        if (d == nb) break;
+        if (level == 0) { pl.xs.len0 = pl.x_len; pl.xs.div0 = make_div(pl.x_len); pl.xs.stride1 = b_out[d]; }
+        else { pl.xs.len1 = pl.x_len / pl.xs.len0; pl.xs.div1 = make_div(pl.xs.len1); pl.xs.stride2 = b_out[d]; }
+        pl.x_len *= bsize[d];
+        batch /= bsize[d];
+        for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
+        nb--;
     }
-    // ... and a short contiguous dim of the output whose neighbour in the output comes from elsewhere in the input.
-    if (elem == 1 && y_len < 64) {
-        for (int d = 0; d < nb; d++) {
-            if (b_out[d] != y_len || static_cast<uint64_t>(y_len) * bsize[d] > 0x7fffffffull) continue;
-            pl.y_split = y_len; pl.y_split_div = make_div(y_len); pl.y_hi_in_stride = b_in[d];
-            pl.y_len = y_len * bsize[d];
-            for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
-            nb--;
-            batch /= (pl.y_len / y_len);
-            break;
-        }
+    // ... and a short contiguous dim of the output whose neighbours in the output come from elsewhere in the input.
+    for (int level = 0; level < 2 && pl.y_len < 64; level++) {
+        int d = 0;
+        while (d < nb && (b_out[d] != pl.y_len || static_cast<uint64_t>(pl.y_len) * bsize[d] > 0x7fffffffull)) d++;
+        if (d == nb) break;
+        if (level == 0) { pl.ys.len0 = pl.y_len; pl.ys.div0 = make_div(pl.y_len); pl.ys.stride1 = b_in[d]; }
+        else { pl.ys.len1 = pl.y_len / pl.ys.len0; pl.ys.div1 = make_div(pl.ys.len1); pl.ys.stride2 = b_in[d]; }
+        pl.y_len *= bsize[d];
+        batch /= bsize[d];
+        for (int k = d; k + 1 < nb; k++) { bsize[k] = bsize[k + 1]; b_in[k] = b_in[k + 1]; b_out[k] = b_out[k + 1]; }
+        nb--;
     }
     if (elem == 3 || elem > 4) {
         RunsPlan rp{};
         const bool vec = elem % 4 == 0;
         rp.run = static_cast<uint32_t>(vec ? elem / 4 : elem);
         rp.tile = elem <= 4 ? 32u : elem <= 16 ? 16u : 8u;
+        if (pl.x_len < rp.tile || pl.y_len < rp.tile) return kTilesDeclined;
         rp.pitch = (rp.tile * rp.run) | 1u;
         rp.in_row_div = make_div(rp.tile * rp.run); rp.out_row_div = rp.in_row_div; rp.run_div = make_div(rp.run);
         rp.unit_row_div = make_div(rp.tile * rp.run / 4);
@@ -811,6 +818,7 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     // Tile shape: narrow along a dim shorter than 64 (the smallest power of two that holds it), square
     // otherwise; vector elements use one shape of 16 KiB.
     uint32_t tx = 64, ty = 64;
+    if ((elem == 2 || elem == 4) && (pl.x_len < 16 || pl.y_len < 16)) return kTilesDeclined;
     if (elem == 4) { tx = 32; ty = 32; }
     else if (elem == 2) { tx = 64; ty = 32; }
     else if (pl.x_len < 64 && pl.x_len <= pl.y_len) { tx = 2; while (tx < pl.x_len) tx <<= 1; ty = kTileElems / tx; }
@@ -833,7 +841,8 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     if (blocks > kMaxElements - 8) return fail(KTH_E_ARGUMENT, "%s: too many tiles", what);
     pl.tiles = static_cast<uint32_t>(blocks);
     const uint32_t line = 128 / (4 * static_cast<uint32_t>(elem));                  // elements per cache line
-    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0 || pl.x_hi_out_stride % line != 0 || pl.y_hi_in_stride % line != 0) ? 1u : 0u;
+    pl.by_xcd = (pl.x_out_stride % line != 0 || pl.y_in_stride % line != 0 || pl.xs.stride1 % line != 0 || pl.xs.stride2 % line != 0 ||
+                 pl.ys.stride1 % line != 0 || pl.ys.stride2 % line != 0) ? 1u : 0u;
     for (int d = 0; d < nb; d++) if (b_in[d] % line != 0 || b_out[d] % line != 0) pl.by_xcd = 1u;
     const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
     LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
@@ -895,31 +904,36 @@ int permute_device(const char* what, const float* in, float* out, const int32_t*
     const StridedDims v = coalesce(raw);
     if (v.stride[0] == 1 && (v.size[0] == 2 || v.size[0] == 4) && v.n >= 3) {
         // An innermost dim of 2 or 4 floats that stays in place: permute float2 / float4 elements
-        // through tiles when the dims that do move are long enough to fill them.
+        // through tiles when the dims that do move (joined with their neighbours) are long enough to fill them.
         const uint64_t elem = v.size[0];
         StridedDims w{};
         for (int d = 1; d < v.n; d++) { w.size[w.n] = v.size[d]; w.stride[w.n] = v.stride[d] / elem; w.n++; }
         int wx = -1;
         for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
-        if (w.stride[0] != 1 && wx > 0 && w.size[0] >= 16 && w.size[wx] >= 16) {
-            if (int rc = launch_tiles(what, w, static_cast<int>(elem), in, out, n)) return rc;
-            KTH_LAUNCH_CHECK("permute_tile_kernel");
-            return KTH_OK;
+        if (w.stride[0] != 1 && wx > 0) {
+            const int rc = launch_tiles(what, w, static_cast<int>(elem), in, out, n);
+            if (rc != kTilesDeclined) {
+                if (rc) return rc;
+                KTH_LAUNCH_CHECK("permute_tile_kernel");
+                return KTH_OK;
+            }
         }
     }
     if (v.stride[0] == 1 && v.size[0] >= 3 && (v.size[0] < 32 || (v.size[0] < 64 && v.size[0] % 4 != 0)) && v.n >= 3) {
         // A run of 3 ... 31 floats that stays innermost (up to 63 when it cannot move as float4s): tiles of
-        // runs, when both transposed dims can fill one.
+        // runs, when both transposed dims (joined with their neighbours) can fill one.
         const uint64_t run = v.size[0];
         StridedDims w{};
         for (int d = 1; d < v.n; d++) { w.size[w.n] = v.size[d]; w.stride[w.n] = v.stride[d] / run; w.n++; }
         int wx = -1;
         for (int d = 1; d < w.n; d++) if (w.stride[d] == 1) wx = d;
-        const uint64_t side = run <= 4 ? 32 : run <= 16 ? 16 : 8;
-        if (w.stride[0] != 1 && wx > 0 && w.size[0] >= side && w.size[wx] >= side) {
-            if (int rc = launch_tiles(what, w, static_cast<int>(run), in, out, n)) return rc;
-            KTH_LAUNCH_CHECK("permute_runs_kernel");
-            return KTH_OK;
+        if (w.stride[0] != 1 && wx > 0) {
+            const int rc = launch_tiles(what, w, static_cast<int>(run), in, out, n);
+            if (rc != kTilesDeclined) {
+                if (rc) return rc;
+                KTH_LAUNCH_CHECK("permute_runs_kernel");
+                return KTH_OK;
+            }
         }
     }
     if (v.stride[0] == 1) {

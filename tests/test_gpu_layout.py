@@ -122,7 +122,10 @@ PERMUTE_SHAPES = [[2, 3, 2], [5, 6, 7], [8, 64, 68], [2, 3, 4, 5], [3, 4, 64, 65
                   [9, 10, 63], [16, 48, 28], [40, 70, 3], [33, 35, 3], [2, 32, 32, 3],
                   # a short contiguous dim of the input (or of the output) whose neighbour there goes elsewhere: the two as one
                   # tile dim; both contiguous dims short with no neighbour to join: the element gather instead of mostly empty tiles
-                  [300, 26, 3], [30, 8, 19, 8], [40, 7, 11, 23], [322, 14, 2, 5], [26, 17, 19, 4], [5, 5, 66, 23], [70, 3, 2, 90]]
+                  [300, 26, 3], [30, 8, 19, 8], [40, 7, 11, 23], [322, 14, 2, 5], [26, 17, 19, 4], [5, 5, 66, 23], [70, 3, 2, 90],
+                  # three dims as one tile dim; joined dims in tiles of runs and of float2 / float4 elements
+                  [155, 19, 3, 3], [3, 3, 19, 155], [470, 31, 3, 6], [3, 31, 470, 6], [60, 5, 7, 4], [90, 3, 3, 3, 2], [37, 3, 5, 2, 12],
+                  [3, 2, 3, 200, 5]]
 
 
 @pytest.mark.parametrize("shape", PERMUTE_SHAPES, ids=lambda s: "x".join(map(str, s)))
