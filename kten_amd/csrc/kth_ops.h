@@ -15,17 +15,25 @@ namespace kth {
 // java.lang.Math.max(float,float): NaN wins, -0 < +0. (JVMRawTensor.kt:159)
 // v_max_f32 / v_min_f32 order the zeros that way themselves (max(+0, -0) = +0 whichever operand holds which) and
 // return the other operand when one is a NaN, so the instruction and one unordered compare make the Java rule.
+// `r` unless an operand is a NaN, then that operand (a first). Written as two selects on the bit patterns: as nested
+// conditions the compiler made branches of it inside the reduction loops (four masked jumps per element).
+__device__ __forceinline__ float java_nan_rule(float a, float b, float r) {
+    const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b), ur = __float_as_uint(r);
+    const uint32_t with_b = (b != b) ? ub : ur;
+    return __uint_as_float((a != a) ? ua : with_b);
+}
+
 __device__ __forceinline__ float jmax(float a, float b) {
     float r;
     asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return (a != a || b != b) ? (a != a ? a : b) : r;
+    return java_nan_rule(a, b, r);
 }
 
 // java.lang.Math.min(float,float). (JVMRawTensor.kt:160)
 __device__ __forceinline__ float jmin(float a, float b) {
     float r;
     asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return (a != a || b != b) ? (a != a ? a : b) : r;
+    return java_nan_rule(a, b, r);
 }
 
 // Float.pow(Float) = Math.pow(double,double).toFloat() (JVMRawTensor.kt:138-140).

@@ -411,7 +411,7 @@ __global__ __launch_bounds__(kBlock) void reduce_strided_kernel(const float* __r
 // One workgroup per (outer index, segment): its slab is one contiguous span. `lanes` groups of
 // inner / VEC threads walk the rows `lanes` apart, so a load instruction of the workgroup covers
 // lanes * inner consecutive floats and every thread stays on its own column(s). The lanes'
-// partials meet in LDS and one thread per column merges them in lane order.
+// partials meet in LDS and are merged pairwise, lane l with lane l + step.
 // VEC = 4: a thread owns four adjacent columns, loaded as 16 bytes from a dword address, for any inner size of
 // at least 4; when inner is not a multiple of 4 the last group starts at inner - 4 and overlaps its neighbour
 // (both fold the same rows, so the columns they share get the same value twice).
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     for (int v = 0; v < VEC; v++) acc[v] = R::init();
     if (lane < lanes) {
         const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
-        constexpr uint32_t kBatch = VEC == 4 ? 4 : 8;
+        constexpr uint32_t kBatch = 8;
         // every pass issues its (up to) kBatch loads before consuming any; the last pass is predicated
         for (uint32_t r = begin + lane; r < end; r += kBatch * lanes) {
             if (VEC == 4) {
@@ -465,11 +465,18 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
         for (int v = 0; v < VEC; v++) fold[lane * g.inner + col + v] = acc[v];
     }
     __syncthreads();
-    for (uint32_t i = t; i < g.inner; i += kBlock) {
-        Acc a = fold[i];
-        for (uint32_t l = 1; l < lanes; l++) a = R::merge(a, fold[l * g.inner + i]);
-        emit<R>(g, o, s, i, a, out, partial);
+    // lane l takes lane l + step, step halving: with an inner size of 4 there are 256 lanes, and one thread per column
+    // merging them in turn was a third of the kernel's time
+    const uint32_t total = lanes * g.inner;
+    uint32_t width = 1;
+    while (width < lanes) width <<= 1;
+    for (uint32_t step = width >> 1; step >= 1; step >>= 1) {
+        const uint32_t half = step * g.inner;
+        for (uint32_t e = t; e < half; e += kBlock)
+            if (e + half < total) fold[e] = R::merge(fold[e], fold[e + half]);
+        __syncthreads();
     }
+    for (uint32_t i = t; i < g.inner; i += kBlock) emit<R>(g, o, s, i, fold[i], out, partial);
 }
 
 // ---------------------------------------------------------------- few rows: axis of 2 ... 7 over wide columns
