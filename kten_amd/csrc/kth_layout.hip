@@ -208,7 +208,7 @@ struct TilePlan {
 // The LDS row pitch TX + 1 is odd: both phases are free of bank conflicts.
 // V is the element: a float, or a float2 / float4 when the permutation keeps an innermost
 // dim of 2 or 4 floats in place (lengths, strides and offsets of the plan then count elements).
-template <int TX, int TY, class V>
+template <int TX, int TY, class V, bool JOINED>
 __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restrict__ in, V* __restrict__ out, TilePlan pl) {
     static_assert(TX * TY * sizeof(V) == kTileElems * sizeof(float), "a tile holds 16 KiB");
     __shared__ V tile[TY * (TX + 1)];
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
         const uint32_t e = k * kBlock + threadIdx.x;
         const uint32_t x = x0 + e % TX, y = y0 + e / TX;
         if (x < pl.x_len && y < pl.y_len) {
-            v[k] = __builtin_nontemporal_load(in + in_off + joined_offset(pl.ys, y, pl.y_in_stride) + x);
+            v[k] = __builtin_nontemporal_load(in + in_off + (JOINED ? joined_offset(pl.ys, y, pl.y_in_stride) : y * pl.y_in_stride) + x);
         }
     }
 #pragma unroll
@@ -255,7 +255,7 @@ __global__ __launch_bounds__(kBlock) void permute_tile_kernel(const V* __restric
         const uint32_t lx = e / TY, ly = e % TY;
         const uint32_t x = x0 + lx, y = y0 + ly;
         if (x < pl.x_len && y < pl.y_len) {
-            out[out_off + joined_offset(pl.xs, x, pl.x_out_stride) + y] = tile[ly * (TX + 1) + lx];
+            out[out_off + (JOINED ? joined_offset(pl.xs, x, pl.x_out_stride) : x * pl.x_out_stride) + y] = tile[ly * (TX + 1) + lx];
         }
     }
 }
@@ -846,22 +846,24 @@ int launch_tiles(const char* what, const StridedDims& v, int elem, const float* 
     for (int d = 0; d < nb; d++) if (b_in[d] % line != 0 || b_out[d] % line != 0) pl.by_xcd = 1u;
     const dim3 grid(static_cast<uint32_t>((blocks + 7) / 8 * 8));
     LaunchScope scope("permute_tile_kernel", elem == 4 ? "float4" : elem == 2 ? "float2" : "", n * 8);
+    const bool joined = pl.xs.len0 != 0 || pl.ys.len0 != 0;                         // (the plain form keeps its address arithmetic free of the test)
+#define KTH_TILE_V(TX, TY, V, J) hipLaunchKernelGGL((permute_tile_kernel<TX, TY, V, J>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const V*>(in), \
+                                                    reinterpret_cast<V*>(out), pl)
+#define KTH_TILE(TX, TY) do { if (joined) KTH_TILE_V(TX, TY, float, true); else KTH_TILE_V(TX, TY, float, false); } while (0)
     if (elem == 4) {
-        hipLaunchKernelGGL((permute_tile_kernel<32, 32, v4f>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const v4f*>(in),
-                           reinterpret_cast<v4f*>(out), pl);
+        if (joined) KTH_TILE_V(32, 32, v4f, true); else KTH_TILE_V(32, 32, v4f, false);
     } else if (elem == 2) {
-        hipLaunchKernelGGL((permute_tile_kernel<64, 32, v2f>), grid, dim3(kBlock), 0, stream, reinterpret_cast<const v2f*>(in),
-                           reinterpret_cast<v2f*>(out), pl);
+        if (joined) KTH_TILE_V(64, 32, v2f, true); else KTH_TILE_V(64, 32, v2f, false);
     } else {
-#define KTH_TILE(TX, TY) hipLaunchKernelGGL((permute_tile_kernel<TX, TY, float>), grid, dim3(kBlock), 0, stream, in, out, pl)
         switch (tx) {
         case 2: KTH_TILE(2, 2048); break;    case 4: KTH_TILE(4, 1024); break;    case 8: KTH_TILE(8, 512); break;
         case 16: KTH_TILE(16, 256); break;   case 32: KTH_TILE(32, 128); break;   case 64: KTH_TILE(64, 64); break;
         case 128: KTH_TILE(128, 32); break;  case 256: KTH_TILE(256, 16); break;  case 512: KTH_TILE(512, 8); break;
         case 1024: KTH_TILE(1024, 4); break; default: KTH_TILE(2048, 2); break;
         }
-#undef KTH_TILE
     }
+#undef KTH_TILE
+#undef KTH_TILE_V
     return KTH_OK;
 }
 
