@@ -124,6 +124,45 @@ def test_permute_matches_checker(sp, seed, hip):
 
 
 @st.composite
+def concat_case(draw):
+    """A shape of 1..4 dims, an axis, and 1..10 lengths along it (empty inputs among them, at least one value in all)."""
+    shape = draw(st.lists(st.sampled_from([1, 2, 3, 4, 5, 7, 8, 16, 33, 64, 257]), min_size=1, max_size=4)
+                 .filter(lambda s: int(np.prod(s)) <= 1 << 14))
+    axis = draw(st.integers(0, len(shape) - 1))
+    lengths = draw(st.lists(st.sampled_from([0, 1, 1, 2, 3, 4, 5, 8, 9, 31]), min_size=1, max_size=10).filter(lambda v: sum(v) > 0))
+    return shape, axis, lengths
+
+
+@settings(**SETTINGS)
+@given(case=concat_case(), seed=st.integers(0, 2 ** 16))
+def test_concat_matches_numpy_and_the_checker(case, seed, hip):
+    """TensorOperations.concat (TensorOperations.kt:41): one launch on the device, a range set per input in the checker
+    (AbstractJVMTensorOperations.kt:106-120), numpy's concatenate as the third opinion."""
+    shape, axis, lengths = case
+    rng = np.random.default_rng(seed)
+    parts = []
+    for length in lengths:
+        sh = list(shape); sh[axis] = length
+        parts.append(rng.standard_normal(sh).astype(np.float32))
+    want = np.concatenate(parts, axis=axis)
+    cpu = jo.JvmOracleOperations()
+    if any(p.size == 0 for p in parts):
+        # an empty input is an empty range to the reference's range set, which it rejects: the same error on both sides
+        with pytest.raises(ValueError) as on_checker:
+            cpu.concat(axis, [cpu.createRaw(list(p.shape), p.reshape(-1)) for p in parts])
+        with hip.garbageCollector(), pytest.raises(ValueError) as on_device:
+            hip.concat(axis, [hip.createRaw(list(p.shape), p) for p in parts])
+        assert str(on_device.value) == str(on_checker.value)
+        return
+    checker = cpu.concat(axis, [cpu.createRaw(list(p.shape), p.reshape(-1)) for p in parts])
+    with hip.garbageCollector():
+        got = hip.concat(axis - len(shape) if seed % 2 else axis, [hip.createRaw(list(p.shape), p) for p in parts])
+        assert got.shape == list(want.shape) == checker.shape
+        assert_bits_equal(got.toArray(), want, f"concat {shape} axis {axis} lengths {lengths}")
+        assert_bits_equal(checker.toArray(), want, f"checker's concat {shape} axis {axis} lengths {lengths}")
+
+
+@st.composite
 def batch_norm_case(draw):
     shape = draw(st.lists(st.sampled_from([1, 2, 3, 4, 5, 8, 17, 64, 70, 130]), min_size=2, max_size=4)
                  .filter(lambda s: 2 <= int(np.prod(s)) <= 1 << 16))
