@@ -643,6 +643,21 @@ inline Raw HipTensorOperations::concat(int axis, const std::vector<Raw>& inputs)
     const Shape resShape = concatShapes(shapes, axis);
     const int a = normalizeAxis(shapes[0], axis);
     Raw res = createRaw(resShape);
+    bool anyEmpty = false;
+    for (const Raw& t : inputs) anyEmpty = anyEmpty || t->size() == 0;
+    if (anyEmpty) {
+        // the reference's construction (AbstractJVMTensorOperations.kt:106-120): an empty input is an empty range, which
+        // the range set rejects as the reference does
+        std::vector<IntRange> target;
+        for (int d : resShape) target.push_back(IntRange{0, d - 1});
+        int last = 0;
+        for (const Raw& t : inputs) {
+            target[a] = IntRange{last, last + t->shape[a] - 1};
+            res->set(target, t);
+            last += t->shape[a];
+        }
+        return res;
+    }
     std::vector<uint64_t> handles;
     std::vector<int32_t> lens;
     for (const Raw& t : inputs) { handles.push_back(t->storeReference); lens.push_back(t->shape[a]); }
