@@ -233,6 +233,38 @@ __global__ __launch_bounds__(kBlock) void bn_stats_cols_kernel(const float* __re
 
 // ---------------------------------------------------------------- finalize
 
+// The sums of one channel straight from the tensor, by one thread: for very many channels of a few items each
+// (per_channel <= 32), where partial sums would be as many as the items themselves ([4194304,4] over axis 0 wrote and
+// re-read 268 MB of them for 67 MB of input). Neighbouring threads read neighbouring channels. Forward: s1 = sum(x - k),
+// s2 = sum((x - k)^2) with k the channel's first item; backward: s1 = sum(g), s2 = sum((x - mean) g).
+__device__ __forceinline__ void fold_items(const float* __restrict__ x, const float* __restrict__ go, const Geometry& g, uint32_t c,
+                                           bool backward, double shift, double& s1, double& s2) {
+    s1 = 0.0; s2 = 0.0;
+    constexpr uint32_t kAhead = 8;
+    for (uint32_t t0 = 0; t0 < g.per_channel; t0 += kAhead) {
+        float vx[kAhead], vg[kAhead];
+#pragma unroll
+        for (uint32_t k = 0; k < kAhead; k++) {
+            const uint32_t t = t0 + k;
+            if (t < g.per_channel) {
+                const uint32_t o = t / g.inner, i = t - o * g.inner;
+                const uint64_t at = (static_cast<uint64_t>(o) * g.channels + c) * g.inner + i;
+                vx[k] = x[at];
+                if (backward) vg[k] = go[at];
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < kAhead; k++) {
+            if (t0 + k < g.per_channel) {
+                const double d = static_cast<double>(vx[k]) - shift;
+                if (backward) { const double gr = static_cast<double>(vg[k]); s1 += gr; s2 += d * gr; }
+                else { s1 += d; s2 += d * d; }
+            }
+        }
+    }
+}
+
+
 // Per-channel parameters for the apply kernels.
 struct ForwardParams { float mean, stdev, gamma, beta; };
 struct BackwardParams { float mean, stdev, gamma, dot_std_sq, grad_mean, pad0, pad1, pad2; };
@@ -288,12 +320,13 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
                                                                     float* __restrict__ current_mean, float* __restrict__ current_std,
                                                                     ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch,
                                                                     int alone) {
-    // one wave per channel, or one thread
+    // one wave per channel, or one thread (alone = 1: over the partials; 2: over the channel's items themselves)
     const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (c >= g.channels) return;
     float mean, stdev = 0.0f;
     double s1 = 0.0, s2 = 0.0;
-    if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    if (training && alone == 2) fold_items(x, nullptr, g, c, false, static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]), s1, s2);
+    else if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
     if (!alone && (threadIdx.x & 63) != 0) return;
     if (training) {
         const double n = static_cast<double>(g.per_channel);
@@ -327,7 +360,8 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float
     soa[c] = p.mean; soa[pitch + c] = p.stdev; soa[2 * pitch + c] = p.gamma; soa[3 * pitch + c] = p.beta;
 }
 
-__global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const double* __restrict__ partial, Geometry g, uint32_t segments,
+__global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const float* __restrict__ x, const float* __restrict__ go,
+                                                                     const double* __restrict__ partial, Geometry g, uint32_t segments,
                                                                      int by_cols, int have_sums, int training, float epsilon,
                                                                      const float* __restrict__ running_mean, const float* __restrict__ running_var,
                                                                      const float* __restrict__ current_mean, const float* __restrict__ current_std,
@@ -337,14 +371,15 @@ __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const doub
     const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (c >= g.channels) return;
     double s1 = 0.0, s2 = 0.0;
-    if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
-    if (!alone && (threadIdx.x & 63) != 0) return;
     float mean, stdev;
     if (training) { mean = current_mean[c]; stdev = current_std[c]; }           // JVMBatchNorm.kt:131-133
     else {                                                                      // :134-137
         mean = running_mean[c];
         stdev = static_cast<float>(1.0 / sqrt(static_cast<double>(running_var[c] + epsilon)));
     }
+    if (have_sums && alone == 2) fold_items(x, go, g, c, true, static_cast<double>(mean), s1, s2);
+    else if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    if (!alone && (threadIdx.x & 63) != 0) return;
     float sum = 0.0f, dot = 0.0f;
     if (have_sums) {
         sum = static_cast<float>(s1);                                           // :139-147
@@ -502,6 +537,9 @@ struct StatsLaunch {
     bool     vec;
 };
 
+// Very many channels of a few items each: no statistics launch, a thread per channel sums its items in the finalize.
+static bool stats_direct(const Geometry& g) { return g.channels >= 16384 && g.per_channel <= 32; }
+
 // A thread per channel folds the partials when there are very many channels of a few items each.
 static bool finalize_alone(const Geometry& g, const StatsLaunch& st) {
     const uint64_t items = st.by_cols ? static_cast<uint64_t>(st.segments) * g.inner : st.segments;
@@ -623,7 +661,8 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     if (int rc = channel_store("kth_batch_norm_forward(current_std)", current_std, g.channels, &cs)) return rc;
     if (!cm || !cs) return fail(KTH_E_ARGUMENT, "kth_batch_norm_forward: current_mean and current_std are outputs and must be given");
 
-    const StatsLaunch st = training ? plan_stats(g) : StatsLaunch{};
+    const bool direct = training && stats_direct(g);
+    const StatsLaunch st = training && !direct ? plan_stats(g) : StatsLaunch{};
     const uint32_t pitch = (g.channels + 3u) & ~3u;
     const uint64_t aos_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(ForwardParams));
     const uint64_t params_bytes = aos_bytes + align256(4ull * pitch * sizeof(float));
@@ -634,10 +673,10 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     ForwardParams* params = reinterpret_cast<ForwardParams*>(ws);
     float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
-    if (training) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
+    if (training && !direct) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
     {
-        LaunchScope scope("bn_finalize_forward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        const int alone = finalize_alone(g, st) ? 1 : 0;
+        LaunchScope scope("bn_finalize_forward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 4 : 0));
+        const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
         const uint32_t per_block = alone ? kBlock : kBlock / 64;
         hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
                            si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params, soa, pitch, alone);
@@ -678,7 +717,8 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     // The two sums feed gradGamma, gradBeta and the training-mode input gradient; the
     // inference-mode input gradient does not use them.
     const bool need_sums = training || gg != nullptr || gb != nullptr;
-    const StatsLaunch st = need_sums ? plan_stats(g) : StatsLaunch{};
+    const bool direct = need_sums && stats_direct(g);
+    const StatsLaunch st = need_sums && !direct ? plan_stats(g) : StatsLaunch{};
     const uint32_t pitch = (g.channels + 3u) & ~3u;
     const uint64_t aos_bytes = align256(static_cast<uint64_t>(g.channels) * sizeof(BackwardParams));
     const uint64_t params_bytes = aos_bytes + align256(5ull * pitch * sizeof(float));
@@ -689,13 +729,13 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     BackwardParams* params = reinterpret_cast<BackwardParams*>(ws);
     float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
-    if (need_sums) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
+    if (need_sums && !direct) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
     {
-        LaunchScope scope("bn_finalize_backward_kernel", "", static_cast<uint64_t>(g.channels) * 32);
-        const int alone = finalize_alone(g, st) ? 1 : 0;
+        LaunchScope scope("bn_finalize_backward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 8 : 0));
+        const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
         const uint32_t per_block = alone ? kBlock : kBlock / 64;
         hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
-                           partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch, alone);
+                           si->ptr, sg ? sg->ptr : nullptr, partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch, alone);
     }
     if (sgi) {
         if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
