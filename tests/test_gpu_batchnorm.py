@@ -46,7 +46,10 @@ LAYOUTS = [([10, 3, 4, 5], 1), ([8, 16, 32, 32], 1), ([4, 6, 67], 1), ([4, 5, 25
            ([20, 12, 13, 13], 1), ([7, 8, 65], 1), ([5, 4, 66], 1), ([3, 5, 71], 1), ([1000, 256], 1), ([33, 4, 7, 12], 3),
            # a matrix of 16, 6, 48 and 3 columns under many rows (the workgroup's threads over several rows at a time), and
            # 20 000 channels of 3 and 12 items (a thread per channel folds them)
-           ([30000, 16], 1), ([5000, 2, 3], 1), ([7000, 48], 1), ([9001, 3], 1), ([3, 20000], 1), ([20000, 12], 0)]
+           ([30000, 16], 1), ([5000, 2, 3], 1), ([7000, 48], 1), ([9001, 3], 1), ([3, 20000], 1), ([20000, 12], 0),
+           # at most 32 items per channel and 16 384 channels or more: no statistics launch, the finalize sums the items
+           # (32 items: the last such shape; 33: the statistics launch again; items of an inner dim under an outer one)
+           ([32, 16384], 1), ([33, 16384], 1), ([2, 17000, 3], 1), ([5, 16390], 1), ([16385, 2], 0)]
 
 
 @pytest.mark.parametrize("affine,running", [(True, True), (False, False)])
