@@ -103,7 +103,7 @@ def test_training_mode_parity(shape, axis, affine, running, gc):
     assert np.abs(ggin.toArray() - cgin.toArray()).max() <= 2e-5 * scale, "gradIn against the checker end to end"
 
 
-@pytest.mark.parametrize("shape,axis", [([10, 3, 4, 5], 2), ([8, 16, 32, 32], 1), ([512, 40], 1), ([4, 6, 67], 1)],
+@pytest.mark.parametrize("shape,axis", [([10, 3, 4, 5], 2), ([8, 16, 32, 32], 1), ([512, 40], 1), ([4, 6, 67], 1), ([3, 20000], 1), ([17000, 2, 2], 0)],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else f"axis{v}")
 def test_inference_mode_is_bit_exact(shape, axis, gc):
     """No reduction feeds the inference output or input gradient, so they match the checker
