@@ -441,11 +441,11 @@ struct BcastPlan {
     bool     a_stream, b_stream;     // operand has as many elements as the output
     // Tile order of the vector kernel. 0: tiles in the order of the output. Otherwise the output is `repeats` slices of
     // `slice` units (the dims inside some dim along which an operand repeats; that dim and those outside it number the
-    // slices), a slice is cut into chunks of 1 << chunk_shift tiles, and the tiles run chunk by chunk: the chunk of slice 0,
+    // slices), a slice is cut into equal chunks of chunk_tiles tiles, and the tiles run chunk by chunk: the chunk of slice 0,
     // the same chunk of slice 1, ... Each XCD takes a contiguous share of that sequence, so that the part of an operand
     // which one slice shares with the next is read from memory once and found in the XCD's L2 by the slices that follow.
-    uint32_t repeats, slice, slice_tiles, tiles, per_xcd, chunk_shift;
-    FastDiv  group_div;              // by repeats << chunk_shift
+    uint32_t repeats, slice, slice_tiles, tiles, per_xcd, chunk_tiles;
+    FastDiv  group_div, chunk_div;   // by repeats * chunk_tiles, by chunk_tiles
 };
 
 __device__ __forceinline__ void decompose(const BcastPlan& pl, uint32_t idx, uint32_t& aoff, uint32_t& boff) {
@@ -484,9 +484,9 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* _
         const uint32_t t = (blockIdx.x & 7u) * pl.per_xcd + (blockIdx.x >> 3);
         if (t >= pl.tiles) return;
         const uint32_t chunk = (__umulhi(t, pl.group_div.mul) + t) >> pl.group_div.shift;
-        const uint32_t in_group = t - ((chunk * pl.repeats) << pl.chunk_shift);
-        const uint32_t rep = in_group >> pl.chunk_shift;
-        const uint32_t tile = (chunk << pl.chunk_shift) + (in_group & ((1u << pl.chunk_shift) - 1u));
+        const uint32_t in_group = t - chunk * pl.repeats * pl.chunk_tiles;
+        const uint32_t rep = (__umulhi(in_group, pl.chunk_div.mul) + in_group) >> pl.chunk_div.shift;
+        const uint32_t tile = chunk * pl.chunk_tiles + (in_group - rep * pl.chunk_tiles);
         if (tile >= pl.slice_tiles) return;                  // the last chunk of a slice may be short
         const uint32_t inner = tile * kBcastTile + threadIdx.x;
         base = rep * pl.slice + inner;
@@ -903,14 +903,19 @@ void order_tiles_for_reuse(BcastPlan* plan, uint32_t n4, dim3* grid) {
     }
     if (!pays || from_slice == 0) return;
     // with both operands repeating, the slices between two uses of a tile bring their own tiles of the other operand
-    const uint32_t shift = (a_in_group && b_in_group) ? kReuseChunkShift - 1 : kReuseChunkShift;
+    const uint64_t longest = 1ull << ((a_in_group && b_in_group) ? kReuseChunkShift - 1 : kReuseChunkShift);
     const uint64_t repeats = n4 / from_slice;
     const uint64_t slice_tiles = (from_slice + kBcastTile - 1) / kBcastTile;
-    const uint64_t tiles = (((slice_tiles + (1u << shift) - 1) >> shift) << shift) * repeats;
-    if (repeats < 6 || tiles > 0xfffffff0ull || (repeats << shift) > 0x7fffffffull) return;      // 4 repeats of 64 MB: 117 us against 115
+    // chunks of equal length, so that the slots past a slice's last tile are few and spread evenly (a last chunk of
+    // 15 tiles out of 32 left the XCDs that took it idle for an eighth of the launch)
+    const uint64_t chunks = (slice_tiles + longest - 1) / longest;
+    const uint64_t chunk_tiles = (slice_tiles + chunks - 1) / chunks;
+    const uint64_t tiles = chunks * chunk_tiles * repeats;
+    if (repeats < 6 || tiles > 0xfffffff0ull) return;        // 4 repeats of 64 MB: 117 us against 115
     plan->repeats = static_cast<uint32_t>(repeats);
-    plan->chunk_shift = shift;
-    plan->group_div = make_div(plan->repeats << shift);
+    plan->chunk_tiles = static_cast<uint32_t>(chunk_tiles);
+    plan->chunk_div = make_div(plan->chunk_tiles);
+    plan->group_div = make_div(static_cast<uint32_t>(repeats * chunk_tiles));
     plan->slice = static_cast<uint32_t>(from_slice);
     plan->slice_tiles = static_cast<uint32_t>(slice_tiles);
     plan->tiles = static_cast<uint32_t>(tiles);

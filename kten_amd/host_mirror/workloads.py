@@ -241,6 +241,25 @@ def _bytes_cat(d):
     return 4 * (2 * n + 2 * n + (d["left"] + d["right"]) + 2 * lb + la)
 
 
+# ---- broadcast of operands that repeat and are too large for one L2 -------------------------------
+
+def _in_reuse(d):
+    g = SplitMix64(16)
+    return {"x": g.uniform([d["n"], d["t"], d["h"]], -1.0, 1.0), "y": g.uniform([1, d["t"], d["h"]], -1.0, 1.0),
+            "a": g.uniform([1, d["q"], d["r"], d["s"]], -1.0, 1.0), "b": g.uniform([d["p"], 1, d["r"], d["s"]], -1.0, 1.0)}
+
+
+def _run_reuse(ops, inp):
+    t = {k: ops.create(list(v.shape), False, v) for k, v in inp.items()}
+    return {"sum": t["x"] + t["y"], "product": t["a"] * t["b"]}
+
+
+def _bytes_reuse(d):
+    x, y = d["n"] * d["t"] * d["h"], d["t"] * d["h"]
+    a, b, out = d["q"] * d["r"] * d["s"], d["p"] * d["r"] * d["s"], d["p"] * d["q"] * d["r"] * d["s"]
+    return 4 * (2 * x + y + a + b + out)
+
+
 # ---- fused batch normalisation ------------------------------------------------------------------
 
 def _in_bn(d):
@@ -474,6 +493,9 @@ WORKLOADS: Dict[str, Workload] = {
                           _in_tr, _run_tr, _bytes_tr),
     "permute": Workload("permute", "x.permute(0,2,3,1) then .permute(0,3,1,2): NCHW [64,128,56,56] to NHWC and back, seed 8",
                         {"n": 64, "c": 128, "h": 56, "w": 56}, _in_perm, _run_perm, _bytes_perm),
+    "broadcast_reuse": Workload("broadcast_reuse", "x[32,2047,1020] + y[1,2047,1020] and a[1,6,4,56860] * b[23,1,4,56860]: operands of 8 MB and "
+                                                   "5-21 MB that repeat along a dim, in shapes that are multiples of nothing; U(-1,1), seed 16",
+                                {"n": 32, "t": 2047, "h": 1020, "p": 23, "q": 6, "r": 4, "s": 56860}, _in_reuse, _run_reuse, _bytes_reuse),
     "concat_mask": Workload("concat_mask", "concat([8192,4096],[8192,4096], axis=1); maskedFill(mask[8192], 0); range get "
                                            "of the right half; range fill of the left half; seed 9",
                             {"rows": 8192, "left": 4096, "right": 4096}, _in_cat, _run_cat, _bytes_cat),

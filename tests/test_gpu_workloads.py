@@ -209,6 +209,20 @@ def test_cfg5_full(gc):
     assert abs(float(got["loss"][0]) - loss_ref) <= 1e-5 * loss_ref
 
 
+@pytest.mark.parametrize("dims", [{"n": 7, "t": 400, "h": 1020, "p": 6, "q": 3, "r": 4, "s": 40000}, None], ids=["small", "full"])
+def test_broadcast_reuse(dims, gc):
+    """Broadcast binary ops whose repeating operand is megabytes large (the tiles of the output are then ordered for
+    reuse in L2): bit for bit against numpy's broadcasting."""
+    wl = WORKLOADS["broadcast_reuse"]
+    inp = wl.make_inputs(dims or wl.full_dims)
+    gc.profileBegin()
+    out = wl.run(gc, inp)
+    launched = " ".join(gc.profileEnd().keys())
+    assert "_chunked" in launched, launched
+    assert_bits_equal(out["sum"].toArray(), inp["x"] + inp["y"], "x + y")
+    assert_bits_equal(out["product"].toArray(), inp["a"] * inp["b"], "a * b")
+
+
 def _check_reduce_shapes(inp, got, scale):
     for i, (shape, axis, op) in enumerate(reduce_shapes_at({"scale": scale})):
         x = inp[f"x{i}"]
