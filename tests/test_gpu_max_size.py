@@ -302,6 +302,30 @@ def test_sorted_and_wave_scatter_near_the_limit(gc):
         gc.release(y)
 
 
+def test_broadcast_with_a_large_repeating_operand_near_the_limit(gc):
+    """x[i, j, k] = r[i] + y[j, k] on [64, 4095, 8188] (2 145 911 040 elements) with y of 134 MB repeating along the outermost
+    dim: the vector kernel takes the output's tiles chunk by chunk across the 64 repeats; then z = x + y with one operand
+    full-size. Values are multiples of 1/8: every sum is exact."""
+    A, B, C = 64, 4095, 8188
+    rng = np.random.default_rng(8)
+    r = (rng.integers(-512, 512, A) / 8.0).astype(np.float32)
+    y = (rng.integers(-512, 512, (B, C)) / 8.0).astype(np.float32)
+    gr, gy = gc.createRaw([A, 1, 1], r), gc.createRaw([1, B, C], y)
+    gc.profileBegin()
+    x = gr.plus(gy)
+    z = x.plus(gy)
+    launched = " ".join(gc.profileEnd().keys())
+    assert launched.count("_chunked") == 2, launched
+    pos = [(0, 0, 0), (A - 1, B - 1, C - 1), (A - 1, 0, 0), (0, B - 1, C - 1), (A - 1, B - 1, 0), (31, 2047, 4093)]
+    pos += [(int(rng.integers(0, A)), int(rng.integers(0, B)), int(rng.integers(0, C))) for _ in range(60)]
+    for i, j, k in pos:
+        assert x.getSingleValue([i, j, k]) == r[i] + y[j, k]
+        assert z.getSingleValue([i, j, k]) == r[i] + y[j, k] + y[j, k]
+    # the last rows of the last slice, whole: the tiles that end with the slice and with the tensor
+    tail = z.get([(A - 1, A - 1), (B - 2, B - 1), ALL]).toArray().reshape(2, C)
+    assert np.array_equal(tail, r[-1] + 2 * y[-2:, :])
+
+
 def test_odd_shaped_tensor_near_the_limit(gc):
     """x[i, j] = r[i] + c[j] on [46339, 46337] (2 147 210 243 elements, rows that start off 16-byte boundaries):
     the forms the kernels take when nothing is a multiple of four -- element gathers in the broadcast, rows read
