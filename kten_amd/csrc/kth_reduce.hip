@@ -631,6 +631,9 @@ void plan_segments(Geom* g, uint64_t base_blocks, uint64_t target, uint32_t quan
     // Cutting the axis costs a second launch (about 4.5 us): only worth it when the
     // outputs alone leave more than half of the machine idle.
     uint32_t want = base_blocks * 2 > target ? 1u : ceil_div(target, base_blocks);
+    // ... and when a workgroup has more than a few passes over its share of the axis (a pass: `quantum` positions, eight
+    // loads in flight each, about a microsecond): six passes or fewer are over before a second launch would have started
+    if (ceil_div(g->axis, quantum * 8u) <= 6u) want = 1u;
     uint32_t max_seg = g->axis / min_len;
     if (max_seg < 1) max_seg = 1;
     if (want > max_seg) want = max_seg;

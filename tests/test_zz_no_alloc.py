@@ -88,18 +88,18 @@ def test_static_reduction_refuses_what_does_not_fit(gc):
     size = ctypes.c_uint64()
     check(gc.lib.kth_reduce_scratch_bytes(ctypes.byref(size)))
     assert size.value == 4 << 20
-    # [128, 200000] over axis 0: 782 column tiles are cut into 3 axis segments -> 200000 * 3 * 8 bytes of partials
-    shape = [128, 200000]
+    # [1024, 200000] over axis 0: 782 column tiles are cut into 3 axis segments -> 200000 * 3 * 8 bytes of partials
+    shape = [1024, 200000]
     t = gc.createRawFill(shape, 1.0)
     out = gc.createRawFill([1, 200000], -7.0)
     assert t.getSingleValue([0, 0]) == 1.0                    # the input is in memory, not a fill still to be launched
     launches = gc.getMetrics()["launches"]
-    rc = gc.lib.kth_reduce_axis_static(Op.SUM, t.storeReference, out.storeReference, 1, 128, 200000)
+    rc = gc.lib.kth_reduce_axis_static(Op.SUM, t.storeReference, out.storeReference, 1, 1024, 200000)
     assert rc == -3, "a plan beyond the scratch array must return KTH_E_ARGUMENT"
     msg = gc.lib.kth_last_error().decode()
     assert "static scratch" in msg and "4800000" in msg, msg
     assert gc.getMetrics()["launches"] == launches, "nothing may be launched for a refused shape"
     assert_bits_equal(out.toArray(), np.full([1, 200000], -7.0, dtype=np.float32), "output of a refused call")
     # the pooled entry point takes the same shape
-    check(gc.lib.kth_reduce_axis(Op.SUM, t.storeReference, out.storeReference, 1, 128, 200000))
-    assert_bits_equal(out.toArray(), np.full([1, 200000], 128.0, dtype=np.float32), "kth_reduce_axis on the refused shape")
+    check(gc.lib.kth_reduce_axis(Op.SUM, t.storeReference, out.storeReference, 1, 1024, 200000))
+    assert_bits_equal(out.toArray(), np.full([1, 200000], 1024.0, dtype=np.float32), "kth_reduce_axis on the refused shape")
