@@ -557,10 +557,14 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float*
                 if (!AL) gather4(a, ao0, pl.astride[0], va);
                 if (!BL) gather4(b, bo0, pl.bstride[0], vb);
             } else {
+                // ... they cross its end: the offsets step along dim 0 and are worked out anew only where it ends
+                uint32_t ao = ao0, bo = bo0, r = r0;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    uint32_t ao, bo;
-                    decompose(pl, e0 + j, ao, bo);
+                    if (j > 0) {
+                        if (++r == pl.size[0]) { r = 0; decompose(pl, e0 + j, ao, bo); }
+                        else { ao += pl.astride[0]; bo += pl.bstride[0]; }
+                    }
                     if (!AL) va[j] = a[ao];
                     if (!BL) vb[j] = b[bo];
                 }
