@@ -749,6 +749,90 @@ __global__ __launch_bounds__(WAVES * kWave) void index_add_long_runs_kernel(floa
     }
 }
 
+// The same long runs when the tensor has few positions beside the axis (a flat tensor: one): the kernel above gives a
+// position a lane and a run's entries to the lanes' registers one after the other, which leaves 63 lanes idle and costs a
+// barrier per 32 entries (9.1 ns an entry). Here a wave owns one (run, position): its lanes fetch 256 entries at a time
+// (the next 256 are on their way meanwhile), park them in LDS, and lane 0 reads them back 64 at a time as sixteen
+// 16-byte words and adds them in order. Nothing crosses a wave, so there is no barrier; the waves of a workgroup take different items.
+constexpr uint32_t kChainWaves = 4;
+constexpr uint32_t kChainPositions = 16;                  // positions up to which a run is taken this way
+__global__ __launch_bounds__(kChainWaves * kWave) void index_add_chain_kernel(float* __restrict__ target, const float* __restrict__ src,
+                                                                             const uint32_t* __restrict__ vals, LongRuns runs, float alpha,
+                                                                             uint32_t from_constant, float constant, uint32_t positions,
+                                                                             RowsPlan pl, FastDiv positions_div) {
+    constexpr uint32_t kDeep = 4;                            // batches of 64 entries in flight: a batch is added in less time than a gather takes
+    constexpr uint32_t kSpan = kDeep * kWave;
+    __shared__ __attribute__((aligned(16))) float staged[kChainWaves][kSpan];
+    const uint32_t lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    const uint64_t n_items = static_cast<uint64_t>(*runs.count) * positions;
+    for (uint64_t item = static_cast<uint64_t>(blockIdx.x) * kChainWaves + w; item < n_items; item += static_cast<uint64_t>(gridDim.x) * kChainWaves) {
+        const uint32_t it = static_cast<uint32_t>(item);                       // (runs * positions stays below 2^32: both are bounded by the entries)
+        const uint32_t slot = (__umulhi(it, positions_div.mul) + it) >> positions_div.shift;
+        const uint32_t p = it - slot * positions;
+        const uint32_t o = (__umulhi(p, pl.inner_div.mul) + p) >> pl.inner_div.shift;
+        const uint32_t col = p - o * pl.inner;
+        const uint32_t first = runs.start[slot], len = runs.len[slot], key = runs.key[slot];
+        float* t = target + (static_cast<size_t>(o) * pl.axis_len + key) * pl.inner + col;
+        const float* s = src + static_cast<size_t>(o) * pl.k * pl.inner + col;
+        float acc = from_constant ? constant : *t;
+        constexpr uint32_t kNone = 0xffffffffu;
+        auto row_at = [&](uint32_t at) -> uint32_t { return at < len ? vals[first + at] : kNone; };
+        auto value_of = [&](uint32_t row) -> float { return row != kNone ? __builtin_nontemporal_load(s + static_cast<size_t>(row) * pl.inner) : 0.0f; };
+        uint32_t row_next[kDeep];
+        float v_next[kDeep];
+#pragma unroll
+        for (uint32_t d = 0; d < kDeep; d++) row_next[d] = row_at(d * kWave + lane);
+#pragma unroll
+        for (uint32_t d = 0; d < kDeep; d++) v_next[d] = value_of(row_next[d]);
+#pragma unroll
+        for (uint32_t d = 0; d < kDeep; d++) row_next[d] = row_at(kSpan + d * kWave + lane);
+        for (uint32_t base = 0; base < len; base += kSpan) {
+#pragma unroll
+            for (uint32_t d = 0; d < kDeep; d++) staged[w][d * kWave + lane] = v_next[d] * alpha;
+#pragma unroll
+            for (uint32_t d = 0; d < kDeep; d++) v_next[d] = value_of(row_next[d]);
+#pragma unroll
+            for (uint32_t d = 0; d < kDeep; d++) row_next[d] = row_at(base + 2 * kSpan + d * kWave + lane);
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");               // the wave's stores before lane 0's loads
+            __builtin_amdgcn_wave_barrier();
+            if (lane == 0) {
+#pragma unroll
+                for (uint32_t d = 0; d < kDeep; d++) {
+                    const uint32_t at = base + d * kWave;
+                    if (at + kWave <= len) {
+                        const float4* q = reinterpret_cast<const float4*>(staged[w] + d * kWave);
+                        float4 f[kWave / 4];
+#pragma unroll
+                        for (uint32_t j = 0; j < kWave / 4; j++) f[j] = q[j];
+#pragma unroll
+                        for (uint32_t j = 0; j < kWave / 4; j++) { acc = acc + f[j].x; acc = acc + f[j].y; acc = acc + f[j].z; acc = acc + f[j].w; }
+                    } else if (at < len) {
+                        for (uint32_t j = 0; j < len - at; j++) acc = acc + staged[w][d * kWave + j];
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");               // ... and its loads before the next stores
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (lane == 0) *t = acc;
+    }
+}
+
+// Launches the kernel that takes the listed long runs: by waves of their own when the positions are few.
+static void launch_long_runs(dim3 long_grid, uint64_t long_items, hipStream_t stream, float* target, const float* src, const uint32_t* vals,
+                             const LongRuns& runs, float alpha, uint32_t from_constant, float constant, uint32_t positions, const RowsPlan& pl) {
+    if (positions <= kChainPositions) {
+        const uint64_t waves = long_items * positions;
+        const uint64_t most = 8ull * static_cast<uint64_t>(state().compute_units);
+        const dim3 grid(static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>((waves + kChainWaves - 1) / kChainWaves, most))));
+        hipLaunchKernelGGL(index_add_chain_kernel, grid, dim3(kChainWaves * kWave), 0, stream, target, src, vals, runs, alpha, from_constant, constant,
+                           positions, pl, make_div(positions));
+        return;
+    }
+    hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, target, src, vals, runs, alpha,
+                       from_constant, constant, positions, pl);
+}
+
 
 // ---- scatter through a sorted list of its entries -----------------------------------------
 // A scatter with few positions and long index rows (a flat tensor, a long axis next to a handful of columns) gives
@@ -1273,8 +1357,7 @@ static int scatter_sorted(int mode, float* target, const int32_t* target_shape, 
         }
         if (long_items > 0) {
             LaunchScope scope("index_add_long_runs_kernel", "scatter", 0);
-            hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, target, psrc, vals_sorted, runs, 1.0f,
-                               0u, 0.0f, 1u, pl);
+            launch_long_runs(long_grid, long_items, stream, target, psrc, vals_sorted, runs, 1.0f, 0u, 0.0f, 1u, pl);
         }
     });
     workspace_release(reinterpret_cast<float*>(keys), cap);
@@ -1556,8 +1639,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
             }
             if (long_items > 0) {
                 LaunchScope scope("index_add_long_runs_kernel", "from a constant", 0);
-                hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 1u, constant,
-                                   static_cast<uint32_t>(positions), long_pl);
+                launch_long_runs(long_grid, long_items, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 1u, constant, static_cast<uint32_t>(positions), long_pl);
             }
         });
         workspace_release(reinterpret_cast<float*>(keys), cap);
@@ -1597,8 +1679,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
         }
         if (long_items > 0) {
             LaunchScope scope("index_add_long_runs_kernel", "", 0);
-            hipLaunchKernelGGL((index_add_long_runs_kernel<kLongWaves, kLongEntries>), long_grid, dim3(kLongWaves * kWave), 0, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 0u, 0.0f,
-                               static_cast<uint32_t>(positions), long_pl);
+            launch_long_runs(long_grid, long_items, stream, st->ptr, ss->ptr, vals_sorted, runs, alpha, 0u, 0.0f, static_cast<uint32_t>(positions), long_pl);
         }
     });
     workspace_release(reinterpret_cast<float*>(keys), cap);

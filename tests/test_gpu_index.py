@@ -315,7 +315,10 @@ LONG_RUN_CASES = [([7], 0, 300, 0.9), ([40], 0, 20000, 0.5), ([5, 64], 0, 2000, 
                   ([3, 1023], 0, 1500, 0.0), ([2, 6, 3], 1, 4000, 0.4), ([3, 50, 8], 1, 30000, 0.7), ([64, 1], 0, 100000, 0.25),
                   ([1, 100], 0, 255, 0.0), ([1, 100], 0, 256, 0.0), ([1, 100], 0, 257, 0.0), ([1, 100], 0, 511, 0.0), ([1, 100], 0, 512, 0.0),
                   ([1, 100], 0, 513, 0.0), ([1, 100], 0, 1024, 0.0), ([1, 100], 0, 1025, 0.0), ([1, 100], 0, 1056, 0.0), ([2, 4], 0, 1537, 0.0),
-                  ([1000, 128], 0, 60000, 0.5), ([12, 2048], 0, 12000, 0.1)]
+                  ([1000, 128], 0, 60000, 0.5), ([12, 2048], 0, 12000, 0.1),
+                  # few positions beside the axis: a wave per (run, position), 64 entries at a time; run lengths around the multiples of 64
+                  ([1, 2], 0, 256, 0.0), ([1, 2], 0, 257, 0.0), ([1, 2], 0, 319, 0.0), ([1, 2], 0, 320, 0.0), ([1, 2], 0, 321, 0.0), ([1], 0, 1025, 0.0),
+                  ([2, 1, 16], 1, 700, 0.0), ([3, 16], 0, 50000, 0.6), ([3, 17], 0, 50000, 0.6), ([9], 0, 300000, 0.8), ([2, 5, 2], 1, 70000, 0.5)]
 
 
 @pytest.mark.parametrize("shape,axis,k,hot", LONG_RUN_CASES, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
