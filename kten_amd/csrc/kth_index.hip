@@ -749,13 +749,13 @@ __global__ __launch_bounds__(WAVES * kWave) void index_add_long_runs_kernel(floa
     }
 }
 
-// The same long runs when the tensor has few positions beside the axis (a flat tensor: one): the kernel above gives a
+// The same long runs when the tensor has one or two positions beside the axis (a flat tensor: one): the kernel above gives a
 // position a lane and a run's entries to the lanes' registers one after the other, which leaves 63 lanes idle and costs a
 // barrier per 32 entries (9.1 ns an entry). Here a wave owns one (run, position): its lanes fetch 256 entries at a time
 // (the next 256 are on their way meanwhile), park them in LDS, and lane 0 reads them back 64 at a time as sixteen
 // 16-byte words and adds them in order. Nothing crosses a wave, so there is no barrier; the waves of a workgroup take different items.
 constexpr uint32_t kChainWaves = 4;
-constexpr uint32_t kChainPositions = 16;                  // positions up to which a run is taken this way
+constexpr uint32_t kChainPositions = 2;                   // positions up to which a run is taken this way (with 8 or 16 and many runs the 4-byte fetches cost more than the barriers: [1024,16] with 2 million rows 437 us against 101)
 __global__ __launch_bounds__(kChainWaves * kWave) void index_add_chain_kernel(float* __restrict__ target, const float* __restrict__ src,
                                                                              const uint32_t* __restrict__ vals, LongRuns runs, float alpha,
                                                                              uint32_t from_constant, float constant, uint32_t positions,
