@@ -15,13 +15,16 @@ op-at-a-time total of the reference's op list (operands at their un-broadcast si
 once) and what the library's launches of that step really read and wrote. The second is smaller
 where a tensor that is one constant (a fresh zerosLike, the broadcast seed gradient) is never
 written out and read back; bytes that did not cross the memory bus are not counted as bandwidth.
-`config` carries both totals and both rates.
+`config` carries both totals.
 
-Timing: a HIP event on the library's own stream before the first and after every one of the K
-timed steps (kth_timer_lap): `value` comes from the time between the first and the last event,
-median and minimum from the steps' own intervals; a host-side wall clock around the same region
-is the cross-check. Per-kernel durations come from HIP event pairs the library records around
-every launch over a second pass of the same K steps (kth_profile_*).
+Timing: W warm-up steps, then exactly K steps between two HIP events on the library's own stream
+(kth_timer_begin / kth_timer_end): `value` and `ms_per_step` come from that region; a host-side wall
+clock around it is the cross-check. Median and minimum come from a second pass of K steps with an
+event after every step (kth_timer_lap; each such event costs the stream about 2 us, so the pass with
+them is not the one `value` is taken from). Per-kernel durations come from HIP event pairs the
+library records around every launch over a third pass of the same K steps (kth_profile_*).
+With the default workload the other BASELINE configurations (cfg1-cfg4) are timed the same way after
+it and reported under config.other_configs.
 
 Two context figures are measured in the same run: the device-to-device copy rate of this GPU
 (`roofline.copy_ceiling`, hipMemcpyAsync and the library's copy kernel on 1 GiB), and the
@@ -58,7 +61,8 @@ def log(*a):
 
 
 def make_step(name, ops, inputs):
-    """Returns a zero-argument callable running one pass of the workload on resident inputs."""
+    """Returns a zero-argument callable running one pass of the workload on resident inputs, and the
+    resident tensors (to be released by the caller when the workload is done)."""
     from kten_amd.host_mirror.workloads import WORKLOADS, cfg5_setup, cfg5_step
     wl = WORKLOADS[name]
     if name == "cfg5":
@@ -68,7 +72,7 @@ def make_step(name, ops, inputs):
 
         def step():
             return cfg5_step(x, w, b)          # backward() opens its own garbage-collector scope
-        return step
+        return step, [x, w, b]
     if name in ("max_backward", "softmax_ce"):
         # Leaves are created once; the step is graph + backward, gradients zeroed in between.
         first = "x" if name == "max_backward" else "logits"
@@ -79,7 +83,7 @@ def make_step(name, ops, inputs):
             out = leaf.max(-1).sum() if other is None else leaf.softmaxCrossEntropy(other)
             out.backward()
             return out
-        return step
+        return step, [t for t in (leaf, other) if t is not None]
     resident = {k: ops.createRaw(list(v.shape), v) for k, v in inputs.items()}
     for r in resident.values():
         r.incrementRef()
@@ -102,7 +106,7 @@ def make_step(name, ops, inputs):
     def step():
         with ops.garbageCollector():
             return wl.run(proxy, inputs)
-    return step
+    return step, list(resident.values())
 
 
 def cold_probe(ops, kernel, nbytes_per_launch, dims, sets=8, rounds=3):
@@ -172,6 +176,33 @@ def cold_probe(ops, kernel, nbytes_per_launch, dims, sets=8, rounds=3):
     return ms / launches * 1e3 if launches else None
 
 
+def launch_floor(ops):
+    """What one more tiny launch costs the stream when it is queued behind running work: the time of three full-size
+    maps followed by k launches on 4096 floats, k = 0 and 16, divided out. No profiler and no event between the
+    launches (an event pair or a tracer adds about 2.5 us to every back-to-back launch)."""
+    import ctypes
+    import numpy as np
+    from kten_amd import abi
+    from kten_amd.abi import Op, check
+    lib = ops.lib
+    n = 1 << 26
+    with ops.garbageCollector():
+        big, big2 = ops.createRaw([n]), ops.createRaw([n])
+        check(lib.kth_fill(big.storeReference, 0, n, 1.5))
+        a, b, c = (ops.createRaw([4096], np.full(4096, 0.25 * (i + 1), dtype=np.float32)) for i in range(3))
+        sh = abi.shape_array([4096])
+        best = {}
+        for k in (0, 16, 0, 16, 0, 16):
+            ops.sync()
+            ops.timerBegin()
+            for _ in range(3):
+                check(lib.kth_unary(Op.NEG, big.storeReference, big2.storeReference, n))
+            for _ in range(k):
+                check(lib.kth_binary(Op.PLUS, a.storeReference, sh, 1, b.storeReference, sh, 1, c.storeReference, sh, 1))
+            best[k] = min(best.get(k, 1e9), ops.timerEnd() * 1e3)
+    return (best[16] - best[0]) / 16
+
+
 def cpu_baseline(name, threads):
     """The CPU restatement of kten-jvm on a bounded sample of the same workload."""
     from kten_amd.host_mirror.workloads import WORKLOADS
@@ -198,6 +229,82 @@ def cpu_baseline(name, threads):
                       f"reference, in-place ops and axis reductions on {threads} threads"}
 
 
+def jvm_probe():
+    """Whether the reference's own toolchain exists on this host: with it, kten-jvm itself could be timed beside the
+    C restatement; without it the restatement is the only CPU baseline. Nothing is installed or run."""
+    import shutil
+    return {tool: shutil.which(tool) for tool in ("java", "kotlinc", "mvn")}
+
+
+def time_steps(ops, step, steps, warmup):
+    """W untimed steps, then exactly K steps between two HIP events on the library's stream, with a host wall clock
+    around the same region and the stream drained on both sides: `ms_per_step` comes from that region alone. Median
+    and minimum come from a second pass of K steps with an event after every step (an event costs the stream about
+    2 us, which the first region therefore does not contain)."""
+    for _ in range(warmup):
+        step()
+    ops.sync()
+    m0 = ops.getMetrics()
+    wall0 = time.perf_counter()
+    ops.timerBegin()
+    for _ in range(steps):
+        step()
+    issued_ms = (time.perf_counter() - wall0) * 1e3          # the host has issued everything; the stream may still be running
+    total_ms = ops.timerEnd()                                # waits for the closing event
+    ops.sync()
+    wall_ms = (time.perf_counter() - wall0) * 1e3
+    m = ops.getMetrics()
+    ops.timerLap()
+    for _ in range(steps):
+        step()
+        ops.timerLap()
+    laps, _ = ops.timerLaps()
+    ops.sync()
+    laps.sort()
+    median_ms = laps[len(laps) // 2] if len(laps) % 2 else 0.5 * (laps[len(laps) // 2 - 1] + laps[len(laps) // 2])
+    return {"ms_per_step": total_ms / steps, "median_ms": median_ms, "min_ms": laps[0], "wall_ms": wall_ms / steps,
+            "host_issue_ms": issued_ms / steps,
+            "moved": (m["bytesMoved"] - m0["bytesMoved"]) / steps, "launches": (m["launches"] - m0["launches"]) / steps}
+
+
+def kernel_events(ops, step, steps):
+    """The same K steps again with a HIP event pair around every launch: {kernel: (launches, bytes, ms)}. Kept out of
+    the region `value` is computed from, because the event pairs themselves cost about a tenth of the step time."""
+    ops.profileBegin()
+    ops.timerBegin()
+    for _ in range(steps):
+        step()
+    ev_ms = ops.timerEnd()
+    return ops.profileEnd(), ev_ms
+
+
+def other_config(ops, name, steps, warmup):
+    """One of the other BASELINE configurations for the same steps / warm-up: its step rate and its largest kernel."""
+    from kten_amd.host_mirror.workloads import WORKLOADS
+    wl = WORKLOADS[name]
+    dims = wl.full_dims
+    nbytes = wl.algorithmic_bytes(dims)
+    inputs = wl.make_inputs(dims)
+    step, resident = make_step(name, ops, inputs)
+    r = time_steps(ops, step, steps, warmup)
+    kernels, _ = kernel_events(ops, step, steps)
+    for t in resident:
+        t.release()
+    ops.sync()
+    counted = min(nbytes, r["moved"])
+    gbps = counted / r["ms_per_step"] / 1e6
+    dom, (n, b, ms) = max(kernels.items(), key=lambda kv: kv[1][2])
+    log(f"{name}: {r['ms_per_step']:.4f} ms/step mean ({r['median_ms']:.4f} median, {r['min_ms']:.4f} min), {gbps:.0f} GB/s "
+        f"({100 * gbps / HBM_PEAK_GBPS:.1f} % of peak), host issue {r['host_issue_ms']:.4f} ms/step; largest kernel {dom} {ms / n * 1e3:.1f} us")
+    return {"workload": wl.description, "algorithmic_bytes_per_step": nbytes, "moved_bytes_per_step": round(r["moved"]),
+            "launches_per_step": r["launches"],
+            "ms_per_step": round(r["ms_per_step"], 4), "ms_per_step_median": round(r["median_ms"], 4), "ms_per_step_min": round(r["min_ms"], 4),
+            "host_issue_ms_per_step": round(r["host_issue_ms"], 4),
+            "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+            "dominant_kernel": dom, "dominant_avg_launch_us": round(ms / n * 1e3, 2), "dominant_GBps": round(b / ms / 1e6, 1),
+            "dominant_frac": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -214,10 +321,16 @@ def main():
                     help="skip the dominant kernel's run over a rotation of untouched buffer sets")
     ap.add_argument("--no-copy-ceiling", dest="ceiling", action="store_false", default=True,
                     help="skip the device-to-device copy measurement")
+    ap.add_argument("--other-configs", dest="others", action="store_true", default=None,
+                    help="after the headline workload, run cfg1-cfg4 for the same steps and warm-up and report them under "
+                         "config.other_configs (the default when the headline is cfg5)")
+    ap.add_argument("--no-other-configs", dest="others", action="store_false")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this backend drives one GPU; the hot path has no cross-GPU step. Run with --gpus 1.")
         sys.exit(2)
+    if args.others is None:
+        args.others = args.config == "cfg5"
 
     import kten_amd
     from kten_amd.host_mirror.workloads import WORKLOADS
@@ -230,49 +343,22 @@ def main():
     t0 = time.perf_counter()
     inputs = wl.make_inputs(dims)
     log(f"inputs generated in {time.perf_counter() - t0:.1f} s")
-    step = make_step(args.config, ops, inputs)
+    step, resident = make_step(args.config, ops, inputs)
 
-    for _ in range(args.warmup):
-        step()
-    ops.sync()
-    m0 = ops.getMetrics()
-    # Timed region: exactly K steps between two events on the library's stream, with a
-    # host wall clock around the same region (stream drained on both sides).
-    wall0 = time.perf_counter()
-    ops.timerLap()
-    for _ in range(args.steps):
-        last = step()
-        ops.timerLap()
-    laps, total_ms = ops.timerLaps()
-    ops.sync()
-    wall_ms = (time.perf_counter() - wall0) * 1e3
-    laps.sort()
-    median_ms = laps[len(laps) // 2] if len(laps) % 2 else 0.5 * (laps[len(laps) // 2 - 1] + laps[len(laps) // 2])
-    min_ms = laps[0]
-    m = ops.getMetrics()
-    counted = (m["bytesMoved"] - m0["bytesMoved"]) / args.steps
-    launches = (m["launches"] - m0["launches"]) / args.steps
-    ms_per_step = total_ms / args.steps
+    r = time_steps(ops, step, args.steps, args.warmup)
+    ms_per_step, median_ms, min_ms, wall_ms = r["ms_per_step"], r["median_ms"], r["min_ms"], r["wall_ms"]
+    counted, launches = r["moved"], r["launches"]
     # `value` never counts bytes that were not moved: where the library folds a constant tensor into its
     # consumer (no fill written, no operand read) its launches move less than the reference's op list names,
     # and the rate is taken on what they moved. Where they move more (transposed copies), the op list stands.
-    algorithmic_gbps = nbytes / ms_per_step / 1e6
     gbps = min(nbytes, counted) / ms_per_step / 1e6
-    log(f"{args.steps} steps: {total_ms:.3f} ms on the stream ({ms_per_step:.4f} ms/step mean, {median_ms:.4f} median, "
-        f"{min_ms:.4f} min), {wall_ms:.3f} ms wall; {launches:.0f} launches/step; "
+    log(f"{args.steps} steps: {ms_per_step * args.steps:.3f} ms on the stream ({ms_per_step:.4f} ms/step mean, {median_ms:.4f} median, "
+        f"{min_ms:.4f} min), {wall_ms:.4f} ms/step wall, host issue {r['host_issue_ms']:.4f} ms/step; {launches:.0f} launches/step; "
         f"library counted {counted:.0f} B/step (formula {nbytes})")
 
-    # Per-kernel durations: the same K steps again, now with a HIP event pair around
-    # every launch. Kept out of the region `value` is computed from, because the event
-    # pairs themselves cost about a tenth of the step time.
     kernels = {}
     if args.events:
-        ops.profileBegin()
-        ops.timerBegin()
-        for _ in range(args.steps):
-            step()
-        ev_ms = ops.timerEnd()
-        kernels = ops.profileEnd()
+        kernels, ev_ms = kernel_events(ops, step, args.steps)
         log(f"{args.steps} steps with per-launch events: {ev_ms:.3f} ms on the stream")
 
     roofline = None
@@ -302,6 +388,11 @@ def main():
             else:
                 roofline["achieved_cold"] = None
     if roofline is not None and args.ceiling:
+        floor_us = launch_floor(ops)
+        roofline["launch_floor_us"] = round(floor_us, 2)
+        roofline["launch_floor_means"] = ("stream time one more launch on 4096 floats adds when it is queued behind running kernels "
+                                          "(slope of 3 full-size maps + k tiny launches, k = 0 and 16; no events between them)")
+        log(f"one more tiny launch queued behind running work costs the stream {floor_us:.2f} us")
         d2d, own = ops.measureCopy(1 << 28, 10)
         roofline["copy_ceiling"] = {"hipMemcpyDtoD_GBps": round(d2d, 1), "copy_kernel_GBps": round(own, 1), "bytes_each_way": 1 << 30,
                                     "note": "read + written bytes over time, 10 copies of 1 GiB back to back on this GPU"}
@@ -320,25 +411,43 @@ def main():
                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
                    "moved_bytes_per_step": round(counted),
                    "GBps_on_moved_bytes": round(counted / ms_per_step / 1e6, 1),
-                   "GBps_on_the_op_list": round(algorithmic_gbps, 1),
                    "value_means": "min(algorithmic_bytes_per_step, moved_bytes_per_step) / ms_per_step. moved_bytes_per_step is what "
                                   "the library's launches of one step read and wrote, summed from their own byte counts; "
                                   "algorithmic_bytes_per_step is the op-at-a-time total of the reference's op list. The two differ "
                                   "where the library does not write out a tensor that is one constant (a fresh zerosLike, the "
                                   "broadcast seed gradient) and hands the constant to the consumer's kernel (fewer bytes moved: "
-                                  "GBps_on_the_op_list would count bytes that never crossed the memory bus, ms_per_step shows the "
-                                  "gain), and where it moves more than the op list names (transposed copies of a scatter along an "
-                                  "outer axis)",
-                   "wall_ms_per_step": round(wall_ms / args.steps, 4),
-                   "per_kernel_durations": "HIP event pair around every launch, over a second pass of the same K steps"
+                                  "the op-list total over time would count bytes that never crossed the memory bus and is not a "
+                                  "bandwidth; ms_per_step shows the gain), and where it moves more than the op list names "
+                                  "(transposed copies of a scatter along an outer axis)",
+                   "wall_ms_per_step": round(wall_ms, 4),
+                   "host_issue_ms_per_step": round(r["host_issue_ms"], 4),
+                   "host_issue_means": "wall time the host took to issue the K timed steps (Python mirror of the autograd layer + "
+                                       "ctypes), per step, before it waited for the stream: close to ms_per_step means that the "
+                                       "stream was waiting for the host at times",
+                   "median_and_min": "from a second pass of K steps with an event after every step",
+                   "per_kernel_durations": "HIP event pair around every launch, over a third pass of the same K steps"
                    if args.events else None},
         "roofline": roofline,
     }
+    if args.others:
+        for t in resident:
+            t.release()
+        ops.sync()
+        line["config"]["other_configs"] = {name: other_config(ops, name, args.steps, args.warmup)
+                                           for name in ("cfg1", "cfg2", "cfg3", "cfg4") if name != args.config}
+        line["config"]["other_configs_note"] = ("the other BASELINE configurations, same steps and warm-up, inputs resident: GBps = "
+                                                "min(algorithmic, moved) bytes / ms_per_step; dominant_* from an event pair around every "
+                                                "launch over a second pass (the pairs add about 2.5 us to a launch); no CPU baseline for them")
     if args.cpu:
         threads = min(16, os.cpu_count() or 1)
         log(f"timing the CPU restatement on {threads} threads of {os.cpu_count()} host cores ...")
         line["cpu_baseline"] = cpu_baseline(args.config, threads)
-        log(f"cpu baseline: {line['cpu_baseline']['value']} GB/s")
+        line["cpu_baseline"]["jvm_available"] = jvm_probe()
+        line["cpu_baseline"]["oracle_used"] = ("the C restatement (kind \"port\"): " + ("a JVM toolchain is on this host but the reference's Maven "
+                                               "dependencies are not, so kten-jvm itself was not built or timed"
+                                               if all(line["cpu_baseline"]["jvm_available"].values()) else
+                                               "java / kotlinc / mvn are not all present on this host, kten-jvm itself cannot be built or timed here"))
+        log(f"cpu baseline: {line['cpu_baseline']['value']} GB/s; jvm toolchain: {line['cpu_baseline']['jvm_available']}")
     print(json.dumps(line), flush=True)
 
 

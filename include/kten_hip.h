@@ -20,8 +20,8 @@
  *   - Shapes travel by value inside the kernel arguments; nothing is uploaded per launch.
  *   - All launches are asynchronous on one internal in-order stream. The only blocking
  *     calls are kth_upload (above 1 MiB), kth_download, kth_read_scalar, kth_contains_nan, kth_sync,
- *     kth_gather / kth_scatter / kth_scatter_fill (they report bad index values), kth_timer_end,
- *     kth_profile_end and kth_shutdown.
+ *     kth_gather / kth_scatter / kth_scatter_fill (they report bad index values) and
+ *     kth_shutdown.
  *   - Shape / argument errors are reported before anything is launched, as the
  *     reference throws IllegalArgumentException host-side before computing
  *     (JVM:89-93, ShapeFunctions.kt:187-201).
@@ -182,8 +182,11 @@ int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t 
 /* sum() / mean() (RAW:121-122; JVM:146-152) of n values into out[0]. op: KTH_SUM, KTH_MEAN. */
 int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
 
-/* kth_reduce_axis for callers that cannot allocate: code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference.
+/* kth_reduce_axis for callers that cannot allocate: tight serving loops, harnesses that forbid
+ * hipMalloc, hosts that keep device memory fixed while a HIP graph is being captured elsewhere in
+ * the process. It has no counterpart in the reference. (The library launches on its own internal
+ * stream, which a caller cannot put under capture: this entry point does not by itself make the
+ * reduction part of a caller's graph; it only guarantees that the call creates nothing.)
  * Same arguments, checks and results (bit for bit: the same kernels and the same plan) as
  * kth_reduce_axis, but the partials of a two-pass reduction go to a fixed array of
  * kth_reduce_scratch_bytes() = 4 MiB in the library's device code instead of a pool
@@ -191,12 +194,14 @@ int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out);
  * events (its launches are counted by kth_metrics but left out of a kth_profile recording).
  * A shape whose plan needs more partial bytes than the array holds (outputs x axis segments
  * x 8 bytes; only reductions whose outputs alone cannot fill the device are cut into
- * segments) returns KTH_E_ARGUMENT before any reduction kernel is launched; single-pass shapes of any
- * size are accepted. An input that is a noted constant (see kth_fill) has its fill launched first:
- * a kernel launch into the store's own memory, nothing is allocated for it. Every call on a device shares that device's array, which keeps the last
- * call's partials; nothing in it needs clearing because every partial is written before it is
- * read. The library's mutex and its one in-order stream keep calls of one process apart;
- * anything that made two such calls overlap on one GPU would race on the array. */
+ * segments) returns KTH_E_ARGUMENT before anything is launched, the fill an operand may still
+ * be owed included (see kth_fill); single-pass shapes of any size are accepted. In an accepted
+ * call an input that is a noted constant has its fill launched first: a kernel launch into the
+ * store's own memory, nothing is allocated for it. Every call on a device shares that device's
+ * array, which keeps the last call's partials; nothing in it needs clearing because every
+ * partial is written before it is read. The library's mutex and its one in-order stream keep
+ * calls of one process apart; anything that made two such calls overlap on one GPU would race
+ * on the array. */
 int kth_reduce_axis_static(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner);
 
 /* Size of that array in bytes. */
@@ -207,8 +212,9 @@ int kth_reduce_scratch_bytes(uint64_t* bytes);
 /* When the indexed moves below report an index value outside its axis. immediate != 0 (the default): every such
  * call waits for its own kernels and returns KTH_E_ARGUMENT itself, as the reference throws IllegalArgumentException
  * at the operation (JVM:238-239,345-346,494-496). immediate == 0: the calls do not wait; an out-of-range index sets a
- * flag on the device and the next blocking call (kth_sync, kth_download, kth_read_scalar) returns KTH_E_ARGUMENT in
- * its place, once. Either way the kernels skip the offending entry and the in-place target of a scatter or indexAdd has
+ * flag on the device and the next blocking call (kth_sync, kth_download, kth_read_scalar, kth_contains_nan) returns
+ * KTH_E_ARGUMENT in its place, once; what that call was asked for (the downloaded floats, the NaN answer) has been
+ * delivered all the same. Either way the kernels skip the offending entry and the in-place target of a scatter or indexAdd has
  * been updated by the entries before it (the JVM, too, has assigned those when it throws).
  * In immediate mode a call does not wait when its index store is known to hold only valid values: an earlier indexed
  * move checked it against an axis no longer than this one (or kth_reduce_axis wrote it as ARG_MAX / ARG_MIN positions
@@ -334,36 +340,6 @@ int kth_sync(void);
  * kernel launches so far, and the algorithmic bytes those launches moved (operands at
  * their un-broadcast size plus the output, 4 bytes each). Any pointer may be NULL. */
 int kth_metrics(uint64_t* live_bytes, uint64_t* pool_bytes, uint64_t* launches, uint64_t* bytes_moved);
-
-/* Device-side stopwatch on the internal stream (a HIP event pair), for benchmarks that
- * must time the stream the kernels run on. No counterpart in the reference, which has
- * no timing facility. kth_timer_end blocks until the second event completes. */
-int kth_timer_begin(void);
-int kth_timer_end(float* milliseconds);
-
-/* Lap timing on the internal stream, for benchmarks that report the spread of a repeated step. No
- * counterpart in the reference. kth_timer_lap records a HIP event (nothing blocks); kth_timer_laps waits for
- * the last one, writes the time between consecutive laps (count = laps - 1; at most `capacity` values are
- * written) and the time from the first lap to the last, and forgets the laps. */
-int kth_timer_lap(void);
-int kth_timer_laps(float* milliseconds, int capacity, int* count, float* total_ms);
-
-/* The device-to-device copy rate of this GPU, the practical ceiling a streaming kernel is measured against:
- * times `reps` copies of n_floats values (a multiple of 4) between two pool buffers, once with hipMemcpyAsync
- * and once with the library's own copy kernel, and returns the milliseconds per copy of each. Blocking; no
- * counterpart in the reference. */
-int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kernel_ms);
-
-/* Per-kernel device timing, for benchmarks that must attribute the time of a region to
- * the kernels in it. No counterpart in the reference. Between kth_profile_begin and
- * kth_profile_end every kernel launch is bracketed by a HIP event pair on the internal
- * stream; kth_profile_end blocks until those launches have finished. Afterwards
- * kth_profile_count gives the number of distinct kernels seen and kth_profile_entry the
- * name ("family<Op>"), launch count, algorithmic bytes and summed duration of one. */
-int kth_profile_begin(void);
-int kth_profile_end(void);
-int kth_profile_count(int* count);
-int kth_profile_entry(int index, char* name, size_t cap, uint64_t* launches, uint64_t* bytes, double* total_ms);
 
 #ifdef __cplusplus
 }

@@ -1,6 +1,6 @@
 """ctypes binding of libkten_hip.so: the same entry points a Kotlin host would bind.
 
-Every function of include/kten_hip.h is declared here with its C signature; `check`
+Every function of include/kten_hip.h and include/kten_hip_bench.h is declared here with its C signature; `check`
 turns a negative status into the Python exception that corresponds to what the
 reference throws for that class of error (IllegalArgumentException -> ValueError,
 IllegalStateException / device failures -> RuntimeError).
@@ -76,6 +76,10 @@ SIGNATURES = {
                                         c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64]),
     "kth_sync": (c_int, []),
     "kth_metrics": (c_int, [POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]),
+}
+
+# The measurement entry points of include/kten_hip_bench.h (same library; no counterpart in the contract).
+BENCH_SIGNATURES = {
     "kth_timer_begin": (c_int, []),
     "kth_timer_end": (c_int, [POINTER(c_float)]),
     "kth_timer_lap": (c_int, []),
@@ -100,7 +104,7 @@ def load():
             f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
             "or `make -C kten_amd/csrc`. There is no CPU fallback for the HIP backend.")
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SIGNATURES.items():
+    for name, (restype, argtypes) in list(SIGNATURES.items()) + list(BENCH_SIGNATURES.items()):
         fn = getattr(lib, name)          # AttributeError here means the .so is stale
         fn.restype = restype
         fn.argtypes = argtypes

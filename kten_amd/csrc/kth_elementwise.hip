@@ -21,7 +21,10 @@ constexpr int kBlock = 256;
 // two and 77 us at four), two for the broadcast kernels.
 constexpr int kUnroll = 1;
 constexpr uint32_t kTile = kBlock * kUnroll;     // float4s per workgroup
-constexpr int kBcastUnroll = 2;
+#ifndef KTH_BCAST_UNROLL
+#define KTH_BCAST_UNROLL 2
+#endif
+constexpr int kBcastUnroll = KTH_BCAST_UNROLL;
 constexpr uint32_t kBcastTile = kBlock * kBcastUnroll;
 constexpr uint32_t kReuseChunkShift = 6;          // 64 tiles (of up to 8 KiB per operand) stay in L2 while the slices pass; half when both operands repeat
 
@@ -1337,7 +1340,10 @@ int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
     if (!st) return KTH_E_HANDLE;
     if (n > st->n_floats) return fail(KTH_E_ARGUMENT, "kth_contains_nan: n=%llu exceeds the store", (unsigned long long)n);
     *out = 0;
-    if (n == 0) return KTH_OK;
+    if (n == 0) {                      // still a blocking call: it drains the stream and reports what is pending
+        KTH_HIP(hipStreamSynchronize(state().stream));
+        return report_deferred_index_error();
+    }
     uint64_t cap;
     int* flag = reinterpret_cast<int*>(workspace_acquire(4, &cap));
     if (!flag) return fail(KTH_E_MEMORY, "kth_contains_nan: no workspace");
@@ -1357,7 +1363,8 @@ int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
     workspace_release(reinterpret_cast<float*>(flag), cap);
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_contains_nan: %s", hipGetErrorString(e));
     *out = host_flag;
-    return KTH_OK;
+    // A pending out-of-range index of deferred checking is reported here, once; *out is valid all the same.
+    return report_deferred_index_error();
 }
 
 }  // extern "C"

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../include/kten_hip.h"
+#include "../../include/kten_hip_bench.h"
 #include "kth_fastdiv.h"
 
 namespace kth {

@@ -61,6 +61,15 @@ __device__ __forceinline__ ArgAcc shfl_xor_acc(ArgAcc a, int m) {
     return r;
 }
 
+__device__ __forceinline__ double shfl_down_acc(double a, int d) { return __shfl_down(a, d); }
+__device__ __forceinline__ float  shfl_down_acc(float a, int d)  { return __shfl_down(a, d); }
+__device__ __forceinline__ ArgAcc shfl_down_acc(ArgAcc a, int d) {
+    ArgAcc r;
+    r.v = __shfl_down(a.v, d);
+    r.i = static_cast<uint32_t>(__shfl_down(static_cast<int>(a.i), d));
+    return r;
+}
+
 template <bool MEAN>
 struct RedSumT {
     static constexpr const char* name = MEAN ? "RedMean" : "RedSum";
@@ -479,6 +488,55 @@ __global__ __launch_bounds__(kBlock) void reduce_stream_kernel(const float* __re
     for (uint32_t i = t; i < g.inner; i += kBlock) emit<R>(g, o, s, i, fold[i], out, partial);
 }
 
+// ---------------------------------------------------------------- small inputs: a wave per slab, no LDS and no barrier
+
+// A tensor of a megabyte or two is over before a workgroup's staging, barriers and LDS fold have paid for themselves:
+// what such a launch costs is its chain of dependent steps (on this part about 1.7 us for load -> store, 3.4 us
+// for the slab-per-workgroup kernel on [128,56,56] -> [128,56]). Here one wave owns the slab [axis, inner] of one
+// outer index: lane = r * groups + c takes the four adjacent columns of group c (16 bytes from a dword address; the
+// last group of an inner size off a multiple of 4 starts at inner - 4 and overlaps its neighbour) on rows
+// r, r + row_lanes, ..., all of them requested before the first is folded when the slab is short, and the row lanes
+// of a column group are merged by shuffles: nothing leaves the wave until the result does.
+constexpr uint32_t kSmallBatch = 16;          // loads in flight per lane
+// A workgroup is one wave: the slabs spread over as many compute units as there are slabs, and a compute unit's
+// share of the loads is one slab's.
+template <class R>
+__global__ __launch_bounds__(kWave) void reduce_wave_slabs_kernel(const float* __restrict__ in, float* __restrict__ out, Geom g,
+                                                                 uint32_t groups, uint32_t row_lanes) {
+    using Acc = typename R::Acc;
+    const uint32_t o = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t r = lane / groups, c = lane - r * groups;
+    const uint32_t own = c * 4;
+    const uint32_t col = own + 4 > g.inner ? g.inner - 4 : own;
+    Acc acc[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) acc[v] = R::init();
+    if (r < row_lanes) {
+        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
+        for (uint32_t a = r; a < g.axis; a += kSmallBatch * row_lanes) {
+            float4 w[kSmallBatch];
+#pragma unroll
+            for (uint32_t k = 0; k < kSmallBatch; k++) if (a + k * row_lanes < g.axis) w[k] = ld4_stream_unaligned(base + static_cast<size_t>(a + k * row_lanes) * g.inner);
+#pragma unroll
+            for (uint32_t k = 0; k < kSmallBatch; k++) {
+                const uint32_t aa = a + k * row_lanes;
+                if (aa < g.axis) { R::step(acc[0], w[k].x, aa); R::step(acc[1], w[k].y, aa); R::step(acc[2], w[k].z, aa); R::step(acc[3], w[k].w, aa); }
+            }
+        }
+    }
+    // row lane r takes row lane r + step (idle lanes hold the identity); row_lanes is a power of two
+    for (uint32_t step = row_lanes >> 1; step >= 1; step >>= 1) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[v] = R::merge(acc[v], shfl_down_acc(acc[v], static_cast<int>(step * groups)));
+    }
+    if (lane < groups) {
+        float* q = out + static_cast<size_t>(o) * g.inner + col;
+#pragma unroll
+        for (uint32_t v = 0; v < 4; v++) if (col + v >= own) q[v] = R::finish(acc[v], g.axis);
+    }
+}
+
 // ---------------------------------------------------------------- few rows: axis of 2 ... 7 over wide columns
 
 // With so short an axis a column gives a thread only a handful of loads, so a thread takes four
@@ -646,11 +704,15 @@ void plan_segments(Geom* g, uint64_t base_blocks, uint64_t target, uint32_t quan
 // Measured: from slabs of about 2048 floats on, streaming a slab per workgroup beats one thread
 // per output (6 TB/s against 1-4.5); below that the per-workgroup fold dominates.
 constexpr uint64_t kStreamMinSlab = 2048;
+// Inputs up to this many floats take the small-input plans.
+constexpr uint64_t kSmallInputFloats = 1u << 20;
+constexpr uint64_t kSmallRowsFloats = 1u << 16;
 
 // use_static: partials go to the static scratch array (no pool, no events, nothing allocated);
 // a plan whose partials do not fit is refused before anything is launched.
+// plan_only: makes the plan, applies that refusal and returns without launching (in and out are not used).
 template <class R>
-int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static) {
+int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static, bool plan_only) {
     using Acc = typename R::Acc;
     State& st = state();
     const bool may_profile = !use_static;
@@ -660,6 +722,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     const uint64_t n_out = static_cast<uint64_t>(outer) * inner;
 
     if (axis == 1) {
+        if (plan_only) return KTH_OK;
         const uint32_t n = static_cast<uint32_t>(n_out);
         hipError_t e;
         {
@@ -671,7 +734,34 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         return KTH_OK;
     }
 
-    if (inner == 1 && axis >= 2 && axis < 256) {
+    // Small inputs (up to 4 MiB): the launch is a chain of latencies, not a stream. Rows get enough lanes each for one
+    // 16-byte load per lane and no LDS tile; slabs get a wave each (reduce_wave_slabs_kernel).
+    const uint64_t n_in = n_out * axis;
+    const bool small_input = n_in <= kSmallInputFloats;
+    if (small_input && inner >= 4 && inner <= 4 * kWave && axis >= 2) {
+        const uint32_t groups = (inner + 3) / 4;
+        uint32_t row_lanes = 1;
+        while (row_lanes * 2 * groups <= kWave && row_lanes * 2 <= axis) row_lanes <<= 1;
+        // a lane's share of the axis in a few batches; enough waves that the tensor is not one wave's work
+        // most lanes of the wave at work; a lane's share of the axis in a few batches; and enough waves that the
+        // tensor is not one wave's work
+        if (groups * row_lanes >= kWave / 2 && static_cast<uint64_t>(axis) * inner >= 512 && ceil_div(axis, row_lanes) <= 4 * kSmallBatch &&
+            (outer >= 16 || static_cast<uint64_t>(axis) * inner <= 16384)) {
+            if (plan_only) return KTH_OK;
+            hipError_t e;
+            {
+                LaunchScope scope("reduce_wave_slabs_kernel", R::name, (n_in + n_out) * 4, may_profile);
+                hipLaunchKernelGGL((reduce_wave_slabs_kernel<R>), dim3(outer), dim3(kWave), 0, stream, in, out, g, groups, row_lanes);
+                e = hipGetLastError();
+            }
+            if (e != hipSuccess) return fail(KTH_E_DEVICE, "kth_reduce: launch failed: %s", hipGetErrorString(e));
+            return KTH_OK;
+        }
+    }
+    const bool small_rows = small_input && inner == 1 && n_in <= kSmallRowsFloats;
+
+    if (inner == 1 && axis >= 2 && axis < 256 && !small_rows) {
+        if (plan_only) return KTH_OK;
         // rows per tile: the largest power of two with rows * axis <= kShortTile, at most kBlock
         ShortPlan pl{};
         uint32_t rows = 16 * kBlock;
@@ -711,6 +801,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         if (ceil_div(outer, slab_rows) < static_cast<uint64_t>(st.compute_units)) slab_rows = 0;
     }
     if (slab_rows > 0) {
+        if (plan_only) return KTH_OK;
         ShortPlan pl{};
         const uint32_t length = axis * inner;
         const uint32_t rows = slab_rows;
@@ -739,6 +830,7 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         const uint32_t tiles = ceil_div(inner, 4u * kBlock);
         const uint64_t few_blocks = static_cast<uint64_t>(tiles) * outer;
         if (few_blocks <= 0x7fffffffull) {
+            if (plan_only) return KTH_OK;
             hipError_t e;
             {
                 LaunchScope scope("reduce_few_kernel", R::name, (static_cast<uint64_t>(outer) * slab + n_out) * 4, may_profile);
@@ -759,6 +851,13 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
         VEC = (axis % 4 == 0) ? 4 : 1;
         const uint32_t per_lane = axis / 4;            // 16-byte loads per row
         G = per_lane >= 1024 ? 256 : per_lane >= 128 ? 64 : per_lane >= 32 ? 16 : per_lane >= 8 ? 4 : per_lane >= 2 ? 2 : 1;
+        if (small_rows && axis < 256) {
+            // a small tensor of short rows: a lane per 16 bytes of the row, so that every lane has one load to wait for
+            G = 1;
+            while (G < 64 && static_cast<uint32_t>(G) * 4 < axis) G <<= 1;
+            if (G == 8) G = 16;                        // (the kernel is built for 1, 2, 4, 16, 64, 256 lanes per row)
+            if (G == 32) G = 64;
+        }
         const uint64_t base_blocks = ceil_div(outer, kBlock / G);
         plan_segments(&g, base_blocks, target / 2, G * VEC, G * VEC * 16);
         blocks = base_blocks * g.segments;
@@ -799,7 +898,9 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
                         "the static scratch holds %llu; use kth_reduce_axis", outer, axis, inner, (unsigned long long)need,
                         (unsigned long long)n_out, g.segments, (unsigned long long)kStaticScratchBytes);
         partial = reinterpret_cast<Acc*>(g_scratch_ptr[st.device]);
-    } else if (g.segments > 1) {
+    }
+    if (plan_only) return KTH_OK;
+    if (g.segments > 1 && !use_static) {
         partial = reinterpret_cast<Acc*>(workspace_acquire(n_out * g.segments * sizeof(Acc), &cap));
         if (!partial) return fail(KTH_E_MEMORY, "kth_reduce: no workspace for %llu partials",
                                   (unsigned long long)(n_out * g.segments));
@@ -856,14 +957,15 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     return KTH_OK;
 }
 
-int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static = false) {
+int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner, bool use_static = false,
+                    bool plan_only = false) {
     switch (op) {
-    case KTH_SUM:     return run_reduce<RedSum>(in, out, outer, axis, inner, use_static);
-    case KTH_MEAN:    return run_reduce<RedMean>(in, out, outer, axis, inner, use_static);
-    case KTH_MAX:     return run_reduce<RedMax>(in, out, outer, axis, inner, use_static);
-    case KTH_MIN:     return run_reduce<RedMin>(in, out, outer, axis, inner, use_static);
-    case KTH_ARG_MAX: return run_reduce<RedArgMax>(in, out, outer, axis, inner, use_static);
-    case KTH_ARG_MIN: return run_reduce<RedArgMin>(in, out, outer, axis, inner, use_static);
+    case KTH_SUM:     return run_reduce<RedSum>(in, out, outer, axis, inner, use_static, plan_only);
+    case KTH_MEAN:    return run_reduce<RedMean>(in, out, outer, axis, inner, use_static, plan_only);
+    case KTH_MAX:     return run_reduce<RedMax>(in, out, outer, axis, inner, use_static, plan_only);
+    case KTH_MIN:     return run_reduce<RedMin>(in, out, outer, axis, inner, use_static, plan_only);
+    case KTH_ARG_MAX: return run_reduce<RedArgMax>(in, out, outer, axis, inner, use_static, plan_only);
+    case KTH_ARG_MIN: return run_reduce<RedArgMin>(in, out, outer, axis, inner, use_static, plan_only);
     default:          return fail(KTH_E_ARGUMENT, "kth_reduce: op %d is not an aggregating operation", op);
     }
 }
@@ -886,8 +988,11 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
                     (unsigned long long)axis, (unsigned long long)inner);
     if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", who);
     if (outer * inner == 0) return KTH_OK;
-    const uint64_t owed_n = so->fill_n;
-    const float owed_value = so->fill_value;
+    // The entry point that creates nothing refuses a plan that does not fit its scratch before it launches anything,
+    // the fill an operand may still be owed included.
+    if (use_static)
+        if (int rc = dispatch_reduce(op, nullptr, nullptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
+                                     static_cast<uint32_t>(inner), true, true)) return rc;
     {
         // A fill the input is still owed is launched here, one the output is owed is dropped if the result
         // covers it; for the entry point that creates nothing, without the event pair of a running profile.
@@ -900,8 +1005,6 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
     }
     const int rc = dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
                                    static_cast<uint32_t>(inner), use_static);
-    // a refused plan has written nothing: the output is still owed what it was owed
-    if (rc != KTH_OK && owed_n != 0 && so->fill_n == 0) { so->fill_n = owed_n; so->fill_value = owed_value; }
     // the positions ARG_MAX / ARG_MIN wrote are index values below the axis length: an indexed move that takes
     // them next (the scatter of a Max / Min backward) need not check them
     if (rc == KTH_OK && (op == KTH_ARG_MAX || op == KTH_ARG_MIN)) {

@@ -191,6 +191,51 @@ extern "C" {
 
 const char* kth_last_error(void) { return tl_error; }
 
+// Frees everything kth_init and the calls after it created and leaves a fresh State. Shared by kth_shutdown and
+// by a kth_init that fails part-way, so that a second kth_init starts from nothing and leaks nothing.
+static void teardown() {
+    State& s = state();
+    if (s.stream) (void)hipStreamSynchronize(s.stream);
+    for (Store& st : s.table)
+        if (st.refs > 0 && st.ptr) (void)hipFree(st.ptr);
+    s.table.clear();
+    s.free_slots.clear();
+    trim_pool();
+    if (s.deferred_index_flag) (void)hipFree(s.deferred_index_flag);
+    if (s.host_index_flag) (void)hipHostFree(const_cast<int*>(s.host_index_flag));
+    s.host_index_flag = nullptr; s.host_index_flag_device = nullptr;
+    for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
+    for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
+    for (hipEvent_t e : s.laps) (void)hipEventDestroy(e);
+    for (int i = 0; i < State::kStageSlots; i++) {
+        if (s.stage[i]) (void)hipHostFree(s.stage[i]);
+        if (s.stage_done[i]) (void)hipEventDestroy(s.stage_done[i]);
+    }
+    if (s.ev_begin) (void)hipEventDestroy(s.ev_begin);
+    if (s.ev_end) (void)hipEventDestroy(s.ev_end);
+    if (s.stream) (void)hipStreamDestroy(s.stream);
+    s = State();
+}
+
+// The fallible part of kth_init after the device was chosen; on any failure the caller tears down.
+static int bring_up(int device) {
+    State& s = state();
+    KTH_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+    KTH_HIP(hipEventCreate(&s.ev_begin));
+    KTH_HIP(hipEventCreate(&s.ev_end));
+    KTH_HIP(init_math_tables());
+    KTH_HIP(reduce_scratch_init(device));
+    KTH_HIP(hipMalloc(reinterpret_cast<void**>(&s.deferred_index_flag), 256));
+    KTH_HIP(hipMemset(s.deferred_index_flag, 0, 256));
+    void* host = nullptr; void* dev = nullptr;
+    KTH_HIP(hipHostMalloc(&host, 256, hipHostMallocDefault));
+    s.host_index_flag = static_cast<volatile int*>(host);
+    KTH_HIP(hipHostGetDevicePointer(&dev, host, 0));
+    s.host_index_flag_device = static_cast<int*>(dev);
+    *s.host_index_flag = 0;
+    return KTH_OK;
+}
+
 int kth_init(int device) {
     std::lock_guard<std::mutex> g(lock());
     State& s = state();
@@ -211,20 +256,9 @@ int kth_init(int device) {
     s.wave_size = prop.warpSize;
     if (s.wave_size != 64)
         return fail(KTH_E_DEVICE, "kernels are written for wave64; device reports wave %d", s.wave_size);
-    KTH_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
-    KTH_HIP(hipEventCreate(&s.ev_begin));
-    KTH_HIP(hipEventCreate(&s.ev_end));
-    KTH_HIP(init_math_tables());
-    KTH_HIP(reduce_scratch_init(device));
-    KTH_HIP(hipMalloc(reinterpret_cast<void**>(&s.deferred_index_flag), 256));
-    KTH_HIP(hipMemset(s.deferred_index_flag, 0, 256));
-    {
-        void* host = nullptr; void* dev = nullptr;
-        KTH_HIP(hipHostMalloc(&host, 256, hipHostMallocDefault));
-        KTH_HIP(hipHostGetDevicePointer(&dev, host, 0));
-        s.host_index_flag = static_cast<volatile int*>(host);
-        s.host_index_flag_device = static_cast<int*>(dev);
-        *s.host_index_flag = 0;
+    if (int rc = bring_up(device)) {
+        teardown();                      // keeps the message `fail` recorded; the next kth_init starts clean
+        return rc;
     }
     s.device = device;
     s.ready = true;
@@ -234,28 +268,8 @@ int kth_init(int device) {
 
 int kth_shutdown(void) {
     std::lock_guard<std::mutex> g(lock());
-    State& s = state();
-    if (!s.ready) return KTH_OK;
-    (void)hipStreamSynchronize(s.stream);
-    for (Store& st : s.table)
-        if (st.refs > 0 && st.ptr) (void)hipFree(st.ptr);
-    s.table.clear();
-    s.free_slots.clear();
-    trim_pool();
-    if (s.deferred_index_flag) (void)hipFree(s.deferred_index_flag);
-    if (s.host_index_flag) (void)hipHostFree(const_cast<int*>(s.host_index_flag));
-    s.host_index_flag = nullptr; s.host_index_flag_device = nullptr;
-    for (LaunchRecord& r : s.records) { (void)hipEventDestroy(r.begin); (void)hipEventDestroy(r.end); }
-    for (hipEvent_t e : s.event_pool) (void)hipEventDestroy(e);
-    for (hipEvent_t e : s.laps) (void)hipEventDestroy(e);
-    for (int i = 0; i < State::kStageSlots; i++) {
-        if (s.stage[i]) (void)hipHostFree(s.stage[i]);
-        if (s.stage_done[i]) (void)hipEventDestroy(s.stage_done[i]);
-    }
-    (void)hipEventDestroy(s.ev_begin);
-    (void)hipEventDestroy(s.ev_end);
-    (void)hipStreamDestroy(s.stream);
-    s = State();
+    if (!state().ready) return KTH_OK;
+    teardown();
     return KTH_OK;
 }
 
@@ -395,11 +409,11 @@ int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n) {
     Store* st = lookup(handle, "kth_download");
     if (!st) return KTH_E_HANDLE;
     if (int rc = check_range(st, offset, n, "kth_download")) return rc;
-    if (n == 0) return KTH_OK;
-    if (!dst) return fail(KTH_E_ARGUMENT, "kth_download: null destination");
+    if (n != 0 && !dst) return fail(KTH_E_ARGUMENT, "kth_download: null destination");
     State& s = state();
-    KTH_HIP(hipMemcpyAsync(dst, st->ptr + offset, n * 4, hipMemcpyDeviceToHost, s.stream));
+    if (n != 0) KTH_HIP(hipMemcpyAsync(dst, st->ptr + offset, n * 4, hipMemcpyDeviceToHost, s.stream));
     KTH_HIP(hipStreamSynchronize(s.stream));
+    // A pending out-of-range index of deferred checking is reported here, once; dst has been filled all the same.
     return report_deferred_index_error();
 }
 
@@ -542,10 +556,14 @@ int kth_timer_end(float* milliseconds) {
     return KTH_OK;
 }
 
+constexpr size_t kMaxPendingLaps = 1u << 16;       // events held until kth_timer_laps reads them
+
 int kth_timer_lap(void) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     State& s = state();
+    if (s.laps.size() >= kMaxPendingLaps)
+        return fail(KTH_E_ARGUMENT, "kth_timer_lap: %zu laps are pending; read them with kth_timer_laps first", s.laps.size());
     hipEvent_t e = take_event();
     if (!e) return fail(KTH_E_DEVICE, "kth_timer_lap: no event");
     KTH_HIP(hipEventRecord(e, s.stream));
@@ -585,6 +603,13 @@ int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kerne
     if (n_floats == 0 || n_floats > kMaxElements || n_floats % 4 != 0 || reps < 1)
         return fail(KTH_E_ARGUMENT, "kth_measure_copy: need a multiple of 4 floats below 2^31 and at least one repetition");
     State& s = state();
+    // Its own event pair: the stopwatch's pair may be open around this call.
+    hipEvent_t ev0 = take_event(), ev1 = take_event();
+    if (!ev0 || !ev1) {
+        if (ev0) s.event_pool.push_back(ev0);
+        if (ev1) s.event_pool.push_back(ev1);
+        return fail(KTH_E_DEVICE, "kth_measure_copy: no event");
+    }
     uint64_t cap_a = 0, cap_b = 0;
     float* a = workspace_acquire(n_floats * 4, &cap_a);
     float* b = a ? workspace_acquire(n_floats * 4, &cap_b) : nullptr;
@@ -594,14 +619,14 @@ int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kerne
         const uint32_t n = static_cast<uint32_t>(n_floats);
         const uint32_t blocks = (n / 4 + 255) / 256;
         for (int i = -1; i < reps; i++) {              // one untimed pass first
-            if (i == 0) { hipError_t e = hipEventRecord(s.ev_begin, s.stream); if (e != hipSuccess) return e; }
+            if (i == 0) { hipError_t e = hipEventRecord(ev0, s.stream); if (e != hipSuccess) return e; }
             if (kernel) hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, s.stream, a, b, n);
             else { hipError_t e = hipMemcpyAsync(b, a, n_floats * 4, hipMemcpyDeviceToDevice, s.stream); if (e != hipSuccess) return e; }
         }
-        hipError_t e = hipEventRecord(s.ev_end, s.stream);
-        if (e == hipSuccess) e = hipEventSynchronize(s.ev_end);
+        hipError_t e = hipEventRecord(ev1, s.stream);
+        if (e == hipSuccess) e = hipEventSynchronize(ev1);
         float ms = 0.0f;
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, s.ev_begin, s.ev_end);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, ev0, ev1);
         if (out_ms) *out_ms = ms / static_cast<float>(reps);
         return e;
     };
@@ -613,6 +638,8 @@ int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kerne
     }
     if (b) workspace_release(b, cap_b);
     if (a) workspace_release(a, cap_a);
+    s.event_pool.push_back(ev0);
+    s.event_pool.push_back(ev1);
     return rc;
 }
 

@@ -500,6 +500,10 @@ def test_deferred_index_check_reports_at_the_next_blocking_call(gc):
         x.indexAdd(1, bad, src)
         with pytest.raises(ValueError, match="invalid index"):
             x.toArray()                              # a download reports it too
+        x.indexAdd(1, bad, src)
+        with pytest.raises(ValueError, match="invalid index"):
+            x.containsNan()                          # and so does the NaN scan, which blocks as well
+        assert x.containsNan() is False              # reported once
     finally:
         abi.check(lib.kth_set_index_check(1))
     with pytest.raises(ValueError):

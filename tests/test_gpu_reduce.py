@@ -111,6 +111,39 @@ def test_special_values_in_reductions(shape, axis, gc):
                           f"{op} {shape} axis {axis}")
 
 
+# Small tensors (up to 4 MiB) whose slabs a wave takes whole, and small tensors of short rows: inner sizes on and off
+# multiples of 4 (the last column group overlaps its neighbour), 1 ... 32 row lanes per column group, slabs of one
+# and of several batches of loads, outer counts that leave a workgroup's last waves without a slab.
+SMALL_SLABS = [([128, 56, 56], 1), ([10, 56, 56], 1), ([1, 64, 200], 1), ([33, 120, 5], 1), ([17, 300, 7], 1), ([64, 9, 255], 1),
+               ([200, 40, 31], 1), ([5, 1000, 4], 1), ([19, 128, 13], 1), ([70, 3, 256], 1), ([2, 2, 40, 129], 2), ([130, 600, 6], 1),
+               ([128, 56, 56], 2), ([16, 2048, 4], 1)]
+SMALL_ROWS = [([128, 56], 1), ([1, 128, 1, 56], 3), ([300, 10], 1), ([77, 255], 1), ([1000, 3], 1), ([40, 129], 1), ([2, 200], 1), ([500, 17], 1)]
+
+
+@pytest.mark.parametrize("shape,axis", SMALL_SLABS + SMALL_ROWS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else str(v))
+def test_small_inputs(shape, axis, gc):
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = rng.standard_normal(shape).astype(np.float32)
+    x.reshape(-1)[::3] = np.round(x.reshape(-1)[::3] * 2) / 2                 # ties for the arg reducers
+    x.reshape(-1)[5::97] = np.nan
+    x.reshape(-1)[11::89] = -np.inf
+    t = raw(gc, x)
+    gc.profileBegin()
+    got = {op: getattr(t, op)(axis).toArray().reshape(-1) for op in OPS}
+    kernels = gc.profileEnd()
+    if (shape, axis) in SMALL_SLABS[:12]:
+        assert any(k.startswith("reduce_wave_slabs_kernel") for k in kernels), f"expected a wave per slab, saw {sorted(kernels)}"
+    if (shape, axis) in SMALL_ROWS:
+        assert all(k.startswith("reduce_rows_kernel") for k in kernels), f"expected the row kernel, saw {sorted(kernels)}"
+    for op in ("max", "min", "argMax", "argMin"):
+        assert_bits_equal(got[op], jo.aggregate(CODE[op], x, axis).reshape(-1), f"{op} {shape} axis {axis}")
+    y = np.nan_to_num(x, nan=0.5, neginf=-2.0)                                 # sums on finite values
+    ty = raw(gc, y)
+    ref64, _ = jo.axis_sum_f64(y, axis)
+    assert_reduction_close(ty.sum(axis).toArray().reshape(-1), ref64, jo.aggregate("sum", y, axis).reshape(-1), f"sum {shape} axis {axis}")
+    assert_reduction_close(ty.mean(axis).toArray().reshape(-1), ref64 / shape[axis], jo.aggregate("mean", y, axis).reshape(-1), f"mean {shape} axis {axis}")
+
+
 @pytest.mark.parametrize("n", [1, 2, 5, 1000, 4099, 300001, 1 << 22])
 def test_full_sum_and_mean(n, gc):
     x = (np.random.default_rng(n).standard_normal(n) * 10 + 0.5).astype(np.float32)

@@ -17,8 +17,8 @@ from kten_amd.host_mirror.workloads import WORKLOADS
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_symbols():
-    text = open(os.path.join(ROOT, "include", "kten_hip.h")).read()
+def header_symbols(name="kten_hip.h"):
+    text = open(os.path.join(ROOT, "include", name)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(kth_[a-z_0-9]+)\s*\(", text)))
 
@@ -30,6 +30,18 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/kten_hip.h but not exported"
     assert sorted(abi.SIGNATURES) == names, "abi.SIGNATURES and include/kten_hip.h declare different entry points"
+
+
+def test_library_exports_the_measurement_entry_points_of_their_own_header():
+    lib = abi.load()
+    names = header_symbols("kten_hip_bench.h")
+    assert len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/kten_hip_bench.h but not exported"
+    assert sorted(abi.BENCH_SIGNATURES) == names
+    # The contract header holds none of them: a host that binds the contract does not meet them.
+    assert not set(names) & set(header_symbols())
+    assert not [n for n in header_symbols() if re.match(r"kth_(timer|profile|measure)_", n)]
 
 
 def test_entry_points_refuse_to_run_before_init():

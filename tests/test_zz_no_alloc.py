@@ -100,6 +100,15 @@ def test_static_reduction_refuses_what_does_not_fit(gc):
     assert "static scratch" in msg and "4800000" in msg, msg
     assert gc.getMetrics()["launches"] == launches, "nothing may be launched for a refused shape"
     assert_bits_equal(out.toArray(), np.full([1, 200000], -7.0, dtype=np.float32), "output of a refused call")
+    # the same refusal while the input is still a noted constant: its fill is not launched either
+    fresh = gc.createRawFill(shape, 2.0)
+    launches = gc.getMetrics()["launches"]
+    rc = gc.lib.kth_reduce_axis_static(Op.SUM, fresh.storeReference, out.storeReference, 1, 1024, 200000)
+    assert rc == -3
+    assert gc.getMetrics()["launches"] == launches, "a refused call must not launch the fill its input is owed"
+    assert_bits_equal(out.toArray(), np.full([1, 200000], -7.0, dtype=np.float32), "output of the second refused call")
+    check(gc.lib.kth_reduce_axis(Op.SUM, fresh.storeReference, out.storeReference, 1, 1024, 200000))
+    assert_bits_equal(out.toArray(), np.full([1, 200000], 2048.0, dtype=np.float32), "the constant input after the refusal")
     # the pooled entry point takes the same shape
     check(gc.lib.kth_reduce_axis(Op.SUM, t.storeReference, out.storeReference, 1, 1024, 200000))
     assert_bits_equal(out.toArray(), np.full([1, 200000], 1024.0, dtype=np.float32), "kth_reduce_axis on the refused shape")
