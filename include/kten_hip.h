@@ -84,6 +84,22 @@ int kth_device_info(char* name, size_t cap, uint64_t* total_mem, int* compute_un
  * (JVM:371-377,387-393). Default 1e-7f. */
 int kth_set_epsilon(float eps);
 
+/* How the transcendental maps (log exp tanh sinh cosh sin cos tan asin acos atan, and pow with a general exponent)
+ * are evaluated. kotlin.math's Float overloads return the f64 libm value rounded once to fp32 (JVM:138-144,395-425).
+ *   KTH_MATH_EXACT         f64 routines that return that float bit for bit (0 of 2^32 inputs differ for 10 of the
+ *                          11 maps, 3 for log; pow a few per 10^8, by 1 ulp); the maps are then bound by f64
+ *                          arithmetic, 1.1 to 1.6 times the time of a copy;
+ *   KTH_MATH_WITHIN_2_ULP  fp32 routines (pow: a shorter f64 one) that stay within 2 units in the last place of that
+ *                          float (measured over all 2^32 inputs: at most 1) at the time of a copy. The default.
+ * Everything else is unaffected: + - x / sqrt abs neg floor ceil trunc round sign reciprocal rsqrt clamp, the
+ * comparisons, pow with the exponents 2, 1, 3, 4, -1, -2, 0.5 and sigmoid (whose float expression, JVM:399, amplifies an
+ * ulp of its exp) are the same bits in both modes. The mode is a property of the library, not of a store; it applies
+ * to the calls made after it is set. */
+#define KTH_MATH_EXACT        0
+#define KTH_MATH_WITHIN_2_ULP 1
+int kth_set_math_mode(int mode);
+int kth_get_math_mode(int* mode);
+
 /* PlatformProvider.memoryUsageScaleHint (PlatformProvider.kt:23-29): fraction of device
  * memory that live + pooled buffers may occupy; pooled buffers are freed first, then
  * kth_alloc fails with KTH_E_MEMORY. Default 0.85. */

@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libkten_hip.so")
 
 KTH_MAX_DIMS = 10
+KTH_MATH_EXACT, KTH_MATH_WITHIN_2_ULP = 0, 1
 KTH_OK, KTH_E_NOT_INIT, KTH_E_HANDLE, KTH_E_ARGUMENT, KTH_E_SHAPE, KTH_E_MEMORY, KTH_E_DEVICE = 0, -1, -2, -3, -4, -5, -6
 
 
@@ -35,6 +36,8 @@ SIGNATURES = {
     "kth_last_error": (c_char_p, []),
     "kth_device_info": (c_int, [ctypes.c_char_p, c_size_t, POINTER(c_uint64), POINTER(c_int), POINTER(c_int)]),
     "kth_set_epsilon": (c_int, [c_float]),
+    "kth_set_math_mode": (c_int, [c_int]),
+    "kth_get_math_mode": (c_int, [POINTER(c_int)]),
     "kth_set_memory_scale_hint": (c_int, [c_double]),
     "kth_alloc": (c_int, [c_uint64, POINTER(c_uint64)]),
     "kth_retain": (c_int, [c_uint64]),

@@ -6,6 +6,7 @@
 #include "kth_ops.h"
 #include "kth_tables.h"
 #include "kth_fast.h"
+#include "kth_f32math.h"
 #include "kth_fold.h"
 
 #include <cmath>
@@ -256,10 +257,38 @@ __device__ __forceinline__ float pow_short_then_long(float a, float b, const Log
     if (!(ok && rounds_safely(y))) r = pow_with_tables(a, b, log_tab, exp_tab);
     return r;
 }
+// The math mode "within 2 ulp": the shorter evaluation decides by itself for a finite base above zero and a finite
+// exponent other than zero with a normal result; every other operand (and a result in the denormal range, where the
+// rounding to fp32 is not relative) takes the routine above as before.
+__device__ __forceinline__ float pow_within_2_ulp(float a, float b, const Log2Entry* log2_tab, const LogEntry* log_tab, const double* exp_tab) {
+    double y;
+    const bool ok = fast_pow<true>(a, b, log2_tab, exp_tab, y);
+    float r = static_cast<float>(y);
+    if (!(ok && y >= 0x1p-126)) r = pow_with_tables(a, b, log_tab, exp_tab);
+    return r;
+}
 struct OpPowT {
     static constexpr const char* name = "OpPow";
     static __device__ __forceinline__ float apply(float a, float b, float) { return pow_short_then_long(a, b, g_log2_table, g_log_table, g_exp_table); }
 };
+
+// The maps of the math mode "within 2 ulp": fp32 evaluations (kth_f32math.h) through the plain unary kernel, no table
+// and no LDS. sin / cos / tan beyond 65536 in magnitude take the long f64 routine in every mode.
+#define KTH_F32_MAP(NAME, EXPR)                                                            \
+    struct NAME { static constexpr const char* name = #NAME;                               \
+        static __device__ __forceinline__ float apply(float x, float, float) { return (EXPR); } };
+KTH_F32_MAP(OpExpF,  f32::exp_(x))
+KTH_F32_MAP(OpLogF,  f32::log_(x))
+KTH_F32_MAP(OpTanhF, f32::tanh_(x))
+KTH_F32_MAP(OpSinhF, f32::sinh_(x))
+KTH_F32_MAP(OpCoshF, f32::cosh_(x))
+KTH_F32_MAP(OpSinF,  fabsf(x) <= f32::kTrigLimit ? f32::sin_short(x) : table_sin(x))
+KTH_F32_MAP(OpCosF,  fabsf(x) <= f32::kTrigLimit ? f32::cos_short(x) : table_cos(x))
+KTH_F32_MAP(OpTanF,  fabsf(x) <= f32::kTrigLimit ? f32::tan_short(x) : table_tan(x))
+KTH_F32_MAP(OpAsinF, f32::asin_(x))
+KTH_F32_MAP(OpAcosF, f32::acos_(x))
+KTH_F32_MAP(OpAtanF, f32::atan_(x))
+#undef KTH_F32_MAP
 
 // Unary map whose op reads a small f64 table through LDS. The data loads of the tile are
 // issued first, the table copy overlaps them. Four float4 per thread, so the 1-2 KiB
@@ -292,7 +321,7 @@ __global__ __launch_bounds__(kBlock) void unary_lds_kernel(const float* a, float
 // pow with both tables (3 KiB) in LDS: the lookups of 64 lanes go to 64 different entries, which as loads from
 // global memory cost more than the arithmetic. MODE 0: out[i] = pow(a[i], c); 1: pow(c, a[i]); 2: pow(a[i], b[i]).
 // out may alias a or b.
-template <int MODE>
+template <int MODE, bool EXACT>
 __global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const float* b, float* out, uint32_t n, float c) {
     constexpr int kLogDoubles = 2 * kLogTableEntries;
     __shared__ double tab[2 * kLogDoubles + kExpTableEntries];       // {1/c, ln c}, 2^(i/128), {1/c, log2 c}
@@ -312,8 +341,8 @@ __global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const f
     const double* exp_tab = tab + kLogDoubles;
     const Log2Entry* log2_tab = reinterpret_cast<const Log2Entry*>(tab + kLogDoubles + kExpTableEntries);
     auto one = [&](float x, float y) {
-        return MODE == 1 ? pow_short_then_long(c, x, log2_tab, log_tab, exp_tab)
-                         : pow_short_then_long(x, MODE == 2 ? y : c, log2_tab, log_tab, exp_tab);
+        const float base_ = MODE == 1 ? c : x, expo = MODE == 1 ? x : MODE == 2 ? y : c;
+        return EXACT ? pow_short_then_long(base_, expo, log2_tab, log_tab, exp_tab) : pow_within_2_ulp(base_, expo, log2_tab, log_tab, exp_tab);
     };
     // four elements through the short routine, then one branch for the lanes of the wave it leaves open
     auto four = [&](float4 x, float4 y) {
@@ -325,9 +354,9 @@ __global__ __launch_bounds__(kBlock) void pow_lds_kernel(const float* a, const f
             const float base_ = MODE == 1 ? c : xs[j];
             const float expo = MODE == 1 ? xs[j] : MODE == 2 ? ys[j] : c;
             double val;
-            const bool ok = fast_pow(base_, expo, log2_tab, exp_tab, val);
+            const bool ok = fast_pow<!EXACT>(base_, expo, log2_tab, exp_tab, val);
             rs[j] = static_cast<float>(val);
-            open[j] = !(ok && rounds_safely(val));
+            open[j] = EXACT ? !(ok && rounds_safely(val)) : !(ok && val >= 0x1p-126);
         }
         if (open[0] | open[1] | open[2] | open[3]) {
 #pragma unroll
@@ -869,9 +898,15 @@ void launch_pow(int mode, const float* a, const float* b, float* out, uint32_t n
     const uint64_t tile = static_cast<uint64_t>(kBlock) * kLdsUnroll;
     const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + tile - 1) / tile);
     const dim3 grid(blocks == 0 ? 1 : blocks);
-    if (mode == 0)      hipLaunchKernelGGL((pow_lds_kernel<0>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
-    else if (mode == 1) hipLaunchKernelGGL((pow_lds_kernel<1>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
-    else                hipLaunchKernelGGL((pow_lds_kernel<2>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+    if (state().math_mode == KTH_MATH_EXACT) {
+        if (mode == 0)      hipLaunchKernelGGL((pow_lds_kernel<0, true>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+        else if (mode == 1) hipLaunchKernelGGL((pow_lds_kernel<1, true>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+        else                hipLaunchKernelGGL((pow_lds_kernel<2, true>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+    } else {
+        if (mode == 0)      hipLaunchKernelGGL((pow_lds_kernel<0, false>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+        else if (mode == 1) hipLaunchKernelGGL((pow_lds_kernel<1, false>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+        else                hipLaunchKernelGGL((pow_lds_kernel<2, false>), grid, dim3(kBlock), 0, state().stream, a, b, out, n, c);
+    }
 }
 
 template <class Op>
@@ -1070,6 +1105,21 @@ int kth_fill(uint64_t handle, uint64_t offset, uint64_t n, float value) {
     return KTH_OK;
 }
 
+int kth_set_math_mode(int mode) {
+    std::lock_guard<std::mutex> g(lock());
+    if (mode != KTH_MATH_EXACT && mode != KTH_MATH_WITHIN_2_ULP)
+        return fail(KTH_E_ARGUMENT, "kth_set_math_mode: %d is neither KTH_MATH_EXACT nor KTH_MATH_WITHIN_2_ULP", mode);
+    state().math_mode = mode;
+    return KTH_OK;
+}
+
+int kth_get_math_mode(int* mode) {
+    std::lock_guard<std::mutex> g(lock());
+    if (!mode) return fail(KTH_E_ARGUMENT, "kth_get_math_mode: null output");
+    *mode = state().math_mode;
+    return KTH_OK;
+}
+
 int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
@@ -1082,26 +1132,32 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
                     (unsigned long long)sa->n_floats, (unsigned long long)so->n_floats);
     const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
 #define U(OP) if (n32) launch_unary<OP>(pa, po, n32, 0.0f, 0.0f)
+    // T: a transcendental map. Mode "exact": the f64 routines behind LDS tables (the float kotlin.math returns, bit
+    // for bit); mode "within 2 ulp": the fp32 routine through the plain kernel.
+#define T(EXACT, FAST) if (n32) { if (exact) launch_unary_lds<EXACT>(pa, po, n32); else launch_unary<FAST>(pa, po, n32, 0.0f, 0.0f); }
+    const bool exact = state().math_mode == KTH_MATH_EXACT;
     switch (op) {
     case KTH_NEG: U(OpNeg); break;           case KTH_RECIPROCAL: U(OpReciprocal); break;
-    case KTH_LOG: if (n32) launch_unary_lds<OpLogT>(pa, po, n32); break;
-    case KTH_EXP: if (n32) launch_unary_lds<OpExpT>(pa, po, n32); break;
-    case KTH_TANH: if (n32) launch_unary_lds<OpTanhT>(pa, po, n32); break;
+    case KTH_LOG: T(OpLogT, OpLogF); break;
+    case KTH_EXP: T(OpExpT, OpExpF); break;
+    case KTH_TANH: T(OpTanhT, OpTanhF); break;
     case KTH_SIGMOID: if (n32) launch_unary_lds<OpSigmoidT>(pa, po, n32); break;
-    case KTH_SINH: if (n32) launch_unary_lds<OpSinhT>(pa, po, n32); break;
-    case KTH_COSH: if (n32) launch_unary_lds<OpCoshT>(pa, po, n32); break;
+    case KTH_SINH: T(OpSinhT, OpSinhF); break;
+    case KTH_COSH: T(OpCoshT, OpCoshF); break;
     case KTH_ABS: U(OpAbs); break;           case KTH_SIGN: U(OpSign); break;
     case KTH_SQRT: U(OpSqrt); break;
-    case KTH_SIN: if (n32) launch_unary_lds<OpSinT>(pa, po, n32); break;
-    case KTH_COS: if (n32) launch_unary_lds<OpCosT>(pa, po, n32); break;
-    case KTH_TAN: if (n32) launch_unary_lds<OpTanT>(pa, po, n32); break;
-    case KTH_ASIN: if (n32) launch_unary_lds<OpAsinT>(pa, po, n32); break;
-    case KTH_ACOS: if (n32) launch_unary_lds<OpAcosT>(pa, po, n32); break;
-    case KTH_ATAN: if (n32) launch_unary_lds<OpAtanT>(pa, po, n32); break;         case KTH_FLOOR: U(OpFloor); break;
+    case KTH_SIN: T(OpSinT, OpSinF); break;
+    case KTH_COS: T(OpCosT, OpCosF); break;
+    case KTH_TAN: T(OpTanT, OpTanF); break;
+    case KTH_ASIN: T(OpAsinT, OpAsinF); break;
+    case KTH_ACOS: T(OpAcosT, OpAcosF); break;
+    case KTH_ATAN: T(OpAtanT, OpAtanF); break;
+    case KTH_FLOOR: U(OpFloor); break;
     case KTH_CEIL: U(OpCeil); break;         case KTH_ROUND: U(OpRound); break;
     case KTH_TRUNC: U(OpTrunc); break;       case KTH_RSQRT: U(OpRsqrt); break;
     default: return fail(KTH_E_ARGUMENT, "kth_unary: op %d is not a unary map", op);
     }
+#undef T
 #undef U
     if (n == 0) return KTH_OK;
     KTH_LAUNCH_CHECK("unary");

@@ -197,6 +197,10 @@ __device__ __forceinline__ bool fast_acos(float x, const double* tab, double& y)
 // next term is below 2^-55). The result is good to 2^-44 for |w| up to 128, beyond which it is 0 or inf anyway.
 struct Log2Entry { double invc, log2c; };
 
+// SHORT (the math mode "within 2 ulp"): log2(1 + r) to r^5 and 2^q - 1 to q^3. The logarithm is then good to 2^-37
+// relative (worst next to a = 1, where log2 a itself is as small as |r|), w = b log2 a to 2^-30 absolute at |w| = 128,
+// the power to 2^-30: the float it rounds to is the exact power's or its neighbour.
+template <bool SHORT = false>
 __device__ __forceinline__ bool fast_pow(float a, float b, const Log2Entry* log2_tab, const double* exp_tab, double& y) {
     const double d = static_cast<double>(a);
     const uint64_t ix = static_cast<uint64_t>(__double_as_longlong(d));
@@ -207,8 +211,11 @@ __device__ __forceinline__ bool fast_pow(float a, float b, const Log2Entry* log2
     const Log2Entry e = log2_tab[i];
     const double r = fma(z, e.invc, -1.0);
     // log2(1 + r) = r (c1 + r (c2 + ...)), c_n = (-1)^(n+1) / (n ln 2)
-    double p = fma(r, 0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3);        // 1/(7 ln2), -1/(6 ln2)
-    p = fma(r, p, 0x1.2776c50ef9bfep-2);                                     // 1/(5 ln2)
+    double p = 0x1.2776c50ef9bfep-2;                                         // 1/(5 ln2)
+    if (!SHORT) {
+        p = fma(r, 0x1.a61762a7aded9p-3, -0x1.ec709dc3a03fdp-3);            // 1/(7 ln2), -1/(6 ln2)
+        p = fma(r, p, 0x1.2776c50ef9bfep-2);
+    }
     p = fma(r, p, -0x1.71547652b82fep-2);                                    // -1/(4 ln2)
     p = fma(r, p, 0x1.ec709dc3a03fdp-2);                                     // 1/(3 ln2)
     p = fma(r, p, -0x1.71547652b82fep-1);                                    // -1/(2 ln2)
@@ -219,8 +226,11 @@ __device__ __forceinline__ bool fast_pow(float a, float b, const Log2Entry* log2
     const int j = static_cast<int>(kd);
     const double q = fma(kd, -0.0078125, w);
     // 2^q - 1 = q (l1 + q (l2 + ...)), l_n = ln2^n / n!
-    double g = fma(q, 0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7);        // ln2^5/120, ln2^4/24
-    g = fma(q, g, 0x1.c6b08d704a0c0p-5);                                     // ln2^3/6
+    double g = 0x1.c6b08d704a0c0p-5;                                         // ln2^3/6
+    if (!SHORT) {
+        g = fma(q, 0x1.5d87fe78a6731p-10, 0x1.3b2ab6fba4e77p-7);            // ln2^5/120, ln2^4/24
+        g = fma(q, g, 0x1.c6b08d704a0c0p-5);
+    }
     g = fma(q, g, 0x1.ebfbdff82c58fp-3);                                     // ln2^2/2
     g = fma(q, g, 0x1.62e42fefa39efp-1);                                     // ln2
     const double s = exp_tab[j & (kExpTableEntries - 1)];

@@ -67,6 +67,7 @@ struct State {
 
     float  epsilon = 1e-7f;
     double mem_hint = 0.85;
+    int    math_mode = KTH_MATH_WITHIN_2_ULP;   // kth_set_math_mode
 
     std::vector<Store>    table;       // handle index -> store
     std::vector<uint32_t> free_slots;

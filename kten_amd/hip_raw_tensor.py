@@ -8,6 +8,7 @@ validates shapes on the host (raising where the reference throws), allocates the
 store from the library's pool and enqueues one kernel through the C ABI. Nothing here
 computes on the CPU; without the shared library the import of `abi.load()` fails.
 """
+import contextlib
 import ctypes
 from contextlib import contextmanager
 from typing import Callable, List, Optional, Sequence
@@ -528,6 +529,31 @@ class HipTensorOperations:
     def setEpsilon(self, eps: float):
         """PlatformProvider.epsilon (PlatformProvider.kt:12)."""
         check(self.lib.kth_set_epsilon(float(eps)))
+
+    def setMathMode(self, mode: str):
+        """How the transcendental maps are evaluated: "exact" (the float kotlin.math returns, bit for bit, by f64
+        routines) or "within_2_ulp" (fp32 routines at the time of a copy; the default). No counterpart in the
+        reference, whose two backends each have one way."""
+        from .abi import KTH_MATH_EXACT, KTH_MATH_WITHIN_2_ULP
+        codes = {"exact": KTH_MATH_EXACT, "within_2_ulp": KTH_MATH_WITHIN_2_ULP}
+        if mode not in codes:
+            raise ValueError(f"math mode {mode!r} is neither 'exact' nor 'within_2_ulp'")
+        check(self.lib.kth_set_math_mode(codes[mode]))
+
+    def getMathMode(self) -> str:
+        m = ctypes.c_int()
+        check(self.lib.kth_get_math_mode(ctypes.byref(m)))
+        return "exact" if m.value == 0 else "within_2_ulp"
+
+    @contextlib.contextmanager
+    def mathMode(self, mode: str):
+        """The math mode for the calls made inside the block; the previous one afterwards."""
+        before = self.getMathMode()
+        self.setMathMode(mode)
+        try:
+            yield self
+        finally:
+            self.setMathMode(before)
 
     def setMemoryUsageScaleHint(self, fraction: float):
         """PlatformProvider.memoryUsageScaleHint (PlatformProvider.kt:23-29)."""

@@ -61,6 +61,26 @@ def test_constant_folding_on_the_host(tmp_path):
     assert "fold ok" in done.stdout
 
 
+def test_fp32_routines_of_the_within_2_ulp_mode_on_the_host(tmp_path):
+    """The fp32 evaluations of exp log tanh sinh cosh sin cos tan asin acos atan (kth_f32math.h: IEEE operations only,
+    so the host computes the device's bits) against (float) libm_f64 on every 509th bit pattern and the special
+    values: none further than 2 ulp (observed: none further than 1)."""
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = tmp_path / "f32math_test"
+    subprocess.run([gxx, "-std=c++17", "-O2", "-ffp-contract=off", "-Wall", "-Wextra", "-Werror",
+                    os.path.join(ROOT, "tests", "cpp", "f32math_test.cpp"), "-o", str(exe), "-lpthread"], check=True)
+    done = subprocess.run([str(exe), "509"], capture_output=True, text=True, timeout=600)
+    print(done.stdout)
+    assert done.returncode == 0, done.stdout + done.stderr
+    rows = [line.split() for line in done.stdout.splitlines()[1:]]
+    assert len(rows) == 11
+    for r in rows:
+        assert int(r[5]) == 0, f"{r[0]}: {r[5]} results further than 2 ulp"
+        assert int(r[4]) == 0, f"{r[0]}: {r[4]} results at 2 ulp (none was observed when this was written)"
+
+
 @pytest.mark.gpu
 def test_cpp_host_mirror_known_answers():
     assert os.path.exists(BINARY), "tests/cpp/host_mirror_test is not built (python __graft_entry__.py build)"
