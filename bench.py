@@ -312,7 +312,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="cfg5",
                     choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "max_backward", "softmax_ce", "transpose", "permute",
-                             "concat_mask", "broadcast_reuse", "batch_norm", "reduce_shapes", "indexed_moves", "indexed_skew", "layout_shapes", "unary_maps"])
+                             "concat_mask", "broadcast_reuse", "broadcast_pairs", "sum0_alone", "batch_norm", "reduce_shapes", "indexed_moves", "indexed_skew", "layout_shapes", "unary_maps"])
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,

@@ -547,6 +547,16 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* _
     }
 }
 
+// Outermost dims taken off a broadcast and run as the grid's y and z: batch item (y, z) is the same problem on the
+// operands and the output moved by these strides (in floats; 0 where an operand does not have the dim).
+struct Batch { uint32_t a[2], b[2], out[2]; };
+
+__device__ __forceinline__ void move_to_batch_item(const Batch& bt, const float*& a, const float*& b, float*& out) {
+    a += static_cast<size_t>(blockIdx.y) * bt.a[0] + static_cast<size_t>(blockIdx.z) * bt.a[1];
+    b += static_cast<size_t>(blockIdx.y) * bt.b[0] + static_cast<size_t>(blockIdx.z) * bt.b[1];
+    out += static_cast<size_t>(blockIdx.y) * bt.out[0] + static_cast<size_t>(blockIdx.z) * bt.out[1];
+}
+
 // Four values of an operand at offsets off, off + stride, ... (stride in elements).
 typedef float v4f_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 __device__ __forceinline__ void gather4(const float* __restrict__ p, uint32_t off, uint32_t stride, float (&v)[4]) {
@@ -566,8 +576,11 @@ __device__ __forceinline__ void gather4(const float* __restrict__ p, uint32_t of
 // as float4; a broadcast operand is gathered element by element through the plan (dim 0 in
 // elements), which the caches serve. The last, partial group of four is done by elements.
 template <class Op, bool AL, bool BL>
-__global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                                   float* __restrict__ out, uint32_t n, float eps, BcastPlan pl) {
+__global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float* __restrict__ a_, const float* __restrict__ b_,
+                                                                   float* __restrict__ out_, uint32_t n, float eps, BcastPlan pl, Batch bt) {
+    const float* a = a_; const float* b = b_; float* out = out_;
+    move_to_batch_item(bt, a, b, out);          // (a batched launch has items of a multiple of 4 floats: the float4s stay aligned)
+    const bool batched = bt.out[1] != 0;
     const uint32_t base = blockIdx.x * kBcastTile + threadIdx.x;
 #pragma unroll
     for (int k = 0; k < kBcastUnroll; k++) {
@@ -575,8 +588,10 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_mixed_kernel(const float*
         if (e0 >= n) continue;
         if (e0 + 4 <= n) {
             float va[4], vb[4];
-            if (AL) { const float4 v = ld4(a, e0 >> 2); va[0] = v.x; va[1] = v.y; va[2] = v.z; va[3] = v.w; }
-            if (BL) { const float4 v = ld4(b, e0 >> 2); vb[0] = v.x; vb[1] = v.y; vb[2] = v.z; vb[3] = v.w; }
+            // an operand laid out like the output: read once in a plain launch (streaming load); in a batched one every
+            // batch item reads it again, so it is loaded through the caches
+            if (AL) { const float4 v = batched ? reinterpret_cast<const float4*>(a)[e0 >> 2] : ld4(a, e0 >> 2); va[0] = v.x; va[1] = v.y; va[2] = v.z; va[3] = v.w; }
+            if (BL) { const float4 v = batched ? reinterpret_cast<const float4*>(b)[e0 >> 2] : ld4(b, e0 >> 2); vb[0] = v.x; vb[1] = v.y; vb[2] = v.z; vb[3] = v.w; }
             // The four outputs are neighbours along dim 0 unless they cross its end. Then a broadcast
             // operand that does not vary along dim 0 needs one load for all four, and one that is
             // contiguous there one 16-byte load from a 4-byte aligned address: four single loads at
@@ -656,8 +671,10 @@ __device__ __forceinline__ void stage_range(float* lds, uint32_t at, const float
 }
 
 template <class Op>
-__global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                             float* __restrict__ out, float eps, OuterPlan pl) {
+__global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __restrict__ a_, const float* __restrict__ b_,
+                                                             float* __restrict__ out_, float eps, OuterPlan pl, Batch bt) {
+    const float* a = a_; const float* b = b_; float* out = out_;
+    move_to_batch_item(bt, a, b, out);
     // sized at launch to what the shape needs (at most 56 KiB), so that short operands leave room for eight workgroups per CU
     extern __shared__ float outer_lds[];
     float* row_lds = outer_lds;
@@ -725,7 +742,8 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
             if (v == pl.run) { v = 0; col++; }
             if (c == pl.span) { c = 0; col = 0; row_base += pl.run; }
         }
-        if (g + 4 <= len) st4(out, e0 >> 2, make_float4(r[0], r[1], r[2], r[3]));
+        // (16 bytes at a dword address: a batch item may start anywhere)
+        if (g + 4 <= len) *reinterpret_cast<v4f_unaligned*>(out + e0) = v4f_unaligned{r[0], r[1], r[2], r[3]};
         else for (uint32_t j = 0; g + j < len; j++) out[e0 + j] = r[j];
     }
 }
@@ -737,8 +755,12 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
 constexpr uint32_t kOuterRows = 8;
 constexpr uint32_t kOuterCols = kOuterTile / kOuterRows;      // 1024 column offsets: four per thread
 template <class Op>
-__global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                                  float* __restrict__ out, float eps, OuterPlan pl, uint32_t rows) {
+__global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* __restrict__ a_, const float* __restrict__ b_,
+                                                                  float* __restrict__ out_, float eps, OuterPlan pl, uint32_t rows, Batch bt) {
+    // (the grid's y counts row blocks here: one batch dim, on z)
+    const float* a = a_ + static_cast<size_t>(blockIdx.z) * bt.a[1];
+    const float* b = b_ + static_cast<size_t>(blockIdx.z) * bt.b[1];
+    float* out = out_ + static_cast<size_t>(blockIdx.z) * bt.out[1];
     extern __shared__ float outer_rows_lds[];
     const float* rowp = pl.a_is_row ? a : b;
     const float* colp = pl.a_is_row ? b : a;
@@ -965,51 +987,110 @@ void order_tiles_for_reuse(BcastPlan* plan, uint32_t n4, dim3* grid) {
     *grid = dim3(plan->per_xcd * 8);
 }
 
+// Whether the d innermost dims of `plan` (d = 2 or 3) are one of the shapes the outer-product kernels take, and the
+// kernel plan for n outputs if so.
+bool match_outer(const BcastPlan& plan, int d, uint32_t n, OuterPlan* op, uint32_t* rows) {
+    if (d != 2 && d != 3) return false;
+    const bool with_run = d == 3;
+    const uint32_t run = with_run ? plan.size[0] : 1u;
+    // the dim next to the outermost one is the column index, the outermost the row index
+    bool run_ok = !with_run || (plan.astride[0] == 1 && plan.bstride[0] == 1 && run <= kOuterMaxRun);
+    bool a_row = plan.astride[d - 2] == 0 && plan.astride[d - 1] == run && plan.bstride[d - 2] == run && plan.bstride[d - 1] == 0;
+    bool b_row = plan.bstride[d - 2] == 0 && plan.bstride[d - 1] == run && plan.astride[d - 2] == run && plan.astride[d - 1] == 0;
+    // or the row operand alone keeps the innermost run and the column operand holds one value per column index
+    bool flat = false;
+    if (with_run && !run_ok && run <= kOuterMaxRun) {
+        const bool a_flat_row = plan.astride[0] == 1 && plan.astride[1] == 0 && plan.astride[2] == run &&
+                                plan.bstride[0] == 0 && plan.bstride[1] == 1 && plan.bstride[2] == 0;
+        const bool b_flat_row = plan.bstride[0] == 1 && plan.bstride[1] == 0 && plan.bstride[2] == run &&
+                                plan.astride[0] == 0 && plan.astride[1] == 1 && plan.astride[2] == 0;
+        flat = run_ok = a_flat_row || b_flat_row;
+        a_row = a_flat_row; b_row = b_flat_row;
+    }
+    if (!(run_ok && (a_row || b_row) && plan.size[d - 2] >= 2)) return false;
+    *op = OuterPlan{};
+    op->n = n; op->run = run; op->span = plan.size[d - 2] * run; op->a_is_row = a_row ? 1u : 0u;
+    op->col_flat = flat ? 1u : 0u; op->cols = plan.size[d - 2];
+    op->span_div = make_div(op->span); op->run_div = make_div(run);
+    op->row_lds = (((kOuterTile - 1) / op->span + 2) * run + 3u) & ~3u;
+    *rows = plan.size[d - 1];
+    return true;
+}
+
+template <class Op>
+void launch_outer(const float* a, const float* b, float* out, float eps, const OuterPlan& op, uint32_t rows, uint64_t bytes,
+                  const Batch& bt, uint32_t batch_y, uint32_t batch_z) {
+    hipStream_t st = state().stream;
+    if (op.span >= 2048u && rows <= 65535u * kOuterRows && batch_y == 1) {
+        LaunchScope scope("binary_outer_rows_kernel", Op::name, bytes);
+        const dim3 grid((op.span + kOuterCols - 1) / kOuterCols, (rows + kOuterRows - 1) / kOuterRows, batch_z);
+        hipLaunchKernelGGL((binary_outer_rows_kernel<Op>), grid, dim3(kBlock), kOuterRows * op.run * sizeof(float), st, a, b, out, eps, op, rows, bt);
+        return;
+    }
+    const uint32_t col_lds = op.col_flat ? std::min(op.cols, kOuterTile / op.run + 2u)
+                                         : op.span <= kOuterTile ? op.span : 4u;  // a longer column operand is not staged
+    LaunchScope scope("binary_outer_kernel", Op::name, bytes);
+    hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((op.n + kOuterTile - 1) / kOuterTile, batch_y, batch_z), dim3(kBlock),
+                       (op.row_lds + col_lds) * sizeof(float), st, a, b, out, eps, op, bt);
+}
+
+template <class Op>
+void launch_mixed(const float* a, const float* b, float* out, uint32_t n, float eps, const BcastPlan& plan, bool al, bool bl,
+                  const Batch& bt, uint32_t batch_y, uint32_t batch_z) {
+    hipStream_t st = state().stream;
+    const uint64_t groups = (static_cast<uint64_t>(n) + 3) / 4;
+    dim3 grid(static_cast<uint32_t>((groups + kBcastTile - 1) / kBcastTile), batch_y, batch_z), block(kBlock);
+    if (al && bl)  hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, true>), grid, block, 0, st, a, b, out, n, eps, plan, bt);
+    else if (al)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, false>), grid, block, 0, st, a, b, out, n, eps, plan, bt);
+    else if (bl)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n, eps, plan, bt);
+    else           hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n, eps, plan, bt);
+}
+
 template <class Op>
 void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n, float eps,
                          BcastPlan plan, bool vec_ok, bool a_vec, bool b_vec, uint64_t bytes) {
-    hipStream_t st = state().stream;
+    const Batch no_batch{};
     // Both operands smaller than the output, in the two- or three-dimensional outer-product shape, and the
     // innermost dim not a multiple of 4 (a multiple of 4 has the float4 kernels): the LDS-staged kernel.
-    if (!vec_ok && !plan.a_stream && !plan.b_stream && n >= 4 * kOuterTile && (plan.ndim == 2 || plan.ndim == 3)) {
-        const int d = plan.ndim;
-        const bool with_run = d == 3;
-        const uint32_t run = with_run ? plan.size[0] : 1u;
-        // the dim next to the outermost one is the column index, the outermost the row index
-        bool run_ok = !with_run || (plan.astride[0] == 1 && plan.bstride[0] == 1 && run <= kOuterMaxRun);
-        bool a_row = plan.astride[d - 2] == 0 && plan.astride[d - 1] == run && plan.bstride[d - 2] == run && plan.bstride[d - 1] == 0;
-        bool b_row = plan.bstride[d - 2] == 0 && plan.bstride[d - 1] == run && plan.astride[d - 2] == run && plan.astride[d - 1] == 0;
-        // or the row operand alone keeps the innermost run and the column operand holds one value per column index
-        bool flat = false;
-        if (with_run && !run_ok && run <= kOuterMaxRun) {
-            const bool a_flat_row = plan.astride[0] == 1 && plan.astride[1] == 0 && plan.astride[2] == run &&
-                                    plan.bstride[0] == 0 && plan.bstride[1] == 1 && plan.bstride[2] == 0;
-            const bool b_flat_row = plan.bstride[0] == 1 && plan.bstride[1] == 0 && plan.bstride[2] == run &&
-                                    plan.astride[0] == 0 && plan.astride[1] == 1 && plan.astride[2] == 0;
-            flat = run_ok = a_flat_row || b_flat_row;
-            a_row = a_flat_row; b_row = b_flat_row;
-        }
-        if (run_ok && (a_row || b_row) && plan.size[d - 2] >= 2) {
-            OuterPlan op{};
-            op.n = n; op.run = run; op.span = plan.size[d - 2] * run; op.a_is_row = a_row ? 1u : 0u;
-            op.col_flat = flat ? 1u : 0u; op.cols = plan.size[d - 2];
-            op.span_div = make_div(op.span); op.run_div = make_div(run);
-            op.row_lds = (((kOuterTile - 1) / op.span + 2) * run + 3u) & ~3u;
-            const uint32_t rows = plan.size[d - 1];
-            if (op.span >= 2048u && rows <= 65535u * kOuterRows) {
-                LaunchScope scope("binary_outer_rows_kernel", Op::name, bytes);
-                const dim3 grid((op.span + kOuterCols - 1) / kOuterCols, (rows + kOuterRows - 1) / kOuterRows);
-                hipLaunchKernelGGL((binary_outer_rows_kernel<Op>), grid, dim3(kBlock), kOuterRows * run * sizeof(float), st, a, b, out, eps, op, rows);
+    if (!vec_ok && !plan.a_stream && !plan.b_stream && n >= 4 * kOuterTile) {
+        OuterPlan op; uint32_t rows;
+        if (match_outer(plan, plan.ndim, n, &op, &rows)) { launch_outer<Op>(a, b, out, eps, op, rows, bytes, no_batch, 1, 1); return; }
+        // Not that shape as a whole (four dims or more, a dim both operands keep outside one that only one keeps):
+        // the one or two outermost dims become the grid's z and y, when what is left inside them is that shape, or a
+        // broadcast in which one operand is as large as the item (the mixed kernel then moves it and the output
+        // as float4s and has one small operand to gather: its fast path).
+        for (int peel = 1; peel <= 2 && plan.ndim - peel >= 2; peel++) {
+            const int d = plan.ndim - peel;
+            uint64_t item = 1;
+            for (int k = 0; k < d; k++) item *= plan.size[k];
+            const uint32_t bz = plan.size[plan.ndim - 1], by = peel == 2 ? plan.size[plan.ndim - 2] : 1u;
+            if (bz > 65535u || by > 65535u || item < 256) continue;
+            Batch bt{};
+            bt.a[1] = plan.astride[plan.ndim - 1]; bt.b[1] = plan.bstride[plan.ndim - 1];
+            bt.out[1] = static_cast<uint32_t>(item * by);
+            if (peel == 2) { bt.a[0] = plan.astride[plan.ndim - 2]; bt.b[0] = plan.bstride[plan.ndim - 2]; bt.out[0] = static_cast<uint32_t>(item); }
+            if (match_outer(plan, d, static_cast<uint32_t>(item), &op, &rows)) {
+                launch_outer<Op>(a, b, out, eps, op, rows, bytes, bt, by, bz);
                 return;
             }
-            const uint32_t col_lds = flat ? std::min(op.cols, kOuterTile / run + 2u)
-                                          : op.span <= kOuterTile ? op.span : 4u;  // a longer column operand is not staged
-            LaunchScope scope("binary_outer_kernel", Op::name, bytes);
-            hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((n + kOuterTile - 1) / kOuterTile), dim3(kBlock),
-                               (op.row_lds + col_lds) * sizeof(float), st, a, b, out, eps, op);
-            return;
+            // an operand that keeps every dim of the item is laid out like the item
+            bool a_full = true, b_full = true;
+            uint64_t dense = 1;
+            for (int k = 0; k < d; k++) {
+                a_full = a_full && plan.astride[k] == dense; b_full = b_full && plan.bstride[k] == dense;
+                dense *= plan.size[k];
+            }
+            if ((a_full || b_full) && item % 4 == 0 && item >= 4096) {
+                BcastPlan inner = plan;
+                inner.ndim = d;
+                inner.a_stream = a_full; inner.b_stream = b_full;
+                LaunchScope scope("binary_bcast_mixed_kernel_batched", Op::name, bytes);
+                launch_mixed<Op>(a, b, out, static_cast<uint32_t>(item), eps, inner, a_full, b_full, bt, by, bz);
+                return;
+            }
         }
     }
+    hipStream_t st = state().stream;
     const uint32_t n4 = n >> 2;
     dim3 vec_grid(static_cast<uint32_t>((static_cast<uint64_t>(n4) + kBcastTile - 1) / kBcastTile));
     if (vec_ok) {
@@ -1029,13 +1110,7 @@ void launch_binary_bcast(const float* a, const float* b, float* out, uint32_t n,
         else if (b_vec)      hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n4, eps, plan);
         else                 hipLaunchKernelGGL((binary_bcast_vec_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n4, eps, plan);
     } else {
-        const uint64_t groups = (static_cast<uint64_t>(n) + 3) / 4;
-        dim3 grid(static_cast<uint32_t>((groups + kBcastTile - 1) / kBcastTile)), block(kBlock);
-        const bool al = plan.a_stream, bl = plan.b_stream;
-        if (al && bl)  hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, true>), grid, block, 0, st, a, b, out, n, eps, plan);
-        else if (al)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, true, false>), grid, block, 0, st, a, b, out, n, eps, plan);
-        else if (bl)   hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, true>), grid, block, 0, st, a, b, out, n, eps, plan);
-        else           hipLaunchKernelGGL((binary_bcast_mixed_kernel<Op, false, false>), grid, block, 0, st, a, b, out, n, eps, plan);
+        launch_mixed<Op>(a, b, out, n, eps, plan, plan.a_stream, plan.b_stream, no_batch, 1, 1);
     }
 }
 

@@ -2,12 +2,15 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
 #include <map>
 #include <mutex>
+#include <tuple>
+#include <utility>
 #include <vector>
 
 #include "../../include/kten_hip.h"
@@ -45,12 +48,22 @@ struct IndexUse {
     uint64_t n = 0;
 };
 
-// One profiled launch: which kernel, the algorithmic bytes it moved, its event pair.
+// One profiled launch: which kernel, the algorithmic bytes it moved, and the event pair that the launch itself
+// carries (hipExtLaunchKernel's start and stop events: the dispatch's own begin and end, no marker of its own on
+// the stream).
 struct LaunchRecord {
     const char* family;
     const char* op;
     uint64_t    bytes;
     hipEvent_t  begin, end;
+};
+
+// The launch bracket that is open (LaunchScope): the kernels launched inside it are recorded under its name.
+struct OpenScope {
+    bool        active = false;
+    const char* family = nullptr;
+    const char* op = nullptr;
+    uint64_t    bytes = 0;          // counted for the first launch of the scope
 };
 
 struct State {
@@ -97,6 +110,7 @@ struct State {
     std::vector<hipEvent_t> laps;           // kth_timer_lap events not yet read by kth_timer_laps
 
     bool profiling = false;
+    OpenScope scope;
     std::vector<LaunchRecord> records;      // launches of the current / last profile
     std::vector<hipEvent_t>   event_pool;   // idle events, reused across profiles
 };
@@ -163,9 +177,29 @@ public:
     ~LaunchScope();
     LaunchScope(const LaunchScope&) = delete;
     LaunchScope& operator=(const LaunchScope&) = delete;
-private:
-    int record_ = -1;
 };
+
+// The event pair for the kernel that is about to be launched, or two nulls: inside an open LaunchScope of a profile
+// that is being recorded, a new record under the scope's name (kth_runtime.hip).
+void events_for_launch(hipEvent_t* begin, hipEvent_t* end);
+
+// Every kernel of the library is launched through this (the macro below puts it in hipLaunchKernelGGL's place): the
+// arguments are converted to the kernel's parameter types and handed to hipExtLaunchKernel, with the event pair of
+// a running profile as the launch's own start and stop events. Outside a profile it is a plain launch.
+template <class... P, class... A, size_t... I>
+inline void launch_kernel_impl(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                               std::index_sequence<I...>, A&&... args) {
+    std::tuple<P...> params{static_cast<P>(std::forward<A>(args))...};
+    void* ptrs[sizeof...(P) > 0 ? sizeof...(P) : 1] = {static_cast<void*>(&std::get<I>(params))...};
+    hipEvent_t begin = nullptr, end = nullptr;
+    events_for_launch(&begin, &end);
+    (void)hipExtLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds, stream, begin, end, 0);
+}
+template <class... P, class... A>
+inline void launch_kernel(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t stream, A&&... args) {
+    static_assert(sizeof...(P) == sizeof...(A), "kernel launched with the wrong number of arguments");
+    launch_kernel_impl(kernel, grid, block, lds, stream, std::index_sequence_for<P...>{}, std::forward<A>(args)...);
+}
 
 #define KTH_REQUIRE_INIT()                                                         \
     do {                                                                           \
@@ -190,3 +224,7 @@ private:
 constexpr uint64_t kMaxElements = 0x7fffffffull;   // store size is a Kotlin Int
 
 }  // namespace kth
+
+#undef hipLaunchKernelGGL
+#define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
+    kth::launch_kernel(kernel, grid, block, lds, stream, __VA_ARGS__)

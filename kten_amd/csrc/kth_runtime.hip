@@ -158,11 +158,22 @@ LaunchScope::LaunchScope(const char* family, const char* op, uint64_t algorithmi
     s.launches += 1;
     s.bytes_moved += algorithmic_bytes;
     if (!s.profiling || !may_profile) return;
-    LaunchRecord r{family, op, algorithmic_bytes, take_event(), take_event()};
-    if (!r.begin || !r.end) return;
-    (void)hipEventRecord(r.begin, s.stream);
+    s.scope.active = true; s.scope.family = family; s.scope.op = op; s.scope.bytes = algorithmic_bytes;
+}
+
+void events_for_launch(hipEvent_t* begin, hipEvent_t* end) {
+    State& s = state();
+    *begin = nullptr; *end = nullptr;
+    if (!s.profiling || !s.scope.active) return;
+    LaunchRecord r{s.scope.family, s.scope.op, s.scope.bytes, take_event(), take_event()};
+    if (!r.begin || !r.end) {
+        if (r.begin) s.event_pool.push_back(r.begin);
+        if (r.end) s.event_pool.push_back(r.end);
+        return;
+    }
+    s.scope.bytes = 0;                       // a scope's bytes are those of all its launches together
     s.records.push_back(r);
-    record_ = static_cast<int>(s.records.size()) - 1;
+    *begin = r.begin; *end = r.end;
 }
 
 int report_deferred_index_error() {
@@ -177,11 +188,7 @@ int report_deferred_index_error() {
                                 "bounds at the axis (its target was updated up to that entry)");
 }
 
-LaunchScope::~LaunchScope() {
-    if (record_ < 0) return;
-    State& s = state();
-    (void)hipEventRecord(s.records[record_].end, s.stream);
-}
+LaunchScope::~LaunchScope() { state().scope.active = false; }
 
 }  // namespace kth
 

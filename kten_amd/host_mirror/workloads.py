@@ -260,6 +260,58 @@ def _bytes_reuse(d):
     return 4 * (2 * x + y + a + b + out)
 
 
+# ---- two operands that are both smaller than the output, in four dims or with a dim both keep ----
+
+# (a shape, b shape) at scale 1; the first dim of each pair's output is what `scale` divides for smaller runs
+BROADCAST_PAIRS = [([1, 196, 1, 2], [4, 1, 20452, 1]), ([246, 1, 4, 1], [1, 206, 4, 165]),
+                   ([111, 5496, 1], [111, 1, 55]), ([2481, 4, 1, 21], [1, 4, 161, 1])]
+
+
+def broadcast_pairs_at(scale):
+    def shrink(shape, lead):
+        s = list(shape)
+        if s[lead] > 1:
+            s[lead] = max(2, s[lead] // scale)
+        return s
+    out = []
+    for k, (sa, sb) in enumerate(BROADCAST_PAIRS):
+        lead = {0: 2, 1: 0, 2: 1, 3: 0}[k]          # the long dim of the pair: 20452, 246, 5496, 2481
+        out.append((shrink(sa, lead), shrink(sb, lead)))
+    return out
+
+
+def _in_pairs(d):
+    g = SplitMix64(17)
+    inp = {}
+    for k, (sa, sb) in enumerate(broadcast_pairs_at(d["scale"])):
+        inp[f"a{k}"] = g.uniform(sa, -1.0, 1.0); inp[f"b{k}"] = g.uniform(sb, 0.5, 1.5)
+    return inp
+
+
+def _run_pairs(ops, inp):
+    t = {k: ops.create(list(v.shape), False, v) for k, v in inp.items()}
+    return {"minus0": t["a0"] - t["b0"], "div1": t["a1"] / t["b1"], "times2": t["a2"] * t["b2"], "plus3": t["a3"] + t["b3"]}
+
+
+def _bytes_pairs(d):
+    total = 0
+    for sa, sb in broadcast_pairs_at(d["scale"]):
+        out = int(np.prod(np.broadcast_shapes(tuple(sa), tuple(sb))))
+        total += int(np.prod(sa)) + int(np.prod(sb)) + out
+    return 4 * total
+
+
+# ---- the column reduction of cfg5 by itself -------------------------------------------------------
+
+def _in_sum0(d):
+    return {"x": SplitMix64(4).normal([d["rows"], d["cols"]])}
+
+
+def _run_sum0(ops, inp):
+    x = ops.create(list(inp["x"].shape), False, inp["x"])
+    return {"sum0": x.sum(0)}
+
+
 # ---- fused batch normalisation ------------------------------------------------------------------
 
 def _in_bn(d):
@@ -496,6 +548,13 @@ WORKLOADS: Dict[str, Workload] = {
     "broadcast_reuse": Workload("broadcast_reuse", "x[32,2047,1020] + y[1,2047,1020] and a[1,6,4,56860] * b[23,1,4,56860]: operands of 8 MB and "
                                                    "5-21 MB that repeat along a dim, in shapes that are multiples of nothing; U(-1,1), seed 16",
                                 {"n": 32, "t": 2047, "h": 1020, "p": 23, "q": 6, "r": 4, "s": 56860}, _in_reuse, _run_reuse, _bytes_reuse),
+    "broadcast_pairs": Workload("broadcast_pairs", "four broadcasts of two operands that are both smaller than the 128-134 MB result and do not "
+                                                   "coalesce to an outer product: [1,196,1,2] - [4,1,20452,1], [246,1,4,1] / [1,206,4,165], "
+                                                   "[111,5496,1] * [111,1,55], [2481,4,1,21] + [1,4,161,1]; seed 17",
+                                {"scale": 1}, _in_pairs, _run_pairs, _bytes_pairs),
+    "sum0_alone": Workload("sum0_alone", "x.sum(0) of x[16384,4096], N(0,1), seed 4: the column reduction of cfg5 with nothing before it "
+                                         "(the tensor was read, never written, by the launches before)",
+                           {"rows": 16384, "cols": 4096}, _in_sum0, _run_sum0, lambda d: 4 * (d["rows"] * d["cols"] + d["cols"])),
     "concat_mask": Workload("concat_mask", "concat([8192,4096],[8192,4096], axis=1); maskedFill(mask[8192], 0); range get "
                                            "of the right half; range fill of the left half; seed 9",
                             {"rows": 8192, "left": 4096, "right": 4096}, _in_cat, _run_cat, _bytes_cat),

@@ -155,6 +155,38 @@ def test_broadcast_of_two_small_operands_in_many_dims_bit_exact(sa, sb, gc):
             assert_bits_equal(raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}")
 
 
+# The same arrangements where the outermost one or two dims become batch dims of the grid and what is left inside them
+# is an outer product or a broadcast with one operand as large as the item: which kernel takes which, and items that
+# are no multiple of 4 floats (the outer-product kernel stores at dword addresses; the mixed kernel is not batched then).
+BATCHED_PAIRS = [
+    (([1, 19, 1, 2], [4, 1, 2045, 1]), "binary_outer_rows_kernel"),           # [N,1,V] o [1,M,1] under a batch dim of 4
+    (([46, 1, 4, 1], [1, 26, 4, 165]), "binary_bcast_mixed_kernel_batched"),  # b is as large as the item [26,4,165]
+    (([111, 549, 1], [111, 1, 55]), "binary_outer_kernel"),                   # a dim of 111 both keep, over [N,1] o [1,M]
+    (([248, 4, 1, 21], [1, 4, 161, 1]), "binary_outer_kernel"),               # two batch dims, items of 3381 floats
+    (([37, 3, 1, 7], [1, 3, 211, 1]), "binary_outer_kernel"),                 # items of 1477 floats
+    (([3, 70001, 1], [3, 1, 5]), "binary_outer_kernel"),
+    (([5, 1, 3, 1], [1, 900, 3, 17]), "binary_bcast_mixed_kernel_batched"),   # items of 45900 floats
+    (([5, 1, 3, 1], [1, 901, 3, 17]), "binary_bcast_mixed_kernel"),           # items of 45951 floats: not batched
+]
+
+
+@pytest.mark.parametrize("pair,kernel", BATCHED_PAIRS,
+                         ids=lambda v: "x".join(map(str, v[0])) + "_" + "x".join(map(str, v[1])) if isinstance(v, tuple) else v)
+def test_broadcast_with_outer_dims_as_batch_dims_bit_exact(pair, kernel, gc):
+    sa, sb = pair
+    rng = np.random.default_rng(sum(sa) * 17 + sum(sb))
+    a = rng.standard_normal(sa).astype(np.float32); b = rng.standard_normal(sb).astype(np.float32)
+    gc.profileBegin()
+    results = []
+    for op, f in (("minus", np.subtract), ("div", np.divide)):
+        for x, y in ((a, b), (b, a)):
+            results.append((raw(gc, x)._binary(op, raw(gc, y)).toArray(), f(x, y), f"{op} {list(x.shape)} {list(y.shape)}"))
+    kernels = gc.profileEnd()
+    assert any(k.startswith(kernel + "<") for k in kernels), f"expected {kernel}, saw {sorted(kernels)}"
+    for got, want, what in results:
+        assert_bits_equal(got, want, what)
+
+
 # An operand that repeats along a dim and holds megabytes inside it: the tiles of the output are taken chunk by chunk
 # across the repeats so that the operand's chunk stays in L2. Slices that end inside a tile and inside a chunk, repeats
 # over two dims, both operands repeating, a scalar innermost dim of the repeating operand.
