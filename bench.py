@@ -2,7 +2,7 @@
 """Benchmark of the kten-hip hot path on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg5] [--cpu-baseline/--no-cpu-baseline]
-                  [--no-kernel-events] [--no-cold] [--no-copy-ceiling]
+                  [--no-kernel-events] [--no-cold] [--no-copy-ceiling] [--no-other-configs] [--math-mode exact|within_2_ulp]
 
 A step is one pass of the chosen workload's raw-op sequence over device-resident
 synthetic inputs (kten_amd/host_mirror/workloads.py). The default workload is cfg5: the autograd
@@ -321,6 +321,8 @@ def main():
                     help="skip the dominant kernel's run over a rotation of untouched buffer sets")
     ap.add_argument("--no-copy-ceiling", dest="ceiling", action="store_false", default=True,
                     help="skip the device-to-device copy measurement")
+    ap.add_argument("--math-mode", default="within_2_ulp", choices=["exact", "within_2_ulp"],
+                    help="how the transcendental maps are evaluated (kth_set_math_mode); the library's default is within_2_ulp")
     ap.add_argument("--other-configs", dest="others", action="store_true", default=None,
                     help="after the headline workload, run cfg1-cfg4 for the same steps and warm-up and report them under "
                          "config.other_configs (the default when the headline is cfg5)")
@@ -338,7 +340,8 @@ def main():
     dims = wl.full_dims
     nbytes = wl.algorithmic_bytes(dims)
     ops = kten_amd.platform(0)
-    log(f"platform {ops.platformKey}: {ops.computeUnits} CUs, wave {ops.waveSize}, {ops.availableMemory / 2**30:.0f} GiB")
+    ops.setMathMode(args.math_mode)
+    log(f"platform {ops.platformKey}: {ops.computeUnits} CUs, wave {ops.waveSize}, {ops.availableMemory / 2**30:.0f} GiB; math mode {args.math_mode}")
     log(f"workload {wl.name}: {wl.description}; {nbytes} algorithmic bytes per step")
     t0 = time.perf_counter()
     inputs = wl.make_inputs(dims)
@@ -406,6 +409,7 @@ def main():
         "config": {"workload": f"{wl.name}: {wl.description}", "algorithmic_bytes_per_step": nbytes,
                    "fused_lower_bound_bytes": wl.fused_lower_bound_bytes(dims) if wl.fused_lower_bound_bytes else None,
                    "launches_per_step": launches,
+                   "math_mode": args.math_mode,
                    "fp32_elements_per_s": round(min(nbytes, counted) / 4 / (ms_per_step / 1e3)),
                    "fp32_elements_per_s_means": "the bytes of `value` / 4 per second: every fp32 value a launch reads or writes",
                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
