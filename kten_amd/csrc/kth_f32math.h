@@ -148,25 +148,20 @@ KTH_F32_FN ExpPair exp_pair(float a) {
     r.t.lo = fmaf(S, e.p, S - r.t.hi) + S * e.p_lo;
     const float rt = approx_rcp(r.t.hi);
     r.u = 0.0625f * rt;
-    r.u_lo = fmaf(-r.u, r.t.hi, 0.0625f) * rt;                            // (1/16 - u t) / t
+    // 1/16 = u (t_hi + t_lo) + residual: u_lo = (1/16 - u t_hi) / t_hi - u t_lo / t_hi
+    r.u_lo = fmaf(-r.u, r.t.hi, 0.0625f) * rt - (r.u * rt) * r.t.lo;
     return r;
 }
 
-// sinh (JVMRawTensor.kt:401). Below 1: x + x^3 H(x^2). From there on 2 (t - u): the difference of the large terms
-// by a fast two-sum (t >= u), the small terms added to its residual.
+// sinh (JVMRawTensor.kt:401): 2 (t - u), the difference of the large terms by a fast two-sum (t >= u), the small terms
+// added to its residual. t and u are each known to 2^-46 of themselves, so the difference holds down to |x| = 2^-12
+// (t - u = 2 sinh |x| >= 2^-11, error 2^-45); below that sinh x rounds to x itself (x^3 / 6 < 2^-26 x).
 KTH_F32_FN float sinh_(float x) {
     const float ax = fabsf(x);
-    const float z = ax * ax;
-    float h = fmaf(z, 1.6059044e-10f, 2.5052108e-08f);
-    h = fmaf(z, h, 2.7557319e-06f);
-    h = fmaf(z, h, 0.00019841270f);
-    h = fmaf(z, h, 0.0083333333f);
-    h = fmaf(z, h, 0.16666667f);
-    const float small = fmaf(ax * z, h, ax);
     const ExpPair v = exp_pair(fminf(ax, 89.5f));
     const float d = v.t.hi - v.u;
     const float large = 2.0f * (d + (((v.t.hi - d) - v.u) + (v.t.lo - v.u_lo)));
-    return x != x ? x : with_sign(ax < 1.0f ? small : large, x);
+    return x != x ? x : with_sign(ax < 0.000244140625f ? ax : large, x);
 }
 
 // cosh (JVMRawTensor.kt:403): 2 (t + u), no cancellation.
