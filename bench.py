@@ -21,8 +21,8 @@ Timing: W warm-up steps, then exactly K steps between two HIP events on the libr
 (kth_timer_begin / kth_timer_end): `value` and `ms_per_step` come from that region; a host-side wall
 clock around it is the cross-check. Median and minimum come from a second pass of K steps with an
 event after every step (kth_timer_lap; each such event costs the stream about 2 us, so the pass with
-them is not the one `value` is taken from). Per-kernel durations come from HIP event pairs the
-library records around every launch over a third pass of the same K steps (kth_profile_*).
+them is not the one `value` is taken from). Per-kernel durations come from the start and stop events
+that every launch of a third pass over the same K steps carries itself (kth_profile_*: the dispatch's own duration).
 With the default workload the other BASELINE configurations (cfg1-cfg4) are timed the same way after
 it and reported under config.other_configs.
 
@@ -268,8 +268,8 @@ def time_steps(ops, step, steps, warmup):
 
 
 def kernel_events(ops, step, steps):
-    """The same K steps again with a HIP event pair around every launch: {kernel: (launches, bytes, ms)}. Kept out of
-    the region `value` is computed from, because the event pairs themselves cost about a tenth of the step time."""
+    """The same K steps again with every launch carrying its own start and stop events (the dispatch's own duration,
+    as a kernel trace shows it): {kernel: (launches, bytes, ms)}. Kept out of the region `value` is computed from."""
     ops.profileBegin()
     ops.timerBegin()
     for _ in range(steps):
@@ -316,7 +316,7 @@ def main():
     ap.add_argument("--cpu-baseline", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu-baseline", dest="cpu", action="store_false")
     ap.add_argument("--no-kernel-events", dest="events", action="store_false", default=True,
-                    help="skip the second pass that brackets every launch with an event pair")
+                    help="skip the pass in which every launch carries its own start and stop events")
     ap.add_argument("--no-cold", dest="cold", action="store_false", default=True,
                     help="skip the dominant kernel's run over a rotation of untouched buffer sets")
     ap.add_argument("--no-copy-ceiling", dest="ceiling", action="store_false", default=True,
@@ -429,7 +429,7 @@ def main():
                                        "ctypes), per step, before it waited for the stream: close to ms_per_step means that the "
                                        "stream was waiting for the host at times",
                    "median_and_min": "from a second pass of K steps with an event after every step",
-                   "per_kernel_durations": "HIP event pair around every launch, over a third pass of the same K steps"
+                   "per_kernel_durations": "start and stop events carried by every launch (the dispatch's own duration), over a third pass of the same K steps"
                    if args.events else None},
         "roofline": roofline,
     }
@@ -440,8 +440,8 @@ def main():
         line["config"]["other_configs"] = {name: other_config(ops, name, args.steps, args.warmup)
                                            for name in ("cfg1", "cfg2", "cfg3", "cfg4") if name != args.config}
         line["config"]["other_configs_note"] = ("the other BASELINE configurations, same steps and warm-up, inputs resident: GBps = "
-                                                "min(algorithmic, moved) bytes / ms_per_step; dominant_* from an event pair around every "
-                                                "launch over a second pass (the pairs add about 2.5 us to a launch); no CPU baseline for them")
+                                                "min(algorithmic, moved) bytes / ms_per_step; dominant_* from the start and stop events every "
+                                                "launch of a further pass carries; no CPU baseline for them")
     if args.cpu:
         threads = min(16, os.cpu_count() or 1)
         log(f"timing the CPU restatement on {threads} threads of {os.cpu_count()} host cores ...")
