@@ -17,7 +17,9 @@
 //            171-177) in its order, writing the per-channel parameters.
 //   apply    one read (+ gradOut) and one write; the float expression of JVMBatchNorm.kt:88-90
 //            / :153-164, evaluated left to right without contraction, so given equal
-//            statistics the output bits equal the reference's.
+//            statistics the output bits equal the reference's. With long runs (NCHW images) the
+//            apply kernel does the finalize step itself, per workgroup, for the few channels
+//            its tile touches: two launches per pass instead of three.
 //
 // Sums accumulate in f64 in a fixed order: deterministic, and closer to the exact sums than
 // the reference's serial float accumulation.
@@ -313,89 +315,137 @@ __device__ __forceinline__ void fold_partials(const double* partial, uint32_t c,
     }
 }
 
-__global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float* __restrict__ x, const double* __restrict__ partial,
-                                                                    Geometry g, uint32_t segments, int by_cols, int training,
-                                                                    float momentum, float epsilon, float* running_mean, float* running_var,
-                                                                    const float* __restrict__ gamma, const float* __restrict__ beta,
-                                                                    float* __restrict__ current_mean, float* __restrict__ current_std,
-                                                                    ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch,
-                                                                    int alone) {
-    // one wave per channel, or one thread (alone = 1: over the partials; 2: over the channel's items themselves)
-    const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    if (c >= g.channels) return;
+// What the per-channel arithmetic of the forward pass needs beside the sums.
+struct ForwardChannelArgs {
+    Geometry g;
+    int training;
+    float momentum, epsilon;
+    float* running_mean;
+    float* running_var;
+    const float* gamma;
+    const float* beta;
+    float* current_mean;
+    float* current_std;
+};
+
+// The scalar float arithmetic of JVMBatchNorm.kt:57-85 for channel c from its two f64 sums, in the reference's order.
+// `publish`: also write the channel's outputs (current mean / std, the running statistics, which are read and
+// rewritten, so exactly one caller per channel may publish).
+__device__ __forceinline__ ForwardParams forward_channel(const float* __restrict__ x, uint32_t c, double s1, double s2,
+                                                         const ForwardChannelArgs& a, bool publish) {
     float mean, stdev = 0.0f;
-    double s1 = 0.0, s2 = 0.0;
-    if (training && alone == 2) fold_items(x, nullptr, g, c, false, static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]), s1, s2);
-    else if (training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
-    if (!alone && (threadIdx.x & 63) != 0) return;
-    if (training) {
-        const double n = static_cast<double>(g.per_channel);
-        const double k = static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]);
+    if (a.training) {
+        const double n = static_cast<double>(a.g.per_channel);
+        const double k = static_cast<double>(x[static_cast<uint64_t>(c) * a.g.inner]);
         mean = static_cast<float>(k + s1 / n);                                  // JVMBatchNorm.kt:57-58
         const double dm = static_cast<double>(mean) - k;
         double ssd = s2 - 2.0 * dm * s1 + n * dm * dm;
         if (ssd < 0.0) ssd = 0.0;
         const float sum = static_cast<float>(ssd);                              // :60-64
-        const float count = static_cast<float>(g.per_channel);
-        if (sum != 0.0f || epsilon != 0.0f) stdev = 1.0f / sqrtf(sum / count + epsilon);   // :66-68
-        current_mean[c] = mean;
-        current_std[c] = stdev;
-        if (running_mean != nullptr && running_var != nullptr) {                // :72-76
-            running_mean[c] = (momentum * mean) + ((1.0f - momentum) * running_mean[c]);
-            const float unbiased = sum / static_cast<float>(g.per_channel - 1);
-            running_var[c] = (momentum * unbiased) + ((1.0f - momentum) * running_var[c]);
+        const float count = static_cast<float>(a.g.per_channel);
+        if (sum != 0.0f || a.epsilon != 0.0f) stdev = 1.0f / sqrtf(sum / count + a.epsilon);   // :66-68
+        if (publish) {
+            a.current_mean[c] = mean;
+            a.current_std[c] = stdev;
+            if (a.running_mean != nullptr && a.running_var != nullptr) {        // :72-76
+                a.running_mean[c] = (a.momentum * mean) + ((1.0f - a.momentum) * a.running_mean[c]);
+                const float unbiased = sum / static_cast<float>(a.g.per_channel - 1);
+                a.running_var[c] = (a.momentum * unbiased) + ((1.0f - a.momentum) * a.running_var[c]);
+            }
         }
     } else {                                                                    // :78-81
-        mean = running_mean[c];
-        stdev = 1.0f / sqrtf(running_var[c] + epsilon);
-        current_mean[c] = 0.0f;
-        current_std[c] = 0.0f;
+        mean = a.running_mean[c];
+        stdev = 1.0f / sqrtf(a.running_var[c] + a.epsilon);
+        if (publish) {
+            a.current_mean[c] = 0.0f;
+            a.current_std[c] = 0.0f;
+        }
     }
     ForwardParams p;
     p.mean = mean; p.stdev = stdev;
-    p.gamma = gamma != nullptr ? gamma[c] : 1.0f;                               // :84-85
-    p.beta = beta != nullptr ? beta[c] : 0.0f;
+    p.gamma = a.gamma != nullptr ? a.gamma[c] : 1.0f;                           // :84-85
+    p.beta = a.beta != nullptr ? a.beta[c] : 0.0f;
+    return p;
+}
+
+__global__ __launch_bounds__(kBlock) void bn_finalize_forward_kernel(const float* __restrict__ x, const double* __restrict__ partial,
+                                                                    ForwardChannelArgs a, uint32_t segments, int by_cols,
+                                                                    ForwardParams* __restrict__ params, float* __restrict__ soa, uint32_t pitch,
+                                                                    int alone) {
+    // one wave per channel, or one thread (alone = 1: over the partials; 2: over the channel's items themselves)
+    const Geometry& g = a.g;
+    const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (c >= g.channels) return;
+    double s1 = 0.0, s2 = 0.0;
+    if (a.training && alone == 2) fold_items(x, nullptr, g, c, false, static_cast<double>(x[static_cast<uint64_t>(c) * g.inner]), s1, s2);
+    else if (a.training) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    if (!alone && (threadIdx.x & 63) != 0) return;
+    const ForwardParams p = forward_channel(x, c, s1, s2, a, true);
     params[c] = p;
     // the same by parameter, for layouts where neighbouring elements belong to neighbouring channels
     soa[c] = p.mean; soa[pitch + c] = p.stdev; soa[2 * pitch + c] = p.gamma; soa[3 * pitch + c] = p.beta;
 }
 
+struct BackwardChannelArgs {
+    Geometry g;
+    int have_sums, training;
+    float epsilon;
+    const float* running_mean;
+    const float* running_var;
+    const float* current_mean;
+    const float* current_std;
+    const float* gamma;
+    float* grad_gamma;
+    float* grad_beta;
+};
+
+// Mean and 1 / std of channel c as the backward pass takes them (JVMBatchNorm.kt:131-137).
+__device__ __forceinline__ void backward_channel_stats(uint32_t c, const BackwardChannelArgs& a, float& mean, float& stdev) {
+    if (a.training) { mean = a.current_mean[c]; stdev = a.current_std[c]; }
+    else {
+        mean = a.running_mean[c];
+        stdev = static_cast<float>(1.0 / sqrt(static_cast<double>(a.running_var[c] + a.epsilon)));
+    }
+}
+
+// The scalar float arithmetic of JVMBatchNorm.kt:139-152,171-177 for channel c; `publish`: also write gradGamma / gradBeta.
+__device__ __forceinline__ BackwardParams backward_channel(uint32_t c, float mean, float stdev, double s1, double s2,
+                                                           const BackwardChannelArgs& a, bool publish) {
+    float sum = 0.0f, dot = 0.0f;
+    if (a.have_sums) {
+        sum = static_cast<float>(s1);                                           // :139-147
+        dot = static_cast<float>(s2);
+    }
+    const float count = static_cast<float>(a.g.per_channel);
+    BackwardParams p;
+    p.mean = mean; p.stdev = stdev;
+    p.gamma = a.gamma != nullptr ? a.gamma[c] : 1.0f;
+    p.dot_std_sq = dot * stdev * stdev / count;                                 // :151
+    p.grad_mean = sum / count;                                                  // :152
+    p.pad0 = p.pad1 = p.pad2 = 0.0f;
+    if (publish) {
+        if (a.grad_gamma != nullptr) a.grad_gamma[c] = dot * stdev;             // :171-173
+        if (a.grad_beta != nullptr) a.grad_beta[c] = sum;                       // :175-177
+    }
+    return p;
+}
+
 __global__ __launch_bounds__(kBlock) void bn_finalize_backward_kernel(const float* __restrict__ x, const float* __restrict__ go,
-                                                                     const double* __restrict__ partial, Geometry g, uint32_t segments,
-                                                                     int by_cols, int have_sums, int training, float epsilon,
-                                                                     const float* __restrict__ running_mean, const float* __restrict__ running_var,
-                                                                     const float* __restrict__ current_mean, const float* __restrict__ current_std,
-                                                                     const float* __restrict__ gamma, float* __restrict__ grad_gamma,
-                                                                     float* __restrict__ grad_beta, BackwardParams* __restrict__ params,
+                                                                     const double* __restrict__ partial, BackwardChannelArgs a,
+                                                                     uint32_t segments, int by_cols, BackwardParams* __restrict__ params,
                                                                      float* __restrict__ soa, uint32_t pitch, int alone) {
+    const Geometry& g = a.g;
     const uint32_t c = alone ? blockIdx.x * kBlock + threadIdx.x : blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (c >= g.channels) return;
     double s1 = 0.0, s2 = 0.0;
     float mean, stdev;
-    if (training) { mean = current_mean[c]; stdev = current_std[c]; }           // JVMBatchNorm.kt:131-133
-    else {                                                                      // :134-137
-        mean = running_mean[c];
-        stdev = static_cast<float>(1.0 / sqrt(static_cast<double>(running_var[c] + epsilon)));
-    }
-    if (have_sums && alone == 2) fold_items(x, go, g, c, true, static_cast<double>(mean), s1, s2);
-    else if (have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
+    backward_channel_stats(c, a, mean, stdev);
+    if (a.have_sums && alone == 2) fold_items(x, go, g, c, true, static_cast<double>(mean), s1, s2);
+    else if (a.have_sums) fold_partials(partial, c, segments, by_cols != 0, g.channels * g.inner, g.inner, alone != 0, s1, s2);
     if (!alone && (threadIdx.x & 63) != 0) return;
-    float sum = 0.0f, dot = 0.0f;
-    if (have_sums) {
-        sum = static_cast<float>(s1);                                           // :139-147
-        dot = static_cast<float>(s2);
-    }
-    const float count = static_cast<float>(g.per_channel);
-    BackwardParams p;
-    p.mean = mean; p.stdev = stdev;
-    p.gamma = gamma != nullptr ? gamma[c] : 1.0f;
-    p.dot_std_sq = dot * stdev * stdev / count;                                 // :151
-    p.grad_mean = sum / count;                                                  // :152
-    p.pad0 = p.pad1 = p.pad2 = 0.0f;
+    const BackwardParams p = backward_channel(c, mean, stdev, s1, s2, a, true);
     params[c] = p;
     soa[c] = p.mean; soa[pitch + c] = p.stdev; soa[2 * pitch + c] = p.gamma; soa[3 * pitch + c] = p.dot_std_sq; soa[4 * pitch + c] = p.grad_mean;
-    if (grad_gamma != nullptr) grad_gamma[c] = dot * stdev;                     // :171-173
-    if (grad_beta != nullptr) grad_beta[c] = sum;                               // :175-177
 }
 
 // ---------------------------------------------------------------- apply
@@ -491,6 +541,75 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float* __restric
                 else if (MODE == 1) out[i] = bn_backward_training(x[i], go[i], bparams[c]);
                 else out[i] = bn_backward_inference(go[i], bparams[c]);
             }
+        }
+    }
+}
+
+// The apply kernel that does the finalize step itself, for tensors whose runs are long (inner % 4 == 0, a tile of a
+// workgroup inside at most kFoldChannels runs): wave w folds the partials of the w-th run the tile touches, in the
+// order the finalize kernel folds them, and lane 0 does the channel's scalar arithmetic: the same functions on the same
+// sums, hence the same parameters in every workgroup and the same bits as the two-launch form. The workgroup whose
+// tile holds the first float of a channel's first run publishes that channel's outputs. The tile's loads are issued
+// before the fold, whose few hundred bytes come from L2.
+constexpr uint32_t kFoldChannels = kBlock / 64;
+
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void bn_apply_folded_kernel(const float* __restrict__ x, const float* __restrict__ go, float* __restrict__ out,
+                                                                const double* __restrict__ partial, uint32_t segments,
+                                                                ForwardChannelArgs fa, BackwardChannelArgs ba, ApplyPlan pl) {
+    __shared__ ForwardParams fpar[kFoldChannels];
+    __shared__ BackwardParams bpar[kFoldChannels];
+    constexpr uint32_t per_block = kBlock * kApplyUnroll;
+    const uint32_t u0 = blockIdx.x * per_block;
+    const uint32_t u1 = u0 + per_block < pl.units ? u0 + per_block : pl.units;
+    const uint32_t base = u0 + threadIdx.x;
+    v4f vx[kApplyUnroll], vg[kApplyUnroll];
+#pragma unroll
+    for (int k = 0; k < kApplyUnroll; k++) {
+        const uint32_t i = base + k * kBlock;
+        if (i < pl.units) {
+            if (MODE != 2) vx[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(x) + i);
+            if (MODE != 0) vg[k] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(go) + i);
+        }
+    }
+    // runs are numbered through the tensor: run q is channel q % channels of outer index q / channels
+    const uint32_t q0 = (__umulhi(u0, pl.inner_div.mul) + u0) >> pl.inner_div.shift;
+    const uint32_t q1 = (__umulhi(u1 - 1, pl.inner_div.mul) + (u1 - 1)) >> pl.inner_div.shift;
+    const uint32_t q = q0 + (threadIdx.x >> 6);
+    if (q <= q1) {
+        const uint32_t o = (__umulhi(q, pl.channel_div.mul) + q) >> pl.channel_div.shift;
+        const uint32_t c = q - o * pl.channels;
+        const Geometry& g = MODE == 0 ? fa.g : ba.g;
+        // the run of outer index 0 starts the channel; its first unit lies in this tile unless the tile begins inside the run
+        const bool publish = o == 0 && (q > q0 || q * (g.inner / 4) == u0);
+        double s1 = 0.0, s2 = 0.0;
+        if (MODE == 0) {
+            if (fa.training) fold_partials(partial, c, segments, false, 0, 0, false, s1, s2);
+            if ((threadIdx.x & 63) == 0) fpar[q - q0] = forward_channel(x, c, s1, s2, fa, publish);
+        } else {
+            float mean, stdev;
+            backward_channel_stats(c, ba, mean, stdev);
+            if (ba.have_sums) fold_partials(partial, c, segments, false, 0, 0, false, s1, s2);
+            if ((threadIdx.x & 63) == 0) bpar[q - q0] = backward_channel(c, mean, stdev, s1, s2, ba, publish);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kApplyUnroll; k++) {
+        const uint32_t i = base + k * kBlock;
+        if (i < pl.units) {
+            const uint32_t at = ((__umulhi(i, pl.inner_div.mul) + i) >> pl.inner_div.shift) - q0;
+            v4f r;
+            if (MODE == 0) {
+                const ForwardParams p = fpar[at];
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = bn_forward(vx[k][e], p);
+            } else {
+                const BackwardParams p = bpar[at];
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = MODE == 1 ? bn_backward_training(vx[k][e], vg[k][e], p) : bn_backward_inference(vg[k][e], p);
+            }
+            reinterpret_cast<v4f*>(out)[i] = r;
         }
     }
 }
@@ -630,6 +749,29 @@ void launch_apply(const Geometry& g, uint64_t n, const float* x, const float* go
     else          hipLaunchKernelGGL((bn_apply_kernel<MODE, false, false>), grid, dim3(kBlock), 0, state().stream, x, go, out, fp, bp, pl);
 }
 
+// The finalize step rides in the apply kernel when the tile of an apply workgroup lies inside at most kFoldChannels runs
+// and a channel's partials are few enough to be folded by every workgroup that needs them.
+static bool can_fold(const Geometry& g, const StatsLaunch& st, bool have_partials) {
+    if (g.inner % 4 != 0 || 3 * (g.inner / 4) < static_cast<uint32_t>(kBlock * kApplyUnroll)) return false;
+    if (have_partials && (st.by_cols || st.segments > 64 || finalize_alone(g, st))) return false;
+    return true;
+}
+
+template <int MODE>
+void launch_apply_folded(const Geometry& g, uint64_t n, const float* x, const float* go, float* out, const double* partial, uint32_t segments,
+                         const ForwardChannelArgs& fa, const BackwardChannelArgs& ba) {
+    ApplyPlan pl{};
+    pl.units = static_cast<uint32_t>(n / 4);
+    pl.channels = g.channels;
+    pl.inner_div = make_div(g.inner / 4);
+    pl.channel_div = make_div(g.channels);
+    const uint32_t per_block = kBlock * kApplyUnroll;
+    const dim3 grid((pl.units + per_block - 1) / per_block);
+    const uint64_t bytes = (MODE == 0 ? 2 : MODE == 1 ? 3 : 2) * n * 4;
+    LaunchScope scope("bn_apply_folded_kernel", MODE == 0 ? "forward" : MODE == 1 ? "backward_training" : "backward_inference", bytes);
+    hipLaunchKernelGGL((bn_apply_folded_kernel<MODE>), grid, dim3(kBlock), 0, state().stream, x, go, out, partial, segments, fa, ba, pl);
+}
+
 uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
 
 }  // namespace
@@ -674,14 +816,22 @@ int kth_batch_norm_forward(uint64_t in, const int32_t* shape, int dims, int axis
     float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
     if (training && !direct) launch_stats<false>(st, si->ptr, nullptr, nullptr, partial, n);
-    {
-        LaunchScope scope("bn_finalize_forward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 4 : 0));
-        const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
-        const uint32_t per_block = alone ? kBlock : kBlock / 64;
-        hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
-                           si->ptr, partial, g, st.segments, st.by_cols ? 1 : 0, training ? 1 : 0, momentum, epsilon, rm, rv, ga, be, cm, cs, params, soa, pitch, alone);
+    ForwardChannelArgs fa{};
+    fa.g = g; fa.training = training ? 1 : 0; fa.momentum = momentum; fa.epsilon = epsilon;
+    fa.running_mean = rm; fa.running_var = rv; fa.gamma = ga; fa.beta = be; fa.current_mean = cm; fa.current_std = cs;
+    // (a result written over its own input keeps the two-launch form: the channel's shift is read from the input)
+    if (!direct && so->ptr != si->ptr && can_fold(g, st, training != 0)) {
+        launch_apply_folded<0>(g, n, si->ptr, nullptr, so->ptr, partial, st.segments, fa, BackwardChannelArgs{});
+    } else {
+        {
+            LaunchScope scope("bn_finalize_forward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 4 : 0));
+            const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
+            const uint32_t per_block = alone ? kBlock : kBlock / 64;
+            hipLaunchKernelGGL(bn_finalize_forward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
+                               si->ptr, partial, fa, st.segments, st.by_cols ? 1 : 0, params, soa, pitch, alone);
+        }
+        launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr, soa, pitch);
     }
-    launch_apply<0>(g, n, si->ptr, nullptr, so->ptr, params, nullptr, soa, pitch);
     workspace_release(reinterpret_cast<float*>(ws), cap);
     KTH_LAUNCH_CHECK("batch_norm_forward");
     return KTH_OK;
@@ -730,16 +880,24 @@ int kth_batch_norm_backward(uint64_t in, const int32_t* shape, int dims, int axi
     float* soa = reinterpret_cast<float*>(ws + aos_bytes);
     double* partial = reinterpret_cast<double*>(ws + params_bytes);
     if (need_sums && !direct) launch_stats<true>(st, si->ptr, sg->ptr, training ? cm : rm, partial, n);
-    {
-        LaunchScope scope("bn_finalize_backward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 8 : 0));
-        const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
-        const uint32_t per_block = alone ? kBlock : kBlock / 64;
-        hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
-                           si->ptr, sg ? sg->ptr : nullptr, partial, g, st.segments, st.by_cols ? 1 : 0, need_sums ? 1 : 0, training ? 1 : 0, epsilon, rm, rv, cm, cs, ga, gg, gb, params, soa, pitch, alone);
-    }
-    if (sgi) {
-        if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
-        else launch_apply<2>(g, n, nullptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
+    BackwardChannelArgs ba{};
+    ba.g = g; ba.have_sums = need_sums ? 1 : 0; ba.training = training ? 1 : 0; ba.epsilon = epsilon;
+    ba.running_mean = rm; ba.running_var = rv; ba.current_mean = cm; ba.current_std = cs; ba.gamma = ga; ba.grad_gamma = gg; ba.grad_beta = gb;
+    if (sgi && !direct && can_fold(g, st, need_sums)) {
+        if (training) launch_apply_folded<1>(g, n, si->ptr, sg->ptr, sgi->ptr, partial, st.segments, ForwardChannelArgs{}, ba);
+        else launch_apply_folded<2>(g, n, nullptr, sg->ptr, sgi->ptr, partial, st.segments, ForwardChannelArgs{}, ba);
+    } else {
+        {
+            LaunchScope scope("bn_finalize_backward_kernel", direct ? "from the items" : "", static_cast<uint64_t>(g.channels) * 32 + (direct ? n * 8 : 0));
+            const int alone = direct ? 2 : finalize_alone(g, st) ? 1 : 0;
+            const uint32_t per_block = alone ? kBlock : kBlock / 64;
+            hipLaunchKernelGGL(bn_finalize_backward_kernel, dim3((g.channels + per_block - 1) / per_block), dim3(kBlock), 0, state().stream,
+                               si->ptr, sg ? sg->ptr : nullptr, partial, ba, st.segments, st.by_cols ? 1 : 0, params, soa, pitch, alone);
+        }
+        if (sgi) {
+            if (training) launch_apply<1>(g, n, si->ptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
+            else launch_apply<2>(g, n, nullptr, sg->ptr, sgi->ptr, nullptr, params, soa, pitch);
+        }
     }
     workspace_release(reinterpret_cast<float*>(ws), cap);
     KTH_LAUNCH_CHECK("batch_norm_backward");
