@@ -670,17 +670,21 @@ __device__ __forceinline__ void stage_range(float* lds, uint32_t at, const float
     }
 }
 
-template <class Op>
+// A_ROW: operand a is the row operand (pl.a_is_row). RUN1: V = 1 (pl.run == 1, hence not pl.col_flat): no position
+// inside a run to keep track of. Both are facts of the launch; as template arguments they take the operand swap (for a
+// division: the second division) and the run's bookkeeping out of the loop over a thread's outputs.
+template <class Op, bool A_ROW, bool RUN1>
 __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __restrict__ a_, const float* __restrict__ b_,
                                                              float* __restrict__ out_, float eps, OuterPlan pl, Batch bt) {
     const float* a = a_; const float* b = b_; float* out = out_;
     move_to_batch_item(bt, a, b, out);
+    if (RUN1) { pl.run = 1; pl.col_flat = 0; }
     // sized at launch to what the shape needs (at most 56 KiB), so that short operands leave room for eight workgroups per CU
     extern __shared__ float outer_lds[];
     float* row_lds = outer_lds;
     float* col_lds = outer_lds + pl.row_lds;
-    const float* rowp = pl.a_is_row ? a : b;
-    const float* colp = pl.a_is_row ? b : a;
+    const float* rowp = A_ROW ? a : b;
+    const float* colp = A_ROW ? b : a;
     const uint32_t s = blockIdx.x * kOuterTile;
     const uint32_t len = min(kOuterTile, pl.n - s);
     const uint32_t i_lo = (__umulhi(s, pl.span_div.mul) + s) >> pl.span_div.shift;
@@ -727,8 +731,8 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
         const uint32_t e0 = s + g;
         const uint32_t i = (__umulhi(e0, pl.span_div.mul) + e0) >> pl.span_div.shift;
         uint32_t c = e0 - i * pl.span;                                     // column operand offset j * V + v
-        uint32_t col = (__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift;   // column index j
-        uint32_t v = c - col * pl.run;
+        uint32_t col = RUN1 ? c : (__umulhi(c, pl.run_div.mul) + c) >> pl.run_div.shift;   // column index j
+        uint32_t v = RUN1 ? 0u : c - col * pl.run;
         uint32_t row_base = (i - i_lo) * pl.run;
         float y[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (!staged) { y[0] = ahead[k].x; y[1] = ahead[k].y; y[2] = ahead[k].z; y[3] = ahead[k].w; }
@@ -737,9 +741,9 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
         for (int j = 0; j < 4; j++) {
             const float x = row_lds[row_base + v];
             const float yy = pl.col_flat ? col_lds[col >= j_lo ? col - j_lo : col + pl.cols - j_lo] : staged ? col_lds[c] : y[j];
-            r[j] = pl.a_is_row ? Op::apply(x, yy, eps) : Op::apply(yy, x, eps);
-            c++; v++;
-            if (v == pl.run) { v = 0; col++; }
+            r[j] = A_ROW ? Op::apply(x, yy, eps) : Op::apply(yy, x, eps);
+            c++;
+            if (!RUN1) { v++; if (v == pl.run) { v = 0; col++; } }
             if (c == pl.span) { c = 0; col = 0; row_base += pl.run; }
         }
         // (16 bytes at a dword address: a batch item may start anywhere)
@@ -754,7 +758,7 @@ __global__ __launch_bounds__(kBlock) void binary_outer_kernel(const float* __res
 // The rows' slice of the row operand (kOuterRows * run floats) is staged in LDS. Grid: (column blocks, row blocks).
 constexpr uint32_t kOuterRows = 8;
 constexpr uint32_t kOuterCols = kOuterTile / kOuterRows;      // 1024 column offsets: four per thread
-template <class Op>
+template <class Op, bool A_ROW>
 __global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* __restrict__ a_, const float* __restrict__ b_,
                                                                   float* __restrict__ out_, float eps, OuterPlan pl, uint32_t rows, Batch bt) {
     // (the grid's y counts row blocks here: one batch dim, on z)
@@ -762,8 +766,8 @@ __global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* 
     const float* b = b_ + static_cast<size_t>(blockIdx.z) * bt.b[1];
     float* out = out_ + static_cast<size_t>(blockIdx.z) * bt.out[1];
     extern __shared__ float outer_rows_lds[];
-    const float* rowp = pl.a_is_row ? a : b;
-    const float* colp = pl.a_is_row ? b : a;
+    const float* rowp = A_ROW ? a : b;
+    const float* colp = A_ROW ? b : a;
     const uint32_t i0 = blockIdx.y * kOuterRows;
     const uint32_t nrows = min(kOuterRows, rows - i0);
     const uint32_t c0 = blockIdx.x * kOuterCols + threadIdx.x * 4;
@@ -791,7 +795,7 @@ __global__ __launch_bounds__(kBlock) void binary_outer_rows_kernel(const float* 
         const float* xs = outer_rows_lds + r * pl.run;
         float res[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) res[j] = pl.a_is_row ? Op::apply(xs[v[j]], y[j], eps) : Op::apply(y[j], xs[v[j]], eps);
+        for (int j = 0; j < 4; j++) res[j] = A_ROW ? Op::apply(xs[v[j]], y[j], eps) : Op::apply(y[j], xs[v[j]], eps);
         float* to = out + static_cast<size_t>(i0 + r) * pl.span + c0;
         if (count == 4) *reinterpret_cast<v4f_unaligned*>(to) = v4f_unaligned{res[0], res[1], res[2], res[3]};
         else for (uint32_t j = 0; j < count; j++) to[j] = res[j];
@@ -1024,14 +1028,23 @@ void launch_outer(const float* a, const float* b, float* out, float eps, const O
     if (op.span >= 2048u && rows <= 65535u * kOuterRows && batch_y == 1) {
         LaunchScope scope("binary_outer_rows_kernel", Op::name, bytes);
         const dim3 grid((op.span + kOuterCols - 1) / kOuterCols, (rows + kOuterRows - 1) / kOuterRows, batch_z);
-        hipLaunchKernelGGL((binary_outer_rows_kernel<Op>), grid, dim3(kBlock), kOuterRows * op.run * sizeof(float), st, a, b, out, eps, op, rows, bt);
+        if (op.a_is_row) hipLaunchKernelGGL((binary_outer_rows_kernel<Op, true>), grid, dim3(kBlock), kOuterRows * op.run * sizeof(float), st, a, b, out, eps, op, rows, bt);
+        else             hipLaunchKernelGGL((binary_outer_rows_kernel<Op, false>), grid, dim3(kBlock), kOuterRows * op.run * sizeof(float), st, a, b, out, eps, op, rows, bt);
         return;
     }
     const uint32_t col_lds = op.col_flat ? std::min(op.cols, kOuterTile / op.run + 2u)
                                          : op.span <= kOuterTile ? op.span : 4u;  // a longer column operand is not staged
     LaunchScope scope("binary_outer_kernel", Op::name, bytes);
-    hipLaunchKernelGGL((binary_outer_kernel<Op>), dim3((op.n + kOuterTile - 1) / kOuterTile, batch_y, batch_z), dim3(kBlock),
-                       (op.row_lds + col_lds) * sizeof(float), st, a, b, out, eps, op, bt);
+    const dim3 grid((op.n + kOuterTile - 1) / kOuterTile, batch_y, batch_z);
+    const size_t lds = (op.row_lds + col_lds) * sizeof(float);
+    const bool run1 = op.run == 1 && !op.col_flat;
+    if (op.a_is_row) {
+        if (run1) hipLaunchKernelGGL((binary_outer_kernel<Op, true, true>), grid, dim3(kBlock), lds, st, a, b, out, eps, op, bt);
+        else      hipLaunchKernelGGL((binary_outer_kernel<Op, true, false>), grid, dim3(kBlock), lds, st, a, b, out, eps, op, bt);
+    } else {
+        if (run1) hipLaunchKernelGGL((binary_outer_kernel<Op, false, true>), grid, dim3(kBlock), lds, st, a, b, out, eps, op, bt);
+        else      hipLaunchKernelGGL((binary_outer_kernel<Op, false, false>), grid, dim3(kBlock), lds, st, a, b, out, eps, op, bt);
+    }
 }
 
 template <class Op>

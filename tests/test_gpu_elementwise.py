@@ -166,6 +166,8 @@ BATCHED_PAIRS = [
     (([37, 3, 1, 7], [1, 3, 211, 1]), "binary_outer_kernel"),                 # items of 1477 floats
     (([3, 70001, 1], [3, 1, 5]), "binary_outer_kernel"),
     (([5, 1, 3, 1], [1, 900, 3, 17]), "binary_bcast_mixed_kernel_batched"),   # items of 45900 floats
+    # two batch dims: the full operand has the outer one too, the small one the dim inside it
+    (([1, 40, 24, 1], [150, 1, 24, 171]), "binary_bcast_mixed_kernel_batched"),
     (([5, 1, 3, 1], [1, 901, 3, 17]), "binary_bcast_mixed_kernel"),           # items of 45951 floats: not batched
 ]
 
