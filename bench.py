@@ -278,6 +278,31 @@ def kernel_events(ops, step, steps):
     return ops.profileEnd(), ev_ms
 
 
+def compiled_host_cfg1(steps, warmup):
+    """cfg1 once more with the C++ mirror of the contract as the host (bench_host.cpp, built by __graft_entry__.build()):
+    with four launches of a few microseconds per step, the Python mirror's issue rate is what bench.py's own cfg1 figure
+    measures. Runs as a child process while this one is idle on the GPU; None (with the reason logged) when the program
+    is not built."""
+    import subprocess
+    exe = os.path.join(ROOT, "bench_host")
+    if not os.path.isfile(exe):
+        log("bench_host is not built (python -c 'import __graft_entry__ as g; g.build()'): no compiled-host figure for cfg1")
+        return None
+    try:
+        out = subprocess.run([exe, str(steps), str(warmup)], capture_output=True, text=True, timeout=120)
+    except (OSError, subprocess.TimeoutExpired) as e:
+        log(f"bench_host did not run: {e}")
+        return None
+    if out.returncode != 0:
+        log(f"bench_host failed ({out.returncode}): {out.stderr.strip()[-300:]}")
+        return None
+    r = json.loads(out.stdout.strip().splitlines()[-1])
+    r["frac_of_hbm_peak"] = round(r["GBps"] / HBM_PEAK_GBPS, 4)
+    log(f"cfg1 with a compiled host: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s ({100 * r['frac_of_hbm_peak']:.1f} % of peak), "
+        f"host issue {r['host_issue_ms_per_step']:.4f} ms/step")
+    return r
+
+
 def other_config(ops, name, steps, warmup):
     """One of the other BASELINE configurations for the same steps / warm-up: its step rate and its largest kernel."""
     from kten_amd.host_mirror.workloads import WORKLOADS
@@ -296,13 +321,16 @@ def other_config(ops, name, steps, warmup):
     dom, (n, b, ms) = max(kernels.items(), key=lambda kv: kv[1][2])
     log(f"{name}: {r['ms_per_step']:.4f} ms/step mean ({r['median_ms']:.4f} median, {r['min_ms']:.4f} min), {gbps:.0f} GB/s "
         f"({100 * gbps / HBM_PEAK_GBPS:.1f} % of peak), host issue {r['host_issue_ms']:.4f} ms/step; largest kernel {dom} {ms / n * 1e3:.1f} us")
-    return {"workload": wl.description, "algorithmic_bytes_per_step": nbytes, "moved_bytes_per_step": round(r["moved"]),
-            "launches_per_step": r["launches"],
-            "ms_per_step": round(r["ms_per_step"], 4), "ms_per_step_median": round(r["median_ms"], 4), "ms_per_step_min": round(r["min_ms"], 4),
-            "host_issue_ms_per_step": round(r["host_issue_ms"], 4),
-            "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
-            "dominant_kernel": dom, "dominant_avg_launch_us": round(ms / n * 1e3, 2), "dominant_GBps": round(b / ms / 1e6, 1),
-            "dominant_frac": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    res = {"workload": wl.description, "algorithmic_bytes_per_step": nbytes, "moved_bytes_per_step": round(r["moved"]),
+           "launches_per_step": r["launches"],
+           "ms_per_step": round(r["ms_per_step"], 4), "ms_per_step_median": round(r["median_ms"], 4), "ms_per_step_min": round(r["min_ms"], 4),
+           "host_issue_ms_per_step": round(r["host_issue_ms"], 4),
+           "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+           "dominant_kernel": dom, "dominant_avg_launch_us": round(ms / n * 1e3, 2), "dominant_GBps": round(b / ms / 1e6, 1),
+           "dominant_frac": round(b / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    if name == "cfg1":
+        res["compiled_host"] = compiled_host_cfg1(steps, warmup)
+    return res
 
 
 def main():
@@ -433,6 +461,9 @@ def main():
                    if args.events else None},
         "roofline": roofline,
     }
+    if args.config == "cfg1":
+        ops.sync()
+        line["config"]["compiled_host"] = compiled_host_cfg1(args.steps, args.warmup)
     if args.others:
         for t in resident:
             t.release()

@@ -40,8 +40,9 @@ int kth_measure_copy(uint64_t n_floats, int reps, float* memcpy_ms, float* kerne
 
 /* Per-kernel device timing, for benchmarks that must attribute the time of a region to
  * the kernels in it. No counterpart in the reference. Between kth_profile_begin and
- * kth_profile_end every kernel launch is bracketed by a HIP event pair on the internal
- * stream; kth_profile_end blocks until those launches have finished. Afterwards
+ * kth_profile_end every kernel launch carries its own start and stop events (the duration of
+ * the dispatch itself, as a kernel trace shows it); kth_profile_end blocks until those
+ * launches have finished. Afterwards
  * kth_profile_count gives the number of distinct kernels seen and kth_profile_entry the
  * name ("family<Op>"), launch count, algorithmic bytes and summed duration of one. */
 int kth_profile_begin(void);
