@@ -59,8 +59,12 @@ LAYOUTS = [([10, 3, 4, 5], 1), ([8, 16, 32, 32], 1), ([4, 6, 67], 1), ([4, 5, 25
 @pytest.mark.parametrize("affine,running", [(True, True), (False, False)])
 @pytest.mark.parametrize("shape,axis", LAYOUTS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else f"axis{v}")
 def test_training_mode_parity(shape, axis, affine, running, gc):
+    check_training_mode(shape, axis, affine, running, sum(shape) * 7 + axis, gc)
+
+
+def check_training_mode(shape, axis, affine, running, seed, gc):
     eps, momentum = 1e-3, 0.1
-    arrays = inputs_for(shape, axis, sum(shape) * 7 + axis, affine, running)
+    arrays = inputs_for(shape, axis, seed, affine, running)
     cpu = jo.JvmOracleOperations()
     g, c = make(gc, arrays), make(cpu, arrays)
     gop, cop = gc.batchNorm(axis, momentum, eps, True), cpu.batchNorm(axis, momentum, eps, True)
@@ -120,13 +124,43 @@ def test_training_mode_parity(shape, axis, affine, running, gc):
         "gradIn against the checker end to end"
 
 
+def long_run_layout(seed):
+    """A random layout whose runs are long enough for the apply kernels to do the finalize step themselves (a multiple
+    of 4 floats, 684 or more), or just not (every fourth seed): one or two dims inside the axis, up to two outside."""
+    rng = np.random.default_rng(9000 + seed)
+    run = int(rng.integers(171, 1200)) * 4
+    if seed % 4 == 3:
+        run = int(rng.integers(100, 171)) * 4 + int(rng.integers(0, 2)) * int(rng.integers(1, 4))
+    channels = int(rng.choice([1, 2, 3, 7, 16, 33, 130]))
+    outer = [int(rng.integers(1, 7)) for _ in range(int(rng.integers(0, 3)))]
+    inner = [run]
+    if run % 8 == 0 and rng.random() < 0.5:
+        inner = [2, run // 2] if rng.random() < 0.5 else [run // 4, 4]
+    while int(np.prod(outer + [channels] + inner)) > 3_000_000 and outer:
+        outer.pop()
+    if int(np.prod(outer, dtype=np.int64)) * run < 2:
+        outer = [2] + outer
+    return outer + [channels] + inner, len(outer)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_layouts_with_long_runs(seed, gc):
+    shape, axis = long_run_layout(seed)
+    check_training_mode(shape, axis, seed % 2 == 0, seed % 3 != 0, 31 * seed + 5, gc)
+    check_inference_mode(shape, axis, 77 * seed + 1, gc)
+
+
 @pytest.mark.parametrize("shape,axis", [([10, 3, 4, 5], 2), ([8, 16, 32, 32], 1), ([512, 40], 1), ([4, 6, 67], 1), ([3, 20000], 1), ([17000, 2, 2], 0)],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v, list) else f"axis{v}")
 def test_inference_mode_is_bit_exact(shape, axis, gc):
+    check_inference_mode(shape, axis, sum(shape) + 100 * axis, gc)
+
+
+def check_inference_mode(shape, axis, seed, gc):
     """No reduction feeds the inference output or input gradient, so they match the checker
     bit for bit; gradGamma / gradBeta are sums and go through the reduction bar."""
     eps = 1e-3
-    arrays = inputs_for(shape, axis, sum(shape) + 100 * axis, True, True)
+    arrays = inputs_for(shape, axis, seed, True, True)
     cpu = jo.JvmOracleOperations()
     g, c = make(gc, arrays), make(cpu, arrays)
     gop, cop = gc.batchNorm(axis, 0.1, eps, False), cpu.batchNorm(axis, 0.1, eps, False)
