@@ -1211,7 +1211,7 @@ int kth_get_math_mode(int* mode) {
 int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* sa = lookup(a, "kth_unary(a)");
+    Store* sa = lookup(a, "kth_unary(a)", true);
     if (!sa) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_unary(out)");
     if (!so) return KTH_E_HANDLE;
@@ -1271,7 +1271,7 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_scalar: op %d is not a binary op", op);
-    Store* sa = lookup_unsettled(a, "kth_scalar(a)");
+    Store* sa = lookup_unsettled(a, "kth_scalar(a)", true);
     if (!sa) return KTH_E_HANDLE;
     Store* so = lookup_unsettled(out, "kth_scalar(out)");
     if (!so) return KTH_E_HANDLE;
@@ -1289,9 +1289,15 @@ int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t 
     }
     settle(sa);
     if (so != sa) settle_for_overwrite(so, n);
+    const bool rev = reverse != 0;
+    // pow(x, 1) into a store of its own (the backward pass of a square asks for it) is a copy, and a copy is put off
+    // until one of the two stores is written
+    if (op == KTH_POW && !rev && c == 1.0f && so != sa && n == so->n_floats) {
+        make_alias(so, sa);
+        return KTH_OK;
+    }
     const float* pa = sa->ptr; float* po = so->ptr; uint32_t n32 = static_cast<uint32_t>(n);
     const float eps = state().epsilon;
-    const bool rev = reverse != 0;
     // pow with an exponent whose f64 result is exact or one correctly rounded operation needs no
     // transcendental: pow(x, 2) is the exact product x*x (48 bits fit a double), pow(x, 1) is x;
     // 3, 4, -1, -2 and 0.5 likewise.
@@ -1314,7 +1320,7 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n) {
     if (!is_binary_op(op)) return fail(KTH_E_ARGUMENT, "kth_binary_inplace: op %d is not a binary op", op);
     Store* sa = lookup_unsettled(a, "kth_binary_inplace(a)");
     if (!sa) return KTH_E_HANDLE;
-    Store* sb = lookup_unsettled(b, "kth_binary_inplace(b)");
+    Store* sb = lookup_unsettled(b, "kth_binary_inplace(b)", true);
     if (!sb) return KTH_E_HANDLE;
     if (n > sa->n_floats || n > sb->n_floats)
         return fail(KTH_E_SHAPE, "kth_binary_inplace: n=%llu exceeds a store (%llu, %llu)", (unsigned long long)n,
@@ -1360,9 +1366,9 @@ int kth_binary(int op,
     if (int rc = check_shape(ashape, adims, "kth_binary(a)", &an)) return rc;
     if (int rc = check_shape(bshape, bdims, "kth_binary(b)", &bn)) return rc;
     if (int rc = check_shape(oshape, odims, "kth_binary(out)", &on)) return rc;
-    Store* sa = lookup_unsettled(a, "kth_binary(a)");
+    Store* sa = lookup_unsettled(a, "kth_binary(a)", true);
     if (!sa) return KTH_E_HANDLE;
-    Store* sb = lookup_unsettled(b, "kth_binary(b)");
+    Store* sb = lookup_unsettled(b, "kth_binary(b)", true);
     if (!sb) return KTH_E_HANDLE;
     Store* so = lookup_unsettled(out, "kth_binary(out)");
     if (!so) return KTH_E_HANDLE;

@@ -39,6 +39,16 @@ struct Store {
     // it, so anything that could have changed the store's contents makes the next use check again.
     uint32_t index_valid_below = 0;
     uint64_t index_valid_n = 0;
+    // A copy that has not been made yet (copy on write). alias_of != 0: this store's n_floats values are those of the
+    // store in table slot alias_of - 1 (the source, which holds at least as many); `ptr` points at the source's memory,
+    // `own_ptr` keeps this store's own buffer, which nothing has touched. Whoever only reads the store reads through
+    // `ptr` and needs to know nothing. Before either side is written the copy is made (`break_aliases`, which every
+    // lookup does unless its caller says that it only reads); when the source is released first, a store that
+    // aliases it takes over its buffer. `dependents` counts the stores that alias this one. A whole-store kth_copy and
+    // pow with the exponent 1 (the backward pass of a square) create aliases instead of copies.
+    uint32_t alias_of = 0;
+    float*   own_ptr = nullptr;
+    uint32_t dependents = 0;
 };
 
 // The index operand of the indexed move that is about to be launched (set by its entry point, taken by the check).
@@ -121,10 +131,18 @@ std::mutex& lock();
 // Records the message for kth_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);
 
-// Handle -> store, or nullptr (with the error recorded). A fill the store is owed is launched first.
-Store* lookup(uint64_t handle, const char* what);
+// Handle -> store, or nullptr (with the error recorded). A fill the store is owed is launched first. Copies that were
+// put off (Store::alias_of) are made first on both sides, the store's own and those of the stores that alias it,
+// unless `only_reads` says that the caller will not write the store's memory: it then reads through `ptr` as ever.
+// A caller that passes only_reads takes `ptr` of its stores after all its lookups (a later lookup may move it).
+Store* lookup(uint64_t handle, const char* what, bool only_reads = false);
 // The same without launching an owed fill: for callers that fold, overwrite or drop it.
-Store* lookup_unsettled(uint64_t handle, const char* what);
+Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads = false);
+// Makes the copies that were put off around `st`: its own, if it aliases another store, and those of its dependents.
+void break_aliases(Store* st);
+// dst (no alias, no dependents, no owed fill: looked up for writing, and about to be overwritten whole) becomes a copy
+// of the first dst->n_floats values of src without a kernel. src holds at least as many values and is owed no fill.
+void make_alias(Store* dst, Store* src);
 // `lookup` for the index operand of an indexed move: keeps the store's record of having been checked as an index.
 Store* lookup_index(uint64_t handle, const char* what);
 // Launches the fill the store is owed, if any, on the library's stream.

@@ -973,9 +973,11 @@ int dispatch_reduce(int op, const float* in, float* out, uint32_t outer, uint32_
 // The argument checks of both axis entry points, then the launch.
 int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner) {
     if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "%s: op %d is not an aggregating operation", who, op);
-    Store* si = lookup_unsettled(in, who);
+    // (neither lookup makes a copy that was put off: the input is only read, and the output's are made below, once the
+    // entry point that launches nothing when it refuses has accepted the plan)
+    Store* si = lookup_unsettled(in, who, true);
     if (!si) return KTH_E_HANDLE;
-    Store* so = lookup_unsettled(out, who);
+    Store* so = lookup_unsettled(out, who, true);
     if (!so) return KTH_E_HANDLE;
     if (axis == 0) return fail(KTH_E_ARGUMENT, "%s: empty axis", who);
     if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
@@ -986,7 +988,7 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
     if (outer * axis * inner > si->n_floats || outer * inner > so->n_floats)
         return fail(KTH_E_ARGUMENT, "%s: [%llu,%llu,%llu] exceeds a store", who, (unsigned long long)outer,
                     (unsigned long long)axis, (unsigned long long)inner);
-    if (si->ptr == so->ptr) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", who);
+    if (si == so) return fail(KTH_E_ARGUMENT, "%s: output aliases the input", who);
     if (outer * inner == 0) return KTH_OK;
     // The entry point that creates nothing refuses a plan that does not fit its scratch before it launches anything,
     // the fill an operand may still be owed included.
@@ -999,6 +1001,7 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
         State& s = state();
         const bool profiling = s.profiling;
         if (use_static) s.profiling = false;
+        break_aliases(so);                // the output is written: copies that were put off around it are made first
         settle(si);
         settle_for_overwrite(so, outer * inner);
         s.profiling = profiling;
@@ -1057,7 +1060,7 @@ int kth_reduce_all(int op, uint64_t in, uint64_t n, uint64_t out) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     if (op != KTH_SUM && op != KTH_MEAN) return fail(KTH_E_ARGUMENT, "kth_reduce_all: op %d is not SUM or MEAN", op);
-    Store* si = lookup(in, "kth_reduce_all(in)");
+    Store* si = lookup(in, "kth_reduce_all(in)", true);
     if (!si) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_reduce_all(out)");
     if (!so) return KTH_E_HANDLE;

@@ -27,7 +27,38 @@ static inline uint64_t make_handle(uint32_t index, uint32_t generation) {
     return (static_cast<uint64_t>(generation) << 32) | static_cast<uint64_t>(index + 1);
 }
 
-Store* lookup_unsettled(uint64_t handle, const char* what) {
+static void launch_store_copy(const float* src, float* dst, uint64_t n);
+
+// The copy that `d` put off is made now: d's own buffer receives the source's values, on the library's stream, ahead
+// of whatever is launched next.
+static void materialize(Store* d) {
+    State& s = state();
+    Store& src = s.table[d->alias_of - 1];
+    d->ptr = d->own_ptr; d->own_ptr = nullptr; d->alias_of = 0;
+    src.dependents -= 1;
+    launch_store_copy(src.ptr, d->ptr, d->n_floats);
+}
+
+void break_aliases(Store* st) {
+    State& s = state();
+    if (st->alias_of != 0) materialize(st);
+    if (st->dependents != 0) {
+        const uint32_t me = static_cast<uint32_t>(st - s.table.data()) + 1;
+        for (Store& d : s.table)
+            if (d.refs > 0 && d.alias_of == me) materialize(&d);
+    }
+}
+
+void make_alias(Store* dst, Store* src) {
+    State& s = state();
+    if (src->alias_of != 0) src = &s.table[src->alias_of - 1];      // an alias of an alias is an alias of its source
+    dst->own_ptr = dst->ptr;
+    dst->ptr = src->ptr;
+    dst->alias_of = static_cast<uint32_t>(src - s.table.data()) + 1;
+    src->dependents += 1;
+}
+
+Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads) {
     State& s = state();
     uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
     uint32_t gen = static_cast<uint32_t>(handle >> 32);
@@ -42,6 +73,7 @@ Store* lookup_unsettled(uint64_t handle, const char* what) {
     }
     st.index_valid_below = 0;          // whoever takes the store may write it: its values are unknown again
     st.index_valid_n = 0;
+    if (!only_reads && (st.alias_of != 0 || st.dependents != 0)) break_aliases(&st);
     return &st;
 }
 
@@ -57,8 +89,8 @@ void settle_for_overwrite(Store* st, uint64_t n) {
     else settle(st);
 }
 
-Store* lookup(uint64_t handle, const char* what) {
-    Store* st = lookup_unsettled(handle, what);
+Store* lookup(uint64_t handle, const char* what, bool only_reads) {
+    Store* st = lookup_unsettled(handle, what, only_reads);
     if (st) settle(st);
     return st;
 }
@@ -203,8 +235,10 @@ const char* kth_last_error(void) { return tl_error; }
 static void teardown() {
     State& s = state();
     if (s.stream) (void)hipStreamSynchronize(s.stream);
-    for (Store& st : s.table)
-        if (st.refs > 0 && st.ptr) (void)hipFree(st.ptr);
+    for (Store& st : s.table) {
+        float* mine = st.alias_of != 0 ? st.own_ptr : st.ptr;       // an aliasing store's `ptr` is its source's buffer
+        if (st.refs > 0 && mine) (void)hipFree(mine);
+    }
     s.table.clear();
     s.free_slots.clear();
     trim_pool();
@@ -324,6 +358,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
     else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); s.table.back().generation = g_epoch << 20; }
     Store& st = s.table[idx];
     st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1; st.fill_n = 0; st.index_valid_below = 0; st.index_valid_n = 0;
+    st.alias_of = 0; st.own_ptr = nullptr; st.dependents = 0;
     s.live_bytes += cap;
     *handle = make_handle(idx, st.generation);
     return KTH_OK;
@@ -332,7 +367,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
 int kth_retain(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup_unsettled(handle, "kth_retain");
+    Store* st = lookup_unsettled(handle, "kth_retain", true);
     if (!st) return KTH_E_HANDLE;
     st->refs += 1;
     return KTH_OK;
@@ -341,11 +376,32 @@ int kth_retain(uint64_t handle) {
 int kth_release(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup_unsettled(handle, "kth_release");      // a fill nobody read is never launched
+    Store* st = lookup_unsettled(handle, "kth_release", true);      // a fill nobody read is never launched, a copy nobody read never made
     if (!st) return KTH_E_HANDLE;
     st->refs -= 1;
     if (st->refs == 0) {
         State& s = state();
+        if (st->alias_of != 0) {
+            s.table[st->alias_of - 1].dependents -= 1;
+            st->ptr = st->own_ptr; st->own_ptr = nullptr; st->alias_of = 0;
+        }
+        if (st->dependents != 0) {
+            // The stores that alias this one need its values: the first whose own buffer is of this one's size class
+            // takes this buffer over and gives its untouched one back in its place; the others get their copies now.
+            const uint32_t me = static_cast<uint32_t>(st - s.table.data()) + 1;
+            Store* heir = nullptr;
+            for (Store& d : s.table) {
+                if (d.refs == 0 || d.alias_of != me) continue;
+                if (!heir && d.cap_bytes == st->cap_bytes) heir = &d;
+                else materialize(&d);
+            }
+            if (heir) {
+                float* values = st->ptr;
+                st->ptr = heir->own_ptr;
+                heir->ptr = values; heir->own_ptr = nullptr; heir->alias_of = 0;
+                st->dependents -= 1;
+            }
+        }
         s.pool[st->cap_bytes].push_back(st->ptr);
         s.live_bytes -= st->cap_bytes;
         s.pool_bytes += st->cap_bytes;
@@ -413,7 +469,7 @@ int kth_upload(uint64_t handle, uint64_t offset, const float* src, uint64_t n) {
 int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup(handle, "kth_download");
+    Store* st = lookup(handle, "kth_download", true);
     if (!st) return KTH_E_HANDLE;
     if (int rc = check_range(st, offset, n, "kth_download")) return rc;
     if (n != 0 && !dst) return fail(KTH_E_ARGUMENT, "kth_download: null destination");
@@ -464,12 +520,23 @@ __global__ __launch_bounds__(256) void copy_any_kernel(const float* __restrict__
 
 }  // namespace
 
+extern "C++" {
+namespace kth {
+static void launch_store_copy(const float* src, float* dst, uint64_t n) {
+    if (n == 0) return;
+    LaunchScope scope("copy_kernel", "copy on write", n * 8);
+    const uint32_t blocks = static_cast<uint32_t>(((n >> 2) + 255) / 256);
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks == 0 ? 1 : blocks), dim3(256), 0, state().stream, src, dst, static_cast<uint32_t>(n));
+}
+}  // namespace kth
+}
+
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     Store* d = lookup_unsettled(dst, "kth_copy(dst)");
     if (!d) return KTH_E_HANDLE;
-    Store* sst = lookup_unsettled(src, "kth_copy(src)");
+    Store* sst = lookup_unsettled(src, "kth_copy(src)", true);
     if (!sst) return KTH_E_HANDLE;
     if (int rc = check_range(d, dst_offset, n, "kth_copy(dst)")) return rc;
     if (int rc = check_range(sst, src_offset, n, "kth_copy(src)")) return rc;
@@ -482,6 +549,11 @@ int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offse
     }
     settle(sst);
     if (d != sst && dst_offset == 0) settle_for_overwrite(d, n); else settle(d);
+    if (d != sst && dst_offset == 0 && src_offset == 0 && n == d->n_floats) {
+        // the whole destination from the head of the source (copy(shallow = false)): put off until one of the two is written
+        make_alias(d, sst);
+        return KTH_OK;
+    }
     if (d->ptr == sst->ptr) {
         uint64_t lo = dst_offset < src_offset ? dst_offset : src_offset;
         uint64_t hi = dst_offset < src_offset ? src_offset : dst_offset;

@@ -156,6 +156,13 @@ class Program:
         i = self.add(sa.g._scalar(name, v, rev), sa.c._scalar(name, v, rev))
         self.note(f"s{i} = s{a} {name} {v}{' reversed' if rev else ''}")
 
+    def op_pow_one(self):
+        """pow with the exponent 1, which the library answers with a copy that it puts off."""
+        a = self.pick()
+        sa = self.slots[a]
+        i = self.add(sa.g._scalar("pow", 1.0), sa.c._scalar("pow", 1.0), sa.bound)
+        self.note(f"s{i} = s{a} pow 1.0")
+
     def op_scalar_assign(self):
         a, name, v = self.pick(), str(self.rng.choice(BINARY)), float(self.rng.choice(CONSTANTS))
         sa = self.slots[a]
@@ -462,7 +469,7 @@ class Program:
             self.note(f"s{x}.store[0:{sx.size}] = new positions below {sx.bound}")
 
     TABLE = [("op_data", 5), ("op_fill", 6), ("op_zeros_like", 3), ("op_single", 2), ("op_binary", 10), ("op_binary_assign", 7),
-             ("op_scalar", 5), ("op_scalar_assign", 4), ("op_unary", 3), ("op_compare", 3), ("op_broadcast_to", 3), ("op_masked_fill", 2),
+             ("op_scalar", 5), ("op_pow_one", 3), ("op_scalar_assign", 4), ("op_unary", 3), ("op_compare", 3), ("op_broadcast_to", 3), ("op_masked_fill", 2),
              ("op_extreme", 5), ("op_gather", 4), ("op_scatter", 6), ("op_index_select", 3), ("op_index_add", 4), ("op_get_ranges", 2),
              ("op_set_ranges", 3), ("op_store_range", 3), ("op_narrow", 2), ("op_transpose", 2), ("op_permute", 2), ("op_concat", 2),
              ("op_copy", 4), ("op_inplace_fill", 3), ("op_resize", 1), ("op_release", 3), ("op_look", 1), ("op_change_an_index", 2)]
