@@ -133,7 +133,11 @@ int kth_download(float* dst, uint64_t handle, uint64_t offset, uint64_t n);
 /* getSingleValue (RAW:166) / Tensor.item(). Blocking. */
 int kth_read_scalar(uint64_t handle, uint64_t index, float* out);
 
-/* copy(shallow=false) (RAW:168, JVM:257-262) and contiguous slice moves. */
+/* copy(shallow=false) (RAW:168, JVM:257-262) and contiguous slice moves. A copy of the head of
+ * `src` that fills the whole of `dst` (what copy() asks for) is put off: dst holds src's values
+ * from this call on, but reads them from src's memory until either store is written, when the
+ * copy is made first; if src is released before that, dst takes over its buffer. Nothing of this
+ * shows in results; kth_metrics counts neither a launch nor bytes for a copy that was never made. */
 int kth_copy(uint64_t dst, uint64_t dst_offset, uint64_t src, uint64_t src_offset, uint64_t n);
 
 /* inplaceFill (RAW:244), zerosLike / zeroOut (OPS:24-26), createRawFill (OPS:18-20),
@@ -171,7 +175,10 @@ int kth_binary_inplace(int op, uint64_t a, uint64_t b, uint64_t n);
  * lt..neq(Float) (RAW:201-206; JVM:379-393): out[i] = a[i] op c. reverse != 0 computes
  * c op a[i]; the contract needs it for TensorOperations.pow(constant, raw) (OPS:39).
  * out == a is allowed and gives plusAssign/timesAssign/divAssign(Float)
- * (RAW:45,59,65; JVM:105-108,116,130,136). */
+ * (RAW:45,59,65; JVM:105-108,116,130,136). pow with c == 1 into a store of its own (the backward
+ * pass of pow(2) asks for it, `input pow constant - 1f`: kten-api/.../autograd/functions/
+ * BasicFunctions.kt:193-198) is a copy of a and
+ * is put off like the whole-store kth_copy. */
 int kth_scalar(int op, uint64_t a, float c, int reverse, uint64_t out, uint64_t n);
 
 /* unaryMinus, reciprocal, log (RAW:51,71,73; JVM:122,142,144) and exp..rsqrt
