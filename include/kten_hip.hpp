@@ -252,6 +252,15 @@ public:
 
     void sync() { check(kth_sync()); }
 
+    // Settings of the platform, as the Kotlin module would hold them as platform properties: the tolerance of eq / neq
+    // (JVMRawTensor.kt:375-377), the share of device memory the store pool may hold, and how the transcendental maps are
+    // evaluated (exact: the float kotlin.math returns, bit for bit; within two ulp: fp32 routines, the default).
+    enum class MathMode { EXACT = KTH_MATH_EXACT, WITHIN_2_ULP = KTH_MATH_WITHIN_2_ULP };
+    void setEpsilon(float eps) { check(kth_set_epsilon(eps)); }
+    void setMemoryUsageScaleHint(double fraction) { check(kth_set_memory_scale_hint(fraction)); }
+    void setMathMode(MathMode mode) { check(kth_set_math_mode(static_cast<int>(mode))); }
+    MathMode getMathMode() { int m = 0; check(kth_get_math_mode(&m)); return static_cast<MathMode>(m); }
+
 private:
     friend class HipRawTensor;
     void collect(const Raw& t) { if (collecting_) instances_.push_back(t); }

@@ -173,6 +173,35 @@ int main() {
         ops.markReleasableInGC(t1);
         t1->release();
     }
+    {
+        // The math mode: exact gives the float of the f64 routine (what kotlin.math's Float overloads return), the
+        // default stays within one ulp of it on these values; a copy is the source's values whoever is written next
+        // (the library puts the copy off until then).
+        auto gc = ops.garbageCollector();
+        std::vector<float> xs;
+        for (int i = 0; i < 4096; i++) xs.push_back(-6.0f + 12.0f * static_cast<float>(i) / 4095.0f);
+        Raw x = ops.createRaw({4096}, [&](int i) { return xs[static_cast<size_t>(i)]; });
+        expect(ops.getMathMode() == HipTensorOperations::MathMode::WITHIN_2_ULP, "the default math mode is within two ulp");
+        const std::vector<float> fast = x->tanh()->toVector();
+        ops.setMathMode(HipTensorOperations::MathMode::EXACT);
+        const std::vector<float> exact = x->tanh()->toVector();
+        ops.setMathMode(HipTensorOperations::MathMode::WITHIN_2_ULP);
+        bool exact_ok = true, fast_ok = true;
+        for (size_t i = 0; i < xs.size(); i++) {
+            const float want = static_cast<float>(std::tanh(static_cast<double>(xs[i])));
+            if (exact[i] != want) exact_ok = false;
+            if (!(std::fabs(fast[i] - want) <= std::fabs(std::nextafter(want, 2.0f) - want))) fast_ok = false;
+        }
+        expect(exact_ok, "tanh in mode exact is the rounded f64 tanh");
+        expect(fast_ok, "tanh in the default mode is within one ulp of it");
+        Raw c = x->copy();
+        Raw p = x->pow(1.0f);
+        x->timesAssign(2.0f);
+        const std::vector<float> cv = c->toVector(), pv = p->toVector(), xv = x->toVector();
+        bool kept = true;
+        for (size_t i = 0; i < xs.size(); i++) if (cv[i] != xs[i] || pv[i] != xs[i] || xv[i] != 2.0f * xs[i]) kept = false;
+        expect(kept, "copy() and pow(1) keep the source's values when the source is written afterwards");
+    }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed == 0 ? 0 : 1;
 }

@@ -77,7 +77,12 @@ SESSION = textwrap.dedent("""
     first = ctypes.c_uint64()
     abi.check(lib.kth_alloc(1000, ctypes.byref(first)))
     abi.check(lib.kth_fill(first, 0, 1000, 1.0))
-    abi.check(lib.kth_shutdown())                                              # frees live stores too
+    source, alias = ctypes.c_uint64(), ctypes.c_uint64()
+    abi.check(lib.kth_alloc(5000, ctypes.byref(source)))
+    abi.check(lib.kth_alloc(5000, ctypes.byref(alias)))
+    abi.check(lib.kth_upload(source, 0, np.ones(5000, np.float32).ctypes.data_as(ctypes.c_void_p), 5000))
+    abi.check(lib.kth_copy(alias, 0, source, 0, 5000))                         # a copy that is still put off ...
+    abi.check(lib.kth_shutdown())                                              # frees live stores too (each its own buffer, once)
     assert lib.kth_release(first) == abi.KTH_E_NOT_INIT
     abi.check(lib.kth_init(0))
     second = ctypes.c_uint64()
