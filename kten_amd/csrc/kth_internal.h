@@ -185,10 +185,10 @@ int report_deferred_index_error();
 // device symbols of the elementwise kernels. Called once from kth_init.
 hipError_t init_math_tables();
 
-// Brackets the launch of one kernel: counts it for kth_metrics and, while a profile is
-// being recorded, puts a HIP event before and after it on the library's stream (the events
-// are created on demand; may_profile = false leaves them out for callers that must not
-// create anything).
+// Brackets the launches of one entry point's kernel: counts it for kth_metrics and, while a profile is
+// being recorded, names the launches inside it, each of which then carries its own start and stop events
+// (events_for_launch; they are created on demand, and may_profile = false leaves them out for callers that
+// must not create anything).
 class LaunchScope {
 public:
     LaunchScope(const char* family, const char* op, uint64_t algorithmic_bytes, bool may_profile = true);
