@@ -946,7 +946,15 @@ int with_index_check(const char* what, F launch) {
     *s.host_index_flag = 0;
     if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: %s", what, hipGetErrorString(e));
     if (host_flag) return fail(KTH_E_ARGUMENT, "%s got invalid index, an index value is out of bounds at the axis", what);
-    if (use.store) { use.store->index_valid_below = use.axis_len; use.store->index_valid_n = use.n; }
+    if (use.store) {
+        use.store->index_valid_below = use.axis_len; use.store->index_valid_n = use.n;
+        // a copy that was put off reads its source's memory: the same holds for the source's first values
+        // (unsqueeze of a targets tensor makes such a copy every step, and the next step's copy inherits the record)
+        if (use.store->alias_of != 0) {
+            Store& src = s.table[use.store->alias_of - 1];
+            src.index_valid_below = use.axis_len; src.index_valid_n = use.n;
+        }
+    }
     return KTH_OK;
 }
 

@@ -35,8 +35,9 @@ struct Store {
     float    fill_value = 0.0f;
     // Set when an indexed move has checked floats [0, index_valid_n) of this store as index values and found every
     // one inside [0, index_valid_below), or when ARG_MAX / ARG_MIN wrote them: the next indexed move with an axis at
-    // least that long skips the check and its wait for the stream. Every lookup other than `lookup_index` clears
-    // it, so anything that could have changed the store's contents makes the next use check again.
+    // least that long skips the check and its wait for the stream. Every lookup other than `lookup_index` and those
+    // whose caller only reads the store clears it, so anything that could have changed the store's contents makes the
+    // next use check again.
     uint32_t index_valid_below = 0;
     uint64_t index_valid_n = 0;
     // A copy that has not been made yet (copy on write). alias_of != 0: this store's n_floats values are those of the
@@ -143,7 +144,8 @@ void break_aliases(Store* st);
 // dst (no alias, no dependents, no owed fill: looked up for writing, and about to be overwritten whole) becomes a copy
 // of the first dst->n_floats values of src without a kernel. src holds at least as many values and is owed no fill.
 void make_alias(Store* dst, Store* src);
-// `lookup` for the index operand of an indexed move: keeps the store's record of having been checked as an index.
+// `lookup` for the index operand of an indexed move, which is only read: keeps the store's record of having been
+// checked as an index.
 Store* lookup_index(uint64_t handle, const char* what);
 // Launches the fill the store is owed, if any, on the library's stream.
 void settle(Store* st);

@@ -56,6 +56,9 @@ void make_alias(Store* dst, Store* src) {
     dst->ptr = src->ptr;
     dst->alias_of = static_cast<uint32_t>(src - s.table.data()) + 1;
     src->dependents += 1;
+    // the same values: what is known of the source as an index tensor holds for the copy
+    dst->index_valid_below = src->index_valid_below;
+    dst->index_valid_n = src->index_valid_n < dst->n_floats ? src->index_valid_n : dst->n_floats;
 }
 
 Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads) {
@@ -71,9 +74,11 @@ Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads) {
         fail(KTH_E_HANDLE, "%s: handle 0x%llx was released", what, (unsigned long long)handle);
         return nullptr;
     }
-    st.index_valid_below = 0;          // whoever takes the store may write it: its values are unknown again
-    st.index_valid_n = 0;
-    if (!only_reads && (st.alias_of != 0 || st.dependents != 0)) break_aliases(&st);
+    if (!only_reads) {
+        st.index_valid_below = 0;      // whoever takes the store may write it: its values are unknown again
+        st.index_valid_n = 0;
+        if (st.alias_of != 0 || st.dependents != 0) break_aliases(&st);
+    }
     return &st;
 }
 
@@ -96,13 +101,8 @@ Store* lookup(uint64_t handle, const char* what, bool only_reads) {
 }
 
 Store* lookup_index(uint64_t handle, const char* what) {
-    State& s = state();
-    const uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
-    uint32_t below = 0; uint64_t n = 0;
-    if (low != 0 && low <= s.table.size()) { below = s.table[low - 1].index_valid_below; n = s.table[low - 1].index_valid_n; }
-    Store* st = lookup(handle, what);
-    if (st) { st->index_valid_below = below; st->index_valid_n = n; }
-    return st;
+    // the index operand is only read: the store keeps what is known of it, and a copy it has put off stays put off
+    return lookup(handle, what, true);
 }
 
 // Size classes: 512-byte granules up to 1 MiB, then 1/8-octave steps (at most 12.5 %

@@ -66,6 +66,45 @@ def test_gather_along_an_outer_axis_goes_through_rows(gc):
         gc.createRaw([5000, 70], x).gather(0, gc.createRaw([4500, 70], bad))
 
 
+def test_copies_of_an_index_share_what_is_known_of_it_until_one_side_changes(gc):
+    """A copy that the library has put off reads its source's memory: a check that passed on either side holds for both
+    (a targets tensor that is unsqueezed every step is checked once, not once per step); a change to either side after
+    the copy concerns that side alone."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal([50, 40]).astype(np.float32)
+    gx = gc.createRaw([50, 40], x)
+    idx = rng.integers(0, 40, size=[50, 12]).astype(np.float32)
+    want = np.take_along_axis(x, idx.astype(np.int64), axis=1)
+    src = gc.createRaw([50, 12], idx)
+    first = src.copy()
+    assert_bits_equal(gx.gather(1, first).toArray(), want, "gather by a copy")            # checked here, for both
+    assert_bits_equal(gx.gather(1, src).toArray(), want, "gather by the source")
+    second = src.copy()                                                                    # inherits the record
+    assert_bits_equal(gx.gather(1, second).toArray(), want, "gather by a later copy")
+    # the source changes: the copies keep the old, valid values; the source is checked again and fails
+    src._scalar_assign("plus", 30.0)
+    assert_bits_equal(gx.gather(1, first).toArray(), want, "first copy after the source changed")
+    assert_bits_equal(gx.gather(1, second).toArray(), want, "second copy after the source changed")
+    with pytest.raises(ValueError):
+        gx.gather(1, src)
+    # a copy changes: it is checked again and fails; source and sibling are untouched
+    src2 = gc.createRaw([50, 12], idx)
+    assert_bits_equal(gx.gather(1, src2).toArray(), want, "gather by a second source")
+    c1, c2 = src2.copy(), src2.copy()
+    c1._set_store_range(7, 1, 40.0)
+    with pytest.raises(ValueError):
+        gx.gather(1, c1)
+    assert_bits_equal(gx.gather(1, c2).toArray(), want, "sibling copy")
+    assert_bits_equal(gx.gather(1, src2).toArray(), want, "second source")
+    # a copy of invalid values is found invalid, and leaves no record on its source
+    bad = idx.copy(); bad[3, 3] = 40.0
+    sb = gc.createRaw([50, 12], bad)
+    with pytest.raises(ValueError):
+        gx.gather(1, sb.copy())
+    with pytest.raises(ValueError):
+        gx.gather(1, sb)
+
+
 def test_an_index_checked_once_is_checked_again_after_any_change(gc):
     """An index tensor that an indexed move found valid is not checked again while nothing touches it; every
     way of changing it (a range fill, an upload, an in-place op, a copy into it, a kernel writing it as its result)
