@@ -1255,7 +1255,7 @@ int kth_unary(int op, uint64_t a, uint64_t out, uint64_t n) {
 int kth_clamp(uint64_t a, uint64_t out, uint64_t n, float lo, float hi) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* sa = lookup(a, "kth_clamp(a)");
+    Store* sa = lookup(a, "kth_clamp(a)", true);
     if (!sa) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_clamp(out)");
     if (!so) return KTH_E_HANDLE;
@@ -1419,9 +1419,9 @@ int kth_masked_fill(uint64_t a, const int32_t* ashape, int adims, uint64_t mask,
     uint64_t an, mn;
     if (int rc = check_shape(ashape, adims, "kth_masked_fill(a)", &an)) return rc;
     if (int rc = check_shape(mshape, mdims, "kth_masked_fill(mask)", &mn)) return rc;
-    Store* sa = lookup(a, "kth_masked_fill(a)");
+    Store* sa = lookup(a, "kth_masked_fill(a)", true);
     if (!sa) return KTH_E_HANDLE;
-    Store* sm = lookup(mask, "kth_masked_fill(mask)");
+    Store* sm = lookup(mask, "kth_masked_fill(mask)", true);
     if (!sm) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_masked_fill(out)");
     if (!so) return KTH_E_HANDLE;
@@ -1449,7 +1449,7 @@ int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
     uint64_t sn, dn;
     if (int rc = check_shape(sshape, sdims, "kth_broadcast_to(src)", &sn)) return rc;
     if (int rc = check_shape(dshape, ddims, "kth_broadcast_to(dst)", &dn)) return rc;
-    Store* ss = lookup_unsettled(src, "kth_broadcast_to(src)");
+    Store* ss = lookup_unsettled(src, "kth_broadcast_to(src)", true);
     if (!ss) return KTH_E_HANDLE;
     Store* sd = lookup_unsettled(dst, "kth_broadcast_to(dst)");
     if (!sd) return KTH_E_HANDLE;
@@ -1486,7 +1486,7 @@ int kth_contains_nan(uint64_t handle, uint64_t n, int* out) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
     if (!out) return fail(KTH_E_ARGUMENT, "kth_contains_nan: null output");
-    Store* st = lookup(handle, "kth_contains_nan");
+    Store* st = lookup(handle, "kth_contains_nan", true);
     if (!st) return KTH_E_HANDLE;
     if (n > st->n_floats) return fail(KTH_E_ARGUMENT, "kth_contains_nan: n=%llu exceeds the store", (unsigned long long)n);
     *out = 0;

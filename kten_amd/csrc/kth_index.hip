@@ -1116,7 +1116,7 @@ int kth_gather(uint64_t in, const int32_t* in_shape, uint64_t index, const int32
     for (int d = 0; d < dims; d++)
         if (d != axis && index_shape[d] > in_shape[d])
             return fail(KTH_E_SHAPE, "kth_gather: index dim %d (%d) exceeds the input's (%d)", d, index_shape[d], in_shape[d]);
-    Store* si = lookup(in, "kth_gather(in)");
+    Store* si = lookup(in, "kth_gather(in)", true);
     if (!si) return KTH_E_HANDLE;
     Store* sx = lookup_index(index, "kth_gather(index)");
     if (!sx) return KTH_E_HANDLE;
@@ -1394,7 +1394,7 @@ static int scatter_common(int mode, uint64_t target, const int32_t* target_shape
     Store* sx = lookup_index(index, "kth_scatter(index)");
     if (!sx) return KTH_E_HANDLE;
     Store* ss = nullptr;
-    if (mode != 2) { ss = lookup(src, "kth_scatter(src)"); if (!ss) return KTH_E_HANDLE; }
+    if (mode != 2) { ss = lookup(src, "kth_scatter(src)", true); if (!ss) return KTH_E_HANDLE; }
     if (t_n > st->n_floats || idx_n > sx->n_floats || (ss && src_n > ss->n_floats))
         return fail(KTH_E_ARGUMENT, "kth_scatter: a shape needs more elements than its store holds");
     if (st->ptr == sx->ptr || (ss && st->ptr == ss->ptr)) return fail(KTH_E_ARGUMENT, "kth_scatter: target aliases an input");
@@ -1453,7 +1453,7 @@ int kth_index_select(uint64_t in, const int32_t* shape, int dims, int axis, uint
     if (int rc = rows_geometry("kth_index_select", shape, dims, axis, &outer, &inner, &total)) return rc;
     const uint64_t n_out = outer * k * inner;
     if (n_out > kMaxElements) return fail(KTH_E_ARGUMENT, "kth_index_select: more than 2^31-1 result elements");
-    Store* si = lookup(in, "kth_index_select(in)");
+    Store* si = lookup(in, "kth_index_select(in)", true);
     if (!si) return KTH_E_HANDLE;
     Store* sx = lookup_index(index, "kth_index_select(index)");
     if (!sx) return KTH_E_HANDLE;
@@ -1522,7 +1522,7 @@ int kth_index_add(uint64_t target, const int32_t* shape, int dims, int axis, uin
     if (!st) return KTH_E_HANDLE;
     Store* sx = lookup_index(index, "kth_index_add(index)");
     if (!sx) return KTH_E_HANDLE;
-    Store* ss = lookup(src, "kth_index_add(src)");
+    Store* ss = lookup(src, "kth_index_add(src)", true);
     if (!ss) return KTH_E_HANDLE;
     if (total > st->n_floats || k > sx->n_floats || n_src > ss->n_floats)
         return fail(KTH_E_ARGUMENT, "kth_index_add: a shape needs more elements than its store holds");

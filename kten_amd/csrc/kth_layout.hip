@@ -876,7 +876,7 @@ int permute_common(const char* what, uint64_t in, const int32_t* shape, int dims
             return fail(KTH_E_ARGUMENT, "%s: axes must name every dimension once", what);
         seen[axes[d]] = true;
     }
-    Store* si = lookup(in, what);
+    Store* si = lookup(in, what, true);
     if (!si) return KTH_E_HANDLE;
     Store* so = lookup(out, what);
     if (!so) return KTH_E_HANDLE;
@@ -964,7 +964,7 @@ int kth_get_range(uint64_t in, const int32_t* shape, int dims, const int32_t* fi
     KTH_REQUIRE_INIT();
     StridedDims box; uint64_t base, count, total;
     if (int rc = box_of("kth_get_range", shape, dims, first, last, &box, &base, &count, &total)) return rc;
-    Store* si = lookup(in, "kth_get_range(in)");
+    Store* si = lookup(in, "kth_get_range(in)", true);
     if (!si) return KTH_E_HANDLE;
     Store* so = lookup(out, "kth_get_range(out)");
     if (!so) return KTH_E_HANDLE;
@@ -987,7 +987,7 @@ int kth_set_range(uint64_t target, const int32_t* shape, int dims, const int32_t
                     static_cast<unsigned long long>(value_n), static_cast<unsigned long long>(count));
     Store* st = lookup(target, "kth_set_range(target)");
     if (!st) return KTH_E_HANDLE;
-    Store* sv = lookup(value, "kth_set_range(value)");
+    Store* sv = lookup(value, "kth_set_range(value)", true);
     if (!sv) return KTH_E_HANDLE;
     if (total > st->n_floats || value_n > sv->n_floats)
         return fail(KTH_E_ARGUMENT, "kth_set_range: a shape needs more elements than its store holds");
@@ -1021,7 +1021,7 @@ int kth_concat(const uint64_t* inputs, const int32_t* axis_lens, int n_inputs, c
     std::vector<const float*> ptrs;
     std::vector<uint64_t> runs;
     for (int i = 0; i < n_inputs; i++) {
-        Store* si = lookup(inputs[i], "kth_concat(input)");
+        Store* si = lookup(inputs[i], "kth_concat(input)", true);
         if (!si) return KTH_E_HANDLE;
         const uint64_t run = static_cast<uint64_t>(axis_lens[i]) * inner;
         if (outer * run > si->n_floats) return fail(KTH_E_ARGUMENT, "kth_concat: input %d needs more elements than its store holds", i);
