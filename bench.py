@@ -14,7 +14,9 @@ Prints ONE JSON line on stdout; everything else goes to stderr.
 op-at-a-time total of the reference's op list (operands at their un-broadcast size, every result
 once) and what the library's launches of that step really read and wrote. The second is smaller
 where a tensor that is one constant (a fresh zerosLike, the broadcast seed gradient) is never
-written out and read back; bytes that did not cross the memory bus are not counted as bandwidth.
+written out and read back, and where a copy (pow with the exponent 1 in the backward pass of a
+square, copy()) is never made because neither side is written while both are alive; bytes that did
+not cross the memory bus are not counted as bandwidth.
 `config` carries both totals.
 
 Timing: W warm-up steps, then exactly K steps between two HIP events on the library's own stream
@@ -447,7 +449,8 @@ def main():
                                   "the library's launches of one step read and wrote, summed from their own byte counts; "
                                   "algorithmic_bytes_per_step is the op-at-a-time total of the reference's op list. The two differ "
                                   "where the library does not write out a tensor that is one constant (a fresh zerosLike, the "
-                                  "broadcast seed gradient) and hands the constant to the consumer's kernel (fewer bytes moved: "
+                                  "broadcast seed gradient) and hands the constant to the consumer's kernel, or does not make a copy "
+                                  "that nobody writes to (pow 1 of a backward pass) (fewer bytes moved: "
                                   "the op-list total over time would count bytes that never crossed the memory bus and is not a "
                                   "bandwidth; ms_per_step shows the gain), and where it moves more than the op list names "
                                   "(transposed copies of a scatter along an outer axis)",
