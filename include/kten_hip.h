@@ -199,7 +199,12 @@ int kth_broadcast_to(uint64_t src, const int32_t* sshape, int sdims,
 /* aggregateOverAxis (RAW:75,92-119; JVM:154-225) on a tensor seen as
  * [outer, axis, inner] -> [outer, 1, inner]. op: KTH_SUM, KTH_MEAN, KTH_MAX, KTH_MIN,
  * KTH_ARG_MAX, KTH_ARG_MIN (indices stored as float, JVM:180; axis must be <= 2^24).
- * Deterministic: the same input gives the same bits on every call. */
+ * Deterministic: the same input gives the same bits on every call.
+ * A small SUM / MEAN may return before anything is launched: `out` is then owed the reduction,
+ * which runs when `out` is next read or `in` next written, or, when the next call sums `out`
+ * over what was the inner dim (the next step of the autograd reduce-to-shape, mayUnexpand, kten-api/.../
+ * autograd/functions/Utils.kt:14-41), as part of that call's one launch over `in`. The
+ * values every call sees are those of the calls made in order; `in` may be released first. */
 int kth_reduce_axis(int op, uint64_t in, uint64_t out, uint64_t outer, uint64_t axis, uint64_t inner);
 
 /* sum() / mean() (RAW:121-122; JVM:146-152) of n values into out[0]. op: KTH_SUM, KTH_MEAN. */

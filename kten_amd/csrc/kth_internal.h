@@ -50,6 +50,16 @@ struct Store {
     uint32_t alias_of = 0;
     float*   own_ptr = nullptr;
     uint32_t dependents = 0;
+    // A small axis SUM / MEAN that has not been launched yet: this store's first outer * inner values are owed the
+    // reduction of the store in table slot owed.src - 1 seen as [outer, axis, inner]. The step of a reduce-to-shape
+    // chain that follows (the same outer index, over what was the inner dim) is then one launch over the source instead
+    // of two, and an intermediate nobody else reads is never computed. The note holds the source (`holds`: the source's
+    // buffer outlives its handle's last release if need be; the handle itself is invalid from then on) and counts among
+    // its `dependents`:
+    // a write to the source launches the reduction first, like a copy that was put off. Whoever needs this store's
+    // values gets them through `lookup`, which launches the reduction unless its caller asks for the note itself.
+    struct OwedReduce { uint32_t src = 0; int op = 0; uint32_t outer = 0, axis = 0, inner = 0; } owed;
+    uint32_t holds = 0;        // notes on other stores that need this one's values: it is freed when refs and holds are both 0
 };
 
 // The index operand of the indexed move that is about to be launched (set by its entry point, taken by the check).
@@ -137,8 +147,15 @@ int fail(int code, const char* fmt, ...);
 // unless `only_reads` says that the caller will not write the store's memory: it then reads through `ptr` as ever.
 // A caller that passes only_reads takes `ptr` of its stores after all its lookups (a later lookup may move it).
 Store* lookup(uint64_t handle, const char* what, bool only_reads = false);
-// The same without launching an owed fill: for callers that fold, overwrite or drop it.
-Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads = false);
+// The same without launching an owed fill: for callers that fold, overwrite or drop it. `no_values`: the caller reads
+// no values either (it counts references, or takes an owed reduction as a note): a reduction the store is owed stays owed.
+Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads = false, bool no_values = false);
+// Launches what `st` put off: the copy of its source, or the reduction it is owed.
+void materialize(Store* st);
+// `out` (looked up for writing; no notes left on it) is owed the SUM / MEAN `op` of `in` seen as [outer, axis, inner].
+void owe_reduce(Store* out, Store* in, int op, uint32_t outer, uint32_t axis, uint32_t inner);
+// The reduction itself, on the library's stream (kth_reduce.hip): out = op over the axis of in[outer, axis, inner].
+int run_owed_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner);
 // Makes the copies that were put off around `st`: its own, if it aliases another store, and those of its dependents.
 void break_aliases(Store* st);
 // dst (no alias, no dependents, no owed fill: looked up for writing, and about to be overwritten whole) becomes a copy

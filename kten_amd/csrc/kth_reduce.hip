@@ -537,6 +537,49 @@ __global__ __launch_bounds__(kWave) void reduce_wave_slabs_kernel(const float* _
     }
 }
 
+// Two steps of a reduce-to-shape chain in one launch: [outer, axis, inner] -> [outer, inner] by R1 as above, and that
+// -> [outer] by R2 (the sum or mean over what was the inner dim), for inner a multiple of 4 below 256. The first step's
+// results are rounded to float as if they had been stored; the second adds them the way the small-rows plan of
+// reduce_rows_kernel would: lane c holds the four floats of 16-byte unit c and adds them in order, then the lanes are
+// folded by xor-shuffles (the lanes beyond the row add exact zeros), so the result has the bits of the two launches.
+template <class R1, class R2>
+__global__ __launch_bounds__(kWave) void reduce_wave_slabs_rows_kernel(const float* __restrict__ in, float* __restrict__ out, Geom g,
+                                                                      uint32_t groups, uint32_t row_lanes) {
+    using Acc = typename R1::Acc;
+    const uint32_t o = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t r = lane / groups, c = lane - r * groups;
+    const uint32_t col = c * 4;                              // inner % 4 == 0: no overlapping last group
+    Acc acc[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) acc[v] = R1::init();
+    if (r < row_lanes) {
+        const float* base = in + static_cast<size_t>(o) * g.axis * g.inner + col;
+        for (uint32_t a = r; a < g.axis; a += kSmallBatch * row_lanes) {
+            float4 w[kSmallBatch];
+#pragma unroll
+            for (uint32_t k = 0; k < kSmallBatch; k++) if (a + k * row_lanes < g.axis) w[k] = ld4_stream_unaligned(base + static_cast<size_t>(a + k * row_lanes) * g.inner);
+#pragma unroll
+            for (uint32_t k = 0; k < kSmallBatch; k++) {
+                const uint32_t aa = a + k * row_lanes;
+                if (aa < g.axis) { R1::step(acc[0], w[k].x, aa); R1::step(acc[1], w[k].y, aa); R1::step(acc[2], w[k].z, aa); R1::step(acc[3], w[k].w, aa); }
+            }
+        }
+    }
+    for (uint32_t step = row_lanes >> 1; step >= 1; step >>= 1) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[v] = R1::merge(acc[v], shfl_down_acc(acc[v], static_cast<int>(step * groups)));
+    }
+    typename R2::Acc second = R2::init();
+    if (lane < groups) {
+#pragma unroll
+        for (uint32_t v = 0; v < 4; v++) R2::step(second, R1::finish(acc[v], g.axis), col + v);
+    }
+#pragma unroll
+    for (int m = kWave / 2; m >= 1; m >>= 1) second = R2::merge(second, shfl_xor_acc(second, m));
+    if (lane == 0) out[o] = R2::finish(second, g.inner);
+}
+
 // ---------------------------------------------------------------- few rows: axis of 2 ... 7 over wide columns
 
 // With so short an axis a column gives a thread only a handful of loads, so a thread takes four
@@ -708,6 +751,21 @@ constexpr uint64_t kStreamMinSlab = 2048;
 constexpr uint64_t kSmallInputFloats = 1u << 20;
 constexpr uint64_t kSmallRowsFloats = 1u << 16;
 
+// Whether [outer, axis, inner] takes reduce_wave_slabs_kernel (a small input whose slabs a wave takes whole), and the
+// kernel's lane layout if so: most lanes of the wave at work, a lane's share of the axis in a few batches, and enough
+// waves that the tensor is not one wave's work.
+static bool wave_slabs_plan(uint32_t outer, uint32_t axis, uint32_t inner, uint32_t* groups_out, uint32_t* row_lanes_out) {
+    const uint64_t n_in = static_cast<uint64_t>(outer) * axis * inner;
+    if (!(n_in <= kSmallInputFloats && inner >= 4 && inner <= 4 * kWave && axis >= 2)) return false;
+    const uint32_t groups = (inner + 3) / 4;
+    uint32_t row_lanes = 1;
+    while (row_lanes * 2 * groups <= kWave && row_lanes * 2 <= axis) row_lanes <<= 1;
+    if (!(groups * row_lanes >= kWave / 2 && static_cast<uint64_t>(axis) * inner >= 512 && ceil_div(axis, row_lanes) <= 4 * kSmallBatch &&
+          (outer >= 16 || static_cast<uint64_t>(axis) * inner <= 16384))) return false;
+    *groups_out = groups; *row_lanes_out = row_lanes;
+    return true;
+}
+
 // use_static: partials go to the static scratch array (no pool, no events, nothing allocated);
 // a plan whose partials do not fit is refused before anything is launched.
 // plan_only: makes the plan, applies that refusal and returns without launching (in and out are not used).
@@ -738,15 +796,9 @@ int run_reduce(const float* in, float* out, uint32_t outer, uint32_t axis, uint3
     // 16-byte load per lane and no LDS tile; slabs get a wave each (reduce_wave_slabs_kernel).
     const uint64_t n_in = n_out * axis;
     const bool small_input = n_in <= kSmallInputFloats;
-    if (small_input && inner >= 4 && inner <= 4 * kWave && axis >= 2) {
-        const uint32_t groups = (inner + 3) / 4;
-        uint32_t row_lanes = 1;
-        while (row_lanes * 2 * groups <= kWave && row_lanes * 2 <= axis) row_lanes <<= 1;
-        // a lane's share of the axis in a few batches; enough waves that the tensor is not one wave's work
-        // most lanes of the wave at work; a lane's share of the axis in a few batches; and enough waves that the
-        // tensor is not one wave's work
-        if (groups * row_lanes >= kWave / 2 && static_cast<uint64_t>(axis) * inner >= 512 && ceil_div(axis, row_lanes) <= 4 * kSmallBatch &&
-            (outer >= 16 || static_cast<uint64_t>(axis) * inner <= 16384)) {
+    {
+        uint32_t groups, row_lanes;
+        if (wave_slabs_plan(outer, axis, inner, &groups, &row_lanes)) {
             if (plan_only) return KTH_OK;
             hipError_t e;
             {
@@ -975,9 +1027,10 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
     if (op < KTH_SUM || op > KTH_ARG_MIN) return fail(KTH_E_ARGUMENT, "%s: op %d is not an aggregating operation", who, op);
     // (neither lookup makes a copy that was put off: the input is only read, and the output's are made below, once the
     // entry point that launches nothing when it refuses has accepted the plan)
-    Store* si = lookup_unsettled(in, who, true);
+    // (... nor do they launch a small reduction that was put off: the step after it may take it along, below)
+    Store* si = lookup_unsettled(in, who, true, true);
     if (!si) return KTH_E_HANDLE;
-    Store* so = lookup_unsettled(out, who, true);
+    Store* so = lookup_unsettled(out, who, true, true);
     if (!so) return KTH_E_HANDLE;
     if (axis == 0) return fail(KTH_E_ARGUMENT, "%s: empty axis", who);
     if (outer > kMaxElements || axis > kMaxElements || inner > kMaxElements ||
@@ -995,16 +1048,54 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
     if (use_static)
         if (int rc = dispatch_reduce(op, nullptr, nullptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
                                      static_cast<uint32_t>(inner), true, true)) return rc;
+    const uint32_t o32 = static_cast<uint32_t>(outer), a32 = static_cast<uint32_t>(axis), i32 = static_cast<uint32_t>(inner);
+    const bool sums = op == KTH_SUM || op == KTH_MEAN;
     {
         // A fill the input is still owed is launched here, one the output is owed is dropped if the result
         // covers it; for the entry point that creates nothing, without the event pair of a running profile.
         State& s = state();
         const bool profiling = s.profiling;
         if (use_static) s.profiling = false;
-        break_aliases(so);                // the output is written: copies that were put off around it are made first
+        break_aliases(so);                // the output is written: what was put off around it is done first
+        so->index_valid_below = 0; so->index_valid_n = 0;      // (it was looked up as if only read)
+        // The input is itself a small sum that was put off, and this is the next step of its chain (the same outer
+        // index, over what was its inner dim): one launch over its source does both. Otherwise it is launched now.
+        const Store::OwedReduce first = si->owed;
+        const bool chain = !use_static && first.src != 0 && sums && first.outer == o32 && first.inner == a32 && i32 == 1;
+        if (first.src != 0 && !chain) materialize(si);
         settle(si);
         settle_for_overwrite(so, outer * inner);
         s.profiling = profiling;
+        if (chain) {
+            Store& src = s.table[first.src - 1];
+            uint32_t groups, row_lanes;
+            if (!wave_slabs_plan(first.outer, first.axis, first.inner, &groups, &row_lanes))
+                return fail(KTH_E_DEVICE, "%s: a reduction was put off that its kernel does not take", who);
+            const Geom g{first.outer, first.axis, first.inner, 1, first.axis};
+            LaunchScope scope("reduce_wave_slabs_rows_kernel", op == KTH_MEAN ? "RedMean" : "RedSum",
+                              (static_cast<uint64_t>(first.outer) * first.axis * first.inner + outer) * 4);
+            const dim3 grid(first.outer), block(kWave);
+            hipStream_t stream = s.stream;
+            if (first.op == KTH_SUM && op == KTH_SUM)        hipLaunchKernelGGL((reduce_wave_slabs_rows_kernel<RedSum, RedSum>), grid, block, 0, stream, src.ptr, so->ptr, g, groups, row_lanes);
+            else if (first.op == KTH_SUM)                    hipLaunchKernelGGL((reduce_wave_slabs_rows_kernel<RedSum, RedMean>), grid, block, 0, stream, src.ptr, so->ptr, g, groups, row_lanes);
+            else if (op == KTH_SUM)                          hipLaunchKernelGGL((reduce_wave_slabs_rows_kernel<RedMean, RedSum>), grid, block, 0, stream, src.ptr, so->ptr, g, groups, row_lanes);
+            else                                             hipLaunchKernelGGL((reduce_wave_slabs_rows_kernel<RedMean, RedMean>), grid, block, 0, stream, src.ptr, so->ptr, g, groups, row_lanes);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail(KTH_E_DEVICE, "%s: launch failed: %s", who, hipGetErrorString(e));
+            return KTH_OK;
+        }
+    }
+    // A small sum or mean that the next step of a reduce-to-shape chain could take along (the plan of a wave per slab;
+    // an inner dim that the small-rows plan would then fold, so that the two launches and the one give the same bits)
+    // is put off: the output is owed it. Whoever reads the output first has it launched; if that is the chain's next
+    // step, the two are one launch and this one's result is never written unless somebody else asks for it.
+    {
+        uint32_t groups, row_lanes;
+        if (!use_static && sums && i32 % 4 == 0 && i32 < 256 && outer * inner <= kSmallRowsFloats && si->alias_of == 0 &&
+            wave_slabs_plan(o32, a32, i32, &groups, &row_lanes)) {
+            owe_reduce(so, si, op, o32, a32, i32);
+            return KTH_OK;
+        }
     }
     const int rc = dispatch_reduce(op, si->ptr, so->ptr, static_cast<uint32_t>(outer), static_cast<uint32_t>(axis),
                                    static_cast<uint32_t>(inner), use_static);
@@ -1020,6 +1111,10 @@ int reduce_axis_checked(const char* who, bool use_static, int op, uint64_t in, u
 }  // namespace
 
 namespace kth {
+
+int run_owed_reduce(int op, const float* in, float* out, uint32_t outer, uint32_t axis, uint32_t inner) {
+    return dispatch_reduce(op, in, out, outer, axis, inner);
+}
 
 // Called by kth_init with `device` current: resolves this device's copy of the scratch array.
 hipError_t reduce_scratch_init(int device) {

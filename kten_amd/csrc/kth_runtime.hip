@@ -29,24 +29,90 @@ static inline uint64_t make_handle(uint32_t index, uint32_t generation) {
 
 static void launch_store_copy(const float* src, float* dst, uint64_t n);
 
-// The copy that `d` put off is made now: d's own buffer receives the source's values, on the library's stream, ahead
-// of whatever is launched next.
-static void materialize(Store* d) {
+static void free_store(Store* st);
+
+// A note (an owed reduction) no longer needs `st`: a store whose handle was released in the meantime is freed now.
+static void drop_hold(Store* st) {
+    st->holds -= 1;
+    if (st->refs == 0 && st->holds == 0) free_store(st);
+}
+
+// What `d` put off is done now, on the library's stream, ahead of whatever is launched next: d's own buffer receives
+// the copy of its source's values, or the reduction it is owed.
+void materialize(Store* d) {
     State& s = state();
-    Store& src = s.table[d->alias_of - 1];
-    d->ptr = d->own_ptr; d->own_ptr = nullptr; d->alias_of = 0;
-    src.dependents -= 1;
-    launch_store_copy(src.ptr, d->ptr, d->n_floats);
+    if (d->alias_of != 0) {
+        Store& src = s.table[d->alias_of - 1];
+        d->ptr = d->own_ptr; d->own_ptr = nullptr; d->alias_of = 0;
+        src.dependents -= 1;
+        launch_store_copy(src.ptr, d->ptr, d->n_floats);
+    } else if (d->owed.src != 0) {
+        Store& src = s.table[d->owed.src - 1];
+        const Store::OwedReduce o = d->owed;
+        d->owed = Store::OwedReduce{};
+        src.dependents -= 1;
+        (void)run_owed_reduce(o.op, src.ptr, d->ptr, o.outer, o.axis, o.inner);
+        drop_hold(&src);
+    }
+}
+
+void owe_reduce(Store* out, Store* in, int op, uint32_t outer, uint32_t axis, uint32_t inner) {
+    State& s = state();
+    out->owed.src = static_cast<uint32_t>(in - s.table.data()) + 1;
+    out->owed.op = op; out->owed.outer = outer; out->owed.axis = axis; out->owed.inner = inner;
+    in->dependents += 1;
+    in->holds += 1;
 }
 
 void break_aliases(Store* st) {
     State& s = state();
-    if (st->alias_of != 0) materialize(st);
+    if (st->alias_of != 0 || st->owed.src != 0) materialize(st);
     if (st->dependents != 0) {
         const uint32_t me = static_cast<uint32_t>(st - s.table.data()) + 1;
         for (Store& d : s.table)
-            if (d.refs > 0 && d.alias_of == me) materialize(&d);
+            if ((d.refs > 0 || d.holds > 0) && (d.alias_of == me || d.owed.src == me)) materialize(&d);
     }
+}
+
+// The last reference to `st` is gone: its notes are dropped, the stores that alias it are served, its buffer goes back
+// to the pool and its table slot is free for the next kth_alloc (a later generation).
+static void free_store(Store* st) {
+    State& s = state();
+    if (st->alias_of != 0) {
+        s.table[st->alias_of - 1].dependents -= 1;
+        st->ptr = st->own_ptr; st->own_ptr = nullptr; st->alias_of = 0;
+    }
+    if (st->owed.src != 0) {
+        Store& src = s.table[st->owed.src - 1];
+        st->owed = Store::OwedReduce{};
+        src.dependents -= 1;
+        drop_hold(&src);
+    }
+    if (st->dependents != 0) {
+        // The stores that alias this one need its values: the first whose own buffer is of this one's size class
+        // takes this buffer over and gives its untouched one back in its place; the others get their copies now.
+        // (A store that is owed a reduction of this one holds a reference to it: none is left when the last goes.)
+        const uint32_t me = static_cast<uint32_t>(st - s.table.data()) + 1;
+        Store* heir = nullptr;
+        for (Store& d : s.table) {
+            if ((d.refs == 0 && d.holds == 0) || d.alias_of != me) continue;
+            if (!heir && d.cap_bytes == st->cap_bytes) heir = &d;
+            else materialize(&d);
+        }
+        if (heir) {
+            float* values = st->ptr;
+            st->ptr = heir->own_ptr;
+            heir->ptr = values; heir->own_ptr = nullptr; heir->alias_of = 0;
+            st->dependents -= 1;
+        }
+    }
+    s.pool[st->cap_bytes].push_back(st->ptr);
+    s.live_bytes -= st->cap_bytes;
+    s.pool_bytes += st->cap_bytes;
+    st->ptr = nullptr;
+    st->fill_n = 0;
+    st->generation += 1;
+    s.free_slots.push_back(static_cast<uint32_t>(st - s.table.data()));
 }
 
 void make_alias(Store* dst, Store* src) {
@@ -61,7 +127,7 @@ void make_alias(Store* dst, Store* src) {
     dst->index_valid_n = src->index_valid_n < dst->n_floats ? src->index_valid_n : dst->n_floats;
 }
 
-Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads) {
+Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads, bool no_values) {
     State& s = state();
     uint32_t low = static_cast<uint32_t>(handle & 0xffffffffu);
     uint32_t gen = static_cast<uint32_t>(handle >> 32);
@@ -77,7 +143,9 @@ Store* lookup_unsettled(uint64_t handle, const char* what, bool only_reads) {
     if (!only_reads) {
         st.index_valid_below = 0;      // whoever takes the store may write it: its values are unknown again
         st.index_valid_n = 0;
-        if (st.alias_of != 0 || st.dependents != 0) break_aliases(&st);
+        if (st.alias_of != 0 || st.dependents != 0 || st.owed.src != 0) break_aliases(&st);
+    } else if (!no_values && st.owed.src != 0) {
+        materialize(&st);              // a reader needs the values
     }
     return &st;
 }
@@ -237,7 +305,7 @@ static void teardown() {
     if (s.stream) (void)hipStreamSynchronize(s.stream);
     for (Store& st : s.table) {
         float* mine = st.alias_of != 0 ? st.own_ptr : st.ptr;       // an aliasing store's `ptr` is its source's buffer
-        if (st.refs > 0 && mine) (void)hipFree(mine);
+        if ((st.refs > 0 || st.holds > 0) && mine) (void)hipFree(mine);
     }
     s.table.clear();
     s.free_slots.clear();
@@ -358,7 +426,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
     else { idx = static_cast<uint32_t>(s.table.size()); s.table.emplace_back(); s.table.back().generation = g_epoch << 20; }
     Store& st = s.table[idx];
     st.ptr = p; st.n_floats = n_floats; st.cap_bytes = cap; st.refs = 1; st.fill_n = 0; st.index_valid_below = 0; st.index_valid_n = 0;
-    st.alias_of = 0; st.own_ptr = nullptr; st.dependents = 0;
+    st.alias_of = 0; st.own_ptr = nullptr; st.dependents = 0; st.owed = Store::OwedReduce{}; st.holds = 0;
     s.live_bytes += cap;
     *handle = make_handle(idx, st.generation);
     return KTH_OK;
@@ -367,7 +435,7 @@ int kth_alloc(uint64_t n_floats, uint64_t* handle) {
 int kth_retain(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup_unsettled(handle, "kth_retain", true);
+    Store* st = lookup_unsettled(handle, "kth_retain", true, true);
     if (!st) return KTH_E_HANDLE;
     st->refs += 1;
     return KTH_OK;
@@ -376,39 +444,15 @@ int kth_retain(uint64_t handle) {
 int kth_release(uint64_t handle) {
     std::lock_guard<std::mutex> g(lock());
     KTH_REQUIRE_INIT();
-    Store* st = lookup_unsettled(handle, "kth_release", true);      // a fill nobody read is never launched, a copy nobody read never made
+    // (a fill nobody read is never launched, a copy nobody read never made, a reduction nobody read never run)
+    Store* st = lookup_unsettled(handle, "kth_release", true, true);
     if (!st) return KTH_E_HANDLE;
     st->refs -= 1;
     if (st->refs == 0) {
-        State& s = state();
-        if (st->alias_of != 0) {
-            s.table[st->alias_of - 1].dependents -= 1;
-            st->ptr = st->own_ptr; st->own_ptr = nullptr; st->alias_of = 0;
-        }
-        if (st->dependents != 0) {
-            // The stores that alias this one need its values: the first whose own buffer is of this one's size class
-            // takes this buffer over and gives its untouched one back in its place; the others get their copies now.
-            const uint32_t me = static_cast<uint32_t>(st - s.table.data()) + 1;
-            Store* heir = nullptr;
-            for (Store& d : s.table) {
-                if (d.refs == 0 || d.alias_of != me) continue;
-                if (!heir && d.cap_bytes == st->cap_bytes) heir = &d;
-                else materialize(&d);
-            }
-            if (heir) {
-                float* values = st->ptr;
-                st->ptr = heir->own_ptr;
-                heir->ptr = values; heir->own_ptr = nullptr; heir->alias_of = 0;
-                st->dependents -= 1;
-            }
-        }
-        s.pool[st->cap_bytes].push_back(st->ptr);
-        s.live_bytes -= st->cap_bytes;
-        s.pool_bytes += st->cap_bytes;
-        st->ptr = nullptr;
-        st->fill_n = 0;
-        st->generation += 1;
-        s.free_slots.push_back(static_cast<uint32_t>((handle & 0xffffffffu) - 1));
+        // The handle is invalid from here on. A store that notes on other stores still hold keeps its values until
+        // they are done with it.
+        if (st->holds == 0) free_store(st);
+        else if (st->alias_of != 0 || st->owed.src != 0) materialize(st);      // (a held store has its values; to be safe)
     }
     return KTH_OK;
 }

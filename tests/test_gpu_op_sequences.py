@@ -218,6 +218,21 @@ class Program:
                      sa.shape[axis] if name.startswith("arg") else sa.bound)
         self.note(f"s{i} = s{a}.{name}({axis}, keep={keep})")
 
+    def op_exact_sum(self):
+        """A sum of whole numbers that no float sum rounds: every order of adding gives the same bits. (The library puts
+        some small sums off and folds two steps of a chain into one launch; what reads or writes the tensors in
+        between must see the plain sequence.)"""
+        a = self.pick(lambda s: s.bound is not None and len(s.shape) >= 1)
+        sa = self.slots[a]
+        axis, keep = int(self.rng.integers(0, len(sa.shape))), bool(self.rng.random() < 0.6)
+        if len(sa.shape) == 1 and not keep:
+            keep = True
+        bound = (sa.bound - 1) * sa.shape[axis] + 1
+        if bound > (1 << 24):
+            raise NotApplicable()
+        i = self.add(sa.g.sum(axis, keep), sa.c.sum(axis, keep), bound)
+        self.note(f"s{i} = s{a}.sum({axis}, keep={keep})")
+
     # ------------------------------------------------------------------ indexed moves
     def index_for(self, target, axis, ishape=None):
         """A slot holding valid positions along `axis` of the slot `target`: an existing one that fits (and is not
@@ -470,7 +485,7 @@ class Program:
 
     TABLE = [("op_data", 5), ("op_fill", 6), ("op_zeros_like", 3), ("op_single", 2), ("op_binary", 10), ("op_binary_assign", 7),
              ("op_scalar", 5), ("op_pow_one", 3), ("op_scalar_assign", 4), ("op_unary", 3), ("op_compare", 3), ("op_broadcast_to", 3), ("op_masked_fill", 2),
-             ("op_extreme", 5), ("op_gather", 4), ("op_scatter", 6), ("op_index_select", 3), ("op_index_add", 4), ("op_get_ranges", 2),
+             ("op_extreme", 5), ("op_exact_sum", 4), ("op_gather", 4), ("op_scatter", 6), ("op_index_select", 3), ("op_index_add", 4), ("op_get_ranges", 2),
              ("op_set_ranges", 3), ("op_store_range", 3), ("op_narrow", 2), ("op_transpose", 2), ("op_permute", 2), ("op_concat", 2),
              ("op_copy", 4), ("op_inplace_fill", 3), ("op_resize", 1), ("op_release", 3), ("op_look", 1), ("op_change_an_index", 2)]
 
@@ -504,7 +519,7 @@ def run_program(seed, hip, cpu, dims, n_ops):
 
 
 SMALL = [[7, 5, 6], [3, 33], [2, 3, 4, 5], [65], [1, 9, 1], [12, 1, 17]]
-MEDIUM = [[64, 48, 40], [300, 257], [16, 8, 24, 20], [70001], [129, 1031], [9, 4096]]
+MEDIUM = [[64, 48, 40], [300, 257], [16, 8, 24, 20], [70001], [129, 1031], [9, 4096], [24, 56, 56], [130, 20, 1, 64]]
 
 
 @pytest.mark.parametrize("seed", range(240))
