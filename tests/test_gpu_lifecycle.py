@@ -82,6 +82,16 @@ SESSION = textwrap.dedent("""
     abi.check(lib.kth_alloc(5000, ctypes.byref(alias)))
     abi.check(lib.kth_upload(source, 0, np.ones(5000, np.float32).ctypes.data_as(ctypes.c_void_p), 5000))
     abi.check(lib.kth_copy(alias, 0, source, 0, 5000))                         # a copy that is still put off ...
+    big, owed, dropped = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
+    abi.check(lib.kth_alloc(64 * 40 * 100, ctypes.byref(big)))
+    abi.check(lib.kth_alloc(64 * 100, ctypes.byref(owed)))
+    abi.check(lib.kth_alloc(64 * 100, ctypes.byref(dropped)))
+    abi.check(lib.kth_fill(big, 0, 64 * 40 * 100, 0.5))
+    abi.check(lib.kth_reduce_axis(abi.Op.SUM, big, owed, 64, 40, 100))          # ... a small sum that is still put off,
+    abi.check(lib.kth_reduce_axis(abi.Op.SUM, big, dropped, 64, 40, 100))
+    abi.check(lib.kth_release(dropped))                                        # one that nobody will ever read
+    abi.check(lib.kth_release(big))                                            # and their source, kept for the first only
+    assert lib.kth_release(big) == abi.KTH_E_HANDLE, "released is released, whatever the library still keeps of it"
     abi.check(lib.kth_shutdown())                                              # frees live stores too (each its own buffer, once)
     assert lib.kth_release(first) == abi.KTH_E_NOT_INIT
     abi.check(lib.kth_init(0))
