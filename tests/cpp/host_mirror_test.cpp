@@ -202,6 +202,29 @@ int main() {
         for (size_t i = 0; i < xs.size(); i++) if (cv[i] != xs[i] || pv[i] != xs[i] || xv[i] != 2.0f * xs[i]) kept = false;
         expect(kept, "copy() and pow(1) keep the source's values when the source is written afterwards");
     }
+    {
+        // The chain of the autograd reduce-to-shape ([64,40,100] -> [64,100] -> [64], each intermediate released after the
+        // next sum, Utils.kt:26-38): whole numbers, so that every order of adding gives the same float. The library puts
+        // the first sum off and runs both in the second call's launch; the source may be written or released in between.
+        auto gc = ops.garbageCollector();
+        Raw x = ops.createRaw({64, 40, 100}, [](int i) { return static_cast<float>(i % 7 - 3); });
+        const std::vector<float> xs = x->toVector();
+        std::vector<float> rows(64 * 100, 0.0f), totals(64, 0.0f);
+        for (int o = 0; o < 64; o++)
+            for (int a = 0; a < 40; a++)
+                for (int i = 0; i < 100; i++) {
+                    rows[static_cast<size_t>(o * 100 + i)] += xs[static_cast<size_t>((o * 40 + a) * 100 + i)];
+                    totals[static_cast<size_t>(o)] += xs[static_cast<size_t>((o * 40 + a) * 100 + i)];
+                }
+        Raw first = x->sum(1, false);
+        Raw second = first->sum(1, false);
+        first->release();
+        expect(second->toVector() == totals, "two steps of a reduce-to-shape chain");
+        Raw kept = x->sum(1, false);
+        x->timesAssign(0.0f);                           // the sum is that of the values at the call
+        x->release();
+        expect(kept->toVector() == rows, "a sum whose source is written and released before anybody reads it");
+    }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed == 0 ? 0 : 1;
 }
