@@ -136,3 +136,29 @@ def test_cfg4_chains_take_three_launches_each(gc):
         x64 = x.astype(np.float64)
         ref = x64.sum((0, 2, 3)) if op == "sum" else x64.mean((0, 2, 3))
         assert np.allclose(got.reshape(-1), ref, rtol=1e-5)
+
+
+def test_the_entry_point_that_allocates_nothing_puts_nothing_off(gc):
+    """kth_reduce_axis_static launches at once, and an input that is still owed its sum has it launched first: the
+    values are those of the plain entry point either way."""
+    from kten_amd.abi import Op, check
+    shape = [128, 56, 56]
+    x = data(shape, 7)
+    t = gc.createRaw(shape, x)
+    mid = t.sum(1)
+    mid_values = mid.toArray()
+    want = mid.sum(1).toArray()
+    # an owed input
+    owed = t.sum(1)
+    out = gc.createRaw([128])
+    before = launches(gc)
+    check(gc.lib.kth_reduce_axis_static(Op.SUM, owed.storeReference, out.storeReference, 128, 56, 1))
+    assert launches(gc) == before + 2, "the owed sum, then this one"
+    assert_bits_equal(out.toArray(), want, "static entry over an owed input")
+    assert_bits_equal(owed.toArray(), mid_values, "the input afterwards")
+    # a geometry that the plain entry point would put off
+    out2 = gc.createRaw([128, 56])
+    before = launches(gc)
+    check(gc.lib.kth_reduce_axis_static(Op.SUM, t.storeReference, out2.storeReference, 128, 56, 56))
+    assert launches(gc) == before + 1
+    assert_bits_equal(out2.toArray(), mid_values, "static entry, first step")
