@@ -525,14 +525,16 @@ __global__ __launch_bounds__(kBlock) void binary_bcast_vec_kernel(const float* _
         n4 = min(n4, rep * pl.slice + pl.slice);             // the tile ends with its slice
     }
     float4 va[kBcastUnroll], vb[kBcastUnroll];
+    // an operand of a small tensor (under 32 MB) is worth keeping in the caches: whoever made it or reads it next is near
+    const bool big = n4 >= (2u << 20);
 #pragma unroll
     for (int k = 0; k < kBcastUnroll; k++) {
         uint32_t i = base + k * kBlock;
         if (i < n4) {
             uint32_t ao, bo;
             decompose(pl, i, ao, bo);
-            va[k] = ld_operand<AV>(a, ao, pl.a_stream);
-            vb[k] = ld_operand<BV>(b, bo, pl.b_stream);
+            va[k] = ld_operand<AV>(a, ao, pl.a_stream && big);
+            vb[k] = ld_operand<BV>(b, bo, pl.b_stream && big);
         }
     }
 #pragma unroll
