@@ -90,6 +90,9 @@ def make_step(name, ops, inputs):
     for r in resident.values():
         r.incrementRef()
 
+    from kten_amd.host_mirror.autograd import NoGradVariable
+    by_identity = {id(v): resident[k] for k, v in inputs.items()}
+
     class Resident:
         """Hands the workload tensors that are already on the device."""
         def __init__(self, ops):
@@ -97,11 +100,7 @@ def make_step(name, ops, inputs):
         def __getattr__(self, k):
             return getattr(self.ops, k)
         def create(self, shape, requiresGrad, init):
-            from kten_amd.host_mirror.autograd import NoGradVariable
-            for key, v in inputs.items():
-                if v is init:
-                    return NoGradVariable(self.ops, resident[key])
-            raise KeyError("unknown input")
+            return NoGradVariable(self.ops, by_identity[id(init)])      # (KeyError: not one of the workload's inputs)
 
     proxy = Resident(ops)
 
